@@ -1,0 +1,173 @@
+"""hipcc -> gfx950 code-object cache.
+
+Stands where the reference calls triton.compile on generated source and keeps
+the result next to the source file (reference
+inductor_x/npu_triton_heuristics.py:111-199, 302-393).  A code object is keyed
+by a hash of the translation unit, the device headers it includes and the
+compiler flags.  Lookups go first to the in-tree store that ships with the
+package (filled ahead of time), then to a per-user store; a miss runs hipcc
+under a per-key file lock so concurrent compile workers do not race.
+"""
+from __future__ import annotations
+
+import fcntl
+import hashlib
+import os
+import shutil
+import subprocess
+import tempfile
+from typing import Iterable, Optional
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC_DIR = os.path.join(_HERE, "csrc")
+HEADER_DIR = os.path.join(CSRC_DIR, "mi")
+AOT_DIR = os.path.join(CSRC_DIR, "aot")
+INTREE_STORE = os.path.join(_HERE, "_hsaco")
+
+ARCH = "gfx950"
+# Packed-fp32 instruction selection is switched off for every device compile.
+HIPCC_FLAGS = (
+    "-O3",
+    f"--offload-arch={ARCH}",
+    "--genco",
+    "-std=c++17",
+    "-Xclang",
+    "-target-feature",
+    "-Xclang",
+    "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+)
+
+
+class CompileError(RuntimeError):
+    pass
+
+
+def hipcc_path() -> str:
+    cand = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(cand):
+        raise CompileError("hipcc not found; cannot build gfx950 code objects")
+    return cand
+
+
+def _headers_digest() -> str:
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(HEADER_DIR)):
+        if name.endswith(".h"):
+            with open(os.path.join(HEADER_DIR, name), "rb") as f:
+                h.update(name.encode())
+                h.update(f.read())
+    return h.hexdigest()
+
+
+_headers_digest_cache: Optional[str] = None
+
+
+def source_key(source: str, extra_flags: Iterable[str] = ()) -> str:
+    global _headers_digest_cache
+    if _headers_digest_cache is None:
+        _headers_digest_cache = _headers_digest()
+    h = hashlib.sha256()
+    h.update(_headers_digest_cache.encode())
+    h.update("\0".join(HIPCC_FLAGS + tuple(extra_flags)).encode())
+    h.update(source.encode())
+    return h.hexdigest()[:32]
+
+
+def user_store() -> str:
+    base = os.environ.get("INDUCTOR_X_AMD_CACHE") or os.path.join(
+        os.environ.get("XDG_CACHE_HOME", os.path.join(os.path.expanduser("~"), ".cache")), "inductor_x_amd"
+    )
+    return base
+
+
+def _stores() -> list[str]:
+    return [INTREE_STORE, user_store()]
+
+
+def lookup(key: str) -> Optional[str]:
+    for d in _stores():
+        p = os.path.join(d, key + ".hsaco")
+        if os.path.exists(p) and os.path.getsize(p) > 0:
+            return p
+    return None
+
+
+def _writable_store(prefer_intree: bool) -> str:
+    order = [INTREE_STORE, user_store()] if prefer_intree else [user_store(), INTREE_STORE]
+    for d in order:
+        try:
+            os.makedirs(d, exist_ok=True)
+            probe = os.path.join(d, f".w{os.getpid()}")
+            with open(probe, "w"):
+                pass
+            os.unlink(probe)
+            return d
+        except OSError:
+            continue
+    return tempfile.mkdtemp(prefix="inductor_x_amd_")
+
+
+def compile_source(
+    source: str,
+    label: str = "kernel",
+    extra_flags: Iterable[str] = (),
+    prefer_intree: bool = False,
+    force: bool = False,
+    include_dir: Optional[str] = None,
+) -> str:
+    """Return the path of the code object for `source`, compiling on a miss.
+
+    `source` may #include "mi/<header>.h".  Raises CompileError with the
+    compiler's stderr when hipcc fails.
+    """
+    extra_flags = tuple(extra_flags)
+    key = source_key(source, extra_flags)
+    if not force:
+        hit = lookup(key)
+        if hit:
+            return hit
+    store = _writable_store(prefer_intree)
+    out = os.path.join(store, key + ".hsaco")
+    lock_path = os.path.join(store, key + ".lock")
+    with open(lock_path, "w") as lock:
+        fcntl.flock(lock, fcntl.LOCK_EX)
+        try:
+            if not force and os.path.exists(out) and os.path.getsize(out) > 0:
+                return out
+            with tempfile.TemporaryDirectory(prefix="mi_hipcc_") as tmp:
+                src = os.path.join(tmp, f"{label}.hip")
+                with open(src, "w") as f:
+                    f.write(source)
+                tmp_out = os.path.join(tmp, "out.hsaco")
+                cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, "-I", include_dir or CSRC_DIR, "-o", tmp_out, src]
+                proc = subprocess.run(cmd, capture_output=True, text=True)
+                if proc.returncode != 0 or not os.path.exists(tmp_out):
+                    raise CompileError(f"hipcc failed for {label} (key {key}):\n{proc.stderr[-4000:]}")
+                final_tmp = out + f".tmp{os.getpid()}"
+                shutil.copyfile(tmp_out, final_tmp)
+                os.replace(final_tmp, out)
+            with open(os.path.join(store, key + ".txt"), "w") as f:
+                f.write(label + "\n")
+            return out
+        finally:
+            fcntl.flock(lock, fcntl.LOCK_UN)
+
+
+def aot_source(name: str) -> str:
+    """Text of one of the hand-written instantiation files under csrc/aot,
+    with its relative includes rewritten to the include root."""
+    with open(os.path.join(AOT_DIR, name)) as f:
+        return f.read().replace('#include "../mi/', '#include "mi/')
+
+
+def aot_files() -> list[str]:
+    return sorted(n for n in os.listdir(AOT_DIR) if n.endswith(".hip"))
+
+
+def build_aot(force: bool = True) -> dict[str, str]:
+    """Compile every file of csrc/aot into the in-tree store."""
+    out = {}
+    for name in aot_files():
+        out[name] = compile_source(aot_source(name), label=name[:-4], prefer_intree=True, force=force)
+    return out

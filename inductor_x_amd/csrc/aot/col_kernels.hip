@@ -1,0 +1,41 @@
+// Split column reduction for the third benchmark graph: per-column mean,
+// variance (correction given at run time) and int64 argmax over dim 0 of an fp32
+// matrix, in one sweep over the input plus a small combine pass.
+#include "../mi/col.h"
+
+using namespace mi;
+
+// Dynamic LDS for pass 1: (RL / 2) * CT * 4 * 5 floats (0 when RL == 1).
+#define COL_PARTIAL_VARIANT(CT, RL, UNROLL)                                                   \
+  extern "C" __global__ __launch_bounds__(CT* RL) void                                        \
+      col_mean_var_argmax_partial_f32_c##CT##_r##RL##_u##UNROLL(                              \
+          const float* x, float* part, int rows, int cols, int rows_per_split, int nsplit) {  \
+    col_stats_partial<CT, RL, UNROLL>(x, part, rows, cols, rows_per_split, nsplit);           \
+  }
+
+COL_PARTIAL_VARIANT(128, 2, 4)
+COL_PARTIAL_VARIANT(128, 2, 8)
+COL_PARTIAL_VARIANT(128, 4, 4)
+COL_PARTIAL_VARIANT(128, 4, 8)
+COL_PARTIAL_VARIANT(128, 8, 4)
+COL_PARTIAL_VARIANT(128, 8, 8)
+COL_PARTIAL_VARIANT(64, 4, 4)
+COL_PARTIAL_VARIANT(64, 4, 8)
+COL_PARTIAL_VARIANT(64, 8, 4)
+COL_PARTIAL_VARIANT(64, 16, 4)
+COL_PARTIAL_VARIANT(64, 1, 8)
+COL_PARTIAL_VARIANT(16, 16, 4)
+COL_PARTIAL_VARIANT(1, 64, 4)
+
+#define COL_FINAL_VARIANT(CPW, SL)                                                            \
+  extern "C" __global__ __launch_bounds__(CPW* SL) void                                       \
+      col_mean_var_argmax_final_f32_c##CPW##_s##SL(const float* part, float* mean_out,        \
+                                                   float* var_out, long long* argmax_out,     \
+                                                   int cols, int nsplit, float correction) {  \
+    col_stats_final<CPW, SL>(part, mean_out, var_out, argmax_out, cols, nsplit, correction);  \
+  }
+
+COL_FINAL_VARIANT(16, 16)
+COL_FINAL_VARIANT(8, 32)
+COL_FINAL_VARIANT(4, 64)
+COL_FINAL_VARIANT(64, 4)

@@ -1,0 +1,251 @@
+// Column ("higher-order") reductions: the reduced axis is the strided outer
+// axis and the kept axis is contiguous
+// (reference inductor_x/codegen/triton.py:1003-1031 for the classification,
+// reference inductor_x/codegen/split_tiling.py:159-165 for the case this file
+// is built for: a reduced axis longer than 32768 that has to be cut across
+// cores).
+//
+// Two-pass workgroup-partial scheme, no atomics:
+//   pass 1  grid (column tiles, SPLITS).  A workgroup owns CT*4 columns and
+//           one slice of rows; thread (ct, rl) walks rows rl, rl+RL, ... of the
+//           slice with float4 loads, so a wavefront reads 1 KiB runs.  Row
+//           lanes are folded through LDS and one partial per (split, column)
+//           goes to a workspace.
+//   pass 2  folds the SPLITS partials of each column.
+// One sweep produces mean, variance and argmax together, so the input is read
+// from HBM exactly once.
+//
+// Variance: each thread accumulates sums of (x - c) and (x - c)^2 with c its
+// first sample, turns them into (n, mean, M2) and every further merge uses
+// Chan's formula.  That is the two-pass definition the reference lowers to
+// (reference inductor_x/lowering.py:270-293) computed without a second read.
+// Argmax follows maximum_with_index: greater wins, NaN beats numbers, ties keep
+// the lower row (reference inductor_x/codegen/triton.py:1217-1233).
+#pragma once
+
+#include "common.h"
+
+namespace mi {
+
+constexpr int kColFields = 5;  // n, mean, m2, best value, best row (int bits)
+
+struct ColState {
+  Moments m;
+  ArgVal a;
+};
+
+__device__ __forceinline__ ColState col_state_empty() {
+  ColState s;
+  s.m.n = 0.f;
+  s.m.mean = 0.f;
+  s.m.m2 = 0.f;
+  s.a.v = -__builtin_inff();
+  s.a.i = 0x7fffffff;
+  return s;
+}
+
+__device__ __forceinline__ ColState col_state_combine(const ColState& a, const ColState& b) {
+  ColState r;
+  r.m = moments_combine(a.m, b.m);
+  r.a = arg_combine<true>(a.a, b.a);
+  return r;
+}
+
+// Fold the RL row lanes of a workgroup.  lds holds (RL/2) * CT * 4 * kColFields
+// floats.  On return the threads with rl == 0 hold the result.
+template <int CT, int RL>
+__device__ __forceinline__ void col_fold_row_lanes(ColState (&st)[4], int ct, int rl, float* lds) {
+  if constexpr (RL > 1) {
+    constexpr int PLANE = (RL / 2) * CT * 4;
+#pragma unroll
+    for (int half = RL / 2; half >= 1; half >>= 1) {
+      if (rl >= half && rl < 2 * half) {
+        const int slot = ((rl - half) * CT + ct) * 4;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          lds[0 * PLANE + slot + k] = st[k].m.n;
+          lds[1 * PLANE + slot + k] = st[k].m.mean;
+          lds[2 * PLANE + slot + k] = st[k].m.m2;
+          lds[3 * PLANE + slot + k] = st[k].a.v;
+          lds[4 * PLANE + slot + k] = __int_as_float(st[k].a.i);
+        }
+      }
+      __syncthreads();
+      if (rl < half) {
+        const int slot = (rl * CT + ct) * 4;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          ColState o;
+          o.m.n = lds[0 * PLANE + slot + k];
+          o.m.mean = lds[1 * PLANE + slot + k];
+          o.m.m2 = lds[2 * PLANE + slot + k];
+          o.a.v = lds[3 * PLANE + slot + k];
+          o.a.i = __float_as_int(lds[4 * PLANE + slot + k]);
+          st[k] = col_state_combine(st[k], o);
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// Pass 1.  Requires cols % 4 == 0 and x 16-byte aligned (checked by the host).
+// part is [kColFields][nsplit][cols] floats.
+template <int CT, int RL, int UNROLL>
+__device__ __forceinline__ void col_stats_partial(const float* __restrict__ x,
+                                                  float* __restrict__ part, int rows, int cols,
+                                                  int rows_per_split, int nsplit) {
+  extern __shared__ float lds_dyn[];
+  const int ct = threadIdx.x % CT;
+  const int rl = threadIdx.x / CT;
+  const int col = (blockIdx.x * CT + ct) * 4;
+  const int split = blockIdx.y;
+  const int r_begin = split * rows_per_split;
+  const int r_end = min(rows, r_begin + rows_per_split);
+  const bool live = col < cols;
+
+  ColState st[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) st[k] = col_state_empty();
+
+  int r = r_begin + rl;
+  if (live && r < r_end) {
+    const float* __restrict__ p = x + static_cast<size_t>(r) * cols + col;
+    const size_t step = static_cast<size_t>(RL) * cols;
+    const Vec<float, 4> first = load_vec<float, 4, true>(p);
+    float c[4], s1[4], s2[4], best[4];
+    int bi[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      c[k] = first[k];
+      s1[k] = 0.f;
+      s2[k] = 0.f;
+      best[k] = first[k];
+      bi[k] = r;
+    }
+    int cnt = 1;
+    r += RL;
+    p += step;
+    for (; r + (UNROLL - 1) * RL < r_end; r += UNROLL * RL, p += UNROLL * step) {
+      Vec<float, 4> v[UNROLL];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) v[u] = load_vec<float, 4, true>(p + u * step);
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const float xv = v[u][k];
+          const float d = xv - c[k];
+          s1[k] += d;
+          s2[k] = fmaf(d, d, s2[k]);
+          const bool upd = (xv > best[k]) || ((xv != xv) && (best[k] == best[k]));
+          best[k] = upd ? xv : best[k];
+          bi[k] = upd ? (r + u * RL) : bi[k];
+        }
+      }
+      cnt += UNROLL;
+    }
+    for (; r < r_end; r += RL, p += step) {
+      const Vec<float, 4> v = load_vec<float, 4, true>(p);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float xv = v[k];
+        const float d = xv - c[k];
+        s1[k] += d;
+        s2[k] = fmaf(d, d, s2[k]);
+        const bool upd = (xv > best[k]) || ((xv != xv) && (best[k] == best[k]));
+        best[k] = upd ? xv : best[k];
+        bi[k] = upd ? r : bi[k];
+      }
+      cnt += 1;
+    }
+    const float n = static_cast<float>(cnt);
+    const float inv_n = 1.0f / n;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      st[k].m.n = n;
+      st[k].m.mean = c[k] + s1[k] * inv_n;
+      // Clamp rounding noise below zero, but let NaN (from NaN or inf inputs) through.
+      const float m2 = s2[k] - s1[k] * s1[k] * inv_n;
+      st[k].m.m2 = (m2 < 0.f) ? 0.f : m2;
+      st[k].a.v = best[k];
+      st[k].a.i = bi[k];
+    }
+  }
+
+  col_fold_row_lanes<CT, RL>(st, ct, rl, lds_dyn);
+
+  if (live && rl == 0) {
+    const size_t plane = static_cast<size_t>(nsplit) * cols;
+    const size_t o = static_cast<size_t>(split) * cols + col;
+    Vec<float, 4> f0, f1, f2, f3, f4;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      f0[k] = st[k].m.n;
+      f1[k] = st[k].m.mean;
+      f2[k] = st[k].m.m2;
+      f3[k] = st[k].a.v;
+      f4[k] = __int_as_float(st[k].a.i);
+    }
+    store_vec<float, 4>(part + 0 * plane + o, f0);
+    store_vec<float, 4>(part + 1 * plane + o, f1);
+    store_vec<float, 4>(part + 2 * plane + o, f2);
+    store_vec<float, 4>(part + 3 * plane + o, f3);
+    store_vec<float, 4>(part + 4 * plane + o, f4);
+  }
+}
+
+// Pass 2.  A workgroup of CPW * SL threads finishes CPW columns; thread
+// (c, sl) folds splits sl, sl+SL, ... in increasing order, then the SL lanes are
+// folded through LDS (CPW * SL * kColFields floats, static).
+template <int CPW, int SL>
+__device__ __forceinline__ void col_stats_final(const float* __restrict__ part,
+                                                float* __restrict__ mean_out,
+                                                float* __restrict__ var_out,
+                                                long long* __restrict__ argmax_out, int cols,
+                                                int nsplit, float correction) {
+  __shared__ float lds[kColFields * CPW * SL];
+  const int c = threadIdx.x % CPW;
+  const int sl = threadIdx.x / CPW;
+  const int col = blockIdx.x * CPW + c;
+  const size_t plane = static_cast<size_t>(nsplit) * cols;
+  ColState st = col_state_empty();
+  if (col < cols) {
+    for (int s = sl; s < nsplit; s += SL) {
+      const size_t o = static_cast<size_t>(s) * cols + col;
+      ColState b;
+      b.m.n = part[0 * plane + o];
+      b.m.mean = part[1 * plane + o];
+      b.m.m2 = part[2 * plane + o];
+      b.a.v = part[3 * plane + o];
+      b.a.i = __float_as_int(part[4 * plane + o]);
+      st = col_state_combine(st, b);
+    }
+  }
+  constexpr int PLANE = CPW * SL;
+  lds[0 * PLANE + threadIdx.x] = st.m.n;
+  lds[1 * PLANE + threadIdx.x] = st.m.mean;
+  lds[2 * PLANE + threadIdx.x] = st.m.m2;
+  lds[3 * PLANE + threadIdx.x] = st.a.v;
+  lds[4 * PLANE + threadIdx.x] = __int_as_float(st.a.i);
+  __syncthreads();
+  if (sl == 0 && col < cols) {
+#pragma unroll
+    for (int j = 1; j < SL; ++j) {
+      const int t = j * CPW + c;
+      ColState b;
+      b.m.n = lds[0 * PLANE + t];
+      b.m.mean = lds[1 * PLANE + t];
+      b.m.m2 = lds[2 * PLANE + t];
+      b.a.v = lds[3 * PLANE + t];
+      b.a.i = __float_as_int(lds[4 * PLANE + t]);
+      st = col_state_combine(st, b);
+    }
+    mean_out[col] = st.m.mean;
+    const float denom = fmaxf(st.m.n - correction, 0.f);
+    var_out[col] = st.m.m2 / denom;
+    argmax_out[col] = static_cast<long long>(st.a.i);
+  }
+}
+
+}  // namespace mi

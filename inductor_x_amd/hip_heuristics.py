@@ -1,0 +1,392 @@
+"""Launch-time side of the backend: launch configurations, the caching
+launcher, grid computation and the CU/occupancy-aware split heuristic.
+
+Counterpart of the reference's launch heuristics module
+(reference inductor_x/npu_triton_heuristics.py):
+  NPUCachingAutotuner.precompile / _precompile_config (:71-266) -> CachingLauncher
+  cached_autotune + .best_config file (:302-435)                -> CachingLauncher.autotune
+  NPUDebugAutotuner bandwidth print (:268-299)                  -> config.profile_bandwidth
+  grid(*numels) (:444-464)                                      -> grid()
+  triton_config_npu_index (:467-544)                            -> *_configs()
+and of the split / tile choosers
+(reference inductor_x/codegen/split_tiling.py:46-182,
+ reference inductor_x/codegen/tile_generator.py:24-130)        -> split_reduction_plan(),
+                                                                   row_reduction_plan(), ...
+The reference sizes everything for `num_vector_core` persistent programs of one
+"warp"; here the unit is a 64-lane wavefront, a CU holds many of them, and the
+aim is enough 16-byte loads in flight per CU to cover HBM latency.
+"""
+from __future__ import annotations
+
+import dataclasses
+import hashlib
+import json
+import logging
+import os
+from typing import Callable, Optional, Sequence
+
+from . import codecache, config, launcher
+
+log = logging.getLogger(__name__)
+
+
+def cdiv(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+def next_power_of_2(n: int) -> int:
+    n = max(int(n), 1)
+    return 1 << (n - 1).bit_length()
+
+
+def prev_power_of_2(n: int) -> int:
+    n = max(int(n), 1)
+    return 1 << (n.bit_length() - 1)
+
+
+# ---------------------------------------------------------------------------
+# Launch configuration and caching launcher
+# ---------------------------------------------------------------------------
+@dataclasses.dataclass
+class LaunchConfig:
+    """One way to run a kernel: which symbol, workgroup shape, how the grid and
+    the dynamic LDS size follow from the call's numels.  `meta` carries the
+    compile-time parameters the symbol was instantiated with (the analogue of a
+    Triton Config's kwargs, e.g. XBLOCK / RBLOCK in the reference)."""
+
+    symbol: str
+    block: int
+    meta: dict = dataclasses.field(default_factory=dict)
+    defines: dict = dataclasses.field(default_factory=dict)
+    lds_bytes: int = 0
+
+    def key(self) -> str:
+        return json.dumps([self.symbol, self.block, self.meta, self.defines, self.lds_bytes], sort_keys=True)
+
+
+def grid(*numels: int) -> Callable[[dict], tuple]:
+    """grid(numel0[, numel1[, numel2]]) -> fn(meta) -> (g0, g1, g2).
+
+    Same call shape as the reference's helper
+    (reference inductor_x/npu_triton_heuristics.py:444-464).  Axis k is covered
+    by cdiv(numel_k, meta["PER_WG<k>"]) workgroups (PER_WG defaults to 1)."""
+
+    def fn(meta: dict) -> tuple:
+        g = [1, 1, 1]
+        for k, n in enumerate(numels[:3]):
+            per = int(meta.get(f"PER_WG{k}", 1))
+            g[k] = max(cdiv(int(n), per), 1)
+        return tuple(g)
+
+    return fn
+
+
+class CachingLauncher:
+    """Compiles (or fetches) a kernel's code object, keeps the usable launch
+    configurations, optionally times them once, and launches the chosen one.
+
+    Behaviour carried over from the reference's NPUCachingAutotuner:
+      - configs are tried in order and those that fail to build or resolve are
+        dropped; it is an error only if none survive (:71-107);
+      - with more than one survivor and autotuning on, each is timed on the
+        first call and the winner is remembered in a `.best_config` JSON next to
+        the code object (:372-390);
+      - run(*args, grid=, stream=) enqueues on the given raw stream and never
+        synchronises (:239-253).
+    """
+
+    def __init__(
+        self,
+        name: str,
+        source: str,
+        signature: str,
+        configs: Sequence[LaunchConfig],
+        bytes_fn: Optional[Callable[..., int]] = None,
+        prefer_intree: bool = False,
+    ):
+        self.name = name
+        self.source = source
+        self.signature = signature
+        self.configs = list(configs)
+        self.bytes_fn = bytes_fn
+        self.prefer_intree = prefer_intree
+        self.launchers: list[tuple[LaunchConfig, launcher.Function]] = []
+        self._best: Optional[int] = None
+        self._modules: dict[str, launcher.Module] = {}
+        self._hsaco_path: Optional[str] = None
+
+    # -- compile / load ----------------------------------------------------
+    def _module_for(self, cfg: LaunchConfig) -> launcher.Module:
+        flags = tuple(f"-D{k}={v}" for k, v in sorted(cfg.defines.items()))
+        key = "|".join(flags)
+        mod = self._modules.get(key)
+        if mod is None:
+            path = codecache.compile_source(
+                self.source, label=self.name, extra_flags=flags, prefer_intree=self.prefer_intree
+            )
+            self._hsaco_path = path
+            with open(path, "rb") as f:
+                mod = launcher.Module(f.read(), label=f"{self.name}[{os.path.basename(path)}]")
+            self._modules[key] = mod
+        return mod
+
+    def precompile(self) -> None:
+        if self.launchers:
+            return
+        errors = []
+        for cfg in self.configs:
+            try:
+                fn = self._module_for(cfg).function(cfg.symbol)
+            except (codecache.CompileError, launcher.LauncherError) as e:
+                errors.append(f"{cfg.symbol}: {e}")
+                log.debug("dropping launch config %s of %s: %s", cfg.symbol, self.name, e)
+                continue
+            self.launchers.append((cfg, fn))
+        if not self.launchers:
+            raise RuntimeError(f"No valid launch configuration for kernel {self.name}:\n" + "\n".join(errors))
+        if len(self.launchers) == 1:
+            self._best = 0
+        else:
+            self._best = self._load_best()
+
+    # -- best-config persistence ------------------------------------------
+    def _configs_hash(self) -> str:
+        h = hashlib.sha256()
+        for cfg in self.configs:
+            h.update(cfg.key().encode())
+        return h.hexdigest()[:16]
+
+    def _best_path(self) -> Optional[str]:
+        return (self._hsaco_path[: -len(".hsaco")] + ".best_config") if self._hsaco_path else None
+
+    def _load_best(self) -> Optional[int]:
+        p = self._best_path()
+        if not p or not os.path.exists(p):
+            return None
+        try:
+            with open(p) as f:
+                rec = json.load(f)
+        except (OSError, ValueError):
+            return None
+        if rec.get("configs_hash") != self._configs_hash():
+            return None
+        for i, (cfg, _) in enumerate(self.launchers):
+            if cfg.symbol == rec.get("symbol") and cfg.defines == rec.get("defines", {}):
+                return i
+        return None
+
+    def _save_best(self, idx: int, timings_ms: dict) -> None:
+        p = self._best_path()
+        if not p:
+            return
+        cfg = self.launchers[idx][0]
+        rec = {
+            "symbol": cfg.symbol,
+            "block": cfg.block,
+            "defines": cfg.defines,
+            **cfg.meta,
+            "configs_hash": self._configs_hash(),
+            "timings_ms": timings_ms,
+        }
+        try:
+            with open(p, "w") as f:
+                json.dump(rec, f)
+        except OSError:
+            pass
+
+    # -- launch -------------------------------------------------------------
+    def _launch(self, idx: int, args, grid_arg, stream: int) -> None:
+        cfg, fn = self.launchers[idx]
+        g = grid_arg(cfg.meta) if callable(grid_arg) else grid_arg
+        fn.launch(self.signature, args, g, (cfg.block,), stream, cfg.lds_bytes)
+
+    def bench(self, idx: int, args, grid_arg, stream: int, warmup: int = 3, rep: int = 10) -> float:
+        """Average milliseconds per launch of configuration idx, timed with
+        events on torch's current stream (which must be `stream`)."""
+        import torch
+
+        for _ in range(warmup):
+            self._launch(idx, args, grid_arg, stream)
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(rep):
+            self._launch(idx, args, grid_arg, stream)
+        end.record()
+        end.synchronize()
+        return start.elapsed_time(end) / rep
+
+    def autotune(self, args, grid_arg, stream: int) -> int:
+        timings = {}
+        best, best_ms = 0, float("inf")
+        for i, (cfg, _) in enumerate(self.launchers):
+            try:
+                ms = self.bench(i, args, grid_arg, stream)
+            except launcher.LauncherError as e:
+                log.debug("config %s of %s failed to launch: %s", cfg.symbol, self.name, e)
+                continue
+            timings[cfg.symbol] = ms
+            if ms < best_ms:
+                best, best_ms = i, ms
+        self._save_best(best, timings)
+        return best
+
+    def run(self, *args, grid, stream: int) -> None:
+        if not self.launchers:
+            self.precompile()
+        if self._best is None:
+            self._best = self.autotune(args, grid, stream) if config.autotune else 0
+        self._launch(self._best, args, grid, stream)
+        if config.profile_bandwidth and self.bytes_fn is not None:
+            ms = self.bench(self._best, args, grid, stream, warmup=1, rep=5)
+            nbytes = self.bytes_fn(*args)
+            print(f"{self.name}: {ms:.4f} ms  {nbytes / 1e9:.4f} GB  {nbytes / 1e6 / ms:.1f} GB/s")
+
+    def select(self, symbol: str) -> None:
+        """Pin the configuration with the given symbol (used by sweeps and tests)."""
+        if not self.launchers:
+            self.precompile()
+        for i, (cfg, _) in enumerate(self.launchers):
+            if cfg.symbol == symbol:
+                self._best = i
+                return
+        raise KeyError(f"{self.name}: no launch configuration {symbol}")
+
+    def best_config(self) -> LaunchConfig:
+        if not self.launchers:
+            self.precompile()
+        return self.launchers[self._best or 0][0]
+
+
+# ---------------------------------------------------------------------------
+# Heuristics
+# ---------------------------------------------------------------------------
+def vector_width(elem_bytes: int, *extents_and_strides: int) -> int:
+    """Largest element count per lane access (<= 16 bytes) that divides every
+    given extent/stride/offset, so every vector stays aligned and in range.
+    Counterpart of the reference's 32-byte block alignment rule
+    (reference inductor_x/codegen/triton_utils.py:22-27)."""
+    vec = max(config.vector_bytes // elem_bytes, 1)
+    while vec > 1 and any(int(e) % vec for e in extents_and_strides):
+        vec //= 2
+    return vec
+
+
+# Bytes a CU wants in flight to cover HBM latency at full bandwidth:
+# 8 TB/s * ~2 us / 256 CUs.
+_BYTES_IN_FLIGHT_PER_CU = 64 * 1024
+
+
+def waves_per_cu_target(unroll: int, vgprs: int = 64, hw: Optional[config.Hardware] = None) -> int:
+    """Resident wavefronts per CU needed so that waves * 64 lanes * 16 B * unroll
+    covers the in-flight byte target, capped by what the register file allows."""
+    hw = hw or config.hardware()
+    need = cdiv(_BYTES_IN_FLIGHT_PER_CU, hw.wave_size * config.vector_bytes * max(unroll, 1))
+    reg_limit = max(hw.regs_per_simd // max(vgprs, 1), 1) * hw.simds_per_cu
+    return max(min(need, reg_limit, hw.max_waves_per_cu), 1)
+
+
+@dataclasses.dataclass(frozen=True)
+class RowPlan:
+    block: int  # threads per workgroup
+    tpr: int  # threads cooperating on one row
+    vec: int  # elements per lane access
+    iters: int  # vectors per thread (persistent form) or 0 (looped form)
+    rows_per_wg: int
+
+
+def row_reduction_plan(xnumel: int, rnumel: int, elem_bytes: int, persistent: bool) -> RowPlan:
+    """Thread mapping for a last-dimension reduction.
+
+    One row gets as many threads as it has 16-byte vectors, up to a whole
+    256-thread workgroup; shorter rows share a workgroup so wavefronts stay
+    full.  Replaces the reference's XBLOCK / XBLOCK_SUB / RBLOCK sweep
+    (reference inductor_x/codegen/tile_generator.py:38-130)."""
+    vec = vector_width(elem_bytes, rnumel)
+    vectors = cdiv(rnumel, vec)
+    block = 256
+    tpr = min(next_power_of_2(vectors), block)
+    # Long rows in the persistent form: keep at most 4 vectors per thread per input.
+    if persistent:
+        while cdiv(vectors, tpr) > 4 and tpr < 1024:
+            tpr *= 2
+        block = max(block, tpr)
+    iters = cdiv(vectors, tpr) if persistent else 0
+    return RowPlan(block=block, tpr=tpr, vec=vec, iters=iters, rows_per_wg=block // tpr)
+
+
+@dataclasses.dataclass(frozen=True)
+class SplitPlan:
+    ct: int  # threads across the kept (contiguous) axis, 4 elements each
+    rl: int  # row lanes per workgroup
+    unroll: int
+    nsplit: int  # workgroups along the reduced axis
+    rows_per_split: int
+    col_tiles: int
+
+    @property
+    def block(self) -> int:
+        return self.ct * self.rl
+
+    @property
+    def lds_bytes(self) -> int:
+        return (self.rl // 2) * self.ct * 4 * 5 * 4
+
+    def workspace_floats(self, cols: int) -> int:
+        return 5 * self.nsplit * cols
+
+
+def split_reduction_plan(
+    rows: int,
+    cols: int,
+    elem_bytes: int = 4,
+    vgprs: int = 48,
+    unroll: int = 4,
+    hw: Optional[config.Hardware] = None,
+    max_workspace_frac: float = 0.05,
+) -> SplitPlan:
+    """CU/occupancy-aware split factor for a column reduction (rows reduced,
+    cols kept and contiguous).
+
+    The reference cuts the reduced axis only above 32768 elements and then into
+    about one slice per vector core (reference
+    inductor_x/codegen/split_tiling.py:159-182).  Here:
+      1. a workgroup spans up to 512 kept elements (128 threads x float4) and
+         as many row lanes as fit in 1024 threads - big workgroups mean few
+         partials, so little workspace traffic;
+      2. the number of wavefronts wanted per CU comes from the in-flight-bytes
+         target and the kernel's register budget (waves_per_cu_target);
+      3. nsplit is the smallest count that gives every CU that many wavefronts,
+         rounded to a multiple of the CU count so the last round of workgroups
+         is full, then capped so that writing and re-reading the partials stays
+         below `max_workspace_frac` of the input bytes and every thread keeps at
+         least one unrolled batch of rows;
+      4. rows_per_split is rounded up to a whole number of unrolled batches.
+    """
+    hw = hw or config.hardware()
+    vec = 4
+    ct = min(next_power_of_2(cdiv(cols, vec)), 128)
+    col_tiles = cdiv(cols, ct * vec)
+    rl = max(min(1024 // ct, prev_power_of_2(max(rows // unroll, 1))), 1)
+    waves_per_wg = max(ct * rl // hw.wave_size, 1)
+    want_waves = hw.cu_count * waves_per_cu_target(unroll, vgprs, hw)
+    nsplit = cdiv(want_waves, waves_per_wg * col_tiles)
+    if nsplit * col_tiles > hw.cu_count:
+        per = max(hw.cu_count // col_tiles, 1)
+        nsplit = cdiv(nsplit, per) * per
+    # workspace traffic cap: 2 * nsplit * cols * 20 B <= frac * rows * cols * elem_bytes
+    cap_ws = int(max_workspace_frac * rows * elem_bytes / 40)
+    # every thread should own at least one unrolled batch
+    cap_rows = rows // (rl * unroll)
+    nsplit = max(min(nsplit, max(cap_ws, 1), max(cap_rows, 1)), 1)
+    batch = rl * unroll
+    rows_per_split = cdiv(cdiv(rows, nsplit), batch) * batch
+    nsplit = cdiv(rows, rows_per_split)
+    return SplitPlan(ct=ct, rl=rl, unroll=unroll, nsplit=nsplit, rows_per_split=rows_per_split, col_tiles=col_tiles)
+
+
+def pointwise_plan(numel: int, elem_bytes: int, inner_extent: int) -> tuple[int, int]:
+    """(block, vec) for a flat pointwise kernel whose innermost contiguous run is
+    `inner_extent` elements long."""
+    vec = vector_width(elem_bytes, inner_extent, numel)
+    return 256, vec

@@ -1,0 +1,385 @@
+"""Host entry points of the hand-written kernel families.
+
+Each function checks shapes, dtypes, contiguity and alignment on the host (a
+kernel is never launched on operands it was not written for), picks a launch
+configuration with the heuristics, and enqueues through the C-ABI launcher on
+torch's current stream.  Outputs are allocated with torch; nothing here
+computes on the CPU and nothing falls back to eager PyTorch.
+
+The code objects come from csrc/aot/*.hip, compiled ahead of time into the
+in-tree store; a missing code object is compiled with hipcc on first use.
+"""
+from __future__ import annotations
+
+import functools
+import math
+from typing import Optional
+
+import torch
+
+from . import codecache, config
+from .hip_heuristics import (
+    CachingLauncher,
+    LaunchConfig,
+    cdiv,
+    next_power_of_2,
+    row_reduction_plan,
+    split_reduction_plan,
+    SplitPlan,
+)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _aligned(t: torch.Tensor, nbytes: int = 16) -> bool:
+    return t.data_ptr() % nbytes == 0
+
+
+def _check_cuda(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        _require(t.is_cuda, "tensor must live on the GPU")
+        _require(t.device == tensors[0].device, "tensors must share a device")
+
+
+# ---------------------------------------------------------------------------
+# code objects (one per aot file), loaded lazily
+# ---------------------------------------------------------------------------
+_ROWSUM_VARIANTS = [(256, 256), (256, 128), (256, 64), (512, 512), (1024, 1024)]
+_RMSNORM_VARIANTS = [
+    (256, 256, 2),
+    (256, 128, 4),
+    (256, 64, 8),
+    (512, 512, 1),
+    (256, 256, 1),
+    (256, 256, 4),
+    (256, 64, 1),
+    (256, 64, 2),
+    (256, 64, 4),
+]
+_COL_PARTIAL_VARIANTS = [
+    (128, 2, 4),
+    (128, 2, 8),
+    (128, 4, 4),
+    (128, 4, 8),
+    (128, 8, 4),
+    (128, 8, 8),
+    (64, 4, 4),
+    (64, 4, 8),
+    (64, 8, 4),
+    (64, 16, 4),
+    (64, 1, 8),
+    (16, 16, 4),
+    (1, 64, 4),
+]
+_COL_FINAL_VARIANTS = [(16, 16), (8, 32), (4, 64), (64, 4)]
+_GATHER_VARIANTS = [(256, 128, 1), (256, 128, 2), (256, 128, 4), (256, 64, 1), (256, 64, 2), (256, 64, 4), (256, 16, 1), (256, 16, 4)]
+_PERMUTE_VARIANTS = [
+    (256, 16, 32, 8),
+    (256, 16, 32, 4),
+    (256, 16, 32, 2),
+    (256, 16, 16, 8),
+    (256, 16, 8, 8),
+    (256, 16, 4, 16),
+    (256, 16, 1, 64),
+    (256, 16, 1, 128),
+    (256, 16, 1, 16),
+    (256, 16, 2, 8),
+    (256, 8, 1, 32),
+    (256, 4, 1, 64),
+    (256, 64, 1, 4),
+    (256, 64, 4, 4),
+]
+
+
+@functools.lru_cache(maxsize=None)
+def _rowsum_launcher() -> CachingLauncher:
+    cfgs = [
+        LaunchConfig(f"fused_relu_sigmoid_rowsum_f32_b{b}_t{t}", b, meta={"BLOCK": b, "TPR": t, "PER_WG0": b // t})
+        for b, t in _ROWSUM_VARIANTS
+    ]
+    return CachingLauncher(
+        "fused_relu_sigmoid_rowsum_f32", codecache.aot_source("row_kernels.hip"), "PPii", cfgs, prefer_intree=True
+    )
+
+
+@functools.lru_cache(maxsize=None)
+def _rmsnorm_launcher() -> CachingLauncher:
+    cfgs = [
+        LaunchConfig(
+            f"add_rmsnorm_bf16_b{b}_t{t}_i{i}", b, meta={"BLOCK": b, "TPR": t, "ITERS": i, "PER_WG0": b // t}
+        )
+        for b, t, i in _RMSNORM_VARIANTS
+    ]
+    return CachingLauncher(
+        "add_rmsnorm_bf16", codecache.aot_source("row_kernels.hip"), "PPPPPiif", cfgs, prefer_intree=True
+    )
+
+
+@functools.lru_cache(maxsize=None)
+def _col_partial_launcher() -> CachingLauncher:
+    cfgs = [
+        LaunchConfig(
+            f"col_mean_var_argmax_partial_f32_c{ct}_r{rl}_u{u}",
+            ct * rl,
+            meta={"CT": ct, "RL": rl, "UNROLL": u},
+            lds_bytes=(rl // 2) * ct * 4 * 5 * 4,
+        )
+        for ct, rl, u in _COL_PARTIAL_VARIANTS
+    ]
+    return CachingLauncher(
+        "col_mean_var_argmax_partial_f32", codecache.aot_source("col_kernels.hip"), "PPiiii", cfgs, prefer_intree=True
+    )
+
+
+@functools.lru_cache(maxsize=None)
+def _col_final_launcher() -> CachingLauncher:
+    cfgs = [
+        LaunchConfig(f"col_mean_var_argmax_final_f32_c{c}_s{s}", c * s, meta={"CPW": c, "SL": s})
+        for c, s in _COL_FINAL_VARIANTS
+    ]
+    return CachingLauncher(
+        "col_mean_var_argmax_final_f32", codecache.aot_source("col_kernels.hip"), "PPPPiif", cfgs, prefer_intree=True
+    )
+
+
+@functools.lru_cache(maxsize=None)
+def _gather_launcher() -> CachingLauncher:
+    cfgs = [
+        LaunchConfig(f"gather_rows_b16_b{b}_t{t}_r{r}", b, meta={"BLOCK": b, "TPR": t, "RPT": r})
+        for b, t, r in _GATHER_VARIANTS
+    ]
+    cfgs.append(LaunchConfig("gather_rows_b32_b256_t64_r2", 256, meta={"BLOCK": 256, "TPR": 64, "RPT": 2, "ELEM": 4}))
+    return CachingLauncher("gather_rows", codecache.aot_source("copy_kernels.hip"), "PPPiii", cfgs, prefer_intree=True)
+
+
+@functools.lru_cache(maxsize=None)
+def _permute_launcher() -> CachingLauncher:
+    cfgs = [
+        LaunchConfig(
+            f"permute_copy_b16_b{b}_p{p}_t{t1}x{t2}", b, meta={"BLOCK": b, "TPC": p, "T1": t1, "T2": t2}
+        )
+        for b, p, t1, t2 in _PERMUTE_VARIANTS
+    ]
+    cfgs.append(
+        LaunchConfig("permute_copy_b32_b256_p16_t8x8", 256, meta={"BLOCK": 256, "TPC": 16, "T1": 8, "T2": 8, "ELEM": 4})
+    )
+    return CachingLauncher(
+        "permute_copy", codecache.aot_source("copy_kernels.hip"), "PPiiiiqqq", cfgs, prefer_intree=True
+    )
+
+
+def _find(l: CachingLauncher, symbol: str) -> int:
+    l.precompile()
+    for i, (cfg, _) in enumerate(l.launchers):
+        if cfg.symbol == symbol:
+            return i
+    raise KeyError(f"{l.name}: no variant {symbol}")
+
+
+# ---------------------------------------------------------------------------
+# graph 1: y = sum(relu(2x+1) * sigmoid(x), -1), fp32
+# ---------------------------------------------------------------------------
+def fused_relu_sigmoid_rowsum(x: torch.Tensor, variant: Optional[tuple] = None) -> torch.Tensor:
+    _check_cuda(x)
+    _require(x.dtype == torch.float32 and x.dim() >= 1, "x must be fp32 with at least one dim")
+    _require(x.is_contiguous(), "x must be contiguous")
+    rnumel = x.shape[-1]
+    xnumel = x.numel() // max(rnumel, 1) if rnumel else 0
+    out = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
+    if xnumel == 0:
+        return out
+    if rnumel == 0:
+        return out.zero_()
+    _require(rnumel % 4 == 0 and _aligned(x), "row length must be a multiple of 4 and x 16-byte aligned")
+    _require(x.numel() < 2**31, "numel must fit int32 indexing")
+    l = _rowsum_launcher()
+    if variant is None:
+        plan = row_reduction_plan(xnumel, rnumel, 4, persistent=False)
+        variant = (plan.block, max(plan.tpr, 64))  # instantiated shapes start at one wavefront per row
+    b, t = variant
+    idx = _find(l, f"fused_relu_sigmoid_rowsum_f32_b{b}_t{t}")
+    l._launch(idx, (x.data_ptr(), out.data_ptr(), xnumel, rnumel), (cdiv(xnumel, b // t), 1, 1), _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
+# graph 2: s = h + r; out = s * rsqrt(mean(s^2, -1) + eps) * w   (bf16)
+# ---------------------------------------------------------------------------
+def add_rmsnorm(
+    h: torch.Tensor, r: torch.Tensor, w: torch.Tensor, eps: float = 1e-6, variant: Optional[tuple] = None
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """Returns (normed, h + r), both bf16."""
+    _check_cuda(h, r, w)
+    _require(h.dtype == r.dtype == w.dtype == torch.bfloat16, "h, r, w must be bf16")
+    _require(h.shape == r.shape and h.dim() >= 1, "h and r must have the same shape")
+    cols = h.shape[-1]
+    _require(w.shape == (cols,), "w must be a vector of the row length")
+    _require(h.is_contiguous() and r.is_contiguous() and w.is_contiguous(), "operands must be contiguous")
+    rows = h.numel() // max(cols, 1) if cols else 0
+    out = torch.empty_like(h)
+    s = torch.empty_like(h)
+    if rows == 0 or cols == 0:
+        return out, s
+    _require(cols % 8 == 0, "row length must be a multiple of 8")
+    _require(all(_aligned(t) for t in (h, r, w, out, s)), "operands must be 16-byte aligned")
+    l = _rmsnorm_launcher()
+    if variant is None:
+        plan = row_reduction_plan(rows, cols, 2, persistent=True)
+        tpr = max(plan.tpr, 64)  # instantiated shapes start at one wavefront per row
+        iters = next_power_of_2(cdiv(cdiv(cols, 8), tpr))
+        block = max(256, tpr)
+        _require(iters <= 8 and block <= 512, f"row length {cols} exceeds the persistent kernel's reach")
+        variant = (block, tpr, iters)
+        # map onto an instantiated variant
+        have = set(_RMSNORM_VARIANTS)
+        while variant not in have and variant[2] < 8:
+            variant = (variant[0], variant[1], variant[2] * 2)
+        _require(variant in have, f"no add_rmsnorm variant for row length {cols}")
+    b, t, i = variant
+    _require(cols <= t * 8 * i, "variant too small for the row length")
+    idx = _find(l, f"add_rmsnorm_bf16_b{b}_t{t}_i{i}")
+    l._launch(
+        idx,
+        (h.data_ptr(), r.data_ptr(), w.data_ptr(), out.data_ptr(), s.data_ptr(), rows, cols, float(eps)),
+        (cdiv(rows, b // t), 1, 1),
+        _stream(),
+    )
+    return out, s
+
+
+def _snap_split_plan(plan: SplitPlan, rows: int, cols: int) -> SplitPlan:
+    """Map a heuristic plan onto the nearest instantiated partial-kernel shape
+    (threads beyond the matrix edge idle, so a wider shape is always valid)."""
+    if (plan.ct, plan.rl, plan.unroll) in set(_COL_PARTIAL_VARIANTS):
+        return plan
+    avail_ct = sorted({v[0] for v in _COL_PARTIAL_VARIANTS})
+    ct = next((c for c in avail_ct if c >= plan.ct), avail_ct[-1])
+    cands = [v for v in _COL_PARTIAL_VARIANTS if v[0] == ct]
+    _, rl, u = min(cands, key=lambda v: (abs(v[1] - plan.rl), abs(v[2] - plan.unroll)))
+    batch = rl * u
+    rps = cdiv(max(plan.rows_per_split, 1), batch) * batch
+    return SplitPlan(ct, rl, u, cdiv(rows, rps), rps, cdiv(cols, ct * 4))
+
+
+
+# ---------------------------------------------------------------------------
+# graph 3: per-column mean, var, argmax over dim 0 (fp32 matrix)
+# ---------------------------------------------------------------------------
+def col_mean_var_argmax(
+    x: torch.Tensor,
+    correction: float = 0.0,
+    plan: Optional[SplitPlan] = None,
+    final_variant: tuple = (16, 16),
+    workspace: Optional[torch.Tensor] = None,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Returns (mean, var, argmax) over dim 0 of a [rows, cols] fp32 matrix."""
+    _check_cuda(x)
+    _require(x.dtype == torch.float32 and x.dim() == 2, "x must be a 2-D fp32 matrix")
+    _require(x.is_contiguous(), "x must be contiguous")
+    rows, cols = x.shape
+    _require(rows > 0, "argmax over an empty axis is undefined")
+    mean = torch.empty(cols, dtype=torch.float32, device=x.device)
+    var = torch.empty(cols, dtype=torch.float32, device=x.device)
+    arg = torch.empty(cols, dtype=torch.int64, device=x.device)
+    if cols == 0:
+        return mean, var, arg
+    _require(cols % 4 == 0 and _aligned(x), "cols must be a multiple of 4 and x 16-byte aligned")
+    _require(x.numel() < 2**31, "numel must fit int32 indexing")
+    if plan is None:
+        plan = _snap_split_plan(split_reduction_plan(rows, cols, 4), rows, cols)
+    _require(plan.rows_per_split * plan.nsplit >= rows, "split plan does not cover all rows")
+    _require(plan.col_tiles * plan.ct * 4 >= cols, "split plan does not cover all columns")
+    need = plan.workspace_floats(cols)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.float32, device=x.device)
+    _require(workspace.numel() >= need and workspace.dtype == torch.float32, "workspace too small")
+    lp, lf = _col_partial_launcher(), _col_final_launcher()
+    ip = _find(lp, f"col_mean_var_argmax_partial_f32_c{plan.ct}_r{plan.rl}_u{plan.unroll}")
+    cpw, sl = final_variant
+    jf = _find(lf, f"col_mean_var_argmax_final_f32_c{cpw}_s{sl}")
+    st = _stream()
+    lp._launch(
+        ip,
+        (x.data_ptr(), workspace.data_ptr(), rows, cols, plan.rows_per_split, plan.nsplit),
+        (plan.col_tiles, plan.nsplit, 1),
+        st,
+    )
+    lf._launch(
+        jf,
+        (workspace.data_ptr(), mean.data_ptr(), var.data_ptr(), arg.data_ptr(), cols, plan.nsplit, float(correction)),
+        (cdiv(cols, cpw), 1, 1),
+        st,
+    )
+    return mean, var, arg
+
+
+# ---------------------------------------------------------------------------
+# graph 4a: out = table[idx]
+# ---------------------------------------------------------------------------
+def gather_rows(table: torch.Tensor, idx: torch.Tensor, variant: Optional[tuple] = None) -> torch.Tensor:
+    _check_cuda(table, idx)
+    _require(table.dim() == 2 and table.is_contiguous(), "table must be a contiguous matrix")
+    _require(idx.dtype == torch.int64 and idx.is_contiguous(), "idx must be contiguous int64")
+    _require(table.element_size() in (2, 4), "gather kernels exist for 2- and 4-byte elements")
+    nrows, width = table.shape
+    out = torch.empty(idx.shape + (width,), dtype=table.dtype, device=table.device)
+    n = idx.numel()
+    if n == 0 or width == 0:
+        return out
+    _require(nrows > 0, "cannot gather from an empty table")
+    vec = 16 // table.element_size()
+    _require(width % vec == 0 and _aligned(table) and _aligned(out), "row bytes must be a multiple of 16")
+    _require(out.numel() < 2**31, "numel must fit int32 indexing")
+    l = _gather_launcher()
+    if table.element_size() == 4:
+        sym, (b, t, r) = "gather_rows_b32_b256_t64_r2", (256, 64, 2)
+    else:
+        if variant is None:
+            t = min(max(next_power_of_2(width // vec), 16), 128)
+            t = 128 if t > 64 else (64 if t > 16 else 16)
+            variant = (256, t, 2 if t >= 64 else 4)
+        b, t, r = variant
+        sym = f"gather_rows_b16_b{b}_t{t}_r{r}"
+    i = _find(l, sym)
+    rows_per_wg = (b // t) * r
+    l._launch(i, (table.data_ptr(), idx.data_ptr(), out.data_ptr(), n, width, nrows), (cdiv(n, rows_per_wg), 1, 1), _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
+# graph 4b: t.permute(0, 2, 1, 3).contiguous()
+# ---------------------------------------------------------------------------
+def permute_0213_contiguous(t: torch.Tensor, variant: Optional[tuple] = None) -> torch.Tensor:
+    """Contiguous copy of t.permute(0, 2, 1, 3) for a contiguous 4-D tensor."""
+    _check_cuda(t)
+    _require(t.dim() == 4 and t.is_contiguous(), "t must be a contiguous 4-D tensor")
+    _require(t.element_size() in (2, 4), "permute kernels exist for 2- and 4-byte elements")
+    n0, n2, n1, inner = t.shape  # output dims are (n0, n1, n2, inner)
+    out = torch.empty((n0, n1, n2, inner), dtype=t.dtype, device=t.device)
+    if out.numel() == 0:
+        return out
+    vec = 16 // t.element_size()
+    _require(inner % vec == 0 and _aligned(t) and _aligned(out), "inner run must be a multiple of 16 bytes")
+    _require(out.numel() < 2**31, "numel must fit int32 indexing")
+    s0, s2, s1, _ = t.stride()  # input strides of output axes a, b, c
+    l = _permute_launcher()
+    if t.element_size() == 4:
+        sym, (b, p, t1, t2) = "permute_copy_b32_b256_p16_t8x8", (256, 16, 8, 8)
+        _require(inner // vec <= 16, "inner run too long for the fp32 permute variant")
+    else:
+        if variant is None:
+            variant = (256, 16, 32, 4)
+        b, p, t1, t2 = variant
+        _require(inner // vec <= p, "inner run too long for this permute variant")
+        sym = f"permute_copy_b16_b{b}_p{p}_t{t1}x{t2}"
+    i = _find(l, sym)
+    tiles = n0 * cdiv(n1, t1) * cdiv(n2, t2)
+    l._launch(i, (t.data_ptr(), out.data_ptr(), n0, n1, n2, inner, s0, s1, s2), (tiles, 1, 1), _stream())
+    return out

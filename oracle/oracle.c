@@ -1,0 +1,216 @@
+/*
+ * CPU oracle -- TEST INFRASTRUCTURE ONLY.
+ *
+ * Plain-C restatement of what the reference's lowering computes for the five
+ * benchmark graphs.  It exists to check the HIP kernels; the product never
+ * calls it (only tests, the smoke check and the benchmark's cpu_baseline leg
+ * may load this library).
+ *
+ * Numerics restated from the reference:
+ *   - sums accumulate in (at least) fp32 and return fp32
+ *       (reference inductor_x/lowering.py:204-215);
+ *   - mean = sum / N computed in fp32 for 16-bit inputs, cast back afterwards
+ *       (reference inductor_x/lowering.py:217-233);
+ *   - var / var_mean are the two-pass form: mean first, then
+ *     sum((x - mean)^2) / max(N - correction, 0)
+ *       (reference inductor_x/lowering.py:270-293);
+ *   - 16-bit loads are widened to fp32, arithmetic stays fp32 inside a fused
+ *     kernel and rounding (RNE) happens at stores only
+ *       (reference inductor_x/codegen/triton.py:1431-1433);
+ *   - argmax: accumulator starts at (-inf, INT64_MAX), a greater value wins,
+ *     NaN beats numbers, equal values keep the lower index
+ *       (reference inductor_x/codegen/triton.py:1217-1233);
+ *   - fused attention: softmax(Q K^T * scale [+ causal mask]) V with fp32
+ *     softmax, plus the row max and row sum the op also returns, each
+ *     broadcast over a trailing axis of 8
+ *       (reference inductor_x/npu_fusion_attention_graph.py:17-35,45-74).
+ *     The arithmetic of that op lives in torch_npu's CANN kernel
+ *     (npu_fusion_attention, no version pinned by the reference), which is not
+ *     part of the reference tree: PARITY UNPINNED against that kernel; this
+ *     function restates the published definition of scaled-dot-product
+ *     attention and is pinned by closed forms in tests/test_oracle.py.
+ *
+ * Accumulations use double so the oracle is the more accurate side of every
+ * comparison; element-wise math is done in float where the kernel does so.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+static inline float bf16_to_f32(uint16_t b) {
+  uint32_t u = ((uint32_t)b) << 16;
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+static inline uint16_t f32_to_bf16(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u); /* quiet NaN */
+  u += 0x7fffu + ((u >> 16) & 1u);                                             /* RNE */
+  return (uint16_t)(u >> 16);
+}
+
+/* y[i] = sum_j relu(2 x[i,j] + 1) * sigmoid(x[i,j]) */
+void oracle_relu_sigmoid_rowsum_f32(const float* x, float* y, int64_t rows, int64_t cols) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < rows; ++i) {
+    double acc = 0.0;
+    const float* p = x + i * cols;
+    for (int64_t j = 0; j < cols; ++j) {
+      const float t = p[j];
+      float a = 2.0f * t + 1.0f;
+      a = a > 0.0f ? a : (a != a ? a : 0.0f); /* relu propagates NaN */
+      const float s = 1.0f / (1.0f + expf(-t));
+      acc += (double)(a * s);
+    }
+    y[i] = (float)acc;
+  }
+}
+
+/* s = h + r (fp32), sum_out = bf16(s), out = bf16(s * rsqrt(mean(s^2) + eps) * w) */
+void oracle_add_rmsnorm_bf16(const uint16_t* h, const uint16_t* r, const uint16_t* w, uint16_t* out,
+                             uint16_t* sum_out, int64_t rows, int64_t cols, float eps) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < rows; ++i) {
+    const uint16_t* hp = h + i * cols;
+    const uint16_t* rp = r + i * cols;
+    double ss = 0.0;
+    for (int64_t j = 0; j < cols; ++j) {
+      const float s = bf16_to_f32(hp[j]) + bf16_to_f32(rp[j]);
+      sum_out[i * cols + j] = f32_to_bf16(s);
+      ss += (double)s * (double)s;
+    }
+    const float mean = (float)(ss / (double)cols);
+    const float rs = (float)(1.0 / sqrt((double)(mean + eps)));
+    for (int64_t j = 0; j < cols; ++j) {
+      const float s = bf16_to_f32(hp[j]) + bf16_to_f32(rp[j]);
+      out[i * cols + j] = f32_to_bf16(s * rs * bf16_to_f32(w[j]));
+    }
+  }
+}
+
+/* Per-column two-pass mean / variance and first-index argmax over dim 0. */
+void oracle_col_mean_var_argmax_f32(const float* x, float* mean_out, float* var_out,
+                                    int64_t* argmax_out, int64_t rows, int64_t cols,
+                                    double correction) {
+#pragma omp parallel for schedule(static)
+  for (int64_t c = 0; c < cols; ++c) {
+    double s = 0.0;
+    float best = -INFINITY;
+    int64_t bi = INT64_MAX;
+    for (int64_t r = 0; r < rows; ++r) {
+      const float v = x[r * cols + c];
+      s += (double)v;
+      const int best_nan = best != best, v_nan = v != v;
+      /* rows come in increasing order, so "equal keeps the lower index" means
+       * an equal value never replaces; the sentinel index loses every tie. */
+      if ((v > best) || (v_nan && !best_nan) || (bi == INT64_MAX && (v == best))) {
+        best = v;
+        bi = r;
+      }
+    }
+    const double mean = rows > 0 ? s / (double)rows : NAN;
+    double m2 = 0.0;
+    for (int64_t r = 0; r < rows; ++r) {
+      const double d = (double)x[r * cols + c] - mean;
+      m2 += d * d;
+    }
+    double denom = (double)rows - correction;
+    if (denom < 0.0) denom = 0.0;
+    mean_out[c] = (float)mean;
+    var_out[c] = (float)(m2 / denom);
+    argmax_out[c] = bi;
+  }
+}
+
+/* out[i, :] = table[idx[i], :]; negative indices wrap once (Python indexing). */
+int oracle_gather_rows(const void* table, const int64_t* idx, void* out, int64_t nidx,
+                       int64_t row_bytes, int64_t table_rows) {
+  int bad = 0;
+#pragma omp parallel for schedule(static) reduction(| : bad)
+  for (int64_t i = 0; i < nidx; ++i) {
+    int64_t k = idx[i];
+    if (k < 0) k += table_rows;
+    if (k < 0 || k >= table_rows) {
+      bad |= 1;
+      continue;
+    }
+    memcpy((char*)out + i * row_bytes, (const char*)table + k * row_bytes, (size_t)row_bytes);
+  }
+  return bad;
+}
+
+/* out = contiguous(in.permute(perm)) for a contiguous 4-D input of `shape`. */
+void oracle_permute4(const void* in, void* out, const int64_t* shape, const int32_t* perm,
+                     int64_t elem_bytes) {
+  int64_t istride[4];
+  istride[3] = 1;
+  for (int d = 2; d >= 0; --d) istride[d] = istride[d + 1] * shape[d + 1];
+  int64_t oshape[4], ostride_in[4];
+  for (int d = 0; d < 4; ++d) {
+    oshape[d] = shape[perm[d]];
+    ostride_in[d] = istride[perm[d]];
+  }
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t a = 0; a < oshape[0]; ++a)
+    for (int64_t b = 0; b < oshape[1]; ++b)
+      for (int64_t c = 0; c < oshape[2]; ++c)
+        for (int64_t d = 0; d < oshape[3]; ++d) {
+          const int64_t o = ((a * oshape[1] + b) * oshape[2] + c) * oshape[3] + d;
+          const int64_t i = a * ostride_in[0] + b * ostride_in[1] + c * ostride_in[2] + d * ostride_in[3];
+          memcpy((char*)out + o * elem_bytes, (const char*)in + i * elem_bytes, (size_t)elem_bytes);
+        }
+}
+
+/*
+ * Attention, layout BNSD: q [B,N,Sq,D], k,v [B,N,Sk,D] bf16 -> out [B,N,Sq,D] bf16,
+ * softmax_max / softmax_sum [B,N,Sq,8] fp32 (value repeated 8 times).
+ * causal != 0 masks key j > query i + (Sk - Sq) (bottom-right aligned; equal to
+ * the usual lower triangle when Sq == Sk).  A fully masked row yields zeros.
+ */
+void oracle_attention_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, uint16_t* out,
+                           float* softmax_max, float* softmax_sum, int64_t B, int64_t N,
+                           int64_t Sq, int64_t Sk, int64_t D, float scale, int causal) {
+#pragma omp parallel for collapse(2) schedule(dynamic, 4)
+  for (int64_t bn = 0; bn < B * N; ++bn) {
+    for (int64_t i = 0; i < Sq; ++i) {
+      const uint16_t* qp = q + (bn * Sq + i) * D;
+      const uint16_t* kb = k + bn * Sk * D;
+      const uint16_t* vb = v + bn * Sk * D;
+      int64_t jend = Sk;
+      if (causal) {
+        jend = i + (Sk - Sq) + 1;
+        if (jend > Sk) jend = Sk;
+        if (jend < 0) jend = 0;
+      }
+      double* s = (double*)malloc(sizeof(double) * (size_t)(jend > 0 ? jend : 1));
+      double* acc = (double*)calloc((size_t)D, sizeof(double));
+      double m = -INFINITY;
+      for (int64_t j = 0; j < jend; ++j) {
+        double dot = 0.0;
+        for (int64_t d = 0; d < D; ++d) dot += (double)bf16_to_f32(qp[d]) * (double)bf16_to_f32(kb[j * D + d]);
+        s[j] = dot * (double)scale;
+        if (s[j] > m) m = s[j];
+      }
+      double l = 0.0;
+      for (int64_t j = 0; j < jend; ++j) {
+        const double p = exp(s[j] - m);
+        l += p;
+        for (int64_t d = 0; d < D; ++d) acc[d] += p * (double)bf16_to_f32(vb[j * D + d]);
+      }
+      for (int64_t d = 0; d < D; ++d)
+        out[(bn * Sq + i) * D + d] = f32_to_bf16(jend > 0 ? (float)(acc[d] / l) : 0.0f);
+      for (int t = 0; t < 8; ++t) {
+        softmax_max[(bn * Sq + i) * 8 + t] = (float)m;
+        softmax_sum[(bn * Sq + i) * 8 + t] = (float)l;
+      }
+      free(s);
+      free(acc);
+    }
+  }
+}
+
+int oracle_abi_version(void) { return 1; }

@@ -1,0 +1,277 @@
+"""Parity of the HIP kernel families (called through the C-ABI launcher)
+against the CPU oracle, on seeded inputs.
+
+Tolerances: bit-exact for integer / index / byte-moving outputs; <= 1e-5
+relative for fp32 outputs; <= 2e-2 absolute for bf16 outputs.  Shapes follow
+the reference's own test shapes where it has them (cited per test).
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import announce, bits
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def K():
+    from inductor_x_amd import kernels
+
+    return kernels
+
+
+@pytest.fixture(scope="module")
+def O():
+    from oracle import oracle
+
+    return oracle
+
+
+# ---------------------------------------------------------------- graph 1
+# last-dim sums incl. odd outer shapes, as reference test/npu_indexing/reduction_test.py:12-33
+@pytest.mark.parametrize("shape", [(3, 8), (1024, 4096), (7, 9, 1024), (2053, 64), (33, 12), (1, 7168), (513, 100)])
+def test_rowsum_vs_oracle(K, O, shape):
+    announce(f"rowsum shape={shape}")
+    torch.manual_seed(0)
+    x = torch.randn(*shape)
+    y = K.fused_relu_sigmoid_rowsum(x.to(DEV)).cpu().numpy()
+    ref = O.relu_sigmoid_rowsum(x.numpy())
+    assert y.shape == ref.shape
+    np.testing.assert_allclose(y, ref, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("variant", [(256, 256), (256, 128), (256, 64), (512, 512), (1024, 1024)])
+def test_rowsum_variants(K, O, variant):
+    announce(f"rowsum variant={variant}")
+    torch.manual_seed(1)
+    x = torch.randn(301, 2048)
+    y = K.fused_relu_sigmoid_rowsum(x.to(DEV), variant=variant).cpu().numpy()
+    np.testing.assert_allclose(y, O.relu_sigmoid_rowsum(x.numpy()), rtol=1e-5, atol=1e-6)
+
+
+def test_rowsum_empty_and_nan(K):
+    announce("rowsum empty / nan")
+    assert K.fused_relu_sigmoid_rowsum(torch.empty(0, 64, device=DEV)).shape == (0,)
+    x = torch.randn(4, 64)
+    x[2, 5] = float("nan")
+    y = K.fused_relu_sigmoid_rowsum(x.to(DEV)).cpu()
+    assert torch.isnan(y[2]) and not torch.isnan(y[[0, 1, 3]]).any()
+
+
+def test_rowsum_rejects_bad_operands(K):
+    with pytest.raises(ValueError):
+        K.fused_relu_sigmoid_rowsum(torch.randn(4, 6, device=DEV))  # row not a multiple of 4
+    with pytest.raises(ValueError):
+        K.fused_relu_sigmoid_rowsum(torch.randn(8, 8, device=DEV).t())  # not contiguous
+    with pytest.raises(ValueError):
+        K.fused_relu_sigmoid_rowsum(torch.randn(8, 8, device=DEV).half())
+
+
+# ---------------------------------------------------------------- graph 2
+@pytest.mark.parametrize("rows,cols", [(1, 8), (5, 64), (64, 4096), (129, 1024), (3, 2056), (257, 512), (8, 8192)])
+def test_add_rmsnorm_vs_oracle(K, O, rows, cols):
+    announce(f"add_rmsnorm rows={rows} cols={cols}")
+    torch.manual_seed(0)
+    h = torch.randn(rows, cols).bfloat16()
+    r = torch.randn(rows, cols).bfloat16()
+    w = (1 + 0.02 * torch.randn(cols)).bfloat16()
+    out, s = K.add_rmsnorm(h.to(DEV), r.to(DEV), w.to(DEV), 1e-6)
+    o_ref, s_ref = O.add_rmsnorm_bf16(bits(h), bits(r), bits(w), 1e-6)
+    assert np.array_equal(bits(s), s_ref)  # h + r is exactly rounded: bit-exact
+    err = np.abs(O.bf16_bits_to_f32(bits(out)) - O.bf16_bits_to_f32(o_ref)).max()
+    assert err <= 2e-2
+    # and almost everywhere identical bits (differences are single bf16 roundings)
+    assert (bits(out) != o_ref).mean() < 0.01
+
+
+@pytest.mark.parametrize("variant", [(256, 256, 2), (256, 128, 4), (256, 64, 8), (512, 512, 1), (256, 256, 4)])
+def test_add_rmsnorm_variants(K, O, variant):
+    announce(f"add_rmsnorm variant={variant}")
+    torch.manual_seed(2)
+    rows, cols = 77, 4096
+    h = torch.randn(rows, cols).bfloat16()
+    r = torch.randn(rows, cols).bfloat16()
+    w = (1 + 0.02 * torch.randn(cols)).bfloat16()
+    out, s = K.add_rmsnorm(h.to(DEV), r.to(DEV), w.to(DEV), 1e-6, variant=variant)
+    o_ref, s_ref = O.add_rmsnorm_bf16(bits(h), bits(r), bits(w), 1e-6)
+    assert np.array_equal(bits(s), s_ref)
+    assert np.abs(O.bf16_bits_to_f32(bits(out)) - O.bf16_bits_to_f32(o_ref)).max() <= 2e-2
+
+
+def test_add_rmsnorm_full_size_properties(K):
+    """BASELINE shape [8192, 4096]: w = 1, r = 0 reduces to textbook RMSNorm
+    (every output row has mean square 1), and h + 0 returns h bit-for-bit."""
+    announce("add_rmsnorm full size properties")
+    torch.manual_seed(0)
+    h = torch.randn(8192, 4096).bfloat16().to(DEV)
+    r = torch.zeros_like(h)
+    w = torch.ones(4096, dtype=torch.bfloat16, device=DEV)
+    out, s = K.add_rmsnorm(h, r, w, 1e-6)
+    assert torch.equal(s, h)
+    ms = out.float().pow(2).mean(-1)
+    assert (ms - 1).abs().max().item() < 5e-3
+    # scale invariance: normalising 4*h gives the same result as h
+    out4, _ = K.add_rmsnorm(h * 4, r, w, 1e-6)
+    assert (out4.float() - out.float()).abs().max().item() <= 2e-2
+
+
+def test_add_rmsnorm_empty(K):
+    out, s = K.add_rmsnorm(
+        torch.empty(0, 64, dtype=torch.bfloat16, device=DEV),
+        torch.empty(0, 64, dtype=torch.bfloat16, device=DEV),
+        torch.ones(64, dtype=torch.bfloat16, device=DEV),
+    )
+    assert out.shape == (0, 64) and s.shape == (0, 64)
+
+
+# ---------------------------------------------------------------- graph 3
+def _check_col(K, O, x, correction=0.0, **kw):
+    mean, var, arg = K.col_mean_var_argmax(x.to(DEV), correction, **kw)
+    m_ref, v_ref, a_ref = O.col_mean_var_argmax(x.numpy(), correction)
+    assert np.array_equal(arg.cpu().numpy(), a_ref)  # bit-exact, first index on ties
+    # means of N(0,1) columns are ~0: relative 1e-5 of the column's scale (its
+    # standard deviation), i.e. an absolute floor of 1e-5 * sqrt(var)
+    scale = np.sqrt(np.maximum(v_ref, 1e-30))
+    assert (np.abs(mean.cpu().numpy() - m_ref) <= 1e-5 * np.maximum(np.abs(m_ref), scale) + 1e-12).all()
+    np.testing.assert_allclose(var.cpu().numpy(), v_ref, rtol=1e-5, atol=1e-12)
+
+
+# shapes: reference test/npu_indexing/var_mean_test.py:28-36 reduces (128,8,64) style
+# tensors; argmax shapes 513x64 / 513x1024 from argmax_unalign_test.py:37,58
+@pytest.mark.parametrize("rows,cols", [(1, 4), (2, 512), (513, 64), (513, 1024), (4096, 512), (65536, 512), (1000, 12), (300, 2048), (70000, 8)])
+def test_col_stats_vs_oracle(K, O, rows, cols):
+    announce(f"col stats rows={rows} cols={cols}")
+    torch.manual_seed(0)
+    _check_col(K, O, torch.randn(rows, cols))
+
+
+def test_col_stats_correction_and_offset(K, O):
+    announce("col stats correction=1, shifted data")
+    torch.manual_seed(3)
+    x = torch.randn(5000, 64) * 0.5 + 100.0  # large mean relative to spread
+    _check_col(K, O, x, correction=1.0)
+
+
+def test_col_argmax_ties_and_nan(K, O):
+    """Planted ties across thread / row-lane / split boundaries and NaNs."""
+    announce("col argmax ties / nan")
+    torch.manual_seed(4)
+    rows, cols = 4096, 64
+    x = torch.randn(rows, cols).clamp_(-3, 3)
+    x[:, 0] = 1.0  # all equal -> index 0
+    x[100, 1] = 10.0
+    x[3000, 1] = 10.0  # tie far apart -> 100
+    x[4095, 2] = 10.0
+    x[17, 2] = 10.0  # later planted first in memory order anyway -> 17
+    x[2000, 3] = float("nan")
+    x[50, 3] = 50.0  # NaN beats numbers -> 2000
+    x[7, 4] = float("nan")
+    x[9, 4] = float("nan")  # first NaN -> 7
+    x[:, 5] = float("-inf")  # all -inf -> 0
+    x[1234, 6] = float("inf")
+    mean, var, arg = K.col_mean_var_argmax(x.to(DEV))
+    a = arg.cpu().numpy()
+    assert list(a[:7]) == [0, 100, 17, 2000, 7, 0, 1234]
+    assert np.array_equal(a, torch.argmax(x, 0).numpy())
+    assert np.array_equal(a, O.col_mean_var_argmax(x.numpy())[2])
+    assert torch.isnan(var.cpu()[3]) and torch.isnan(mean.cpu()[3])
+
+
+@pytest.mark.parametrize("ct,rl,u", [(128, 2, 4), (128, 4, 8), (128, 8, 4), (64, 16, 4), (64, 1, 8), (16, 16, 4), (1, 64, 4)])
+def test_col_stats_variants(K, O, ct, rl, u):
+    from inductor_x_amd.hip_heuristics import SplitPlan, cdiv
+
+    announce(f"col stats variant ct={ct} rl={rl} u={u}")
+    torch.manual_seed(5)
+    rows, cols = 3001, 256
+    x = torch.randn(rows, cols)
+    rps = cdiv(cdiv(rows, 7), rl * u) * rl * u
+    plan = SplitPlan(ct, rl, u, cdiv(rows, rps), rps, cdiv(cols, ct * 4))
+    for fv in [(16, 16), (8, 32), (4, 64), (64, 4)]:
+        _check_col(K, O, x, plan=plan, final_variant=fv)
+
+
+def test_col_stats_invariants_full_size(K):
+    """BASELINE shape: var(x + c) == var(x), var(k x) == k^2 var(x), argmax unchanged."""
+    announce("col stats invariants 65536x512")
+    torch.manual_seed(0)
+    x = torch.randn(65536, 512).to(DEV)
+    m0, v0, a0 = K.col_mean_var_argmax(x)
+    m1, v1, a1 = K.col_mean_var_argmax(x + 3.0)
+    m2, v2, a2 = K.col_mean_var_argmax(x * 2.0)
+    assert torch.equal(a0, a2)
+    assert ((v1 - v0).abs() / v0).max().item() < 1e-4  # x + 3 rounds the inputs themselves
+    assert ((v2 - 4 * v0).abs() / (4 * v0)).max().item() < 1e-6
+    assert (m1 - m0 - 3.0).abs().max().item() < 1e-5
+    assert torch.equal(a0, torch.argmax(x, 0))
+
+
+# ---------------------------------------------------------------- graph 4
+@pytest.mark.parametrize("nrows,width,n", [(10, 8, 1), (50304, 1024, 4096), (17, 128, 1000), (3, 2048, 33), (100, 264, 77)])
+def test_gather_vs_oracle(K, O, nrows, width, n):
+    announce(f"gather nrows={nrows} width={width} n={n}")
+    torch.manual_seed(0)
+    table = (0.02 * torch.randn(nrows, width)).bfloat16()
+    idx = torch.randint(0, nrows, (n,), dtype=torch.int64)
+    idx[0] = 0
+    idx[-1] = nrows - 1
+    out = K.gather_rows(table.to(DEV), idx.to(DEV))
+    assert np.array_equal(bits(out), O.gather_rows(bits(table), idx.numpy()))
+
+
+def test_gather_duplicates_negative_2d_index_fp32(K, O):
+    announce("gather duplicates / negative / 2-D idx / fp32")
+    torch.manual_seed(1)
+    table = torch.randn(9, 64).bfloat16()
+    idx = torch.tensor([[0, 0, 8, -1], [3, 3, -9, 8]], dtype=torch.int64)
+    out = K.gather_rows(table.to(DEV), idx.to(DEV))
+    assert out.shape == (2, 4, 64)
+    assert torch.equal(out.cpu(), table[idx])
+    t32 = torch.randn(9, 64)
+    assert torch.equal(K.gather_rows(t32.to(DEV), idx.to(DEV)).cpu(), t32[idx])
+    assert K.gather_rows(table.to(DEV), torch.empty(0, dtype=torch.int64, device=DEV)).shape == (0, 64)
+
+
+@pytest.mark.parametrize("variant", [(256, 128, 1), (256, 128, 4), (256, 64, 2), (256, 16, 4)])
+def test_gather_variants(K, variant):
+    announce(f"gather variant={variant}")
+    torch.manual_seed(2)
+    table = torch.randn(301, 1024).bfloat16()
+    idx = torch.randint(0, 301, (999,), dtype=torch.int64)
+    out = K.gather_rows(table.to(DEV), idx.to(DEV), variant=variant)
+    assert torch.equal(out.cpu(), table[idx])
+
+
+# permute (0,2,1,3): reference test/npu_indexing/permute_test.py:19 on (8,8,512,128)
+@pytest.mark.parametrize("shape", [(8, 8, 512, 128), (2, 3, 5, 8), (1, 33, 7, 64), (16, 2048, 32, 128), (3, 100, 9, 120)])
+def test_permute_vs_oracle(K, O, shape):
+    announce(f"permute shape={shape}")
+    torch.manual_seed(0)
+    t = torch.randn(*shape).bfloat16()
+    out = K.permute_0213_contiguous(t.to(DEV))
+    assert out.shape == (shape[0], shape[2], shape[1], shape[3])
+    assert np.array_equal(bits(out), O.permute4(bits(t), (0, 2, 1, 3)))
+
+
+def test_permute_involution_full_size_and_fp32(K):
+    announce("permute involution 16x2048x32x128")
+    torch.manual_seed(0)
+    t = torch.randn(16, 2048, 32, 128, device=DEV).bfloat16()
+    once = K.permute_0213_contiguous(t)
+    assert torch.equal(K.permute_0213_contiguous(once), t)
+    assert torch.equal(once, t.permute(0, 2, 1, 3).contiguous())
+    f = torch.randn(4, 50, 6, 64, device=DEV)
+    assert torch.equal(K.permute_0213_contiguous(f), f.permute(0, 2, 1, 3).contiguous())
+
+
+@pytest.mark.parametrize("variant", [(256, 16, 32, 8), (256, 16, 8, 8), (256, 16, 1, 64), (256, 16, 2, 8), (256, 64, 4, 4), (256, 8, 1, 32)])
+def test_permute_variants(K, variant):
+    announce(f"permute variant={variant}")
+    torch.manual_seed(1)
+    inner = min(variant[1] * 8, 128)
+    t = torch.randn(3, 70, 37, inner, device=DEV).bfloat16()
+    out = K.permute_0213_contiguous(t, variant=variant)
+    assert torch.equal(out, t.permute(0, 2, 1, 3).contiguous())
