@@ -51,6 +51,14 @@ __device__ __forceinline__ ColState col_state_combine(const ColState& a, const C
   return r;
 }
 
+// True when a later row's value x must replace the running best: x is greater,
+// or x is NaN while best is not.  !(x <= best) covers "greater or unordered";
+// the second term keeps a NaN best in place.  Written with bitwise operators so
+// it compiles to two compares and a mask AND instead of branches.
+__device__ __forceinline__ bool col_argmax_update(float x, float best) {
+  return static_cast<bool>(static_cast<int>(!(x <= best)) & static_cast<int>(best == best));
+}
+
 // Fold the RL row lanes of a workgroup.  lds holds (RL/2) * CT * 4 * kColFields
 // floats.  On return the threads with rl == 0 hold the result.
 template <int CT, int RL>
@@ -126,10 +134,23 @@ __device__ __forceinline__ void col_stats_partial(const float* __restrict__ x,
     int cnt = 1;
     r += RL;
     p += step;
-    for (; r + (UNROLL - 1) * RL < r_end; r += UNROLL * RL, p += UNROLL * step) {
-      Vec<float, 4> v[UNROLL];
+    // Software pipeline: the next batch of UNROLL loads is in flight while the
+    // current batch is folded.
+    Vec<float, 4> v[UNROLL];
+    bool have = r + (UNROLL - 1) * RL < r_end;
+    if (have) {
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) v[u] = load_vec<float, 4, true>(p + u * step);
+    }
+    while (have) {
+      const int rn = r + UNROLL * RL;
+      const float* __restrict__ pn = p + UNROLL * step;
+      const bool have_next = rn + (UNROLL - 1) * RL < r_end;
+      Vec<float, 4> vn[UNROLL];
+      if (have_next) {
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) vn[u] = load_vec<float, 4, true>(pn + u * step);
+      }
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
 #pragma unroll
@@ -138,12 +159,17 @@ __device__ __forceinline__ void col_stats_partial(const float* __restrict__ x,
           const float d = xv - c[k];
           s1[k] += d;
           s2[k] = fmaf(d, d, s2[k]);
-          const bool upd = (xv > best[k]) || ((xv != xv) && (best[k] == best[k]));
+          const bool upd = col_argmax_update(xv, best[k]);
           best[k] = upd ? xv : best[k];
           bi[k] = upd ? (r + u * RL) : bi[k];
         }
       }
       cnt += UNROLL;
+      r = rn;
+      p = pn;
+      have = have_next;
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) v[u] = vn[u];
     }
     for (; r < r_end; r += RL, p += step) {
       const Vec<float, 4> v = load_vec<float, 4, true>(p);
@@ -153,7 +179,7 @@ __device__ __forceinline__ void col_stats_partial(const float* __restrict__ x,
         const float d = xv - c[k];
         s1[k] += d;
         s2[k] = fmaf(d, d, s2[k]);
-        const bool upd = (xv > best[k]) || ((xv != xv) && (best[k] == best[k]));
+        const bool upd = col_argmax_update(xv, best[k]);
         best[k] = upd ? xv : best[k];
         bi[k] = upd ? r : bi[k];
       }
@@ -196,9 +222,11 @@ __device__ __forceinline__ void col_stats_partial(const float* __restrict__ x,
 }
 
 // Pass 2.  A workgroup of CPW * SL threads finishes CPW columns; thread
-// (c, sl) folds splits sl, sl+SL, ... in increasing order, then the SL lanes are
-// folded through LDS (CPW * SL * kColFields floats, static).
-template <int CPW, int SL>
+// (c, sl) folds splits sl, sl+SL, ... in increasing order.  The partials are
+// fetched in batches of BATCH independent loads so the fold is not a chain of
+// memory round trips.  The SL lanes are then folded through LDS
+// (CPW * SL * kColFields floats, static).
+template <int CPW, int SL, int BATCH = 8>
 __device__ __forceinline__ void col_stats_final(const float* __restrict__ part,
                                                 float* __restrict__ mean_out,
                                                 float* __restrict__ var_out,
@@ -211,15 +239,27 @@ __device__ __forceinline__ void col_stats_final(const float* __restrict__ part,
   const size_t plane = static_cast<size_t>(nsplit) * cols;
   ColState st = col_state_empty();
   if (col < cols) {
-    for (int s = sl; s < nsplit; s += SL) {
-      const size_t o = static_cast<size_t>(s) * cols + col;
-      ColState b;
-      b.m.n = part[0 * plane + o];
-      b.m.mean = part[1 * plane + o];
-      b.m.m2 = part[2 * plane + o];
-      b.a.v = part[3 * plane + o];
-      b.a.i = __float_as_int(part[4 * plane + o]);
-      st = col_state_combine(st, b);
+    for (int s0 = sl; s0 < nsplit; s0 += SL * BATCH) {
+      float f[BATCH][kColFields];
+#pragma unroll
+      for (int b = 0; b < BATCH; ++b) {
+        const int s = s0 + b * SL;
+        const size_t o = static_cast<size_t>(s < nsplit ? s : s0) * cols + col;
+#pragma unroll
+        for (int k = 0; k < kColFields; ++k) f[b][k] = part[k * plane + o];
+      }
+#pragma unroll
+      for (int b = 0; b < BATCH; ++b) {
+        if (s0 + b * SL < nsplit) {
+          ColState t;
+          t.m.n = f[b][0];
+          t.m.mean = f[b][1];
+          t.m.m2 = f[b][2];
+          t.a.v = f[b][3];
+          t.a.i = __float_as_int(f[b][4]);
+          st = col_state_combine(st, t);
+        }
+      }
     }
   }
   constexpr int PLANE = CPW * SL;
@@ -229,10 +269,11 @@ __device__ __forceinline__ void col_stats_final(const float* __restrict__ part,
   lds[3 * PLANE + threadIdx.x] = st.a.v;
   lds[4 * PLANE + threadIdx.x] = __int_as_float(st.a.i);
   __syncthreads();
-  if (sl == 0 && col < cols) {
+  // tree over the SL lanes: log2(SL) rounds instead of SL serial steps
 #pragma unroll
-    for (int j = 1; j < SL; ++j) {
-      const int t = j * CPW + c;
+  for (int half = SL / 2; half >= 1; half >>= 1) {
+    if (sl < half) {
+      const int t = (sl + half) * CPW + c;
       ColState b;
       b.m.n = lds[0 * PLANE + t];
       b.m.mean = lds[1 * PLANE + t];
@@ -240,7 +281,15 @@ __device__ __forceinline__ void col_stats_final(const float* __restrict__ part,
       b.a.v = lds[3 * PLANE + t];
       b.a.i = __float_as_int(lds[4 * PLANE + t]);
       st = col_state_combine(st, b);
+      lds[0 * PLANE + threadIdx.x] = st.m.n;
+      lds[1 * PLANE + threadIdx.x] = st.m.mean;
+      lds[2 * PLANE + threadIdx.x] = st.m.m2;
+      lds[3 * PLANE + threadIdx.x] = st.a.v;
+      lds[4 * PLANE + threadIdx.x] = __int_as_float(st.a.i);
     }
+    __syncthreads();
+  }
+  if (sl == 0 && col < cols) {
     mean_out[col] = st.m.mean;
     const float denom = fmaxf(st.m.n - correction, 0.f);
     var_out[col] = st.m.m2 / denom;

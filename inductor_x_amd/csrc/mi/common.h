@@ -225,7 +225,7 @@ __device__ __forceinline__ Moments moments_combine(Moments a, Moments b) {
   const float n = a.n + b.n;
   if (n == 0.f) return a;
   const float delta = b.mean - a.mean;
-  const float wb = b.n / n;
+  const float wb = b.n * __builtin_amdgcn_rcpf(n);
   Moments r;
   r.n = n;
   r.mean = a.mean + delta * wb;

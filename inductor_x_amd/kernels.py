@@ -383,3 +383,61 @@ def permute_0213_contiguous(t: torch.Tensor, variant: Optional[tuple] = None) ->
     tiles = n0 * cdiv(n1, t1) * cdiv(n2, t2)
     l._launch(i, (t.data_ptr(), out.data_ptr(), n0, n1, n2, inner, s0, s1, s2), (tiles, 1, 1), _stream())
     return out
+
+
+# ---------------------------------------------------------------------------
+# graph 5: fused attention forward (bf16, head dim 128)
+# ---------------------------------------------------------------------------
+_ATTN_LDS_BYTES = (64 * 136 + 128 * 72) * 2
+
+
+@functools.lru_cache(maxsize=None)
+def _attention_launcher() -> CachingLauncher:
+    cfgs = [
+        LaunchConfig("fused_attention_fwd_bf16_d128_causal", 256, meta={"CAUSAL": 1}, lds_bytes=_ATTN_LDS_BYTES),
+        LaunchConfig("fused_attention_fwd_bf16_d128_full", 256, meta={"CAUSAL": 0}, lds_bytes=_ATTN_LDS_BYTES),
+    ]
+    return CachingLauncher(
+        "fused_attention_fwd_bf16_d128",
+        codecache.aot_source("attention_kernels.hip"),
+        "PPPPPPiif",
+        cfgs,
+        prefer_intree=True,
+    )
+
+
+def fused_attention(
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """softmax(q k^T * scale [+ causal mask]) v for [B, N, S, 128] bf16 tensors.
+
+    Returns (out bf16 [B,N,S,128], softmax_max fp32 [B,N,S,8], softmax_sum fp32
+    [B,N,S,8]); the statistics are the row maximum of the scaled scores and the
+    row sum of exp(score - max), each repeated over the trailing axis."""
+    _check_cuda(q, k, v)
+    _require(q.dtype == k.dtype == v.dtype == torch.bfloat16, "q, k, v must be bf16")
+    _require(q.dim() == 4 and q.shape == k.shape == v.shape, "q, k, v must share a [B, N, S, D] shape")
+    B, N, S, D = q.shape
+    _require(D == 128, "head dimension must be 128")
+    _require(S % 128 == 0 and S > 0, "sequence length must be a positive multiple of 128")
+    _require(q.is_contiguous() and k.is_contiguous() and v.is_contiguous(), "q, k, v must be contiguous (BNSD)")
+    _require(all(_aligned(t) for t in (q, k, v)), "q, k, v must be 16-byte aligned")
+    _require(scale > 0 and math.isfinite(scale), "scale must be positive and finite")
+    _require(B * N * S * D < 2**31, "numel must fit int32 indexing")
+    out = torch.empty_like(q)
+    smax = torch.empty((B, N, S, 8), dtype=torch.float32, device=q.device)
+    ssum = torch.empty((B, N, S, 8), dtype=torch.float32, device=q.device)
+    if B * N == 0:
+        return out, smax, ssum
+    l = _attention_launcher()
+    i = _find(l, "fused_attention_fwd_bf16_d128_causal" if causal else "fused_attention_fwd_bf16_d128_full")
+    heads = B * N
+    grid = 8 * cdiv(heads, 8) * (S // 128)
+    l._launch(
+        i,
+        (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), smax.data_ptr(), ssum.data_ptr(), heads, S,
+         float(scale) * 1.4426950408889634),
+        (grid, 1, 1),
+        _stream(),
+    )
+    return out, smax, ssum

@@ -1,0 +1,98 @@
+"""Fused attention (bf16 MFMA kernel) against the CPU oracle and against the
+closed-form properties of softmax attention.  Tolerance: 2e-2 absolute on the
+bf16 output; the fp32 statistics to 1e-3 relative (they depend only on q, k).
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import announce, bits
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def K():
+    from inductor_x_amd import kernels
+
+    return kernels
+
+
+@pytest.fixture(scope="module")
+def O():
+    from oracle import oracle
+
+    return oracle
+
+
+@pytest.mark.parametrize("B,N,S,causal", [(1, 1, 128, True), (1, 2, 256, True), (2, 3, 384, True), (1, 2, 256, False), (1, 9, 128, False), (1, 1, 512, True)])
+def test_attention_vs_oracle(K, O, B, N, S, causal):
+    announce(f"attention B={B} N={N} S={S} causal={causal}")
+    torch.manual_seed(0)
+    q, k, v = (torch.randn(B, N, S, 128).bfloat16() for _ in range(3))
+    scale = 128 ** -0.5
+    out, smax, ssum = K.fused_attention(q.to(DEV), k.to(DEV), v.to(DEV), scale, causal)
+    o_ref, m_ref, l_ref = O.attention_bf16(bits(q), bits(k), bits(v), scale, causal)
+    err = np.abs(O.bf16_bits_to_f32(bits(out)) - O.bf16_bits_to_f32(o_ref)).max()
+    assert err <= 2e-2, err
+    np.testing.assert_allclose(smax.cpu().numpy(), m_ref, rtol=1e-3, atol=1e-3)
+    np.testing.assert_allclose(ssum.cpu().numpy(), l_ref, rtol=2e-3)
+
+
+def test_attention_closed_forms(K):
+    """V = 1 gives O = 1 (probabilities sum to one); with a causal mask the first
+    query row returns V[0]; identical keys give the running mean of V."""
+    announce("attention closed forms")
+    torch.manual_seed(1)
+    B, N, S = 1, 2, 256
+    q = torch.randn(B, N, S, 128, device=DEV).bfloat16()
+    k = torch.randn(B, N, S, 128, device=DEV).bfloat16()
+    v = torch.randn(B, N, S, 128, device=DEV).bfloat16()
+    ones = torch.ones_like(v)
+    for causal in (True, False):
+        out, _, _ = K.fused_attention(q, k, ones, 0.1, causal)
+        assert (out.float() - 1).abs().max().item() <= 8e-3
+    out, smax, ssum = K.fused_attention(q, k, v, 0.1, True)
+    assert torch.equal(out[:, :, 0], v[:, :, 0])
+    assert (ssum[:, :, 0] - 1).abs().max().item() < 1e-6  # one key: sum of exp(0)
+    kc = k[:, :, :1].expand(-1, -1, S, -1).contiguous()  # all keys equal -> uniform weights
+    out, _, ssum = K.fused_attention(q, kc, v, 0.1, True)
+    mean = torch.cumsum(v.float(), 2) / torch.arange(1, S + 1, device=DEV).view(1, 1, S, 1)
+    assert (out.float() - mean).abs().max().item() <= 2e-2
+    n = torch.arange(1, S + 1, device=DEV, dtype=torch.float32).view(1, 1, S, 1).expand(B, N, S, 8)
+    assert torch.allclose(ssum, n, rtol=1e-5)
+
+
+def test_attention_causality_and_sdpa_full_size_slice(K):
+    """Causal output must not depend on later keys/values; and one head at the
+    BASELINE sequence length matches PyTorch's math-backend attention on the GPU."""
+    announce("attention causality / S=4096")
+    torch.manual_seed(2)
+    B, N, S = 1, 2, 4096
+    q, k, v = (torch.randn(B, N, S, 128, device=DEV).bfloat16() for _ in range(3))
+    scale = 128 ** -0.5
+    out, smax, ssum = K.fused_attention(q, k, v, scale, True)
+    k2, v2 = k.clone(), v.clone()
+    k2[:, :, 2048:] = torch.randn_like(k2[:, :, 2048:])
+    v2[:, :, 2048:] = torch.randn_like(v2[:, :, 2048:])
+    out2, _, _ = K.fused_attention(q, k2, v2, scale, True)
+    assert torch.equal(out[:, :, :2048], out2[:, :, :2048])
+    s = (q.float() @ k.float().transpose(-1, -2)) * scale
+    s = s.masked_fill(torch.ones(S, S, device=DEV, dtype=torch.bool).triu(1), float("-inf"))
+    ref = torch.softmax(s, -1) @ v.float()
+    assert (out.float() - ref).abs().max().item() <= 2e-2
+    assert torch.allclose(smax[..., 0], s.max(-1).values, rtol=1e-3, atol=1e-3)
+    assert torch.allclose(ssum[..., 0], torch.exp(s - s.max(-1, keepdim=True).values).sum(-1), rtol=2e-3)
+
+
+def test_attention_rejects_bad_operands(K):
+    q = torch.randn(1, 1, 128, 64, device=DEV).bfloat16()
+    with pytest.raises(ValueError):
+        K.fused_attention(q, q, q, 0.1, True)  # head dim
+    q = torch.randn(1, 1, 100, 128, device=DEV).bfloat16()
+    with pytest.raises(ValueError):
+        K.fused_attention(q, q, q, 0.1, True)  # sequence length
+    q = torch.randn(1, 1, 128, 128, device=DEV)
+    with pytest.raises(ValueError):
+        K.fused_attention(q, q, q, 0.1, True)  # dtype
