@@ -9,12 +9,12 @@
 
 using namespace mi;
 
-template <bool CAUSAL>
+template <bool CAUSAL, int WAVES>
 __device__ __forceinline__ void attention_entry(const bf16_t* q, const bf16_t* k, const bf16_t* v,
                                                 bf16_t* o, float* smax, float* ssum, int n_heads,
                                                 int S, float scale_log2e) {
   constexpr int XCDS = 8;
-  const int n_qb = S / kAttnBM;
+  const int n_qb = S / (kAttnRowsPerWave * WAVES);
   const int id = blockIdx.x;
   const int xcd = id % XCDS;
   const int slot = id / XCDS;
@@ -22,17 +22,19 @@ __device__ __forceinline__ void attention_entry(const bf16_t* q, const bf16_t* k
   int qb = slot % n_qb;
   if (head >= n_heads) return;
   if (CAUSAL) qb = n_qb - 1 - qb;
-  attention_fwd_d128<CAUSAL>(q, k, v, o, smax, ssum, S, qb, head, scale_log2e);
+  attention_fwd_d128<CAUSAL, WAVES>(q, k, v, o, smax, ssum, S, qb, head, scale_log2e);
 }
 
-extern "C" __global__ __launch_bounds__(kAttnThreads) void fused_attention_fwd_bf16_d128_causal(
-    const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
-    int n_heads, int S, float scale_log2e) {
-  attention_entry<true>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
-}
+// w4: 256 threads, 128 queries per workgroup, two workgroups per CU.
+// w8: 512 threads, 256 queries per workgroup, one workgroup per CU.
+#define ATTENTION_VARIANT(NAME, CAUSAL, WAVES, MINBLOCKS)                                      \
+  extern "C" __global__ __launch_bounds__(64 * WAVES, MINBLOCKS) void NAME(                    \
+      const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,  \
+      int n_heads, int S, float scale_log2e) {                                                 \
+    attention_entry<CAUSAL, WAVES>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);           \
+  }
 
-extern "C" __global__ __launch_bounds__(kAttnThreads) void fused_attention_fwd_bf16_d128_full(
-    const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
-    int n_heads, int S, float scale_log2e) {
-  attention_entry<false>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
-}
+ATTENTION_VARIANT(fused_attention_fwd_bf16_d128_causal_w4, true, 4, 2)
+ATTENTION_VARIANT(fused_attention_fwd_bf16_d128_full_w4, false, 4, 2)
+ATTENTION_VARIANT(fused_attention_fwd_bf16_d128_causal_w8, true, 8, 1)
+ATTENTION_VARIANT(fused_attention_fwd_bf16_d128_full_w8, false, 8, 1)

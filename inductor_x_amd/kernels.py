@@ -388,14 +388,20 @@ def permute_0213_contiguous(t: torch.Tensor, variant: Optional[tuple] = None) ->
 # ---------------------------------------------------------------------------
 # graph 5: fused attention forward (bf16, head dim 128)
 # ---------------------------------------------------------------------------
-_ATTN_LDS_BYTES = (64 * 136 + 128 * 72) * 2
+_ATTN_LDS_BYTES = 2 * (64 * 136 + 128 * 64) * 2  # two K + V^T tiles
 
 
 @functools.lru_cache(maxsize=None)
 def _attention_launcher() -> CachingLauncher:
     cfgs = [
-        LaunchConfig("fused_attention_fwd_bf16_d128_causal", 256, meta={"CAUSAL": 1}, lds_bytes=_ATTN_LDS_BYTES),
-        LaunchConfig("fused_attention_fwd_bf16_d128_full", 256, meta={"CAUSAL": 0}, lds_bytes=_ATTN_LDS_BYTES),
+        LaunchConfig(
+            f"fused_attention_fwd_bf16_d128_{'causal' if c else 'full'}_w{w}",
+            64 * w,
+            meta={"CAUSAL": c, "WAVES": w},
+            lds_bytes=_ATTN_LDS_BYTES,
+        )
+        for c in (1, 0)
+        for w in (4, 8)
     ]
     return CachingLauncher(
         "fused_attention_fwd_bf16_d128",
@@ -407,7 +413,7 @@ def _attention_launcher() -> CachingLauncher:
 
 
 def fused_attention(
-    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool, waves: Optional[int] = None
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """softmax(q k^T * scale [+ causal mask]) v for [B, N, S, 128] bf16 tensors.
 
@@ -429,10 +435,13 @@ def fused_attention(
     ssum = torch.empty((B, N, S, 8), dtype=torch.float32, device=q.device)
     if B * N == 0:
         return out, smax, ssum
+    if waves is None:
+        waves = _ATTN_DEFAULT_WAVES if S % 256 == 0 else 4
+    _require(waves in (4, 8) and S % (32 * waves) == 0, "waves must be 4 or 8 and 32*waves must divide S")
     l = _attention_launcher()
-    i = _find(l, "fused_attention_fwd_bf16_d128_causal" if causal else "fused_attention_fwd_bf16_d128_full")
+    i = _find(l, f"fused_attention_fwd_bf16_d128_{'causal' if causal else 'full'}_w{waves}")
     heads = B * N
-    grid = 8 * cdiv(heads, 8) * (S // 128)
+    grid = 8 * cdiv(heads, 8) * (S // (32 * waves))
     l._launch(
         i,
         (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), smax.data_ptr(), ssum.data_ptr(), heads, S,
@@ -441,3 +450,6 @@ def fused_attention(
         _stream(),
     )
     return out, smax, ssum
+
+
+_ATTN_DEFAULT_WAVES = 8

@@ -26,13 +26,25 @@ def O():
     return oracle
 
 
-@pytest.mark.parametrize("B,N,S,causal", [(1, 1, 128, True), (1, 2, 256, True), (2, 3, 384, True), (1, 2, 256, False), (1, 9, 128, False), (1, 1, 512, True)])
-def test_attention_vs_oracle(K, O, B, N, S, causal):
-    announce(f"attention B={B} N={N} S={S} causal={causal}")
+@pytest.mark.parametrize(
+    "B,N,S,causal,waves",
+    [
+        (1, 1, 128, True, 4),
+        (1, 2, 256, True, 4),
+        (1, 2, 256, True, 8),
+        (2, 3, 384, True, 4),
+        (1, 2, 256, False, 4),
+        (1, 9, 128, False, 4),
+        (1, 1, 512, True, 8),
+        (1, 3, 512, False, 8),
+    ],
+)
+def test_attention_vs_oracle(K, O, B, N, S, causal, waves):
+    announce(f"attention B={B} N={N} S={S} causal={causal} waves={waves}")
     torch.manual_seed(0)
     q, k, v = (torch.randn(B, N, S, 128).bfloat16() for _ in range(3))
     scale = 128 ** -0.5
-    out, smax, ssum = K.fused_attention(q.to(DEV), k.to(DEV), v.to(DEV), scale, causal)
+    out, smax, ssum = K.fused_attention(q.to(DEV), k.to(DEV), v.to(DEV), scale, causal, waves=waves)
     o_ref, m_ref, l_ref = O.attention_bf16(bits(q), bits(k), bits(v), scale, causal)
     err = np.abs(O.bf16_bits_to_f32(bits(out)) - O.bf16_bits_to_f32(o_ref)).max()
     assert err <= 2e-2, err
@@ -73,6 +85,8 @@ def test_attention_causality_and_sdpa_full_size_slice(K):
     q, k, v = (torch.randn(B, N, S, 128, device=DEV).bfloat16() for _ in range(3))
     scale = 128 ** -0.5
     out, smax, ssum = K.fused_attention(q, k, v, scale, True)
+    out8, smax8, ssum8 = K.fused_attention(q, k, v, scale, True, waves=8)
+    assert torch.equal(out, out8) and torch.equal(smax, smax8) and torch.equal(ssum, ssum8)
     k2, v2 = k.clone(), v.clone()
     k2[:, :, 2048:] = torch.randn_like(k2[:, :, 2048:])
     v2[:, :, 2048:] = torch.randn_like(v2[:, :, 2048:])
