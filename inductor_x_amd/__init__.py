@@ -1,9 +1,103 @@
-"""MI355X-native TorchInductor backend (gfx950).  Importing the package has
-side effects only, like the reference's import hook
-(reference inductor_x/__init__.py:1-63); see `_register` below.
+"""MI355X-native TorchInductor backend (gfx950).
+
+Importing the package has side effects only, like the reference's import hook
+(reference inductor_x/__init__.py:1-63): it registers the HIP scheduling and a
+wrapper code generator for the GPU device type, a device-op override whose
+generated wrappers fetch the raw stream from this package, a device interface,
+the lowering / decomposition table patches and the fused-attention graph
+pattern.  After `import inductor_x_amd`, `torch.compile(fn)` on PyTorch-ROCm
+emits hand-templated HIP kernels launched through the C-ABI launcher; no Triton
+is generated.
 """
 from __future__ import annotations
 
 __version__ = "0.1.0"
 
+import torch
+
 from . import config  # noqa: F401
+
+DEVICE_TYPE = "cuda"  # PyTorch-ROCm exposes AMD GPUs under this device type
+
+
+def get_current_raw_stream(device) -> int:
+    """Raw hipStream_t of torch's current stream as an integer
+    (reference inductor_x/__init__.py:26-27)."""
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _inductor_register_backend_for_device() -> None:
+    from torch._inductor.codegen.common import register_backend_for_device
+
+    from .codegen.scheduling import HipScheduling
+    from .codegen.wrapper import HipWrapperCodegen
+
+    register_backend_for_device(DEVICE_TYPE, HipScheduling, HipWrapperCodegen)
+
+
+def _inductor_register_device_op_overrides() -> None:
+    from torch._inductor.codegen.common import get_device_op_overrides, register_device_op_overrides
+
+    # Inductor fills its table of per-device overrides lazily and only while the
+    # table is empty (importing any one device's module makes it non-empty); ask
+    # for an entry first so the CPU and other defaults are in place before the
+    # GPU entry is replaced.
+    get_device_op_overrides("cpu")
+    from torch._inductor.codegen.cuda.device_op_overrides import CUDADeviceOpOverrides
+
+    class HipDeviceOpOverrides(CUDADeviceOpOverrides):
+        def import_get_raw_stream_as(self, name: str) -> str:
+            return f"from inductor_x_amd import get_current_raw_stream as {name}"
+
+    register_device_op_overrides(DEVICE_TYPE, HipDeviceOpOverrides())
+
+
+def _register_device_interface() -> None:
+    from torch._dynamo.device_interface import CudaInterface, register_interface_for_device
+
+    class HipInterface(CudaInterface):
+        """reference inductor_x/__init__.py:40-52"""
+
+        @staticmethod
+        def is_available() -> bool:
+            return torch.cuda.device_count() > 0
+
+        @staticmethod
+        def get_compute_capability(device=None):
+            # the code object target, e.g. "gfx950"
+            if torch.cuda.device_count() == 0:
+                return "gfx950"
+            return torch.cuda.get_device_properties(device).gcnArchName.split(":")[0]
+
+    register_interface_for_device(DEVICE_TYPE, HipInterface)
+
+
+_registered = False
+
+
+def _register() -> None:
+    global _registered
+    if _registered:
+        return
+    _registered = True
+    from torch._inductor import lowering as inductor_lowering
+
+    from . import codegen  # noqa: F401  (installs the Reduction.num_splits stub)
+    from .codegen.ir import install_num_splits_stub
+    from .decomposition import _register_inductor_decompositions
+    from .lowering import _register_inductor_fallbacks, make_reduction
+
+    config.apply_inductor_settings()
+    _inductor_register_backend_for_device()
+    _inductor_register_device_op_overrides()
+    _register_device_interface()
+    install_num_splits_stub()
+    inductor_lowering.make_reduction = make_reduction
+    _register_inductor_fallbacks()
+    _register_inductor_decompositions()
+    from . import fusion_attention_graph
+
+    fusion_attention_graph.register_fx_pass()
+
+
+_register()

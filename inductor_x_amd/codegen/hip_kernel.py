@@ -1,0 +1,1175 @@
+"""Fused Inductor node -> HIP source for gfx950.
+
+Counterpart of the reference's kernel code generator
+(reference inductor_x/codegen/triton.py): where that file prints Triton text
+with N-D block indices, this one prints C++ against the hand-written template
+library in csrc/mi/codegen.h.  Three code shapes exist:
+
+  pointwise  (reference family F1/F2, triton.py:693-815)    one 16-byte vector per thread
+  row        (F3/F4/F6, triton.py:1103-1262)                TPR threads per row, DPP + LDS combine
+  column     (F5 + the outer-reduce hint, triton.py:1003-1031,
+              split_tiling.py:159-165)                      two-pass workgroup partials
+
+The shape is chosen from the strides of the accesses (which axis is the
+contiguous one), not from tags put on the IR node.
+
+Values are either thread-uniform scalars or mi::V<T, VEC> register vectors
+along the contiguous axis.  The generator tracks which is which only where it
+must (to choose between a vector load, a scalar load and a gather); the C++
+overloads do the rest.
+"""
+from __future__ import annotations
+
+import dataclasses
+import itertools
+import math
+from typing import Any, Optional, Sequence, Union
+
+import sympy
+
+import torch
+from torch._inductor import config as inductor_config, ir
+from torch._inductor.codegen.common import (
+    CSEVariable,
+    DeferredLine,
+    IndentedBuffer,
+    OpOverrides,
+    SizeArg,
+    TensorArg,
+    WorkspaceArg,
+)
+from torch._inductor.codegen.simd import (
+    DisableReduction,
+    EnableReduction,
+    IterationRangesEntry,
+    SIMDKernel,
+)
+from torch._inductor.ops_handler import StoreMode
+from torch._inductor.utils import sympy_subs
+from torch._inductor.virtualized import V
+from torch.utils._ordered_set import OrderedSet
+from torch.utils._sympy.functions import FloorDiv, ModularIndexing
+from torch.utils._sympy.printers import ExprPrinter
+from torch.utils._sympy.value_ranges import ValueRanges
+
+from .. import config as backend_config
+
+DTYPE_TO_HIP = {
+    torch.float32: "float",
+    torch.float64: "double",
+    torch.float16: "mi::f16_t",
+    torch.bfloat16: "mi::bf16_t",
+    torch.int8: "signed char",
+    torch.uint8: "unsigned char",
+    torch.int16: "short",
+    torch.int32: "int",
+    torch.int64: "mi::i64",
+    torch.bool: "bool",
+}
+
+# struct codes for the launcher's argument packing
+DTYPE_TO_STRUCT = {torch.int32: "i", torch.int64: "q", torch.float32: "f", torch.float64: "d"}
+
+
+class VecConstraintError(Exception):
+    """The chosen vector width does not fit an index that showed up late."""
+
+
+class UnsupportedHipCodegen(NotImplementedError):
+    pass
+
+
+def dtype_nbytes(dtype: torch.dtype) -> int:
+    return torch.empty((), dtype=dtype).element_size()
+
+
+# ---------------------------------------------------------------------------
+# index expression printer
+# ---------------------------------------------------------------------------
+class HipExprPrinter(ExprPrinter):
+    """sympy index expression -> C++.  Indices are non-negative, so floor
+    division and modular indexing are the plain C operators; the same text
+    works for scalars and for mi::V<int, N> lane vectors."""
+
+    def _print_FloorDiv(self, expr: sympy.Expr) -> str:
+        x, div = expr.args
+        return f"(({self.doprint(x)}) / ({self.doprint(div)}))"
+
+    def _print_ModularIndexing(self, expr: sympy.Expr) -> str:
+        x, div, mod = expr.args
+        xs = self.doprint(x)
+        if div != 1:
+            xs = f"(({xs}) / ({self.doprint(div)}))"
+        return f"(({xs}) % ({self.doprint(mod)}))"
+
+    def _print_Min(self, expr: sympy.Expr) -> str:
+        args = [self.doprint(a) for a in expr.args]
+        out = args[0]
+        for a in args[1:]:
+            out = f"mi::minimum({out}, {a})"
+        return out
+
+    def _print_Max(self, expr: sympy.Expr) -> str:
+        args = [self.doprint(a) for a in expr.args]
+        out = args[0]
+        for a in args[1:]:
+            out = f"mi::maximum({out}, {a})"
+        return out
+
+    def _print_Abs(self, expr: sympy.Expr) -> str:
+        return f"mi::abs({self.doprint(expr.args[0])})"
+
+    def _print_Where(self, expr: sympy.Expr) -> str:
+        c, p, q = (self.doprint(a) for a in expr.args)
+        return f"mi::where({c}, {p}, {q})"
+
+    def _print_ToFloat(self, expr: sympy.Expr) -> str:
+        return f"mi::cast<float>({self.doprint(expr.args[0])})"
+
+    def _print_Float(self, expr: sympy.Expr) -> str:
+        return f"{float(expr)!r}f"
+
+    def _print_PowByNatural(self, expr: sympy.Expr) -> str:
+        x, y = expr.args
+        if isinstance(y, sympy.Integer) and 0 <= int(y) <= 8:
+            xs = self.doprint(x)
+            return "(" + " * ".join([f"({xs})"] * int(y)) + ")" if int(y) else "1"
+        return f"mi::pow({self.doprint(x)}, {self.doprint(y)})"
+
+    def _print_IntTrueDiv(self, expr: sympy.Expr) -> str:
+        a, b = expr.args
+        return f"mi::truediv({self.doprint(a)}, {self.doprint(b)})"
+
+    def _print_FloorToInt(self, expr: sympy.Expr) -> str:
+        return f"mi::cast<mi::i64>(mi::floor({self.doprint(expr.args[0])}))"
+
+    def _print_TruncToInt(self, expr: sympy.Expr) -> str:
+        return f"mi::cast<mi::i64>(mi::trunc({self.doprint(expr.args[0])}))"
+
+
+hexpr = HipExprPrinter().doprint
+
+
+def value_to_hip(val: Union[float, int, bool, str, CSEVariable], dtype: Optional[torch.dtype] = None) -> str:
+    if isinstance(val, bool):
+        return "true" if val else "false"
+    if isinstance(val, float):
+        if math.isinf(val):
+            return "__builtin_inff()" if val > 0 else "(-__builtin_inff())"
+        if val != val:
+            return "__builtin_nanf(\"\")"
+        if dtype == torch.float64:
+            return repr(val)
+        return f"{val!r}f"
+    if isinstance(val, int):
+        if dtype is not None and dtype.is_floating_point:
+            return f"{float(val)!r}" + ("" if dtype == torch.float64 else "f")
+        if abs(val) > 2**31 - 1:
+            return f"{val}LL"
+        return str(val)
+    return str(val)
+
+
+# ---------------------------------------------------------------------------
+# op overrides
+# ---------------------------------------------------------------------------
+class HipOverrides(OpOverrides):
+    """One C++ expression per Inductor op.  16-bit floats are computed in fp32
+    and only rounded at stores (reference inductor_x/codegen/triton.py:1431-1433),
+    so to_dtype to a 16-bit float is a cast to float.  maximum / minimum
+    propagate NaN as torch does (the reference's helper drops it,
+    reference inductor_x/npu_triton_helpers.py:8-18)."""
+
+    @staticmethod
+    def _compute_type(dtype: torch.dtype) -> str:
+        if dtype in (torch.float16, torch.bfloat16):
+            return "float"
+        return DTYPE_TO_HIP[dtype]
+
+    @staticmethod
+    def to_dtype(x, dtype: torch.dtype, src_dtype: Optional[torch.dtype] = None, use_compute_types: bool = True) -> str:
+        if dtype == torch.bool:
+            return f"({x} != 0)"
+        return f"mi::cast<{HipOverrides._compute_type(dtype)}>({x})"
+
+    @staticmethod
+    def to_dtype_bitcast(x, dtype: torch.dtype, src_dtype: torch.dtype) -> str:
+        if src_dtype in (torch.float16, torch.bfloat16):
+            x = f"mi::cast<{DTYPE_TO_HIP[src_dtype]}>({x})"
+        out = f"mi::bitcast<{DTYPE_TO_HIP[dtype]}>({x})"
+        if dtype in (torch.float16, torch.bfloat16):
+            out = f"mi::cast<float>({out})"
+        return out
+
+    @staticmethod
+    def constant(val, dtype: torch.dtype) -> str:
+        text = value_to_hip(val, dtype)
+        if dtype in (torch.int64,) and isinstance(val, int) and not isinstance(val, bool):
+            return f"static_cast<mi::i64>({text})"
+        return text
+
+    @staticmethod
+    def index_expr(expr: sympy.Expr, dtype: torch.dtype) -> str:
+        kernel: HipKernel = V.kernel
+        idx = kernel.prepare_indexing(expr)
+        text = kernel.index_to_vec_str(idx) if kernel.index_is_lane_varying(idx) else kernel.index_to_str(idx)
+        var = kernel.cse.generate(kernel.compute, f"mi::cast<{HipOverrides._compute_type(dtype)}>({text})", dtype=dtype)
+        var.is_vec = kernel.index_is_lane_varying(idx)
+        return var
+
+    @staticmethod
+    def masked(mask, body, other) -> str:
+        # Evaluate the body with loads guarded by the mask, then select.
+        kernel: HipKernel = V.kernel
+        with kernel.mask_loads(mask, other) as new_mask:
+            result = body()
+        if isinstance(result, CSEVariable) and result.dtype is not None:
+            other_s = value_to_hip(other, result.dtype)
+        else:
+            other_s = value_to_hip(other)
+        return f"mi::where({new_mask}, {result}, {other_s})"
+
+    @staticmethod
+    def where(a, b, c) -> str:
+        return f"mi::where({a}, {b}, {c})"
+
+    @staticmethod
+    def maximum(a, b) -> str:
+        return f"mi::maximum({a}, {b})"
+
+    @staticmethod
+    def minimum(a, b) -> str:
+        return f"mi::minimum({a}, {b})"
+
+    @staticmethod
+    def relu(x) -> str:
+        return f"mi::relu({x})"
+
+    @staticmethod
+    def sigmoid(x) -> str:
+        return f"mi::sigmoid({x})"
+
+    @staticmethod
+    def logical_and(a, b) -> str:
+        return f"mi::logical_and({a}, {b})"
+
+    @staticmethod
+    def logical_or(a, b) -> str:
+        return f"mi::logical_or({a}, {b})"
+
+    @staticmethod
+    def logical_xor(a, b) -> str:
+        return f"mi::logical_xor({a}, {b})"
+
+    @staticmethod
+    def logical_not(a) -> str:
+        return f"mi::logical_not({a})"
+
+    @staticmethod
+    def truediv(a, b) -> str:
+        return f"mi::truediv({a}, {b})"
+
+    @staticmethod
+    def floordiv(a, b) -> str:
+        return f"mi::floordiv({a}, {b})"
+
+    @staticmethod
+    def truncdiv(a, b) -> str:
+        return f"mi::truncdiv({a}, {b})"
+
+    @staticmethod
+    def remainder(a, b) -> str:
+        if isinstance(a, CSEVariable) and a.dtype is not None and a.dtype.is_floating_point:
+            return f"mi::remainder_f({a}, {b})"
+        return f"mi::pymod({a}, {b})"
+
+    @staticmethod
+    def mod(a, b) -> str:
+        if isinstance(a, CSEVariable) and a.dtype is not None and a.dtype.is_floating_point:
+            return f"mi::fmod({a}, {b})"
+        return f"({a} % {b})"
+
+    @staticmethod
+    def fmod(a, b) -> str:
+        return f"mi::fmod({a}, {b})"
+
+    @staticmethod
+    def pow(a, b) -> str:
+        return f"mi::pow({a}, {b})"
+
+    @staticmethod
+    def square(x) -> str:
+        return f"({x} * {x})"
+
+    @staticmethod
+    def neg(x) -> str:
+        return f"(-{x})"
+
+    @staticmethod
+    def fma(a, b, c) -> str:
+        return f"mi::fma({a}, {b}, {c})"
+
+    @staticmethod
+    def isnan(x) -> str:
+        return f"mi::isnan({x})"
+
+    @staticmethod
+    def isinf(x) -> str:
+        return f"mi::isinf({x})"
+
+    @staticmethod
+    def signbit(x) -> str:
+        return f"mi::signbit({x})"
+
+    @staticmethod
+    def sign(x) -> str:
+        return f"mi::sign({x})"
+
+    @staticmethod
+    def copysign(a, b) -> str:
+        return f"mi::copysign({a}, {b})"
+
+    @staticmethod
+    def atan2(a, b) -> str:
+        return f"mi::atan2({a}, {b})"
+
+    @staticmethod
+    def reciprocal(x) -> str:
+        return f"mi::reciprocal({x})"
+
+    @staticmethod
+    def libdevice_exp(x) -> str:
+        return f"mi::exp({x})"
+
+    @staticmethod
+    def libdevice_sqrt(x) -> str:
+        return f"mi::sqrt({x})"
+
+    @staticmethod
+    def libdevice_sigmoid(x) -> str:
+        return f"mi::sigmoid({x})"
+
+    @staticmethod
+    def libdevice_log(x) -> str:
+        return f"mi::log({x})"
+
+    @staticmethod
+    def libdevice_abs(x) -> str:
+        return f"mi::abs({x})"
+
+    @staticmethod
+    def identity(x) -> str:
+        return f"{x}"
+
+    @staticmethod
+    def load_seed(name: str, offset) -> str:
+        raise UnsupportedHipCodegen("random number generation is not generated; the op falls back to eager")
+
+
+def _add_unary(name: str) -> None:
+    def fn(x) -> str:
+        return f"mi::{name}({x})"
+
+    fn.__name__ = name
+    setattr(HipOverrides, name, staticmethod(fn))
+
+
+for _n in (
+    "exp", "exp2", "expm1", "log", "log2", "log10", "log1p", "sqrt", "rsqrt", "sin", "cos", "tan", "tanh",
+    "sinh", "cosh", "asin", "acos", "atan", "erf", "erfc", "lgamma", "floor", "ceil", "trunc", "round", "abs",
+):
+    _add_unary(_n)
+
+
+# ---------------------------------------------------------------------------
+# CSE variable with vector-ness
+# ---------------------------------------------------------------------------
+class HipCSEVariable(CSEVariable):
+    def __init__(self, name: str, bounds: ValueRanges[Any], dtype: Optional[torch.dtype] = None, shape=None):
+        super().__init__(name, bounds, dtype, shape=shape)
+        # True when the value differs between the lanes of the thread's vector
+        self.is_vec = False
+
+    def update_on_args(self, name: str, args: Any, kwargs: Any) -> None:
+        def any_vec(a) -> bool:
+            if isinstance(a, HipCSEVariable):
+                return a.is_vec
+            if isinstance(a, (list, tuple)):
+                return any(any_vec(b) for b in a)
+            return False
+
+        if any_vec(args) or any_vec(list(kwargs.values())):
+            self.is_vec = True
+
+
+REDUCTION_KIND = {
+    "sum": "mi::RedSum",
+    "prod": "mi::RedProd",
+    "max": "mi::RedMax",
+    "min": "mi::RedMin",
+    "any": "mi::RedAny",
+    "argmax": "mi::RedArgMax",
+    "argmin": "mi::RedArgMin",
+    "welford_reduce": "mi::RedWelford",
+}
+REDUCTION_WORDS = {"sum": 1, "prod": 1, "max": 1, "min": 1, "any": 1, "argmax": 2, "argmin": 2, "welford_reduce": 3}
+
+
+@dataclasses.dataclass
+class ColReduction:
+    kind: str  # key of REDUCTION_KIND
+    acc: str  # accumulator variable in the partial kernel
+    result: str  # merged state variable in the final kernel
+    value: str
+    ws_offset_words: int  # offset in units of nsplit * xnumel floats
+
+
+class HipKernel(SIMDKernel):
+    overrides = HipOverrides  # type: ignore[assignment]
+    suffix = ";"
+    newvar_prefix = "auto "
+    kexpr = staticmethod(hexpr)
+    sexpr = staticmethod(hexpr)
+    allow_block_ptr = False
+
+    MAX_ROW_THREADS = 1024
+
+    def __init__(self, tiling: dict[str, sympy.Expr], force_vec: Optional[int] = None, **kwargs: Any) -> None:
+        self.force_vec = force_vec
+        self.mode = "pointwise"
+        self.vec = 1
+        self.block = 256
+        self.tpr = 256
+        self.col_ct = 128
+        self.col_rl = 8
+        self.vec_tree_prefix = "x"
+        self.lane_syms: OrderedSet[sympy.Symbol] = OrderedSet()
+        self.x_entries: list[IterationRangesEntry] = []
+        self.r_entries: list[IterationRangesEntry] = []
+        self.r_full = False
+        self.prologue = IndentedBuffer()
+        self.row_loop_accs: list[str] = []
+        self.col_reductions: list[ColReduction] = []
+        self.partial_body = IndentedBuffer()
+        self.final_body = IndentedBuffer()
+        self.ws_words = 0
+        self.phase_bodies_started = False
+        self.acc_ids = itertools.count()
+        self.red_stores = IndentedBuffer()
+        self._result_defs: list[str] = []
+        self._result_defs_col: list[str] = []
+        self.mode_decided = False
+        super().__init__(tiling, **kwargs)
+        self.n_reduction_phases = self._count_reduction_phases()
+
+    # -- framework hooks --------------------------------------------------
+    def create_cse_var(self, *args: Any, **kwargs: Any) -> HipCSEVariable:
+        return HipCSEVariable(*args, **kwargs)
+
+    def dtype_to_str(self, dtype: torch.dtype) -> str:
+        return DTYPE_TO_HIP[dtype]
+
+    def should_use_persistent_reduction(self) -> bool:
+        """Rows that fit one register vector per thread of a single workgroup are
+        kept in registers (the reference's limit is 1024 elements,
+        reference inductor_x/codegen/triton.py:401-424)."""
+        if not self.features.is_reduction():
+            return False
+        rnumel = self.features.reduction_numel
+        if not isinstance(rnumel, (int, sympy.Integer)):
+            return False
+        return int(rnumel) <= self.MAX_ROW_THREADS * 8 and int(rnumel) <= backend_config.persistent_reduction_max
+
+    def _col_split_ok(self) -> bool:
+        """The two-kernel column shape needs everything that follows the (single)
+        reduction loop to be a function of the kept axis only: the second kernel
+        has no loop over the reduced axis."""
+        seen_reduction = False
+        xnumel = self.numels.get("x")
+        for n in self.features.node_schedule:
+            if n is EnableReduction or n is DisableReduction:
+                continue
+            if getattr(n, "is_reduction", lambda: False)():
+                seen_reduction = True
+                continue
+            if seen_reduction:
+                try:
+                    numel = n.group[1][0]
+                except Exception:
+                    return False
+                if V.graph.sizevars.simplify(numel - xnumel) != 0:
+                    return False
+        return seen_reduction
+
+    def _count_reduction_phases(self) -> int:
+        phases, inside = 0, False
+        for n in self.features.node_schedule:
+            if n is EnableReduction or n is DisableReduction:
+                inside = False
+                continue
+            is_red = getattr(n, "is_reduction", lambda: False)()
+            if is_red and not inside:
+                phases += 1
+            inside = is_red
+        return phases
+
+    # -- mode / vector width ----------------------------------------------
+    def _tree(self, prefix: str):
+        for t in self.range_trees:
+            if t.prefix == prefix:
+                return t
+        return None
+
+    def _static_numel(self, prefix: str) -> Optional[int]:
+        t = self._tree(prefix)
+        if t is None:
+            return None
+        n = V.graph.sizevars.simplify(t.numel)
+        return int(n) if isinstance(n, (int, sympy.Integer)) else None
+
+    def _unit_stride_symbols(self, index: sympy.Expr) -> list[sympy.Symbol]:
+        out = []
+        for s in index.free_symbols:
+            if s in self.range_tree_nodes:
+                try:
+                    c = index.coeff(s)
+                except Exception:
+                    continue
+                if c == 1 and s not in (index - s).free_symbols:
+                    out.append(s)
+        return out
+
+    def finalize_indexing(self, indices: Sequence[sympy.Expr]) -> None:
+        """Choose the code shape and the vector width from every index the fused
+        node will use (the reference's find_lowest_dimension / select_tiling_axis
+        step, reference inductor_x/codegen/split_tiling.py:85-154,188-239)."""
+        prepared = []
+        for idx in indices:
+            try:
+                prepared.append(self.prepare_indexing(idx))
+            except Exception:
+                continue
+        is_red = self.features.is_reduction()
+        r_tree = self._tree("r0_")
+        if not is_red:
+            self.mode = "pointwise"
+            self.vec_tree_prefix = "x"
+        else:
+            r_unit = x_unit = 0
+            for idx in prepared:
+                for s in self._unit_stride_symbols(idx):
+                    entry = self.range_tree_nodes[s]
+                    if entry.divisor != 1:
+                        continue
+                    if entry.root.prefix == "r0_":
+                        r_unit += 1
+                    elif entry.root.prefix == "x":
+                        x_unit += 1
+            if (
+                r_unit == 0
+                and x_unit > 0
+                and self.n_reduction_phases == 1
+                and self._col_split_ok()
+                and not self.persistent_reduction_blocks_col()
+            ):
+                self.mode = "col"
+                self.vec_tree_prefix = "x"
+                # the reduced axis is always walked in a loop here, and what
+                # follows the loop goes to the second kernel
+                self.persistent_reduction = False
+                for t in self.range_trees:
+                    if t.is_reduction:
+                        t.is_loop = True
+            else:
+                self.mode = "row"
+                self.vec_tree_prefix = "r0_"
+        self._choose_vec(prepared)
+        self._choose_geometry()
+        self.mode_decided = True
+
+    def persistent_reduction_blocks_col(self) -> bool:
+        """Column shape is for long reduced axes; a short strided reduction is
+        cheaper as a (gathering) row kernel with no workspace round trip."""
+        rnumel = self._static_numel("r0_")
+        return rnumel is not None and rnumel < 64
+
+    def _buffers_min_itemsize(self) -> int:
+        size = 4
+        for n in self.features.scheduler_nodes():
+            for dep in itertools.chain(n.read_writes.reads, n.read_writes.writes):
+                try:
+                    size = min(size, dtype_nbytes(V.graph.get_dtype(dep.name)))
+                except Exception:
+                    pass
+        return max(size, 1)
+
+    def _choose_vec(self, prepared: Sequence[sympy.Expr]) -> None:
+        vec = max(backend_config.vector_bytes // self._buffers_min_itemsize(), 1)
+        if self.force_vec is not None:
+            vec = self.force_vec
+        numel = self._static_numel(self.vec_tree_prefix)
+        if numel is None:
+            vec = 1
+        while vec > 1 and not self._vec_ok(vec, numel):
+            vec //= 2
+        self.vec = vec
+
+    def _vec_ok(self, vec: int, numel: Optional[int]) -> bool:
+        if numel is None or numel % vec:
+            return False
+        for entry in self.range_tree_nodes.values():
+            if entry.root.prefix != self.vec_tree_prefix:
+                continue
+            if not self._entry_fits_vec(entry, vec):
+                return False
+        return True
+
+    @staticmethod
+    def _entry_fits_vec(entry: IterationRangesEntry, vec: int) -> bool:
+        div, length = entry.divisor, entry.length
+        if not isinstance(div, (int, sympy.Integer)) or not isinstance(length, (int, sympy.Integer)):
+            return vec == 1
+        div, length = int(div), int(length)
+        if div == 1:
+            return length % vec == 0
+        return div % vec == 0
+
+    def _choose_geometry(self) -> None:
+        from ..hip_heuristics import next_power_of_2
+
+        if self.mode == "row":
+            rnumel = self._static_numel("r0_")
+            vectors = max(-(-rnumel // self.vec), 1) if rnumel is not None else 256
+            if self.persistent_reduction:
+                self.tpr = min(max(next_power_of_2(vectors), 1), self.MAX_ROW_THREADS)
+                self.r_full = rnumel is not None and self.tpr * self.vec == rnumel
+                if self.tpr * self.vec < (rnumel or 0):
+                    # cannot hold the row in one vector per thread: walk it instead
+                    self.persistent_reduction = False
+                    for t in self.range_trees:
+                        if t.is_reduction:
+                            t.is_loop = True
+                    self.tpr = 256
+            else:
+                self.tpr = min(max(next_power_of_2(vectors), 1), 256)
+            self.block = max(256, self.tpr)
+        elif self.mode == "col":
+            xnumel = self._static_numel("x")
+            groups = max(-(-(xnumel or 512) // self.vec), 1)
+            self.col_ct = min(next_power_of_2(groups), 128)
+            self.col_rl = max(1024 // self.col_ct, 1)
+            self.block = self.col_ct * self.col_rl
+        else:
+            self.block = 256
+
+    # -- lane-varying index handling --------------------------------------
+    def _is_lane_symbol(self, s: sympy.Symbol) -> bool:
+        entry = self.range_tree_nodes.get(s)
+        return (
+            entry is not None
+            and self.vec > 1
+            and entry.root.prefix == self.vec_tree_prefix
+            and entry.divisor == 1
+        )
+
+    def index_is_lane_varying(self, index: sympy.Expr) -> bool:
+        if self.vec == 1:
+            return False
+        for s in index.free_symbols:
+            if self._is_lane_symbol(s):
+                return True
+            v = self.cse.varname_map.get(str(s)) if hasattr(self.cse, "varname_map") else None
+            if isinstance(v, HipCSEVariable) and v.is_vec:
+                return True
+        return False
+
+    def index_to_vec_str(self, index: sympy.Expr) -> str:
+        """Index with every lane-varying range variable replaced by its lane
+        vector (x0 -> x0_v = x0 + iota)."""
+        repl = {s: sympy.Symbol(f"{s}_v", integer=True) for s in index.free_symbols if self._is_lane_symbol(s)}
+        return self.index_to_str(sympy_subs(index, repl))
+
+    def classify_index(self, index: sympy.Expr) -> str:
+        """'uniform' (same address for all lanes), 'contiguous' (lane i reads
+        base + i) or 'gather'."""
+        if self.vec == 1:
+            return "uniform"
+        lane_syms = [s for s in index.free_symbols if self._is_lane_symbol(s)]
+        tmp_vec = False
+        for s in index.free_symbols:
+            v = self.cse.varname_map.get(str(s))
+            if isinstance(v, HipCSEVariable) and v.is_vec:
+                tmp_vec = True
+        if tmp_vec:
+            return "gather"
+        if not lane_syms:
+            return "uniform"
+        lane = sympy.Symbol("lane_", integer=True, nonnegative=True)
+        shifted = sympy_subs(index, {s: s + lane for s in lane_syms})
+        diff = sympy.expand(shifted - index)
+        if diff == lane:
+            return "contiguous"
+        if diff == 0:
+            return "uniform"
+        return "gather"
+
+    def index_is_aligned(self, index: sympy.Expr) -> bool:
+        """True when the address of lane 0 is provably a multiple of the vector
+        width (lane-varying variables are multiples of it by construction)."""
+        lane_syms = [s for s in index.free_symbols if self._is_lane_symbol(s)]
+        base = sympy.expand(sympy_subs(index, {s: sympy.Integer(0) for s in lane_syms}))
+        try:
+            return bool(V.graph.sizevars.statically_known_multiple_of(base, self.vec))
+        except Exception:
+            return False
+
+    def _buffer_aligned(self, name: str) -> bool:
+        return name not in V.graph.unaligned_buffers
+
+    # -- range variables ---------------------------------------------------
+    def codegen_iteration_ranges_entry(self, entry: IterationRangesEntry) -> None:
+        """Range variables are only recorded here; their text is produced when a
+        body is assembled, once the code shape and the vector width are known."""
+        if self.mode_decided and entry.root.prefix == self.vec_tree_prefix and not self._entry_fits_vec(entry, self.vec):
+            raise VecConstraintError(f"{entry.name}: divisor {entry.divisor}, length {entry.length}, vec {self.vec}")
+        (self.r_entries if entry.root.is_reduction else self.x_entries).append(entry)
+
+    def _entry_code(self, entries: Sequence[IterationRangesEntry], lane_vectors: bool = True) -> IndentedBuffer:
+        buf = IndentedBuffer()
+        for entry in entries:
+            expr = self.rename_indexing(entry.expr)
+            buf.writeline(f"const {self.index_dtype} {entry.name} = {self.kexpr(expr)};")
+            if entry.divisor == 1 and entry.root.prefix == self.vec_tree_prefix:
+                rhs = f"{entry.name} + mi::iota<VEC>()" if (lane_vectors and self.vec > 1) else entry.name
+                buf.writeline(f"const auto {entry.name}_v = {rhs};")
+        return buf
+
+    # -- masks ---------------------------------------------------------------
+    def _load_mask_for(self, index: sympy.Expr) -> Optional[str]:
+        """Guard for a load: the row shape masks accesses that move along the
+        reduced axis (the tail of the last vector round); an enclosing
+        ops.masked adds its own condition.  Kept-axis indices are clamped into
+        range instead of masked, and the column shape only runs live columns."""
+        parts = []
+        if self.mode == "row" and self.inside_reduction and not self.r_full and self._index_uses_tree(index, "r0_"):
+            parts.append("rmask")
+        if self._load_mask:
+            parts.append(str(self._load_mask))
+        if not parts:
+            return None
+        return parts[0] if len(parts) == 1 else f"({parts[0]} && {parts[1]})"
+
+    # -- loads / stores ------------------------------------------------------
+    def load(self, name: str, index: sympy.Expr) -> CSEVariable:
+        var = self.args.input(name)
+        indirect = self.is_indirect_indexing(index)
+        index = self.prepare_indexing(index)
+        dtype = V.graph.get_dtype(name)
+        kind = self.classify_index(index)
+        mask = self._load_mask_for(index)
+        other = value_to_hip(self._load_other if self._load_mask else 0, dtype if dtype.is_floating_point else None)
+        if kind == "contiguous":
+            aligned = self.index_is_aligned(index) and self._buffer_aligned(name)
+            ptr = f"{var} + ({self.index_to_str(index)})"
+            if mask is None:
+                line = f"mi::vload<VEC>({ptr})" if aligned else f"mi::vload_u<VEC>({ptr})"
+            else:
+                line = f"mi::vload_m<VEC>({ptr}, {mask}, {other})"
+            is_vec = True
+        elif kind == "uniform":
+            if mask is None:
+                line = f"{var}[{self.index_to_str(index)}]"
+            else:
+                line = f"mi::gather_m({var}, {self.index_to_str(index)}, {mask}, {other})"
+            is_vec = False
+        else:
+            idx = self.index_to_vec_str(index)
+            line = f"mi::gather({var}, {idx})" if mask is None else f"mi::gather_m({var}, {idx}, {mask}, {other})"
+            is_vec = True
+        if dtype in (torch.float16, torch.bfloat16):
+            line = f"mi::cast<float>({line})"
+            dtype = torch.float32
+        # a load whose address or guard is itself computed must follow that computation
+        buf = self.compute if (indirect or self._load_mask) else self.loads
+        out = self.cse.generate(buf, line, dtype=dtype)
+        if isinstance(out, HipCSEVariable):
+            out.is_vec = out.is_vec or is_vec
+        return out
+
+    def _index_uses_tree(self, index: sympy.Expr, prefix: str) -> bool:
+        for s in index.free_symbols:
+            e = self.range_tree_nodes.get(s)
+            if e is not None and e.root.prefix == prefix:
+                return True
+        return False
+
+    def store(self, name: str, index: sympy.Expr, value: CSEVariable, mode: StoreMode = None) -> None:
+        var = self.args.output(name)
+        index = self.prepare_indexing(index)
+        if mode is not None:
+            raise UnsupportedHipCodegen(f"store mode {mode}")
+        kind = self.classify_index(index)
+        if self.mode == "row":
+            if self.inside_reduction:
+                mask = "xmask" if self.r_full else "(rmask && xmask)"
+            else:
+                mask = "(xmask && rlane == 0)"
+        elif self.mode == "col":
+            # inside the reduction loop only live columns run; afterwards (final
+            # kernel) one of the SL lanes of a column stores
+            mask = None if (self.inside_reduction and not self.phase_bodies_started) else "(live && sl == 0)"
+        else:
+            mask = None
+        if kind == "contiguous":
+            aligned = self.index_is_aligned(index) and self._buffer_aligned(name)
+            ptr = f"{var} + ({self.index_to_str(index)})"
+            if mask is None:
+                line = f"mi::vstore<VEC>({ptr}, {value});" if aligned else f"mi::vstore_u<VEC>({ptr}, {value});"
+            else:
+                line = f"mi::vstore_m<VEC>({ptr}, {value}, {mask});"
+        elif kind == "uniform":
+            line = f"mi::vstore<1>({var} + ({self.index_to_str(index)}), {value});"
+            if mask is not None:
+                line = f"if ({mask}) {{ {line} }}"
+        else:
+            idx = self.index_to_vec_str(index)
+            line = f"mi::scatter_m<VEC>({var}, {idx}, {value}, {mask or 'true'});"
+        self.stores.writeline(DeferredLine(name, line))
+
+    def store_reduction(self, name: str, index: sympy.Expr, value: CSEVariable) -> None:
+        """The reduced value is uniform for the row (or column); one thread writes it."""
+        var = self.args.output(name)
+        index = self.prepare_indexing(index)
+        guard = "(live && sl == 0)" if self.mode == "col" else "(xmask && rlane == 0)"
+        line = f"if {guard} {{ mi::vstore<1>({var} + ({self.index_to_str(index)}), {value}); }}"
+        self.red_stores.writeline(DeferredLine(name, line))
+
+    def check_bounds(self, expr: sympy.Expr, size: sympy.Expr, lower: bool, upper: bool) -> None:
+        # Out-of-range indices are undefined behaviour in the source program; no
+        # device-side assert is generated.
+        return
+
+    # -- reductions -----------------------------------------------------------
+    def reduction(self, dtype, src_dtype, reduction_type, value):
+        cache_key = (src_dtype, reduction_type, value)
+        if cache_key in self.cse.reduction_cache:
+            return self.cse.reduction_cache[cache_key]
+        result = self._reduction_nocache(dtype, src_dtype, reduction_type, value)
+        self.cse.reduction_cache[cache_key] = result
+        return result
+
+    def _r_index_str(self) -> str:
+        return "(r0_index + mi::iota<VEC>())" if (self.mode == "row" and self.vec > 1) else "r0_index"
+
+    def _reduction_nocache(self, dtype, src_dtype, reduction_type, value):
+        assert self.inside_reduction
+        if reduction_type not in REDUCTION_KIND:
+            raise UnsupportedHipCodegen(f"reduction {reduction_type}")
+        if reduction_type in ("sum", "prod", "max", "min") and not src_dtype.is_floating_point and src_dtype != torch.bool:
+            raise UnsupportedHipCodegen(f"integer {reduction_type} reduction")
+        if isinstance(value, tuple):
+            raise UnsupportedHipCodegen(f"tuple-valued reduction input for {reduction_type}")
+        kind = REDUCTION_KIND[reduction_type]
+        if self._load_mask:
+            raise UnsupportedHipCodegen("reduction under a load mask")
+        n = next(self.acc_ids)
+        if self.mode == "row":
+            if self.persistent_reduction:
+                if reduction_type == "sum":
+                    merged = self.cse.generate(
+                        self.compute, f"mi::row_sum<BLOCK, TPR>({value}, rmask, lds_red)", dtype=torch.float32
+                    )
+                    return self._cast_result(merged, dtype)
+                merged_name = f"red{n}"
+                self.compute.writeline(
+                    f"const auto {merged_name} = mi::group_merge<{kind}, BLOCK, TPR>({kind}::finish("
+                    f"mi::thread_step<{kind}>({kind}::init(), {value}, {self._r_index_str()}, rmask)), lds_red);"
+                )
+            else:
+                acc = f"acc{n}"
+                self.prologue.writeline(f"typename {kind}::T {acc} = {kind}::init();")
+                self.compute.writeline(
+                    f"{acc} = mi::thread_step<{kind}>({acc}, {value}, {self._r_index_str()}, rmask);"
+                )
+                merged_name = f"red{n}"
+                self.row_loop_accs.append(
+                    f"const auto {merged_name} = mi::group_merge<{kind}, BLOCK, TPR>({kind}::finish({acc}), lds_red);"
+                )
+            return self._unpack_result(merged_name, reduction_type, dtype)
+        if self.mode == "col":
+            acc = f"acc{n}"
+            merged_name = f"red{n}"
+            self.col_reductions.append(ColReduction(reduction_type, acc, merged_name, str(value), self.ws_words))
+            self.ws_words += REDUCTION_WORDS[reduction_type]
+            self.compute.writeline(f"{acc}.step({value}, r0_index, xmask);")
+            return self._unpack_result(merged_name, reduction_type, dtype)
+        raise UnsupportedHipCodegen("reduction in a pointwise kernel")
+
+    def _result_var(self, text: str, dtype: torch.dtype) -> CSEVariable:
+        """A value that exists once the reduction is complete.  With the whole
+        row in registers the code is straight-line, so the definition goes where
+        the reduction stands; otherwise it is placed after the loop."""
+        name = f"rv{next(self.acc_ids)}"
+        var = self.create_cse_var(name, ValueRanges.unknown(), dtype)
+        if self.mode == "row" and self.persistent_reduction:
+            self.compute.writeline(f"const auto {name} = {text};")
+        else:
+            self._result_defs.append(f"const auto {name} = {text};")
+        return var
+
+    def _cast_result(self, var: CSEVariable, dtype: torch.dtype) -> CSEVariable:
+        return var
+
+    def _unpack_result(self, merged: str, reduction_type: str, dtype: torch.dtype):
+        if reduction_type in ("argmax", "argmin"):
+            return self._result_var(f"static_cast<mi::i64>({merged}.i)", torch.int64)
+        if reduction_type == "welford_reduce":
+            return (
+                self._result_var(f"{merged}.mean", torch.float32),
+                self._result_var(f"{merged}.m2", torch.float32),
+                self._result_var(f"{merged}.n", torch.float32),
+            )
+        if reduction_type == "any":
+            return self._result_var(f"({merged} != 0.f)", torch.bool)
+        return self._result_var(f"{merged}", torch.float32)
+
+    # -- body assembly ----------------------------------------------------------
+    def _take_result_defs(self) -> list[str]:
+        defs = self._result_defs
+        self._result_defs = []
+        return defs
+
+    def codegen_body(self) -> None:
+        if not (self.loads or self.compute or self.stores or self.row_loop_accs or self._result_defs or self.red_stores):
+            return
+        if self.mode == "col":
+            if self.inside_reduction and not self.phase_bodies_started:
+                # loop body of the partial kernel; what follows belongs to the final kernel
+                self.partial_body.splice(self._entry_code(self.r_entries))
+                self.partial_body.splice(self.loads)
+                self.partial_body.splice(self.compute)
+                self.partial_body.splice(self.stores)
+                self.phase_bodies_started = True
+                self._result_defs_col = self._take_result_defs()
+                self.final_body.splice(self.red_stores)
+                keep = OrderedSet()
+                for item in self.cse.reduction_cache.values():
+                    for v in item if isinstance(item, tuple) else (item,):
+                        keep.add(v)
+                self.cse.invalidate(keep)
+            else:
+                self.final_body.splice(self.loads)
+                self.final_body.splice(self.compute)
+                self.final_body.splice(self.stores)
+                self.final_body.splice(self.red_stores)
+        elif self.mode == "row" and self.inside_reduction and not self.persistent_reduction:
+            # one pass over the reduced axis
+            self.body.writeline(
+                f"for ({self.index_dtype} r0_base = 0; r0_base < rnumel; r0_base += TPR * VEC) {{"
+            )
+            with self.body.indent():
+                self.body.writeline(f"const {self.index_dtype} r0_index = r0_base + rlane * VEC;")
+                self.body.writeline("const bool rmask = r0_index < rnumel;")
+                self.body.splice(self._entry_code(self.r_entries))
+                self.body.splice(self.loads)
+                self.body.splice(self.compute)
+                self.body.splice(self.stores)
+            self.body.writeline("}")
+            for line in self.row_loop_accs:
+                self.body.writeline(line)
+            self.row_loop_accs.clear()
+            for line in self._take_result_defs():
+                self.body.writeline(line)
+            self.body.splice(self.red_stores)
+            # values computed inside the loop die with it; reduction results survive
+            keep = OrderedSet()
+            for item in self.cse.reduction_cache.values():
+                for v in item if isinstance(item, tuple) else (item,):
+                    keep.add(v)
+            self.cse.invalidate(keep)
+        else:
+            self.body.splice(self.loads)
+            self.body.splice(self.compute)
+            for line in self._take_result_defs():
+                self.body.writeline(line)
+            self.body.splice(self.stores)
+            self.body.splice(self.red_stores)
+        self.loads.clear()
+        self.compute.clear()
+        self.stores.clear()
+        self.red_stores.clear()
+
+    # -- signature -----------------------------------------------------------------
+    def _signature(self):
+        """C parameter list, struct codes for packing, python call arguments."""
+        _, call_args, signature, _ = self.args.python_argdefs()
+        params, codes = [], []
+        for arg in signature:
+            if isinstance(arg, TensorArg):
+                const = "" if (arg.name.startswith("out_ptr") or arg.name.startswith("in_out_ptr")) else "const "
+                params.append(f"{const}{DTYPE_TO_HIP[arg.dtype]}* __restrict__ {arg.name}")
+                codes.append("P")
+            elif isinstance(arg, SizeArg):
+                params.append(f"const mi::i64 {arg.name}")
+                codes.append("q")
+            elif isinstance(arg, WorkspaceArg):
+                raise UnsupportedHipCodegen("Inductor-managed workspace arguments")
+            else:
+                raise UnsupportedHipCodegen(f"kernel argument {type(arg).__name__}")
+        return params, "".join(codes), [str(a) for a in call_args]
+
+    def codegen_kernel(self, name: Optional[str] = None) -> str:
+        self.codegen_body()
+        params, codes, _ = self._signature()
+        idx_t = self.index_dtype
+        idx_code = "i" if idx_t == "int" else "q"
+        kname = name or "KERNEL_NAME"
+        src = IndentedBuffer()
+        src.writeline('#include "mi/codegen.h"')
+        src.writeline("")
+        meta: dict[str, Any] = {"mode": self.mode, "vec": self.vec, "block": self.block, "index_code": idx_code}
+        if self.mode == "pointwise":
+            plist = ", ".join(params + [f"const {idx_t} xnumel"])
+            src.writeline(f'extern "C" __global__ __launch_bounds__({self.block}) void {kname}({plist}) {{')
+            with src.indent():
+                src.writeline(f"constexpr int VEC = {self.vec};")
+                src.writeline(
+                    f"const {idx_t} xindex = (static_cast<{idx_t}>(blockIdx.x) * {self.block} + threadIdx.x) * VEC;"
+                )
+                src.writeline("if (xindex >= xnumel) return;")
+                src.splice(self._entry_code(self.x_entries))
+                src.splice(self.body)
+            src.writeline("}")
+            sig = codes + idx_code
+        elif self.mode == "row":
+            plist = ", ".join(params + [f"const {idx_t} xnumel", f"const {idx_t} rnumel"])
+            src.writeline(f'extern "C" __global__ __launch_bounds__({self.block}) void {kname}({plist}) {{')
+            with src.indent():
+                src.writeline(f"constexpr int VEC = {self.vec};")
+                src.writeline(f"constexpr int BLOCK = {self.block};")
+                src.writeline(f"constexpr int TPR = {self.tpr};")
+                src.writeline("__shared__ float lds_red[(BLOCK / 64) * 4];")
+                src.writeline(f"const {idx_t} xrow = static_cast<{idx_t}>(blockIdx.x) * (BLOCK / TPR) + threadIdx.x / TPR;")
+                src.writeline("const bool xmask = xrow < xnumel;")
+                src.writeline(f"const {idx_t} xindex = xmask ? xrow : xnumel - 1;")
+                src.writeline("const int rlane = threadIdx.x % TPR;")
+                if self.persistent_reduction:
+                    src.writeline(f"const {idx_t} r0_index = rlane * VEC;")
+                    src.writeline("const bool rmask = r0_index < rnumel;")
+                src.splice(self._entry_code(self.x_entries))
+                if self.persistent_reduction:
+                    src.splice(self._entry_code(self.r_entries))
+                src.splice(self.prologue)
+                src.splice(self.body)
+            src.writeline("}")
+            sig = codes + idx_code + idx_code
+            meta.update({"tpr": self.tpr, "persistent": bool(self.persistent_reduction)})
+        else:  # col
+            sig = self._codegen_col(src, kname, params, codes, idx_t, idx_code, meta)
+        meta["signature"] = sig
+        meta["n_buffer_args"] = len(codes)
+        self.meta = meta
+        return src.getvalue()
+
+    def _codegen_col(self, src, kname, params, codes, idx_t, idx_code, meta) -> str:
+        if not self.col_reductions:
+            raise UnsupportedHipCodegen("column kernel without a reduction")
+        ct, rl, vec = self.col_ct, self.col_rl, self.vec
+        max_words = max(REDUCTION_WORDS[c.kind] for c in self.col_reductions)
+        extra = [f"float* __restrict__ ws", f"const {idx_t} xnumel", f"const {idx_t} rnumel",
+                 "const int rows_per_split", "const int nsplit"]
+        plist = ", ".join(params + extra)
+        # ---- pass 1
+        src.writeline(f'extern "C" __global__ __launch_bounds__({ct * rl}) void {kname}_partial({plist}) {{')
+        with src.indent():
+            src.writeline(f"constexpr int VEC = {vec};")
+            src.writeline(f"constexpr int CT = {ct};")
+            src.writeline(f"constexpr int RL = {rl};")
+            src.writeline("extern __shared__ float lds_dyn[];")
+            src.writeline("const int ct = threadIdx.x % CT;")
+            src.writeline("const int rl = threadIdx.x / CT;")
+            src.writeline(f"const {idx_t} xindex = (static_cast<{idx_t}>(blockIdx.x) * CT + ct) * VEC;")
+            src.writeline("const int split = blockIdx.y;")
+            src.writeline("const bool xmask = xindex < xnumel;")
+            src.writeline(f"const {idx_t} r_begin = static_cast<{idx_t}>(split) * rows_per_split;")
+            src.writeline(f"const {idx_t} r_end = (r_begin + rows_per_split < rnumel) ? r_begin + rows_per_split : rnumel;")
+            for c in self.col_reductions:
+                kind = REDUCTION_KIND[c.kind]
+                src.writeline(f"mi::ColAcc<{kind}, VEC> {c.acc};")
+                src.writeline(f"{c.acc}.init();")
+            src.writeline("if (xmask) {")
+            with src.indent():
+                src.splice(self._entry_code(self.x_entries))
+                src.writeline("#pragma unroll 4")
+                src.writeline(f"for ({idx_t} r0_index = r_begin + rl; r0_index < r_end; r0_index += RL) {{")
+                with src.indent():
+                    src.splice(self.partial_body)
+                src.writeline("}")
+            src.writeline("}")
+            for c in self.col_reductions:
+                kind = REDUCTION_KIND[c.kind]
+                src.writeline(f"typename {kind}::M {c.acc}_m[VEC];")
+                src.writeline("#pragma unroll")
+                src.writeline(f"for (int i = 0; i < VEC; ++i) {c.acc}_m[i] = {kind}::finish({c.acc}.s[i]);")
+                src.writeline(f"mi::col_fold<{kind}, VEC, CT, RL>({c.acc}_m, ct, rl, lds_dyn);")
+                src.writeline(
+                    f"if (rl == 0) mi::col_store_partial<{kind}, VEC>(ws + {c.ws_offset_words} * "
+                    f"static_cast<mi::i64>(nsplit) * xnumel, {c.acc}_m, xindex, xnumel, split, nsplit);"
+                )
+        src.writeline("}")
+        src.writeline("")
+        # ---- pass 2
+        cpw, sl = 16, 16
+        src.writeline(f'extern "C" __global__ __launch_bounds__({cpw * sl}) void {kname}_final({plist}) {{')
+        with src.indent():
+            src.writeline("constexpr int VEC = 1;")
+            src.writeline(f"constexpr int CPW = {cpw};")
+            src.writeline(f"constexpr int SL = {sl};")
+            src.writeline(f"__shared__ float lds_fin[CPW * SL * {max_words}];")
+            src.writeline("const int slot = threadIdx.x % CPW;")
+            src.writeline("const int sl = threadIdx.x / CPW;")
+            src.writeline(f"const {idx_t} xraw = static_cast<{idx_t}>(blockIdx.x) * CPW + slot;")
+            src.writeline("const bool live = xraw < xnumel;")
+            src.writeline(f"const {idx_t} xindex = live ? xraw : xnumel - 1;")
+            for c in self.col_reductions:
+                kind = REDUCTION_KIND[c.kind]
+                src.writeline(
+                    f"const auto {c.result} = mi::col_final<{kind}, CPW, SL>(ws + {c.ws_offset_words} * "
+                    f"static_cast<mi::i64>(nsplit) * xnumel, xindex, xnumel, nsplit, slot, sl, live, lds_fin);"
+                )
+            for line in self._result_defs_col:
+                src.writeline(line)
+            src.splice(self._final_indexing_code())
+            src.splice(self.final_body)
+        src.writeline("}")
+        meta.update({"ct": ct, "rl": rl, "cpw": cpw, "sl": sl, "ws_words": self.ws_words,
+                     "lds_partial": (rl // 2) * ct * vec * max_words * 4})
+        return codes + "P" + idx_code + idx_code + "ii"
+
+    def _final_indexing_code(self) -> IndentedBuffer:
+        """Range variables of the kept axis for the final kernel (one column per
+        thread there, so lane vectors collapse to scalars)."""
+        return self._entry_code(self.x_entries, lane_vectors=False)
+
+    # -- call ---------------------------------------------------------------------
+    def call_kernel(self, name: str, node: Any = None, deallocate_ws: bool = True) -> None:
+        wrapper = V.graph.wrapper_code
+        for v in self.args.sizevars:
+            wrapper.ensure_size_computed(v)
+        _, _, call_args = self._signature()
+        numels = []
+        for tree in self.range_trees:
+            if isinstance(tree.numel, (sympy.Integer, int)):
+                expr = str(int(tree.numel))
+            elif isinstance(tree.numel, sympy.Symbol):
+                expr = wrapper.val_to_arg_str(tree.numel) if hasattr(wrapper, "val_to_arg_str") else str(tree.numel)
+            else:
+                expr = str(wrapper.generate_numel_expr(name, tree).inner)
+            numels.append(f"{tree.prefix}numel={expr}")
+        device = V.graph.get_current_device_or_throw()
+        if device.type == "cpu":
+            stream = "0"
+        else:
+            stream = wrapper.write_get_raw_stream(device.index, V.graph.name)
+        args = ", ".join(call_args + numels + [f"stream={stream}"])
+        wrapper.writeline(f"{name}.run({args})")

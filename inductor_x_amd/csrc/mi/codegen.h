@@ -1,0 +1,690 @@
+// Building blocks for kernels emitted by the Inductor code generator.
+//
+// A generated kernel is straight-line C++ over two kinds of values: scalars
+// (uniform for the thread) and V<T, N> register vectors (N consecutive
+// elements along the contiguous axis).  Every operator and math function below
+// accepts any mix of the two, so the generator prints one expression per
+// Inductor op and lets overload resolution widen scalars where needed.
+//
+// Three code shapes are built from these pieces (they mirror the reference's
+// pointwise / row-reduction / higher-order-reduction kernel bodies,
+// reference inductor_x/codegen/triton.py:693-815, 1103-1262):
+//   pointwise  one V per thread, 128-bit loads and stores where the index
+//              is contiguous along the vector axis, gathers elsewhere;
+//   row        TPR threads share a row, each holds one V of it (or walks
+//              the row in a loop), results meet through DPP and LDS;
+//   column     every vector lane is its own output column, row lanes of the
+//              workgroup meet through LDS, slices of the reduced axis meet
+//              through a workspace and a second kernel.
+#pragma once
+
+#include <type_traits>
+
+#include "common.h"
+
+namespace mi {
+
+typedef long long i64;
+
+// ---------------------------------------------------------------------------
+// register vector + scalar/vector-generic elementwise application
+// ---------------------------------------------------------------------------
+template <typename T, int N>
+struct V {
+  T v[N];
+  __device__ __forceinline__ T& operator[](int i) { return v[i]; }
+  __device__ __forceinline__ const T& operator[](int i) const { return v[i]; }
+};
+
+template <class A>
+struct Tr {
+  static constexpr int n = 0;
+  typedef A elem;
+};
+template <class T, int N>
+struct Tr<V<T, N>> {
+  static constexpr int n = N;
+  typedef T elem;
+};
+
+template <class A>
+__device__ __forceinline__ auto at(const A& a, int i) {
+  if constexpr (Tr<A>::n != 0) {
+    return a.v[i];
+  } else {
+    return a;
+  }
+}
+
+template <int... Ns>
+struct MaxN;
+template <int A>
+struct MaxN<A> {
+  static constexpr int value = A;
+};
+template <int A, int... Rest>
+struct MaxN<A, Rest...> {
+  static constexpr int value = A > MaxN<Rest...>::value ? A : MaxN<Rest...>::value;
+};
+
+template <class F, class... A>
+__device__ __forceinline__ auto apply(F f, const A&... a) {
+  constexpr int n = MaxN<Tr<A>::n...>::value;
+  if constexpr (n == 0) {
+    return f(a...);
+  } else {
+    V<decltype(f(at(a, 0)...)), n> r;
+#pragma unroll
+    for (int i = 0; i < n; ++i) r.v[i] = f(at(a, i)...);
+    return r;
+  }
+}
+
+template <class A, class B>
+using EnableIfAnyVec = typename std::enable_if<(Tr<A>::n != 0 || Tr<B>::n != 0), int>::type;
+
+#define MI_BINARY_OPERATOR(OP)                                                         \
+  template <class A, class B, EnableIfAnyVec<A, B> = 0>                                \
+  __device__ __forceinline__ auto operator OP(const A& a, const B& b) {                \
+    return apply([](auto x, auto y) { return x OP y; }, a, b);                         \
+  }
+MI_BINARY_OPERATOR(+)
+MI_BINARY_OPERATOR(-)
+MI_BINARY_OPERATOR(*)
+MI_BINARY_OPERATOR(/)
+MI_BINARY_OPERATOR(%)
+MI_BINARY_OPERATOR(<)
+MI_BINARY_OPERATOR(<=)
+MI_BINARY_OPERATOR(>)
+MI_BINARY_OPERATOR(>=)
+MI_BINARY_OPERATOR(==)
+MI_BINARY_OPERATOR(!=)
+MI_BINARY_OPERATOR(&)
+MI_BINARY_OPERATOR(|)
+MI_BINARY_OPERATOR(^)
+MI_BINARY_OPERATOR(<<)
+MI_BINARY_OPERATOR(>>)
+MI_BINARY_OPERATOR(&&)
+MI_BINARY_OPERATOR(||)
+#undef MI_BINARY_OPERATOR
+
+template <class T, int N>
+__device__ __forceinline__ auto operator-(const V<T, N>& a) {
+  return apply([](auto x) { return -x; }, a);
+}
+template <class T, int N>
+__device__ __forceinline__ auto operator!(const V<T, N>& a) {
+  return apply([](auto x) { return !x; }, a);
+}
+template <class T, int N>
+__device__ __forceinline__ auto operator~(const V<T, N>& a) {
+  return apply([](auto x) { return ~x; }, a);
+}
+
+// 0, 1, ..., N-1 as a vector (N == 1 gives a plain 0 so scalar code stays scalar)
+template <int N>
+__device__ __forceinline__ auto iota() {
+  if constexpr (N == 1) {
+    return 0;
+  } else {
+    V<int, N> r;
+#pragma unroll
+    for (int i = 0; i < N; ++i) r.v[i] = i;
+    return r;
+  }
+}
+
+template <class T, class A>
+__device__ __forceinline__ auto cast(const A& a) {
+  return apply([](auto x) { return static_cast<T>(x); }, a);
+}
+template <class T, class A>
+__device__ __forceinline__ auto bitcast(const A& a) {
+  return apply([](auto x) { return __builtin_bit_cast(T, x); }, a);
+}
+template <class C, class A, class B>
+__device__ __forceinline__ auto where(const C& c, const A& a, const B& b) {
+  return apply(
+      [](bool cc, auto x, auto y) {
+        typedef decltype(true ? x : y) R;
+        return cc ? static_cast<R>(x) : static_cast<R>(y);
+      },
+      c, a, b);
+}
+
+// ---------------------------------------------------------------------------
+// math (fp32 unless noted)
+// ---------------------------------------------------------------------------
+#define MI_UNARY_FN(NAME, EXPR)                                   \
+  template <class A>                                              \
+  __device__ __forceinline__ auto NAME(const A& a) {              \
+    return apply([](auto x) { return EXPR; }, a);                 \
+  }
+MI_UNARY_FN(exp, __expf(static_cast<float>(x)))
+MI_UNARY_FN(exp2, __builtin_amdgcn_exp2f(static_cast<float>(x)))
+MI_UNARY_FN(expm1, ::expm1f(static_cast<float>(x)))
+MI_UNARY_FN(log, ::logf(static_cast<float>(x)))
+MI_UNARY_FN(log2, ::log2f(static_cast<float>(x)))
+MI_UNARY_FN(log10, ::log10f(static_cast<float>(x)))
+MI_UNARY_FN(log1p, ::log1pf(static_cast<float>(x)))
+MI_UNARY_FN(sqrt, ::sqrtf(static_cast<float>(x)))
+MI_UNARY_FN(rsqrt, ::rsqrtf(static_cast<float>(x)))
+MI_UNARY_FN(sin, ::sinf(static_cast<float>(x)))
+MI_UNARY_FN(cos, ::cosf(static_cast<float>(x)))
+MI_UNARY_FN(tan, ::tanf(static_cast<float>(x)))
+MI_UNARY_FN(tanh, ::tanhf(static_cast<float>(x)))
+MI_UNARY_FN(sinh, ::sinhf(static_cast<float>(x)))
+MI_UNARY_FN(cosh, ::coshf(static_cast<float>(x)))
+MI_UNARY_FN(asin, ::asinf(static_cast<float>(x)))
+MI_UNARY_FN(acos, ::acosf(static_cast<float>(x)))
+MI_UNARY_FN(atan, ::atanf(static_cast<float>(x)))
+MI_UNARY_FN(erf, ::erff(static_cast<float>(x)))
+MI_UNARY_FN(erfc, ::erfcf(static_cast<float>(x)))
+MI_UNARY_FN(lgamma, ::lgammaf(static_cast<float>(x)))
+MI_UNARY_FN(floor, ::floorf(static_cast<float>(x)))
+MI_UNARY_FN(ceil, ::ceilf(static_cast<float>(x)))
+MI_UNARY_FN(trunc, ::truncf(static_cast<float>(x)))
+MI_UNARY_FN(round, ::nearbyintf(static_cast<float>(x)))
+MI_UNARY_FN(reciprocal, 1.0f / static_cast<float>(x))
+MI_UNARY_FN(sigmoid, __builtin_amdgcn_rcpf(1.0f + __expf(-static_cast<float>(x))))
+MI_UNARY_FN(isnan, (x != x))
+MI_UNARY_FN(isinf, (::isinf(static_cast<float>(x)) != 0))
+MI_UNARY_FN(signbit, (::signbit(static_cast<float>(x)) != 0))
+MI_UNARY_FN(abs, (x < 0 ? -x : x))
+MI_UNARY_FN(logical_not, (!x))
+// relu keeps NaN (a plain fmaxf would drop it)
+MI_UNARY_FN(relu, (x != x ? x : (x > 0 ? x : static_cast<decltype(x)>(0))))
+#undef MI_UNARY_FN
+
+template <class A>
+__device__ __forceinline__ auto sign(const A& a) {
+  return apply([](auto x) { return static_cast<decltype(x)>((x > 0) - (x < 0)); }, a);
+}
+
+#define MI_BINARY_FN(NAME, EXPR)                                   \
+  template <class A, class B>                                      \
+  __device__ __forceinline__ auto NAME(const A& a, const B& b) {   \
+    return apply([](auto x, auto y) { return EXPR; }, a, b);       \
+  }
+// NaN-propagating, as torch.maximum / torch.minimum
+MI_BINARY_FN(maximum, (x != x ? x : (y != y ? static_cast<decltype(x)>(y) : (x > y ? x : static_cast<decltype(x)>(y)))))
+MI_BINARY_FN(minimum, (x != x ? x : (y != y ? static_cast<decltype(x)>(y) : (x < y ? x : static_cast<decltype(x)>(y)))))
+MI_BINARY_FN(pow, ::powf(static_cast<float>(x), static_cast<float>(y)))
+MI_BINARY_FN(atan2, ::atan2f(static_cast<float>(x), static_cast<float>(y)))
+MI_BINARY_FN(fmod, ::fmodf(static_cast<float>(x), static_cast<float>(y)))
+MI_BINARY_FN(copysign, ::copysignf(static_cast<float>(x), static_cast<float>(y)))
+MI_BINARY_FN(truediv, static_cast<float>(x) / static_cast<float>(y))
+// Python-style integer floor division and modulo
+MI_BINARY_FN(floordiv, ((x / y) - ((x % y != 0) && ((x < 0) != (y < 0)) ? 1 : 0)))
+MI_BINARY_FN(pymod, (((x % y) != 0 && ((x % y) < 0) != (y < 0)) ? (x % y) + y : (x % y)))
+MI_BINARY_FN(truncdiv, (x / y))
+MI_BINARY_FN(logical_and, (static_cast<bool>(x) && static_cast<bool>(y)))
+MI_BINARY_FN(logical_or, (static_cast<bool>(x) || static_cast<bool>(y)))
+MI_BINARY_FN(logical_xor, (static_cast<bool>(x) != static_cast<bool>(y)))
+// float remainder with the sign of the divisor (torch.remainder)
+MI_BINARY_FN(remainder_f, (::fmodf(static_cast<float>(x), static_cast<float>(y)) != 0.f &&
+                                   ((::fmodf(static_cast<float>(x), static_cast<float>(y)) < 0.f) != (static_cast<float>(y) < 0.f))
+                               ? ::fmodf(static_cast<float>(x), static_cast<float>(y)) + static_cast<float>(y)
+                               : ::fmodf(static_cast<float>(x), static_cast<float>(y))))
+#undef MI_BINARY_FN
+
+template <class A, class B, class C>
+__device__ __forceinline__ auto fma(const A& a, const B& b, const C& c) {
+  return apply([](float x, float y, float z) { return ::fmaf(x, y, z); }, a, b, c);
+}
+
+// ---------------------------------------------------------------------------
+// loads / stores
+// ---------------------------------------------------------------------------
+// Contiguous, aligned run of N elements starting at p (N * sizeof(T) bytes,
+// moved in 16-byte pieces).  The generator proves contiguity and alignment.
+template <int N, class T>
+__device__ __forceinline__ auto vload(const T* __restrict__ p) {
+  if constexpr (N == 1) {
+    return *p;
+  } else {
+    constexpr int PER = (16 / sizeof(T)) < N ? (16 / sizeof(T)) : N;
+    V<T, N> r;
+#pragma unroll
+    for (int c = 0; c < N / PER; ++c) {
+      const Vec<T, PER> t = load_vec<T, PER>(p + c * PER);
+#pragma unroll
+      for (int i = 0; i < PER; ++i) r.v[c * PER + i] = t[i];
+    }
+    return r;
+  }
+}
+
+// Contiguous run with no alignment guarantee.
+template <int N, class T>
+__device__ __forceinline__ auto vload_u(const T* __restrict__ p) {
+  if constexpr (N == 1) {
+    return *p;
+  } else {
+    V<T, N> r;
+#pragma unroll
+    for (int i = 0; i < N; ++i) r.v[i] = p[i];
+    return r;
+  }
+}
+
+// Element-wise indexed load: idx scalar -> scalar, idx vector -> vector.
+template <class T, class I>
+__device__ __forceinline__ auto gather(const T* __restrict__ p, const I& idx) {
+  return apply([p](auto i) { return p[i]; }, idx);
+}
+
+// Masked forms: lanes whose mask is false read nothing and yield `other`.
+template <int N, class T, class M, class O>
+__device__ __forceinline__ auto vload_m(const T* __restrict__ p, const M& mask, O other) {
+  if constexpr (N == 1) {
+    return static_cast<bool>(at(mask, 0)) ? *p : static_cast<T>(other);
+  } else {
+    V<T, N> r;
+    bool all = true;
+#pragma unroll
+    for (int i = 0; i < N; ++i) all = all && static_cast<bool>(at(mask, i));
+    if (all) {
+      r = vload<N, T>(p);
+    } else {
+#pragma unroll
+      for (int i = 0; i < N; ++i) r.v[i] = static_cast<bool>(at(mask, i)) ? p[i] : static_cast<T>(other);
+    }
+    return r;
+  }
+}
+template <class T, class I, class M, class O>
+__device__ __forceinline__ auto gather_m(const T* __restrict__ p, const I& idx, const M& mask, O other) {
+  return apply([p, other](auto i, bool m) { return m ? p[i] : static_cast<T>(other); }, idx, mask);
+}
+
+template <int N, class T, class A>
+__device__ __forceinline__ void vstore(T* __restrict__ p, const A& val) {
+  if constexpr (N == 1) {
+    *p = static_cast<T>(at(val, 0));
+  } else {
+    constexpr int PER = (16 / sizeof(T)) < N ? (16 / sizeof(T)) : N;
+#pragma unroll
+    for (int c = 0; c < N / PER; ++c) {
+      Vec<T, PER> t;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) t[i] = static_cast<T>(at(val, c * PER + i));
+      store_vec<T, PER>(p + c * PER, t);
+    }
+  }
+}
+template <int N, class T, class A>
+__device__ __forceinline__ void vstore_u(T* __restrict__ p, const A& val) {
+#pragma unroll
+  for (int i = 0; i < (N < 1 ? 1 : N); ++i) p[i] = static_cast<T>(at(val, i));
+}
+template <int N, class T, class A, class M>
+__device__ __forceinline__ void vstore_m(T* __restrict__ p, const A& val, const M& mask) {
+  bool all = true;
+#pragma unroll
+  for (int i = 0; i < N; ++i) all = all && static_cast<bool>(at(mask, i));
+  if (all) {
+    vstore<N, T>(p, val);
+  } else {
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+      if (static_cast<bool>(at(mask, i))) p[i] = static_cast<T>(at(val, i));
+  }
+}
+// Element-wise indexed store (scatter): idx and/or val may be vectors.
+template <int N, class T, class I, class A, class M>
+__device__ __forceinline__ void scatter_m(T* __restrict__ p, const I& idx, const A& val, const M& mask) {
+#pragma unroll
+  for (int i = 0; i < (N < 1 ? 1 : N); ++i)
+    if (static_cast<bool>(at(mask, i))) p[at(idx, i)] = static_cast<T>(at(val, i));
+}
+
+// ---------------------------------------------------------------------------
+// reduction kinds.  Thread-level state T (cheap per-element step), merge-level
+// state M (what travels between threads), W floats per M on the wire.
+// Combination rules for arg-reductions and NaN handling follow
+// reference inductor_x/codegen/triton.py:1217-1233 (maximum_with_index).
+// ---------------------------------------------------------------------------
+struct RedSum {
+  typedef float T;
+  typedef float M;
+  static constexpr int W = 1;
+  __device__ static T init() { return 0.f; }
+  __device__ static T step(T s, float v, int) { return s + v; }
+  __device__ static M finish(T s) { return s; }
+  __device__ static M empty() { return 0.f; }
+  __device__ static M merge(M a, M b) { return a + b; }
+  __device__ static void enc(M m, float* w) { w[0] = m; }
+  __device__ static M dec(const float* w) { return w[0]; }
+};
+struct RedProd {
+  typedef float T;
+  typedef float M;
+  static constexpr int W = 1;
+  __device__ static T init() { return 1.f; }
+  __device__ static T step(T s, float v, int) { return s * v; }
+  __device__ static M finish(T s) { return s; }
+  __device__ static M empty() { return 1.f; }
+  __device__ static M merge(M a, M b) { return a * b; }
+  __device__ static void enc(M m, float* w) { w[0] = m; }
+  __device__ static M dec(const float* w) { return w[0]; }
+};
+struct RedMax {
+  typedef float T;
+  typedef float M;
+  static constexpr int W = 1;
+  __device__ static T init() { return -__builtin_inff(); }
+  __device__ static T step(T s, float v, int) { return MaxOp()(s, v); }
+  __device__ static M finish(T s) { return s; }
+  __device__ static M empty() { return -__builtin_inff(); }
+  __device__ static M merge(M a, M b) { return MaxOp()(a, b); }
+  __device__ static void enc(M m, float* w) { w[0] = m; }
+  __device__ static M dec(const float* w) { return w[0]; }
+};
+struct RedMin {
+  typedef float T;
+  typedef float M;
+  static constexpr int W = 1;
+  __device__ static T init() { return __builtin_inff(); }
+  __device__ static T step(T s, float v, int) { return MinOp()(s, v); }
+  __device__ static M finish(T s) { return s; }
+  __device__ static M empty() { return __builtin_inff(); }
+  __device__ static M merge(M a, M b) { return MinOp()(a, b); }
+  __device__ static void enc(M m, float* w) { w[0] = m; }
+  __device__ static M dec(const float* w) { return w[0]; }
+};
+struct RedAny {
+  typedef float T;
+  typedef float M;
+  static constexpr int W = 1;
+  __device__ static T init() { return 0.f; }
+  __device__ static T step(T s, float v, int) { return (s != 0.f || v != 0.f) ? 1.f : 0.f; }
+  __device__ static M finish(T s) { return s; }
+  __device__ static M empty() { return 0.f; }
+  __device__ static M merge(M a, M b) { return (a != 0.f || b != 0.f) ? 1.f : 0.f; }
+  __device__ static void enc(M m, float* w) { w[0] = m; }
+  __device__ static M dec(const float* w) { return w[0]; }
+};
+template <bool IS_MAX>
+struct RedArg {
+  typedef ArgVal T;
+  typedef ArgVal M;
+  static constexpr int W = 2;
+  __device__ static T init() {
+    ArgVal a;
+    a.v = IS_MAX ? -__builtin_inff() : __builtin_inff();
+    a.i = 0x7fffffff;
+    return a;
+  }
+  __device__ static T step(T s, float v, int idx) {
+    ArgVal b;
+    b.v = v;
+    b.i = idx;
+    return arg_combine<IS_MAX>(s, b);
+  }
+  __device__ static M finish(T s) { return s; }
+  __device__ static M empty() { return init(); }
+  __device__ static M merge(M a, M b) { return arg_combine<IS_MAX>(a, b); }
+  __device__ static void enc(M m, float* w) {
+    w[0] = m.v;
+    w[1] = __int_as_float(m.i);
+  }
+  __device__ static M dec(const float* w) {
+    ArgVal a;
+    a.v = w[0];
+    a.i = __float_as_int(w[1]);
+    return a;
+  }
+};
+typedef RedArg<true> RedArgMax;
+typedef RedArg<false> RedArgMin;
+
+// Mean / M2 / count.  A thread accumulates shifted sums (shift = its first
+// sample), which costs three flops per element and is as stable as Welford's
+// update; merges use Chan's formula.  The definition restated is the two-pass
+// one of reference inductor_x/lowering.py:270-293.
+struct RedWelford {
+  struct T {
+    float n, c, s1, s2;
+  };
+  typedef Moments M;
+  static constexpr int W = 3;
+  __device__ static T init() {
+    T t;
+    t.n = 0.f;
+    t.c = 0.f;
+    t.s1 = 0.f;
+    t.s2 = 0.f;
+    return t;
+  }
+  __device__ static T step(T s, float v, int) {
+    s.c = (s.n == 0.f) ? v : s.c;
+    const float d = v - s.c;
+    s.s1 += d;
+    s.s2 = fmaf(d, d, s.s2);
+    s.n += 1.f;
+    return s;
+  }
+  __device__ static M finish(T s) {
+    Moments m;
+    m.n = s.n;
+    if (s.n == 0.f) {
+      m.mean = 0.f;
+      m.m2 = 0.f;
+      return m;
+    }
+    const float inv = 1.0f / s.n;
+    m.mean = s.c + s.s1 * inv;
+    const float m2 = s.s2 - s.s1 * s.s1 * inv;
+    m.m2 = (m2 < 0.f) ? 0.f : m2;
+    return m;
+  }
+  __device__ static M empty() {
+    Moments m;
+    m.n = 0.f;
+    m.mean = 0.f;
+    m.m2 = 0.f;
+    return m;
+  }
+  __device__ static M merge(M a, M b) { return moments_combine(a, b); }
+  __device__ static void enc(M m, float* w) {
+    w[0] = m.n;
+    w[1] = m.mean;
+    w[2] = m.m2;
+  }
+  __device__ static M dec(const float* w) {
+    Moments m;
+    m.n = w[0];
+    m.mean = w[1];
+    m.m2 = w[2];
+    return m;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// row shape: reduce a thread's vector, then the TPR threads of the row
+// ---------------------------------------------------------------------------
+// Butterfly over the low lanes of a wavefront for any merge state.
+template <class R, int WIDTH>
+__device__ __forceinline__ typename R::M wave_merge(typename R::M m) {
+#pragma unroll
+  for (int off = 1; off < WIDTH; off <<= 1) {
+    float w[R::W], o[R::W];
+    R::enc(m, w);
+#pragma unroll
+    for (int k = 0; k < R::W; ++k) o[k] = __shfl_xor(w[k], off, kWave);
+    // keep the operand order fixed by lane so every lane computes the same value
+    const bool low = (threadIdx.x & off) == 0;
+    const typename R::M other = R::dec(o);
+    m = low ? R::merge(m, other) : R::merge(other, m);
+  }
+  return m;
+}
+
+// lds: at least (BLOCK / 64) * R::W floats.  All threads of the group receive
+// the result.
+template <class R, int BLOCK, int TPR>
+__device__ __forceinline__ typename R::M group_merge(typename R::M m, float* lds) {
+  if constexpr (TPR <= kWave) {
+    return wave_merge<R, TPR>(m);
+  } else {
+    constexpr int WPG = TPR / kWave;
+    m = wave_merge<R, kWave>(m);
+    const int wave = threadIdx.x / kWave;
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+      float w[R::W];
+      R::enc(m, w);
+#pragma unroll
+      for (int k = 0; k < R::W; ++k) lds[wave * R::W + k] = w[k];
+    }
+    __syncthreads();
+    const int first = (wave / WPG) * WPG;
+    typename R::M total = R::dec(lds + first * R::W);
+#pragma unroll
+    for (int j = 1; j < WPG; ++j) total = R::merge(total, R::dec(lds + (first + j) * R::W));
+    return total;
+  }
+}
+
+// Fold one vector of values (with their reduction indices and a validity mask)
+// into a thread state.
+template <class R, class VT, class IT, class MT>
+__device__ __forceinline__ typename R::T thread_step(typename R::T s, const VT& val, const IT& idx, const MT& mask) {
+  constexpr int n = Tr<VT>::n == 0 ? (Tr<IT>::n == 0 ? (Tr<MT>::n == 0 ? 1 : Tr<MT>::n) : Tr<IT>::n) : Tr<VT>::n;
+#pragma unroll
+  for (int i = 0; i < n; ++i)
+    if (static_cast<bool>(at(mask, i))) s = R::step(s, static_cast<float>(at(val, i)), static_cast<int>(at(idx, i)));
+  return s;
+}
+
+// Plain fp32 sums and maxima take the DPP path of common.h.
+template <int BLOCK, int TPR, class VT, class MT>
+__device__ __forceinline__ float row_sum(const VT& val, const MT& mask, float* lds) {
+  constexpr int n = Tr<VT>::n == 0 ? 1 : Tr<VT>::n;
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < n; ++i) s += static_cast<bool>(at(mask, i)) ? static_cast<float>(at(val, i)) : 0.f;
+  return group_reduce<BLOCK, TPR>(s, SumOp(), lds);
+}
+
+// ---------------------------------------------------------------------------
+// column shape
+// ---------------------------------------------------------------------------
+// Per-thread: N independent columns, each with its own thread state.
+template <class R, int N>
+struct ColAcc {
+  typename R::T s[N];
+  __device__ __forceinline__ void init() {
+#pragma unroll
+    for (int i = 0; i < N; ++i) s[i] = R::init();
+  }
+  template <class VT, class MT>
+  __device__ __forceinline__ void step(const VT& val, int ridx, const MT& mask) {
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+      if (static_cast<bool>(at(mask, i))) s[i] = R::step(s[i], static_cast<float>(at(val, i)), ridx);
+  }
+};
+
+// Fold the RL row lanes of a workgroup (thread = rl * CT + ct).  lds holds
+// (RL / 2) * CT * N * R::W floats.  Afterwards threads with rl == 0 own the result.
+template <class R, int N, int CT, int RL>
+__device__ __forceinline__ void col_fold(typename R::M (&m)[N], int ct, int rl, float* lds) {
+  if constexpr (RL > 1) {
+    constexpr int PLANE = (RL / 2) * CT * N;
+#pragma unroll
+    for (int half = RL / 2; half >= 1; half >>= 1) {
+      __syncthreads();
+      if (rl >= half && rl < 2 * half) {
+        const int slot = ((rl - half) * CT + ct) * N;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+          float w[R::W];
+          R::enc(m[i], w);
+#pragma unroll
+          for (int k = 0; k < R::W; ++k) lds[k * PLANE + slot + i] = w[k];
+        }
+      }
+      __syncthreads();
+      if (rl < half) {
+        const int slot = (rl * CT + ct) * N;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+          float w[R::W];
+#pragma unroll
+          for (int k = 0; k < R::W; ++k) w[k] = lds[k * PLANE + slot + i];
+          m[i] = R::merge(m[i], R::dec(w));
+        }
+      }
+    }
+  }
+}
+
+// Workspace layout for one reduction: [R::W][nsplit][xnumel] floats.
+template <class R, int N>
+__device__ __forceinline__ void col_store_partial(float* __restrict__ ws, const typename R::M (&m)[N], i64 x0,
+                                                  i64 xnumel, int split, int nsplit) {
+  const i64 plane = static_cast<i64>(nsplit) * xnumel;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    if (x0 + i < xnumel) {
+      float w[R::W];
+      R::enc(m[i], w);
+#pragma unroll
+      for (int k = 0; k < R::W; ++k) ws[k * plane + static_cast<i64>(split) * xnumel + x0 + i] = w[k];
+    }
+  }
+}
+
+// Second pass for one column x: thread sl of SL folds splits sl, sl+SL, ...
+// (batched loads), then the SL lanes are folded through LDS (SL * W floats per
+// column slot; `slot` = the column's index inside the workgroup, CPW of them).
+template <class R, int CPW, int SL>
+__device__ __forceinline__ typename R::M col_final(const float* __restrict__ ws, i64 x, i64 xnumel, int nsplit,
+                                                   int slot, int sl, bool live, float* lds) {
+  constexpr int BATCH = 4;
+  const i64 plane = static_cast<i64>(nsplit) * xnumel;
+  typename R::M m = R::empty();
+  if (live) {
+    for (int s0 = sl; s0 < nsplit; s0 += SL * BATCH) {
+      float w[BATCH][R::W];
+#pragma unroll
+      for (int b = 0; b < BATCH; ++b) {
+        const int s = s0 + b * SL;
+        const i64 o = static_cast<i64>(s < nsplit ? s : s0) * xnumel + x;
+#pragma unroll
+        for (int k = 0; k < R::W; ++k) w[b][k] = ws[k * plane + o];
+      }
+#pragma unroll
+      for (int b = 0; b < BATCH; ++b)
+        if (s0 + b * SL < nsplit) m = R::merge(m, R::dec(w[b]));
+    }
+  }
+  constexpr int PLANE = CPW * SL;
+  const int me = sl * CPW + slot;
+  __syncthreads();
+  {
+    float w[R::W];
+    R::enc(m, w);
+#pragma unroll
+    for (int k = 0; k < R::W; ++k) lds[k * PLANE + me] = w[k];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int half = SL / 2; half >= 1; half >>= 1) {
+    if (sl < half) {
+      float w[R::W];
+#pragma unroll
+      for (int k = 0; k < R::W; ++k) w[k] = lds[k * PLANE + (sl + half) * CPW + slot];
+      m = R::merge(m, R::dec(w));
+      R::enc(m, w);
+#pragma unroll
+      for (int k = 0; k < R::W; ++k) lds[k * PLANE + me] = w[k];
+    }
+    __syncthreads();
+  }
+  return m;  // valid where sl == 0
+}
+
+}  // namespace mi

@@ -1,0 +1,257 @@
+"""Fused-attention custom op and graph pattern.
+
+Counterpart of reference inductor_x/npu_fusion_attention_graph.py: the same
+operator library and schemas (`npu_graph::npu_fa`, `npu_graph::npu_fa_backward`,
+:13-18), a device implementation (:20-42), Meta implementations giving the
+output shapes (:45-86), an autograd.Function wrapper (:88-123), the public
+npu_fusion_attention_graph() (:125-132) and the replacement of
+    matmul(q, k^T).div(inv_scale).softmax(-1)[.dropout].matmul(v)
+with q, k, v given as [B, S, N, D] and permuted (0, 2, 1, 3) (:134-230).
+
+The device implementation runs the MFMA kernel of this package.  As in the
+reference the op receives the *inverse* scale from the pattern and inverts it
+(:20-35, :162).  The reference's pattern carries no mask; a causal mask enters
+through the op's own arguments: sparse_mode 2 or 3, or next_tockens == 0 with
+pre_tockens covering the sequence.  Supported: layout "BNSD", bf16, head
+dimension 128, no pse / padding mask / dropout; anything else raises.
+"""
+from __future__ import annotations
+
+import functools
+
+import torch
+from torch.autograd import Function
+from torch.library import Library
+
+TOKEN_MAX = 2147483647
+
+npu_def = Library("npu_graph", "DEF")
+gpu_lib = Library("npu_graph", "IMPL", "CUDA")
+meta_lib = Library("npu_graph", "IMPL", "Meta")
+
+npu_def.define(
+    "npu_fa(Tensor query, Tensor key, Tensor value, int head_num, str input_layout, Tensor? pse=None, "
+    "Tensor? padding_mask=None, Tensor? atten_mask=None, float scale=1., float keep_prob=1., "
+    "int pre_tockens=2147483647, int next_tockens=2147483647, int inner_precise=0, int[]? prefix=None, "
+    "int[]? actual_seq_qlen=None, int[]? actual_seq_kvlen=None, int sparse_mode=0, bool gen_mask_parallel=True, "
+    "bool sync=False) -> (Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor)"
+)
+npu_def.define(
+    "npu_fa_backward(Tensor query, Tensor key, Tensor value, Tensor dy, int head_num, str input_layout, *, "
+    "Tensor? pse=None, Tensor? padding_mask=None, Tensor? atten_mask=None, Tensor? softmax_max=None, "
+    "Tensor? softmax_sum=None, Tensor? softmax_in=None, Tensor? attention_in=None, float scale_value=1., "
+    "float keep_prob=1., int pre_tockens=2147483647, int next_tockens=2147483647, int inner_precise=0, "
+    "Tensor? seed=None, Tensor? offset=None, Tensor? numels=None, int[]? prefix=None, int[]? actual_seq_qlen=None, "
+    "int[]? actual_seq_kvlen=None, int sparse_mode=0, bool gen_mask_parallel=True, bool sync=False) "
+    "-> (Tensor, Tensor, Tensor, Tensor)"
+)
+
+
+def _is_causal(seq_len: int, atten_mask, pre_tockens: int, next_tockens: int, sparse_mode: int) -> bool:
+    if sparse_mode in (2, 3):
+        return True
+    if sparse_mode == 0 and next_tockens == 0 and pre_tockens >= seq_len:
+        return True
+    if atten_mask is not None:
+        raise NotImplementedError(
+            "npu_fa: an attention mask is only supported as the causal mask "
+            "(sparse_mode 2/3, or next_tockens=0 with pre_tockens >= sequence length)"
+        )
+    return False
+
+
+def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask=None, atten_mask=None, scale=1.0,
+               keep_prob=1.0, pre_tockens=TOKEN_MAX, next_tockens=TOKEN_MAX, inner_precise=0, prefix=None,
+               actual_seq_qlen=None, actual_seq_kvlen=None, sparse_mode=0, gen_mask_parallel=True, sync=False):
+    from . import kernels
+
+    if input_layout != "BNSD":
+        raise NotImplementedError(f"npu_fa: layout {input_layout!r} (only 'BNSD')")
+    if pse is not None or padding_mask is not None or prefix or actual_seq_qlen or actual_seq_kvlen:
+        raise NotImplementedError("npu_fa: pse / padding_mask / prefix / variable sequence lengths")
+    if keep_prob != 1.0:
+        raise NotImplementedError("npu_fa: dropout (keep_prob != 1)")
+    if query.size(1) != head_num:
+        raise ValueError(f"npu_fa: head_num {head_num} does not match query of shape {tuple(query.shape)}")
+    if scale == 0:
+        raise ZeroDivisionError("npu_fa: the inverse scale factor is zero")
+    # the graph pattern passes the divisor of the scores; the kernel multiplies
+    real_scale = 1.0 / scale
+    causal = _is_causal(query.size(2), atten_mask, pre_tockens, next_tockens, sparse_mode)
+    out, smax, ssum = kernels.fused_attention(
+        query.contiguous(), key.contiguous(), value.contiguous(), real_scale, causal
+    )
+    softmax_out = torch.empty([0], dtype=query.dtype, device=query.device)
+    zero = lambda: torch.zeros([1], dtype=torch.int64)  # noqa: E731  seed / offset / numel: no dropout
+    return out, smax, ssum, softmax_out, zero(), zero(), zero()
+
+
+gpu_lib.impl("npu_fa", npu_fa_gpu)
+
+
+def npu_fa_backward_gpu(*args, **kwargs):
+    raise NotImplementedError("npu_fa_backward: the attention backward kernel is not part of this build")
+
+
+gpu_lib.impl("npu_fa_backward", npu_fa_backward_gpu)
+
+
+def npu_fa_meta(query, key, value, head_num, input_layout, pse=None, padding_mask=None, atten_mask=None, scale=1.0,
+                keep_prob=1.0, pre_tockens=TOKEN_MAX, next_tockens=TOKEN_MAX, inner_precise=0, prefix=None,
+                actual_seq_qlen=None, actual_seq_kvlen=None, sparse_mode=0, gen_mask_parallel=True, sync=False):
+    B, S1 = query.size(0), query.size(2)
+    if input_layout == "BSH":
+        B, S1 = query.size(0), query.size(1)
+    if input_layout == "SBH":
+        B, S1 = query.size(1), query.size(0)
+    dev = query.device
+    return (
+        torch.empty_like(query).contiguous(),
+        torch.empty([B, head_num, S1, 8], dtype=torch.float32, device=dev),
+        torch.empty([B, head_num, S1, 8], dtype=torch.float32, device=dev),
+        torch.empty([0], dtype=query.dtype, device=dev),
+        torch.empty([1], dtype=torch.int64, device="meta"),
+        torch.empty([1], dtype=torch.int64, device="meta"),
+        torch.empty([1], dtype=torch.int64, device="meta"),
+    )
+
+
+meta_lib.impl("npu_fa", npu_fa_meta)
+
+
+def npu_fa_backward_meta(query, key, value, dy, head_num, input_layout, *, pse=None, padding_mask=None,
+                         atten_mask=None, softmax_max=None, softmax_sum=None, softmax_in=None, attention_in=None,
+                         scale_value=1.0, keep_prob=1.0, pre_tockens=TOKEN_MAX, next_tockens=TOKEN_MAX,
+                         inner_precise=0, seed=None, offset=None, numels=None, prefix=None, actual_seq_qlen=None,
+                         actual_seq_kvlen=None, sparse_mode=0, gen_mask_parallel=True, sync=False):
+    return (
+        torch.empty_like(query).contiguous(),
+        torch.empty_like(key).contiguous(),
+        torch.empty_like(value).contiguous(),
+        torch.empty([0], dtype=query.dtype, device=query.device),
+    )
+
+
+meta_lib.impl("npu_fa_backward", npu_fa_backward_meta)
+
+
+class GraphAttentionFunction(Function):
+    """autograd wrapper of npu_graph::npu_fa (reference
+    inductor_x/npu_fusion_attention_graph.py:88-123)."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, head_num, input_layout, pse=None, padding_mask=None, atten_mask=None,
+                scale=1.0, keep_prob=1.0, pre_tockens=TOKEN_MAX, next_tockens=TOKEN_MAX, inner_precise=0,
+                prefix=None, actual_seq_qlen=None, actual_seq_kvlen=None, sparse_mode=0, gen_mask_parallel=True,
+                sync=False):
+        res = torch.ops.npu_graph.npu_fa(
+            query, key, value, head_num, input_layout, pse=pse, padding_mask=padding_mask, atten_mask=atten_mask,
+            scale=scale, keep_prob=keep_prob, pre_tockens=pre_tockens, next_tockens=next_tockens,
+            inner_precise=inner_precise, prefix=prefix, actual_seq_qlen=actual_seq_qlen,
+            actual_seq_kvlen=actual_seq_kvlen, sparse_mode=sparse_mode, gen_mask_parallel=gen_mask_parallel, sync=sync,
+        )
+        ctx.save_for_backward(query, key, value, pse, padding_mask, atten_mask, res[1], res[2], res[3], res[0],
+                              res[4], res[5], res[6])
+        ctx.attrs = dict(head_num=head_num, input_layout=input_layout, scale=scale, keep_prob=keep_prob,
+                         pre_tockens=pre_tockens, next_tockens=next_tockens, inner_precise=inner_precise,
+                         prefix=prefix, actual_seq_qlen=actual_seq_qlen, actual_seq_kvlen=actual_seq_kvlen,
+                         sparse_mode=sparse_mode, gen_mask_parallel=gen_mask_parallel, sync=sync)
+        return res
+
+    @staticmethod
+    def backward(ctx, grad0, *unused):
+        (query, key, value, pse, padding_mask, atten_mask, smax, ssum, sout, out, seed, offset, numels) = ctx.saved_tensors
+        a = ctx.attrs
+        dq, dk, dv, dpse = torch.ops.npu_graph.npu_fa_backward(
+            query, key, value, grad0, a["head_num"], a["input_layout"], pse=pse, padding_mask=padding_mask,
+            atten_mask=atten_mask, softmax_max=smax, softmax_sum=ssum, softmax_in=sout, attention_in=out,
+            scale_value=a["scale"], keep_prob=a["keep_prob"], pre_tockens=a["pre_tockens"],
+            next_tockens=a["next_tockens"], inner_precise=a["inner_precise"], seed=seed, offset=offset, numels=numels,
+            prefix=a["prefix"], actual_seq_qlen=a["actual_seq_qlen"], actual_seq_kvlen=a["actual_seq_kvlen"],
+            sparse_mode=a["sparse_mode"], gen_mask_parallel=a["gen_mask_parallel"], sync=a["sync"],
+        )
+        return (dq, dk, dv, None, None, dpse) + (None,) * 13
+
+
+def npu_fusion_attention_graph(query, key, value, head_num, input_layout, pse=None, padding_mask=None,
+                               atten_mask=None, scale=1.0, keep_prob=1.0, pre_tockens=TOKEN_MAX,
+                               next_tockens=TOKEN_MAX, inner_precise=0, prefix=None, actual_seq_qlen=None,
+                               actual_seq_kvlen=None, sparse_mode=0, gen_mask_parallel=True, sync=False):
+    """Public entry (reference inductor_x/npu_fusion_attention_graph.py:125-132).
+    `scale` is the divisor applied to the scores, as the graph pattern passes it."""
+    return GraphAttentionFunction.apply(
+        query, key, value, head_num, input_layout, pse, padding_mask, atten_mask, scale, keep_prob, pre_tockens,
+        next_tockens, inner_precise, prefix, actual_seq_qlen, actual_seq_kvlen, sparse_mode, gen_mask_parallel, sync,
+    )
+
+
+# ---------------------------------------------------------------------------
+# graph pattern
+# ---------------------------------------------------------------------------
+def _attention_pattern_1(query, key, value, inv_scale_factor, dropout_p):
+    q = query.permute(0, 2, 1, 3)
+    k = key.permute(0, 2, 1, 3)
+    v = value.permute(0, 2, 1, 3)
+    return torch.nn.functional.dropout(
+        torch.matmul(q, k.transpose(-2, -1)).div(inv_scale_factor).softmax(dim=-1), p=dropout_p
+    ).matmul(v)
+
+
+def _attention_replacement_1(query, key, value, inv_scale_factor, dropout_p):
+    from torch._dynamo.utils import counters
+
+    counters["inductor"]["fuse_attention"] += 1
+    head_num = query.size(2)
+    return npu_fusion_attention_graph(
+        query.transpose(1, 2), key.transpose(1, 2), value.transpose(1, 2), head_num, "BNSD", None,
+        atten_mask=None, scale=inv_scale_factor, keep_prob=1.0 - dropout_p,
+    )[0]
+
+
+def _extra_check(match) -> bool:
+    """Only rewrite what the kernel can run: bf16 GPU tensors with head dim 128."""
+    try:
+        q = match.kwargs["query"].meta["val"]
+    except Exception:
+        return False
+    return (
+        q.device.type == "cuda" and q.dtype == torch.bfloat16 and q.dim() == 4 and q.size(3) == 128
+        and q.size(1) % 128 == 0
+    )
+
+
+_registered = False
+
+
+def register_fx_pass() -> None:
+    """Register the replacement with Inductor's joint-graph pattern pass
+    (reference inductor_x/npu_fusion_attention_graph.py:134-230).  Inference
+    only: the training variant needs npu_fa_backward."""
+    global _registered
+    if _registered:
+        return
+    _registered = True
+    from torch._inductor.fx_passes import joint_graph
+    from torch._inductor.fx_passes.fuse_attention import partialize_and_update_signature
+    from torch._inductor.pattern_matcher import fwd_only, init_once_fakemode, register_replacement
+
+    @init_once_fakemode
+    def _init():
+        device = "cuda" if torch.cuda.is_available() else "cpu"
+        g = functools.partial(torch.empty, (2, 4, 8, 16), device=device, dtype=torch.float)
+        c = functools.partial(torch.tensor, 2.0, device=device, dtype=torch.float)
+        pattern = partialize_and_update_signature(_attention_pattern_1, dropout_p=0.0)
+        replacement = partialize_and_update_signature(_attention_replacement_1, dropout_p=0.0)
+        register_replacement(
+            pattern, replacement, [g(), g(), g(), c()], fwd_only, joint_graph.patterns,
+            extra_check=_extra_check, scalar_workaround={},
+        )
+
+    original_lazy_init = joint_graph.lazy_init
+
+    @functools.wraps(original_lazy_init)
+    def lazy_init_with_attention():
+        original_lazy_init()
+        _init()
+
+    joint_graph.lazy_init = lazy_init_with_attention

@@ -390,3 +390,99 @@ def pointwise_plan(numel: int, elem_bytes: int, inner_extent: int) -> tuple[int,
     `inner_extent` elements long."""
     vec = vector_width(elem_bytes, inner_extent, numel)
     return 256, vec
+
+
+# ---------------------------------------------------------------------------
+# Kernels emitted by the Inductor code generator
+# ---------------------------------------------------------------------------
+def split_factor(rows: int, cols: int, ct: int, rl: int, vec: int, elem_bytes: int = 4, unroll: int = 4,
+                 words: int = 5, hw: Optional[config.Hardware] = None) -> tuple[int, int]:
+    """(nsplit, rows_per_split) for a generated column kernel whose workgroup
+    shape (ct x rl threads, vec columns per thread) is already fixed.  Same
+    rules as split_reduction_plan."""
+    hw = hw or config.hardware()
+    col_tiles = cdiv(cols, ct * vec)
+    waves_per_wg = max(ct * rl // hw.wave_size, 1)
+    want_waves = hw.cu_count * waves_per_cu_target(unroll, 64, hw)
+    nsplit = cdiv(want_waves, waves_per_wg * col_tiles)
+    if nsplit * col_tiles > hw.cu_count:
+        per = max(hw.cu_count // col_tiles, 1)
+        nsplit = cdiv(nsplit, per) * per
+    cap_ws = int(0.05 * rows * elem_bytes / (8 * max(words, 1)))
+    cap_rows = rows // (rl * unroll)
+    nsplit = max(min(nsplit, max(cap_ws, 1), max(cap_rows, 1)), 1)
+    batch = rl * unroll
+    rows_per_split = cdiv(cdiv(rows, nsplit), batch) * batch
+    return cdiv(rows, rows_per_split), rows_per_split
+
+
+_DRYRUN = os.environ.get("INDUCTOR_X_AMD_DRYRUN", "0") == "1"
+
+
+class GeneratedKernel:
+    """Run-time side of one generated kernel: compiles (or fetches) its code
+    object on first use and launches it through the C-ABI launcher.  This is the
+    object the generated wrapper calls, in the place of the reference's
+    `kernel.run(*args, grid=grid(...), stream=stream0)`
+    (reference test/npu_indexing/issue61_test.py:62)."""
+
+    def __init__(self, name: str, meta: dict, source: str):
+        self.name = name
+        self.meta = dict(meta)
+        self.source = source
+        self.mode = meta["mode"]
+        self._fns: Optional[dict] = None
+
+    def precompile(self) -> None:
+        if self._fns is not None:
+            return
+        path = codecache.compile_source(self.source, label=self.name)
+        self.hsaco_path = path
+        if _DRYRUN:
+            self._fns = {}
+            return
+        with open(path, "rb") as f:
+            mod = launcher.Module(f.read(), label=self.name)
+        if self.mode == "col":
+            self._fns = {"partial": mod.function(self.name + "_partial"), "final": mod.function(self.name + "_final")}
+        else:
+            self._fns = {"main": mod.function(self.name)}
+        self._module = mod
+
+    @staticmethod
+    def _raw(a):
+        return a.data_ptr() if hasattr(a, "data_ptr") else int(a)
+
+    def run(self, *args, xnumel: int, r0_numel: int = 1, stream: int = 0) -> None:
+        self.precompile()
+        if _DRYRUN:
+            return
+        xnumel, rnumel = int(xnumel), int(r0_numel)
+        if xnumel == 0:
+            return
+        m = self.meta
+        raw = tuple(self._raw(a) for a in args)
+        if self.mode == "pointwise":
+            grid = (cdiv(xnumel, m["block"] * m["vec"]), 1, 1)
+            self._fns["main"].launch(m["signature"], raw + (xnumel,), grid, (m["block"],), stream)
+        elif self.mode == "row":
+            grid = (cdiv(xnumel, m["block"] // m["tpr"]), 1, 1)
+            self._fns["main"].launch(m["signature"], raw + (xnumel, rnumel), grid, (m["block"],), stream)
+        else:
+            import torch
+
+            nsplit, rps = split_factor(rnumel, xnumel, m["ct"], m["rl"], m["vec"], words=m["ws_words"])
+            dev = next(a.device for a in args if hasattr(a, "device"))
+            ws = torch.empty(m["ws_words"] * nsplit * xnumel, dtype=torch.float32, device=dev)
+            full = raw + (ws.data_ptr(), xnumel, rnumel, rps, nsplit)
+            self._fns["partial"].launch(
+                m["signature"], full, (cdiv(xnumel, m["ct"] * m["vec"]), nsplit, 1), (m["block"],), stream,
+                m["lds_partial"],
+            )
+            self._fns["final"].launch(
+                m["signature"], full, (cdiv(xnumel, m["cpw"]), 1, 1), (m["cpw"] * m["sl"],), stream
+            )
+
+
+def generated_kernel(name: str, meta: dict, source: str) -> GeneratedKernel:
+    return GeneratedKernel(name, meta, source)

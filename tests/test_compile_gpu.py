@@ -1,0 +1,235 @@
+"""torch.compile through the backend's import hook vs eager and vs the oracle.
+
+These read like the reference's own tests (compile with backend="inductor",
+compare with eager, rtol = atol = 1e-3: reference
+test/npu_indexing/reduction_test.py:28-30, permute_test.py:23-27,
+argmax_test.py:19-23), plus the oracle comparison at the tolerances of the
+benchmark definition.  Each test also checks that the generated wrapper calls
+generated HIP kernels and no Triton kernel.
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import announce, bits
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def backend():
+    import inductor_x_amd  # noqa: F401  registration side effects
+
+    return inductor_x_amd
+
+
+@pytest.fixture(scope="module")
+def O():
+    from oracle import oracle
+
+    return oracle
+
+
+def compile_and_code(fn, *args):
+    from torch._inductor.utils import run_and_get_code
+
+    torch._dynamo.reset()
+    out, codes = run_and_get_code(torch.compile(fn, backend="inductor"), *args)
+    code = "\n".join(codes)
+    assert "generated_kernel(" in code, "no generated HIP kernel in the wrapper"
+    assert "triton.jit" not in code and "@triton" not in code, "Triton code was generated"
+    return out, code
+
+
+def test_pointwise_add_shapes():
+    # reference test/npu_indexing/pointwise_test.py:12-31
+    for shape in [(8, 8, 256, 128), (3, 5, 7), (1024,), (2, 3, 5, 9)]:
+        announce(f"compile a+b {shape}")
+        a, b = torch.randn(*shape, device=DEV), torch.randn(*shape, device=DEV)
+        out, _ = compile_and_code(lambda a, b: a + b, a, b)
+        torch.testing.assert_close(out, a + b, rtol=1e-3, atol=1e-3)
+
+
+def test_graph1_pointwise_rowsum(O):
+    announce("compile graph 1")
+    torch.manual_seed(0)
+    x = torch.randn(1024, 4096)
+    f = lambda x: (torch.relu(2 * x + 1) * torch.sigmoid(x)).sum(-1)  # noqa: E731
+    out, code = compile_and_code(f, x.to(DEV))
+    assert code.count("generated_kernel(") == 1 and "'mode': 'row'" in code
+    np.testing.assert_allclose(out.cpu().numpy(), O.relu_sigmoid_rowsum(x.numpy()), rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(out, f(x.to(DEV)), rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("shape", [(9, 1024), (32, 8, 2048), (2053, 7, 9), (8, 16, 512, 64), (1, 1, 7168), (77, 33000)])
+def test_last_dim_sum_and_mean(shape):
+    # reference test/npu_indexing/reduction_test.py:12-33, issue70_test.py:11-23
+    announce(f"compile sum/mean {shape}")
+    a, b = torch.randn(*shape, device=DEV), torch.randn(*shape, device=DEV)
+    out, _ = compile_and_code(lambda a, b: ((a + b).sum(-1), (a + b).mean(-1)), a, b)
+    torch.testing.assert_close(out[0], (a + b).sum(-1), rtol=1e-3, atol=1e-3)
+    torch.testing.assert_close(out[1], (a + b).mean(-1), rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("dim", [0, 1, 2, 3])
+def test_sum_every_dim(dim):
+    # reference test/npu_indexing/reduction_test.py:36-42
+    announce(f"compile sum dim={dim}")
+    a = torch.randn(8, 16, 512, 64, device=DEV)
+    out, _ = compile_and_code(lambda a: a.sum(dim), a)
+    torch.testing.assert_close(out, a.sum(dim), rtol=1e-3, atol=1e-3)
+
+
+def test_graph2_add_rmsnorm(O):
+    announce("compile graph 2")
+    torch.manual_seed(0)
+    rows, cols = 2048, 4096
+    h = torch.randn(rows, cols).bfloat16()
+    r = torch.randn(rows, cols).bfloat16()
+    w = (1 + 0.02 * torch.randn(cols)).bfloat16()
+
+    def f(h, r, w):
+        s = h + r
+        sf = s.float()
+        out = (sf * torch.rsqrt(sf.pow(2).mean(-1, keepdim=True) + 1e-6) * w.float()).to(torch.bfloat16)
+        return out, s
+
+    (out, s), code = compile_and_code(f, h.to(DEV), r.to(DEV), w.to(DEV))
+    assert code.count("generated_kernel(") == 1 and "'mode': 'row'" in code
+    o_ref, s_ref = O.add_rmsnorm_bf16(bits(h), bits(r), bits(w), 1e-6)
+    assert np.array_equal(bits(s), s_ref)
+    assert np.abs(O.bf16_bits_to_f32(bits(out)) - O.bf16_bits_to_f32(o_ref)).max() <= 2e-2
+
+
+def test_graph3_col_mean_var_argmax(O):
+    announce("compile graph 3")
+    torch.manual_seed(0)
+    x = torch.randn(65536, 512)
+    f = lambda x: (x.mean(0), x.var(0, unbiased=False), x.argmax(0))  # noqa: E731
+    (mean, var, arg), code = compile_and_code(f, x.to(DEV))
+    assert "'mode': 'col'" in code
+    m_ref, v_ref, a_ref = O.col_mean_var_argmax(x.numpy(), 0.0)
+    assert np.array_equal(arg.cpu().numpy(), a_ref)
+    scale = np.sqrt(v_ref)
+    assert (np.abs(mean.cpu().numpy() - m_ref) <= 1e-5 * np.maximum(np.abs(m_ref), scale)).all()
+    np.testing.assert_allclose(var.cpu().numpy(), v_ref, rtol=1e-5)
+
+
+@pytest.mark.parametrize("shape,dim", [((512, 64), -1), ((513, 64), -1), ((513, 1024), -1), ((4096, 64), 0), ((300, 7, 12), 1)])
+def test_argmax(shape, dim):
+    # reference test/npu_indexing/argmax_test.py:10-25, argmax_unalign_test.py:36-58
+    announce(f"compile argmax {shape} dim={dim}")
+    torch.manual_seed(1)
+    x = torch.randn(*shape, device=DEV) * 2000
+    x[3] = x[1]  # ties between rows
+    out, _ = compile_and_code(lambda x: torch.argmax(x, dim), x)
+    assert torch.equal(out, torch.argmax(x, dim))
+
+
+@pytest.mark.parametrize("dims", [[0, 2], [0, 1], [1, 2], [0], [1], [2]])
+def test_var_mean_dims(dims):
+    # reference test/npu_indexing/var_mean_test.py:8-36 (default correction)
+    announce(f"compile var_mean {dims}")
+    x = torch.randn(128, 8, 64, device=DEV)
+    out, _ = compile_and_code(lambda x: torch.var_mean(x, dims), x)
+    ref = torch.var_mean(x, dims)
+    torch.testing.assert_close(out[0], ref[0], rtol=1e-3, atol=1e-3)
+    torch.testing.assert_close(out[1], ref[1], rtol=1e-3, atol=1e-3)
+
+
+def test_graph4_gather_and_permute(O):
+    announce("compile graph 4")
+    torch.manual_seed(0)
+    table = (0.02 * torch.randn(50304, 1024)).bfloat16()
+    idx = torch.randint(0, 50304, (4096,), dtype=torch.int64)
+    out, code = compile_and_code(lambda t, i: t[i], table.to(DEV), idx.to(DEV))
+    assert np.array_equal(bits(out), O.gather_rows(bits(table), idx.numpy()))
+    emb, _ = compile_and_code(lambda t, i: torch.nn.functional.embedding(i, t), table.to(DEV), idx.to(DEV))
+    assert torch.equal(emb, out)
+    t = torch.randn(4, 2048, 32, 128).bfloat16()
+    out, code = compile_and_code(lambda t: t.permute(0, 2, 1, 3).contiguous(), t.to(DEV))
+    assert "mi::vload<VEC>" in code and "mi::vstore<VEC>" in code  # 16-byte accesses on both sides
+    assert np.array_equal(bits(out), O.permute4(bits(t), (0, 2, 1, 3)))
+
+
+@pytest.mark.parametrize("perm", [(0, 2, 1, 3), (0, 1, 3, 2), (3, 2, 1, 0), (1, 0, 2, 3), (0, 3, 1, 2)])
+def test_permute_variants(perm):
+    # reference test/npu_indexing/permute_test.py:7-30
+    announce(f"compile permute {perm}")
+    x = torch.randn(8, 8, 64, 128, device=DEV)
+    out, _ = compile_and_code(lambda x: x.permute(*perm).contiguous() + 1.0, x)
+    assert torch.equal(out, x.permute(*perm).contiguous() + 1.0)
+
+
+def test_reduction_broadcast_permute():
+    # reference test/npu_indexing/reduction_broadcast_permute_test.py:9-33
+    announce("compile sum -> broadcast -> permute")
+    a = torch.randn(8, 16, 64, 32, device=DEV)
+
+    def f(a):
+        s = a.sum(2, keepdim=True)
+        return (a - s).permute(0, 2, 1, 3).contiguous()
+
+    out, _ = compile_and_code(f, a)
+    torch.testing.assert_close(out, f(a), rtol=1e-3, atol=1e-3)
+
+
+def test_layernorm_fp16_and_softmax():
+    # reference test/npu_indexing/issue62_test.py:8-47 (LayerNorm through var_mean + rsqrt)
+    announce("compile layernorm / softmax")
+    x = torch.randn(64, 1024, device=DEV, dtype=torch.float16)
+    w = torch.randn(1024, device=DEV, dtype=torch.float16)
+    b = torch.randn(1024, device=DEV, dtype=torch.float16)
+    f = lambda x, w, b: torch.nn.functional.layer_norm(x, (1024,), w, b, 1e-5)  # noqa: E731
+    out, _ = compile_and_code(f, x, w, b)
+    torch.testing.assert_close(out, f(x, w, b), rtol=1e-2, atol=1e-2)
+    y = torch.randn(33, 5000, device=DEV)
+    out, _ = compile_and_code(lambda y: torch.softmax(y, -1), y)
+    torch.testing.assert_close(out, torch.softmax(y, -1), rtol=1e-3, atol=1e-5)
+
+
+def test_clamp_where_dtypes():
+    # reference test/npu_indexing/clamp_test.py:28-114
+    announce("compile clamp / where / dtypes")
+    for dtype in (torch.float32, torch.bfloat16, torch.int32, torch.int64):
+        x = (torch.randn(37, 129, device=DEV) * 10).to(dtype)
+        f = lambda x: torch.where(x > 1, x.clamp(-3, 3), x * 2)  # noqa: E731
+        out, _ = compile_and_code(f, x)
+        torch.testing.assert_close(out, f(x), rtol=1e-3, atol=1e-3)
+
+
+def test_attention_op_and_pattern():
+    """The custom op under torch.compile, and the graph pattern rewriting the
+    unfused matmul-softmax-matmul into it."""
+    announce("compile attention op / pattern")
+    from torch._dynamo.utils import counters
+
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
+    torch.manual_seed(0)
+    B, S, N, D = 2, 256, 4, 128
+    q, k, v = (torch.randn(B, N, S, D, device=DEV).bfloat16() for _ in range(3))
+    inv_scale = D ** 0.5
+
+    def f(q, k, v):
+        return npu_fusion_attention_graph(q, k, v, N, "BNSD", scale=inv_scale, sparse_mode=3)[0]
+
+    torch._dynamo.reset()
+    out = torch.compile(f)(q, k, v)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float(), is_causal=True)
+    assert (out.float() - ref).abs().max().item() <= 2e-2
+
+    qs, ks, vs = (t.transpose(1, 2).contiguous() for t in (q, k, v))  # [B, S, N, D]
+
+    def g(q, k, v):
+        q, k, v = (t.permute(0, 2, 1, 3) for t in (q, k, v))
+        return torch.matmul(q, k.transpose(-2, -1)).div(inv_scale).softmax(dim=-1).matmul(v)
+
+    torch._dynamo.reset()
+    counters.clear()
+    with torch.no_grad():
+        out = torch.compile(g)(qs, ks, vs)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
+    assert (out.float() - ref).abs().max().item() <= 2e-2
+    assert counters["inductor"]["fuse_attention"] >= 1
