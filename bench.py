@@ -91,53 +91,87 @@ def _graph_time_ms(fn, launches_per_graph: int = 20, replays: int = 5) -> float:
 
 
 def _all_configs(K, torch) -> list:
+    """Every graph of the benchmark definition, two ways: the hand-written kernel
+    family called directly through the launcher ("kernel"), and the same graph
+    written in PyTorch and compiled through the backend's import hook
+    ("torch.compile": generated HIP kernels; the attention graph reaches the
+    MFMA kernel through the custom op)."""
+    import inductor_x_amd  # noqa: F401  registers the Inductor backend
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
     dev = "cuda:0"
     out = []
 
-    def add(name, fn, work, bound):
+    def add(name, path, fn, work, bound):
         try:
             ms = _graph_time_ms(fn)
             how = "hip-graph replay"
         except Exception as e:  # capture unsupported: time the plain loop instead
-            ms = _event_time_ms(fn, 20)
-            how = f"event loop ({type(e).__name__})"
+            try:
+                ms = _event_time_ms(fn, 20)
+                how = f"event loop ({type(e).__name__})"
+            except Exception as e2:
+                out.append({"config": name, "path": path, "error": f"{type(e2).__name__}: {e2}"[:200]})
+                return
         if bound == "hbm":
             ach = work / ms / 1e6
-            out.append({"config": name, "ms": round(ms, 5), "bound": "hbm", "achieved": round(ach, 1),
+            out.append({"config": name, "path": path, "ms": round(ms, 5), "bound": "hbm", "achieved": round(ach, 1),
                         "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "timing": how})
         else:
             ach = work / ms / 1e9
-            out.append({"config": name, "ms": round(ms, 5), "bound": "mfma", "achieved": round(ach, 1),
+            out.append({"config": name, "path": path, "ms": round(ms, 5), "bound": "mfma", "achieved": round(ach, 1),
                         "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "timing": how})
+
+    def both(name, direct, graph_fn, args, work, bound):
+        add(name, "kernel", lambda: direct(*args), work, bound)
+        try:
+            torch._dynamo.reset()
+            cf = torch.compile(graph_fn)
+            cf(*args)
+            add(name, "torch.compile", lambda: cf(*args), work, bound)
+        except Exception as e:
+            out.append({"config": name, "path": "torch.compile", "error": f"{type(e).__name__}: {e}"[:200]})
 
     torch.manual_seed(0)
     x = torch.randn(1024, 4096).to(dev)
-    add("1 pointwise+rowsum fp32 [1024,4096] (cache-warm)", lambda: K.fused_relu_sigmoid_rowsum(x), ALGO_BYTES["rowsum"], "hbm")
+    both("1 pointwise+rowsum fp32 [1024,4096] (cache-warm)", K.fused_relu_sigmoid_rowsum,
+         lambda x: (torch.relu(2 * x + 1) * torch.sigmoid(x)).sum(-1), (x,), ALGO_BYTES["rowsum"], "hbm")
     del x
     torch.manual_seed(0)
     h = torch.randn(8192, 4096).bfloat16().to(dev)
     r = torch.randn(8192, 4096).bfloat16().to(dev)
     w = (1 + 0.02 * torch.randn(4096)).bfloat16().to(dev)
-    add("2 add+rmsnorm bf16 [8192,4096]", lambda: K.add_rmsnorm(h, r, w, 1e-6), ALGO_BYTES["add_rmsnorm"], "hbm")
+
+    def rms(h, r, w):
+        s = h + r
+        sf = s.float()
+        return (sf * torch.rsqrt(sf.pow(2).mean(-1, keepdim=True) + 1e-6) * w.float()).to(torch.bfloat16), s
+
+    both("2 add+rmsnorm bf16 [8192,4096]", lambda h, r, w: K.add_rmsnorm(h, r, w, 1e-6), rms, (h, r, w),
+         ALGO_BYTES["add_rmsnorm"], "hbm")
     del h, r, w
     torch.manual_seed(0)
     x = torch.randn(65536, 512).to(dev)
-    add("3 col mean/var/argmax fp32 [65536,512]", lambda: K.col_mean_var_argmax(x), ALGO_BYTES["col_mean_var_argmax"], "hbm")
+    both("3 col mean/var/argmax fp32 [65536,512]", K.col_mean_var_argmax,
+         lambda x: (x.mean(0), x.var(0, unbiased=False), x.argmax(0)), (x,), ALGO_BYTES["col_mean_var_argmax"], "hbm")
     del x
     torch.manual_seed(0)
     table = (0.02 * torch.randn(50304, 1024)).bfloat16().to(dev)
     idx = torch.randint(0, 50304, (32768,), dtype=torch.int64).to(dev)
-    add("4a gather bf16 [50304,1024][32768]", lambda: K.gather_rows(table, idx), ALGO_BYTES["gather"], "hbm")
+    both("4a gather bf16 [50304,1024][32768]", K.gather_rows, lambda t, i: t[i], (table, idx), ALGO_BYTES["gather"], "hbm")
     del table, idx
     torch.manual_seed(0)
     t = torch.randn(16, 2048, 32, 128).bfloat16().to(dev)
-    add("4b permute(0,2,1,3) bf16 [16,2048,32,128]", lambda: K.permute_0213_contiguous(t), ALGO_BYTES["permute"], "hbm")
+    both("4b permute(0,2,1,3) bf16 [16,2048,32,128]", K.permute_0213_contiguous,
+         lambda t: t.permute(0, 2, 1, 3).contiguous(), (t,), ALGO_BYTES["permute"], "hbm")
     del t
     torch.manual_seed(0)
     q = torch.randn(4, 32, 4096, 128).bfloat16().to(dev)
     k = torch.randn(4, 32, 4096, 128).bfloat16().to(dev)
     v = torch.randn(4, 32, 4096, 128).bfloat16().to(dev)
-    add("5 causal attention bf16 [4,32,4096,128]", lambda: K.fused_attention(q, k, v, 128 ** -0.5, True), ATTN_FLOPS_CAUSAL, "mfma")
+    both("5 causal attention bf16 [4,32,4096,128]", lambda q, k, v: K.fused_attention(q, k, v, 128 ** -0.5, True),
+         lambda q, k, v: npu_fusion_attention_graph(q, k, v, 32, "BNSD", scale=128 ** 0.5, sparse_mode=3)[0],
+         (q, k, v), ATTN_FLOPS_CAUSAL, "mfma")
     return out
 
 

@@ -23,6 +23,9 @@ CSRC_DIR = os.path.join(_HERE, "csrc")
 HEADER_DIR = os.path.join(CSRC_DIR, "mi")
 AOT_DIR = os.path.join(CSRC_DIR, "aot")
 INTREE_STORE = os.path.join(_HERE, "_hsaco")
+# Code objects of generated (torch.compile) kernels that ship with the tree, so a
+# machine that has seen a graph before does not invoke hipcc for it again.
+GENERATED_STORE = os.path.join(_HERE, "_hsaco_gen")
 
 ARCH = "gfx950"
 # Packed-fp32 instruction selection is switched off for every device compile.
@@ -82,7 +85,7 @@ def user_store() -> str:
 
 
 def _stores() -> list[str]:
-    return [INTREE_STORE, user_store()]
+    return [INTREE_STORE, GENERATED_STORE, user_store()]
 
 
 def lookup(key: str) -> Optional[str]:

@@ -23,6 +23,7 @@ from __future__ import annotations
 import dataclasses
 import itertools
 import math
+import os
 from typing import Any, Optional, Sequence, Union
 
 import sympy
@@ -657,7 +658,8 @@ class HipKernel(SIMDKernel):
             xnumel = self._static_numel("x")
             groups = max(-(-(xnumel or 512) // self.vec), 1)
             self.col_ct = min(next_power_of_2(groups), 128)
-            self.col_rl = max(1024 // self.col_ct, 1)
+            # 8 wavefronts per workgroup: the measured sweet spot for streaming column sweeps
+            self.col_rl = max(int(os.environ.get("INDUCTOR_X_AMD_COL_THREADS", "512")) // self.col_ct, 1)
             self.block = self.col_ct * self.col_rl
         else:
             self.block = 256
@@ -796,6 +798,17 @@ class HipKernel(SIMDKernel):
             out.is_vec = out.is_vec or is_vec
         return out
 
+    STREAMING_BYTES = 32 << 20
+
+    def _is_streaming_buffer(self, name: str) -> bool:
+        """Outputs far larger than L2 are written with the non-temporal hint."""
+        try:
+            buf = V.graph.get_buffer(name)
+            numel = V.graph.sizevars.size_hint(buf.get_numel())
+            return int(numel) * dtype_nbytes(V.graph.get_dtype(name)) >= self.STREAMING_BYTES
+        except Exception:
+            return False
+
     def _index_uses_tree(self, index: sympy.Expr, prefix: str) -> bool:
         for s in index.free_symbols:
             e = self.range_tree_nodes.get(s)
@@ -823,10 +836,13 @@ class HipKernel(SIMDKernel):
         if kind == "contiguous":
             aligned = self.index_is_aligned(index) and self._buffer_aligned(name)
             ptr = f"{var} + ({self.index_to_str(index)})"
+            stream = ", true" if self._is_streaming_buffer(name) else ""
             if mask is None:
-                line = f"mi::vstore<VEC>({ptr}, {value});" if aligned else f"mi::vstore_u<VEC>({ptr}, {value});"
+                line = f"mi::vstore<VEC{stream}>({ptr}, {value});" if aligned else f"mi::vstore_u<VEC>({ptr}, {value});"
+            elif aligned:
+                line = f"mi::vstore_m<VEC{stream}>({ptr}, {value}, {mask});"
             else:
-                line = f"mi::vstore_m<VEC>({ptr}, {value}, {mask});"
+                line = f"mi::scatter_m<VEC>({var}, {self.index_to_vec_str(index)}, {value}, {mask});"
         elif kind == "uniform":
             line = f"mi::vstore<1>({var} + ({self.index_to_str(index)}), {value});"
             if mask is not None:
@@ -1100,7 +1116,7 @@ class HipKernel(SIMDKernel):
             src.writeline("if (xmask) {")
             with src.indent():
                 src.splice(self._entry_code(self.x_entries))
-                src.writeline("#pragma unroll 4")
+                src.writeline(f"#pragma unroll {int(os.environ.get('INDUCTOR_X_AMD_COL_UNROLL', '4'))}")
                 src.writeline(f"for ({idx_t} r0_index = r_begin + rl; r0_index < r_end; r0_index += RL) {{")
                 with src.indent():
                     src.splice(self.partial_body)
@@ -1110,7 +1126,7 @@ class HipKernel(SIMDKernel):
                 kind = REDUCTION_KIND[c.kind]
                 src.writeline(f"typename {kind}::M {c.acc}_m[VEC];")
                 src.writeline("#pragma unroll")
-                src.writeline(f"for (int i = 0; i < VEC; ++i) {c.acc}_m[i] = {kind}::finish({c.acc}.s[i]);")
+                src.writeline(f"for (int i = 0; i < VEC; ++i) {c.acc}_m[i] = {c.acc}.finish(i);")
                 src.writeline(f"mi::col_fold<{kind}, VEC, CT, RL>({c.acc}_m, ct, rl, lds_dyn);")
                 src.writeline(
                     f"if (rl == 0) mi::col_store_partial<{kind}, VEC>(ws + {c.ws_offset_words} * "

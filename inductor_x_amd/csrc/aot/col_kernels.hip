@@ -26,6 +26,11 @@ COL_PARTIAL_VARIANT(64, 16, 4)
 COL_PARTIAL_VARIANT(64, 1, 8)
 COL_PARTIAL_VARIANT(16, 16, 4)
 COL_PARTIAL_VARIANT(1, 64, 4)
+COL_PARTIAL_VARIANT(16, 64, 4)
+COL_PARTIAL_VARIANT(32, 32, 4)
+COL_PARTIAL_VARIANT(32, 16, 4)
+COL_PARTIAL_VARIANT(16, 32, 4)
+COL_PARTIAL_VARIANT(64, 8, 8)
 
 #define COL_FINAL_VARIANT(CPW, SL)                                                            \
   extern "C" __global__ __launch_bounds__(CPW* SL) void                                       \

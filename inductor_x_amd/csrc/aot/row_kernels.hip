@@ -120,3 +120,5 @@ RMSNORM_VARIANT(256, 256, 4)
 RMSNORM_VARIANT(256, 64, 1)
 RMSNORM_VARIANT(256, 64, 2)
 RMSNORM_VARIANT(256, 64, 4)
+RMSNORM_VARIANT(512, 512, 2)
+RMSNORM_VARIANT(512, 512, 4)

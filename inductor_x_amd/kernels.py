@@ -62,6 +62,8 @@ _RMSNORM_VARIANTS = [
     (256, 64, 1),
     (256, 64, 2),
     (256, 64, 4),
+    (512, 512, 2),
+    (512, 512, 4),
 ]
 _COL_PARTIAL_VARIANTS = [
     (128, 2, 4),
@@ -77,6 +79,11 @@ _COL_PARTIAL_VARIANTS = [
     (64, 1, 8),
     (16, 16, 4),
     (1, 64, 4),
+    (16, 64, 4),
+    (32, 32, 4),
+    (32, 16, 4),
+    (16, 32, 4),
+    (64, 8, 8),
 ]
 _COL_FINAL_VARIANTS = [(16, 16), (8, 32), (4, 64), (64, 4)]
 _GATHER_VARIANTS = [(256, 128, 1), (256, 128, 2), (256, 128, 4), (256, 64, 1), (256, 64, 2), (256, 64, 4), (256, 16, 1), (256, 16, 4)]
@@ -234,14 +241,11 @@ def add_rmsnorm(
         plan = row_reduction_plan(rows, cols, 2, persistent=True)
         tpr = max(plan.tpr, 64)  # instantiated shapes start at one wavefront per row
         iters = next_power_of_2(cdiv(cdiv(cols, 8), tpr))
-        block = max(256, tpr)
-        _require(iters <= 8 and block <= 512, f"row length {cols} exceeds the persistent kernel's reach")
-        variant = (block, tpr, iters)
-        # map onto an instantiated variant
+        variant = (max(256, tpr), tpr, iters)
         have = set(_RMSNORM_VARIANTS)
         while variant not in have and variant[2] < 8:
             variant = (variant[0], variant[1], variant[2] * 2)
-        _require(variant in have, f"no add_rmsnorm variant for row length {cols}")
+        _require(variant in have, f"row length {cols} exceeds the persistent kernel's reach")
     b, t, i = variant
     _require(cols <= t * 8 * i, "variant too small for the row length")
     idx = _find(l, f"add_rmsnorm_bf16_b{b}_t{t}_i{i}")
