@@ -33,9 +33,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
 
 # HBM bytes per launch of add_rmsnorm_bf16 at [8192, 4096], from rocprofv3 --pmc
 # FETCH_SIZE and WRITE_SIZE runs scaled by the same counters on a plain copy
-# kernel of known size; summary in profiles/add_rmsnorm_bf16_8192x4096_pmc.txt.
-# None until that profile has been taken.
-MEASURED_TRAFFIC_BYTES = {"add_rmsnorm": None}
+# kernel of known size (scale factors 1.99984 and 0.99922); summary in
+# profiles/add_rmsnorm_bf16_8192x4096_pmc.txt.
+MEASURED_TRAFFIC_BYTES = {"add_rmsnorm": 268_550_300}
 
 ALGO_BYTES = {
     "rowsum": 16_781_312,
@@ -272,6 +272,8 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-all-configs", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 256 MiB copy kernel 10 times (calibrates HBM byte counters under rocprofv3 --pmc)")
     ap.add_argument("--cpu-baseline-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
 
@@ -343,6 +345,14 @@ def main() -> None:
         },
     }
     del h, r, w
+    if args.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            K.copy_bytes(dst, src)
+        torch.cuda.synchronize()
+        line["copy_probe"] = {"kernel": "copy_b128", "bytes_read": 256 << 20, "bytes_written": 256 << 20, "launches": 10}
+        del src, dst
     if not args.no_all_configs:
         line["all_configs"] = _all_configs(K, torch)
     line["cpu_baseline"] = (

@@ -57,3 +57,11 @@ extern "C" __global__ __launch_bounds__(256) void permute_copy_b32_b256_p16_t8x8
     long long s1, long long s2) {
   permute_copy_tiled<uint32_t, 4, 256, 16, 8, 8>(in, out, n0, n1, n2, inner, s0, s1, s2);
 }
+
+// Plain contiguous copy, 16 bytes per thread.  Used as the known-size probe that
+// calibrates the HBM byte counters (FETCH_SIZE / WRITE_SIZE) in profiles.
+extern "C" __global__ __launch_bounds__(256) void copy_b128(const uint32_t* in, uint32_t* out,
+                                                            long long n_vec) {
+  const long long i = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+  if (i < n_vec) store_vec<uint32_t, 4, true>(out + 4 * i, load_vec<uint32_t, 4>(in + 4 * i));
+}

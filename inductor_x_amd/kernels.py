@@ -182,6 +182,31 @@ def _permute_launcher() -> CachingLauncher:
     )
 
 
+@functools.lru_cache(maxsize=None)
+def _copy_launcher() -> CachingLauncher:
+    return CachingLauncher(
+        "copy_b128", codecache.aot_source("copy_kernels.hip"), "PPq", [LaunchConfig("copy_b128", 256)],
+        prefer_intree=True,
+    )
+
+
+def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
+    """dst <- src for two contiguous tensors of equal byte size (a multiple of
+    16).  A known-size streaming kernel: the probe that calibrates HBM byte
+    counters when profiling."""
+    _check_cuda(dst, src)
+    nbytes = src.numel() * src.element_size()
+    _require(dst.numel() * dst.element_size() == nbytes, "size mismatch")
+    _require(nbytes % 16 == 0 and dst.is_contiguous() and src.is_contiguous(), "contiguous, multiple of 16 bytes")
+    _require(_aligned(dst) and _aligned(src), "16-byte alignment")
+    if nbytes == 0:
+        return
+    n_vec = nbytes // 16
+    l = _copy_launcher()
+    l.precompile()
+    l._launch(0, (src.data_ptr(), dst.data_ptr(), n_vec), (cdiv(n_vec, 256), 1, 1), _stream())
+
+
 def _find(l: CachingLauncher, symbol: str) -> int:
     l.precompile()
     for i, (cfg, _) in enumerate(l.launchers):

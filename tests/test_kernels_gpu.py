@@ -275,3 +275,11 @@ def test_permute_variants(K, variant):
     t = torch.randn(3, 70, 37, inner, device=DEV).bfloat16()
     out = K.permute_0213_contiguous(t, variant=variant)
     assert torch.equal(out, t.permute(0, 2, 1, 3).contiguous())
+
+
+def test_copy_probe(K):
+    announce("copy probe")
+    src = torch.randint(0, 255, (1 << 20,), dtype=torch.uint8, device=DEV)
+    dst = torch.zeros_like(src)
+    K.copy_bytes(dst, src)
+    assert torch.equal(dst, src)
