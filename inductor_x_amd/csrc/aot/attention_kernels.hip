@@ -5,7 +5,7 @@
 // Ids that land on one die walk the query blocks of one head before moving to
 // the next head, so a head's K and V are fetched into a single L2.  With a
 // causal mask the heaviest query blocks (most key tiles) are issued first.
-#include "../mi/attention.h"
+#include "../mi/attention_pp.h"
 
 using namespace mi;
 
@@ -38,3 +38,44 @@ ATTENTION_VARIANT(fused_attention_fwd_bf16_d128_causal_w4, true, 4, 2)
 ATTENTION_VARIANT(fused_attention_fwd_bf16_d128_full_w4, false, 4, 2)
 ATTENTION_VARIANT(fused_attention_fwd_bf16_d128_causal_w8, true, 8, 1)
 ATTENTION_VARIANT(fused_attention_fwd_bf16_d128_full_w8, false, 8, 1)
+
+// pp: 512 threads, 256 queries per workgroup, the two wavefronts of every SIMD
+// alternate between the matrix phase and the softmax phase (attention_pp.h).
+template <bool CAUSAL>
+__device__ __forceinline__ void attention_entry_pp(const bf16_t* q, const bf16_t* k, const bf16_t* v,
+                                                   bf16_t* o, float* smax, float* ssum, int n_heads,
+                                                   int S, float scale_log2e) {
+  constexpr int XCDS = 8;
+  const int n_qb = S / (kAttnRowsPerWave * kAttnPPWaves);
+  const int id = blockIdx.x;
+  const int xcd = id % XCDS;
+  const int slot = id / XCDS;
+  if (CAUSAL) {
+    // Under a causal mask query block b visits 4 b + 4 key tiles.  A workgroup
+    // takes blocks b and n_qb - 1 - b one after the other, so every workgroup
+    // does the same amount of work and the last round of the launch is full.
+    const int n_pair = (n_qb + 1) / 2;
+    const int head = (slot / n_pair) * XCDS + xcd;
+    const int lo = slot % n_pair;
+    const int hi = n_qb - 1 - lo;
+    if (head >= n_heads) return;
+    attention_fwd_d128_pingpong<true>(q, k, v, o, smax, ssum, S, hi, head, scale_log2e);
+    if (lo != hi) attention_fwd_d128_pingpong<true>(q, k, v, o, smax, ssum, S, lo, head, scale_log2e);
+  } else {
+    const int head = (slot / n_qb) * XCDS + xcd;
+    const int qb = slot % n_qb;
+    if (head >= n_heads) return;
+    attention_fwd_d128_pingpong<false>(q, k, v, o, smax, ssum, S, qb, head, scale_log2e);
+  }
+}
+
+extern "C" __global__ __launch_bounds__(512, 1) void fused_attention_fwd_bf16_d128_causal_pp(
+    const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
+    int n_heads, int S, float scale_log2e) {
+  attention_entry_pp<true>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
+}
+extern "C" __global__ __launch_bounds__(512, 1) void fused_attention_fwd_bf16_d128_full_pp(
+    const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
+    int n_heads, int S, float scale_log2e) {
+  attention_entry_pp<false>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
+}

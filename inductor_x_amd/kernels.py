@@ -431,6 +431,14 @@ def _attention_launcher() -> CachingLauncher:
         )
         for c in (1, 0)
         for w in (4, 8)
+    ] + [
+        LaunchConfig(
+            f"fused_attention_fwd_bf16_d128_{'causal' if c else 'full'}_pp",
+            512,
+            meta={"CAUSAL": c, "WAVES": 8, "PINGPONG": 1},
+            lds_bytes=_ATTN_LDS_BYTES,
+        )
+        for c in (1, 0)
     ]
     return CachingLauncher(
         "fused_attention_fwd_bf16_d128",
@@ -442,7 +450,8 @@ def _attention_launcher() -> CachingLauncher:
 
 
 def fused_attention(
-    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool, waves: Optional[int] = None
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool, waves: Optional[int] = None,
+    pingpong: Optional[bool] = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """softmax(q k^T * scale [+ causal mask]) v for [B, N, S, 128] bf16 tensors.
 
@@ -467,10 +476,17 @@ def fused_attention(
     if waves is None:
         waves = _ATTN_DEFAULT_WAVES if S % 256 == 0 else 4
     _require(waves in (4, 8) and S % (32 * waves) == 0, "waves must be 4 or 8 and 32*waves must divide S")
+    if pingpong is None:
+        pingpong = _ATTN_DEFAULT_PINGPONG and waves == 8
+    _require(not pingpong or waves == 8, "the ping-pong schedule needs 8 wavefronts per workgroup")
     l = _attention_launcher()
-    i = _find(l, f"fused_attention_fwd_bf16_d128_{'causal' if causal else 'full'}_w{waves}")
+    suffix = "pp" if pingpong else f"w{waves}"
+    i = _find(l, f"fused_attention_fwd_bf16_d128_{'causal' if causal else 'full'}_{suffix}")
     heads = B * N
-    grid = 8 * cdiv(heads, 8) * (S // (32 * waves))
+    n_qb = S // (32 * waves)
+    # the causal ping-pong kernel pairs query blocks (b, n_qb - 1 - b) in one workgroup
+    per_head = (n_qb + 1) // 2 if (pingpong and causal) else n_qb
+    grid = 8 * cdiv(heads, 8) * per_head
     l._launch(
         i,
         (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), smax.data_ptr(), ssum.data_ptr(), heads, S,
@@ -482,3 +498,4 @@ def fused_attention(
 
 
 _ATTN_DEFAULT_WAVES = 8
+_ATTN_DEFAULT_PINGPONG = True

@@ -85,8 +85,14 @@ def test_attention_causality_and_sdpa_full_size_slice(K):
     q, k, v = (torch.randn(B, N, S, 128, device=DEV).bfloat16() for _ in range(3))
     scale = 128 ** -0.5
     out, smax, ssum = K.fused_attention(q, k, v, scale, True)
-    out8, smax8, ssum8 = K.fused_attention(q, k, v, scale, True, waves=8)
+    out8, smax8, ssum8 = K.fused_attention(q, k, v, scale, True, waves=8, pingpong=False)
     assert torch.equal(out, out8) and torch.equal(smax, smax8) and torch.equal(ssum, ssum8)
+    outp, smaxp, ssump = K.fused_attention(q, k, v, scale, True, waves=8, pingpong=True)
+    assert torch.equal(out, outp) and torch.equal(smax, smaxp) and torch.equal(ssum, ssump)
+    for causal in (False,):
+        a = K.fused_attention(q, k, v, scale, causal, waves=4)
+        b = K.fused_attention(q, k, v, scale, causal, waves=8, pingpong=True)
+        assert all(torch.equal(x, y) for x, y in zip(a, b))
     k2, v2 = k.clone(), v.clone()
     k2[:, :, 2048:] = torch.randn_like(k2[:, :, 2048:])
     v2[:, :, 2048:] = torch.randn_like(v2[:, :, 2048:])
