@@ -233,3 +233,46 @@ def test_attention_op_and_pattern():
     ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
     assert (out.float() - ref).abs().max().item() <= 2e-2
     assert counters["inductor"]["fuse_attention"] >= 1
+
+
+def test_ring_attention_forward_update():
+    """Merge step of ring attention: online-softmax rescale of two partial
+    attention outputs (reference test/npu_indexing/attn_cp_test.py:19-59, shapes
+    from :86-98 scaled down), compiled through the backend."""
+    announce("compile ring-attention forward_update")
+    F32_BLK = 8
+
+    def trans_bnsd2sbh(x):
+        b, n, s, d = x.shape
+        return x.permute(2, 0, 1, 3).reshape(s, b, n * d)
+
+    def broadcast_and_trans(x, h):
+        n = x.shape[1]
+        d = h // n
+        new_x = x[..., 0].unsqueeze(3).repeat(1, 1, 1, d)
+        return trans_bnsd2sbh(new_x)
+
+    def forward_update(prev_out, prev_max, prev_sum, cur_out, cur_max, cur_sum):
+        org = prev_out.dtype
+        smax = torch.maximum(prev_max, cur_max)
+        prev_scale = torch.exp(prev_max - smax)
+        cur_scale = torch.exp(cur_max - smax)
+        ps = prev_sum * prev_scale
+        cs = cur_sum * cur_scale
+        ssum = ps + cs
+        pso = broadcast_and_trans(ps / ssum, prev_out.shape[-1])
+        cso = broadcast_and_trans(cs / ssum, prev_out.shape[-1])
+        return (prev_out * pso + cur_out * cso).to(org), smax, ssum
+
+    torch.manual_seed(0)
+    S, B, H, N = 1024, 1, 1536, 12
+    mk = lambda: torch.rand((B, N, S), device=DEV).unsqueeze(3).repeat(1, 1, 1, F32_BLK)  # noqa: E731
+    args = (torch.randn(S, B, H, device=DEV), mk(), mk() + 0.5, torch.randn(S, B, H, device=DEV), mk(), mk() + 0.5)
+    out, code = compile_and_code(forward_update, *args)
+    ref = forward_update(*args)
+    for a, b in zip(out, ref):
+        torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-6)
+    bf = tuple(a.bfloat16() if i in (0, 3) else a for i, a in enumerate(args))  # bf16 outputs, fp32 statistics
+    out, _ = compile_and_code(forward_update, *bf)
+    ref = forward_update(*bf)
+    assert out[0].dtype == torch.bfloat16 and (out[0].float() - ref[0].float()).abs().max().item() <= 2e-2
