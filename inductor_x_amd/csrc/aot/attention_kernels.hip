@@ -6,6 +6,7 @@
 // the next head, so a head's K and V are fetched into a single L2.  With a
 // causal mask the heaviest query blocks (most key tiles) are issued first.
 #include "../mi/attention_pp.h"
+#include "../mi/attention_v2.h"
 
 using namespace mi;
 
@@ -78,4 +79,44 @@ extern "C" __global__ __launch_bounds__(512, 1) void fused_attention_fwd_bf16_d1
     const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
     int n_heads, int S, float scale_log2e) {
   attention_entry_pp<false>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
+}
+
+// v2: 256 threads, 64 queries per wavefront, one wavefront per SIMD (attention_v2.h).
+template <bool CAUSAL>
+__device__ __forceinline__ void attention_entry_v2(const bf16_t* q, const bf16_t* k, const bf16_t* v,
+                                                   bf16_t* o, float* smax, float* ssum, int n_heads,
+                                                   int S, float scale_log2e) {
+  constexpr int XCDS = 8;
+  const int n_qb = S / kAttnV2BM;
+  const int id = blockIdx.x;
+  const int xcd = id % XCDS;
+  const int slot = id / XCDS;
+  if (CAUSAL) {
+    const int n_pair = (n_qb + 1) / 2;
+    const int head = (slot / n_pair) * XCDS + xcd;
+    const int lo = slot % n_pair;
+    const int hi = n_qb - 1 - lo;
+    if (head >= n_heads) return;
+    // one copy of the code for both members of the pair (the longer one first)
+    const int n_pass = lo != hi ? 2 : 1;
+#pragma nounroll
+    for (int pass = 0; pass < n_pass; ++pass)
+      attention_fwd_d128_v2<true>(q, k, v, o, smax, ssum, S, pass == 0 ? hi : lo, head, scale_log2e);
+  } else {
+    const int head = (slot / n_qb) * XCDS + xcd;
+    const int qb = slot % n_qb;
+    if (head >= n_heads) return;
+    attention_fwd_d128_v2<false>(q, k, v, o, smax, ssum, S, qb, head, scale_log2e);
+  }
+}
+
+extern "C" __global__ __launch_bounds__(256, 1) void fused_attention_fwd_bf16_d128_causal_v2(
+    const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
+    int n_heads, int S, float scale_log2e) {
+  attention_entry_v2<true>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
+}
+extern "C" __global__ __launch_bounds__(256, 1) void fused_attention_fwd_bf16_d128_full_v2(
+    const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
+    int n_heads, int S, float scale_log2e) {
+  attention_entry_v2<false>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
 }

@@ -439,6 +439,14 @@ def _attention_launcher() -> CachingLauncher:
             lds_bytes=_ATTN_LDS_BYTES,
         )
         for c in (1, 0)
+    ] + [
+        LaunchConfig(
+            f"fused_attention_fwd_bf16_d128_{'causal' if c else 'full'}_v2",
+            256,
+            meta={"CAUSAL": c, "WAVES": 4, "QUERIES_PER_WAVE": 64},
+            lds_bytes=_ATTN_LDS_BYTES,
+        )
+        for c in (1, 0)
     ]
     return CachingLauncher(
         "fused_attention_fwd_bf16_d128",
@@ -451,7 +459,7 @@ def _attention_launcher() -> CachingLauncher:
 
 def fused_attention(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool, waves: Optional[int] = None,
-    pingpong: Optional[bool] = None,
+    pingpong: Optional[bool] = None, variant: Optional[str] = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """softmax(q k^T * scale [+ causal mask]) v for [B, N, S, 128] bf16 tensors.
 
@@ -473,6 +481,25 @@ def fused_attention(
     ssum = torch.empty((B, N, S, 8), dtype=torch.float32, device=q.device)
     if B * N == 0:
         return out, smax, ssum
+    if variant is None and waves is None and pingpong is None:
+        variant = _ATTN_DEFAULT_VARIANT if S % 256 == 0 else None
+    if variant == "v2":
+        # 4 wavefronts of 64 queries: 256 queries per workgroup, causal query blocks paired
+        _require(S % 256 == 0, "the 64-queries-per-wavefront kernel needs S to be a multiple of 256")
+        l = _attention_launcher()
+        i = _find(l, f"fused_attention_fwd_bf16_d128_{'causal' if causal else 'full'}_v2")
+        heads = B * N
+        n_qb = S // 256
+        per_head = (n_qb + 1) // 2 if causal else n_qb
+        l._launch(
+            i,
+            (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), smax.data_ptr(), ssum.data_ptr(), heads, S,
+             float(scale) * 1.4426950408889634),
+            (8 * cdiv(heads, 8) * per_head, 1, 1),
+            _stream(),
+        )
+        return out, smax, ssum
+    _require(variant is None, "variant must be None or 'v2'")
     if waves is None:
         waves = _ATTN_DEFAULT_WAVES if S % 256 == 0 else 4
     _require(waves in (4, 8) and S % (32 * waves) == 0, "waves must be 4 or 8 and 32*waves must divide S")
@@ -499,3 +526,4 @@ def fused_attention(
 
 _ATTN_DEFAULT_WAVES = 8
 _ATTN_DEFAULT_PINGPONG = True
+_ATTN_DEFAULT_VARIANT = None  # "v2" selects the 64-queries-per-wavefront kernel when S % 256 == 0

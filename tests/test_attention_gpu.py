@@ -52,6 +52,58 @@ def test_attention_vs_oracle(K, O, B, N, S, causal, waves):
     np.testing.assert_allclose(ssum.cpu().numpy(), l_ref, rtol=2e-3)
 
 
+@pytest.mark.parametrize(
+    "B,N,S,causal,qmul",
+    [
+        (1, 2, 256, True, 1.0),
+        (1, 2, 256, False, 1.0),
+        (2, 3, 512, True, 1.0),
+        (1, 9, 512, False, 1.0),  # heads not a multiple of the 8 dies
+        (1, 2, 768, True, 1.0),  # odd number of query blocks: the middle one has no partner
+        (1, 2, 1024, True, 8.0),  # large scores: the reference maximum moves more than once
+        (1, 2, 512, False, 8.0),
+    ],
+)
+def test_attention_64_queries_per_wave_vs_oracle(K, O, B, N, S, causal, qmul):
+    """The kernel with 64 queries per wavefront (inline-assembly MFMAs, lazily updated
+    reference maximum) against the oracle, to the same bars as the default kernel."""
+    announce(f"attention v2 B={B} N={N} S={S} causal={causal} qmul={qmul}")
+    torch.manual_seed(3)
+    q, k, v = (torch.randn(B, N, S, 128).bfloat16() for _ in range(3))
+    q = (q.float() * qmul).bfloat16()
+    scale = 128 ** -0.5
+    out, smax, ssum = K.fused_attention(q.to(DEV), k.to(DEV), v.to(DEV), scale, causal, variant="v2")
+    o_ref, m_ref, l_ref = O.attention_bf16(bits(q), bits(k), bits(v), scale, causal)
+    err = np.abs(O.bf16_bits_to_f32(bits(out)) - O.bf16_bits_to_f32(o_ref)).max()
+    assert err <= 2e-2, err
+    np.testing.assert_allclose(smax.cpu().numpy(), m_ref, rtol=1e-3, atol=1e-3)
+    np.testing.assert_allclose(ssum.cpu().numpy(), l_ref, rtol=2e-3)
+
+
+def test_attention_64_queries_per_wave_full_length(K):
+    """S = 4096: statistics equal to the default kernel's to fp32 rounding, outputs within
+    bf16 rounding of it, causal output independent of later keys."""
+    announce("attention v2 S=4096")
+    torch.manual_seed(4)
+    B, N, S = 1, 3, 4096
+    q, k, v = (torch.randn(B, N, S, 128, device=DEV).bfloat16() for _ in range(3))
+    scale = 128 ** -0.5
+    for causal in (True, False):
+        o1, m1, l1 = K.fused_attention(q, k, v, scale, causal, waves=8, pingpong=True)
+        o2, m2, l2 = K.fused_attention(q, k, v, scale, causal, variant="v2")
+        assert (o1.float() - o2.float()).abs().max().item() <= 1.6e-2
+        assert torch.equal(m1, m2)
+        assert torch.allclose(l1, l2, rtol=1e-5)
+    k2, v2 = k.clone(), v.clone()
+    k2[:, :, 2048:] = torch.randn_like(k2[:, :, 2048:])
+    v2[:, :, 2048:] = torch.randn_like(v2[:, :, 2048:])
+    oa, _, _ = K.fused_attention(q, k, v, scale, True, variant="v2")
+    ob, _, _ = K.fused_attention(q, k2, v2, scale, True, variant="v2")
+    assert torch.equal(oa[:, :, :2048], ob[:, :, :2048])
+    with pytest.raises(ValueError):
+        K.fused_attention(q[:, :, :128], k[:, :, :128], v[:, :, :128], scale, True, variant="v2")
+
+
 def test_attention_closed_forms(K):
     """V = 1 gives O = 1 (probabilities sum to one); with a causal mask the first
     query row returns V[0]; identical keys give the running mean of V."""
