@@ -8,11 +8,11 @@
 // bandwidth).  A workgroup is 4 wavefronts (256 queries); with ~450 registers
 // per lane a SIMD holds a single wavefront, so the matrix core and the vector
 // ALU are kept busy from one instruction stream.  Iteration t is two phases:
-//     A   matrix:  O += V^T(t-1) P(t-1)      vector:  row max of S(t), 3/4 of P(t)
-//     B   matrix:  S(t+1) = K(t+1) Q^T       vector:  last 1/4 of P(t); K(t+2), V(t) -> LDS
+//     A   matrix:  O += V^T(t-1) P(t-1)      vector:  row max of S(t), first half of P(t)
+//     B   matrix:  S(t+1) = K(t+1) Q^T       vector:  second half of P(t); K(t+2), V(t) -> LDS
 // P lives in one set of registers: the words for key slice j of P(t) are produced only
-// after the MFMAs that read slice j of P(t-1) have been issued (slice 3 at the start of
-// phase B, before S's second key block is overwritten).
+// after the MFMAs that read slice j of P(t-1) have been issued, and the second half
+// before the MFMAs of phase B overwrite S's second key block.
 // Each phase is written as 16 chunks of {one LDS fragment read two chunks
 // ahead, two MFMAs, one slice of the vector work}; a scheduling fence between
 // chunks keeps the compiler from regrouping them, which both fixes the
@@ -91,11 +91,11 @@ __device__ __forceinline__ void attn_mfma_vacc_first(f32x16_t& acc, bf16x8_t a, 
   asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b));
 }
 // The hardware does not interlock a vector-ALU access to registers that an MFMA in flight
-// is still going to write (11 idle issue slots after an 8-pass MFMA, 19 after a 16-pass
-// one), and the compiler cannot see MFMAs inside inline assembly.  The fence takes S as
+// is still going to write (12 idle issue slots after an 8-pass MFMA such as this one; the
+// fence gives 16), and the compiler cannot see MFMAs inside inline assembly.  The fence takes S as
 // in/out operands so that data flow orders it after the last MFMA and before every read.
 __device__ __forceinline__ void attn_mfma_result_fence(f32x16_t& a, f32x16_t& b, f32x16_t& c, f32x16_t& d) {
-  asm volatile("s_nop 15\n\ts_nop 3" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+  asm volatile("s_nop 15" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
 }
 
 template <bool CAUSAL>
@@ -160,21 +160,25 @@ __device__ __forceinline__ void attention_fwd_d128_v2(const bf16_t* __restrict__
   const int v_kg = tid >> 4;
   const int v_dg = tid & 15;
   const int v_pos = attn_vt_pos(4 * v_kg);
-  auto load_k = [&](int tile) {
+  auto load_k_part = [&](int tile, int u) {
     const bf16_t* kp = Kh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
+    kst[u] = *reinterpret_cast<const u32x4_t*>(kp + static_cast<size_t>(k_row + 16 * u) * kAttnD + k_col);
+  };
+  auto load_k = [&](int tile) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
-      kst[u] = *reinterpret_cast<const u32x4_t*>(kp + static_cast<size_t>(k_row + 16 * u) * kAttnD + k_col);
+    for (int u = 0; u < 4; ++u) load_k_part(tile, u);
   };
   auto store_k_part = [&](int buf, int u) {
     bf16_t* Ks = Kbuf + buf * kAttnV2KElems;
     *reinterpret_cast<u32x4_t*>(Ks + (k_row + 16 * u) * kAttnKStride + k_col) = kst[u];
   };
-  auto load_v = [&](int tile) {
+  auto load_v_part = [&](int tile, int u) {
     const bf16_t* vp = Vh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
+    vst[u] = *reinterpret_cast<const u32x4_t*>(vp + static_cast<size_t>(4 * v_kg + u) * kAttnD + 8 * v_dg);
+  };
+  auto load_v = [&](int tile) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
-      vst[u] = *reinterpret_cast<const u32x4_t*>(vp + static_cast<size_t>(4 * v_kg + u) * kAttnD + 8 * v_dg);
+    for (int u = 0; u < 4; ++u) load_v_part(tile, u);
   };
   // dword e2 of each staged V row holds d = 2 e2 (low half, odd = 0) and 2 e2 + 1 (high half)
   auto store_v_half = [&](int buf, int e2, int odd) {
@@ -235,7 +239,10 @@ __device__ __forceinline__ void attention_fwd_d128_v2(const bf16_t* __restrict__
       mpart[sub] = a;
     } else {
       a = fmaxf(a, mpart[sub]);
-      mx[sub] = fmaxf(a, __shfl_xor(a, 32, kWave));
+      // lanes l and l + 32 hold the two halves of a query's keys: exchange through the
+      // vector ALU (no LDS round trip to wait for)
+      const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(a), false, false);
+      mx[sub] = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
     }
   };
   // reference maximum and rescale factor (slice 2 of phase A)
@@ -280,7 +287,7 @@ __device__ __forceinline__ void attention_fwd_d128_v2(const bf16_t* __restrict__
 
   // ---- phase A: O += V^T(tile-1) P(tile-1) alongside the first part of the softmax step on S(tile) ----
   // odd_c: parity of `tile` (LDS buffer indices become compile-time constants)
-  auto phase_a = [&](auto pv_c, auto odd_c) {
+  auto phase_a = [&](auto pv_c, auto odd_c, int k_tile, int v_tile) {
     constexpr bool DO_PV = decltype(pv_c)::value;
     constexpr int ODD = decltype(odd_c)::value ? 1 : 0;
     const bf16_t* Vt = Vbuf + (1 - ODD) * kAttnV2VElems;
@@ -300,12 +307,22 @@ __device__ __forceinline__ void attention_fwd_d128_v2(const bf16_t* __restrict__
           if constexpr (h == 0 && i + kAttnV2Prefetch < 16) f[i + kAttnV2Prefetch] = v_frag(Vt, i + kAttnV2Prefetch);
           oacc[h][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], attn_as_bf16x8(pf.w[h][t4]), oacc[h][db], 0, 0, 0);
         }
+        // the global loads of the tiles that phase B stores to LDS, one per half chunk so
+        // that the memory pipeline's queue never fills
+        if constexpr (i < 4) {
+          if constexpr (h == 0) load_k_part(k_tile, i);
+          else load_v_part(v_tile, i);
+        }
         if constexpr (i == 0) softmax_rowmax(std::integral_constant<int, 0>(), hc);
         if constexpr (i == 1) softmax_rowmax(std::integral_constant<int, 1>(), hc);
         if constexpr (i == 2 && h == 0) softmax_ref();
-        // slice j of P may be rewritten once chunk 4 j + 3 has issued its MFMAs
-        if constexpr (i >= 4)
-          softmax_word(std::integral_constant<int, (i >> 2) - 1>(), std::integral_constant<int, 2 * (i & 3) + h>());
+        // Key slice j of P may be rewritten once chunk 4 j + 3 has issued its MFMAs.  Slices 0
+        // and 1 (S's first key block) are done here, slices 2 and 3 in phase B, which leaves
+        // both phases with about as many vector instructions as fit beside their MFMAs.
+        if constexpr (i >= 4 && i < 8)
+          softmax_word(std::integral_constant<int, 0>(), std::integral_constant<int, (i >= 4 && i < 8 ? 2 * (i - 4) + h : 0)>());
+        if constexpr (i >= 8 && h == 0)
+          softmax_word(std::integral_constant<int, 1>(), std::integral_constant<int, (i >= 8 ? i - 8 : 0)>());
         __builtin_amdgcn_sched_barrier(0);
       });
     });
@@ -344,11 +361,12 @@ __device__ __forceinline__ void attention_fwd_d128_v2(const bf16_t* __restrict__
           if constexpr (ks == 0) attn_mfma_vacc_first(sacc[h][kb], f[i], qf[h][ks]);
           else attn_mfma_vacc(sacc[h][kb], f[i], qf[h][ks]);
         }
-        // key slice 3 of P reads S's second key block, which chunk 8 starts to overwrite
-        if constexpr (i < 4) softmax_word(std::integral_constant<int, 3>(), std::integral_constant<int, 2 * i + h>());
-        if constexpr (i == 3 && h == 1) softmax_finish();
-        if constexpr (i >= 4 && i < 8 && h == 0) store_k_part(wbuf, i - 4);
-        if constexpr (i >= 8 && i < 12) store_v_half(wbuf, i - 8, h);
+        // key slices 2 and 3 of P read S's second key block, which chunk 8 starts to overwrite
+        if constexpr (i < 8)
+          softmax_word(std::integral_constant<int, 2 + (i >> 2)>(), std::integral_constant<int, 2 * (i & 3) + h>());
+        if constexpr (i == 7 && h == 1) softmax_finish();
+        if constexpr (i >= 8 && i < 12 && h == 0) store_k_part(wbuf, i - 8);
+        if constexpr (i >= 12) store_v_half(wbuf, i - 12, h);
         __builtin_amdgcn_sched_barrier(0);
       });
     });
@@ -386,30 +404,24 @@ __device__ __forceinline__ void attention_fwd_d128_v2(const bf16_t* __restrict__
   using F = std::false_type;
 
   // ---- iteration 0: no previous tile to multiply ----
-  load_k(2);
-  load_v(0);
   if (CAUSAL && 0 >= first_masked) apply_mask(0);
-  phase_a(F(), F());
+  phase_a(F(), F(), 2, 0);
   phase_b(T(), F());
   __syncthreads();
 
   // ---- iterations 1 .. n_tiles-2, two per trip (odd tile, even tile) ----
   for (int t = 1; t < n_tiles - 1; t += 2) {
     {
-      load_k(min(t + 2, n_tiles - 1));  // past the end: a harmless reload of the last tile
-      load_v(t);
       if (CAUSAL && t >= first_masked) apply_mask(t);
-      phase_a(T(), T());
+      phase_a(T(), T(), min(t + 2, n_tiles - 1), t);  // K past the end: a harmless reload
       rescale();
       phase_b(T(), T());
       __syncthreads();
     }
     {
       const int u = t + 1;
-      load_k(min(u + 2, n_tiles - 1));
-      load_v(u);
       if (CAUSAL && u >= first_masked) apply_mask(u);
-      phase_a(T(), F());
+      phase_a(T(), F(), min(u + 2, n_tiles - 1), u);
       rescale();
       phase_b(T(), F());
       __syncthreads();
@@ -419,10 +431,8 @@ __device__ __forceinline__ void attention_fwd_d128_v2(const bf16_t* __restrict__
   // ---- last iteration (n_tiles - 1 is odd): no next S; then the final product ----
   {
     const int t = n_tiles - 1;
-    load_k(t);
-    load_v(t);
     if (CAUSAL) apply_mask(t);
-    phase_a(T(), T());
+    phase_a(T(), T(), t, t);
     rescale();
     phase_b(F(), T());
     __syncthreads();
