@@ -410,9 +410,13 @@ __device__ __forceinline__ void attention_fwd_d128_v2(const bf16_t* __restrict__
   __syncthreads();
 
   // ---- iterations 1 .. n_tiles-2, two per trip (odd tile, even tile) ----
-  for (int t = 1; t < n_tiles - 1; t += 2) {
+  // Two copies of the loop: tiles wholly below the diagonal need no mask, and keeping the
+  // masking out of that loop keeps it free of branches; the second copy masks every tile
+  // (a no-op for a tile that lies below the diagonal after all).
+  auto pair = [&](int t, auto mask_c) {
+    constexpr bool MASK = decltype(mask_c)::value;
     {
-      if (CAUSAL && t >= first_masked) apply_mask(t);
+      if constexpr (MASK) apply_mask(t);
       phase_a(T(), T(), min(t + 2, n_tiles - 1), t);  // K past the end: a harmless reload
       rescale();
       phase_b(T(), T());
@@ -420,17 +424,22 @@ __device__ __forceinline__ void attention_fwd_d128_v2(const bf16_t* __restrict__
     }
     {
       const int u = t + 1;
-      if (CAUSAL && u >= first_masked) apply_mask(u);
+      if constexpr (MASK) apply_mask(u);
       phase_a(T(), F(), min(u + 2, n_tiles - 1), u);
       rescale();
       phase_b(T(), F());
       __syncthreads();
     }
+  };
+  int t = 1;
+  for (; t + 1 < first_masked; t += 2) pair(t, F());
+  if constexpr (CAUSAL) {
+    for (; t < n_tiles - 1; t += 2) pair(t, T());
   }
 
   // ---- last iteration (n_tiles - 1 is odd): no next S; then the final product ----
   {
-    const int t = n_tiles - 1;
+    t = n_tiles - 1;
     if (CAUSAL) apply_mask(t);
     phase_a(T(), T(), t, t);
     rescale();

@@ -526,4 +526,4 @@ def fused_attention(
 
 _ATTN_DEFAULT_WAVES = 8
 _ATTN_DEFAULT_PINGPONG = True
-_ATTN_DEFAULT_VARIANT = None  # "v2" selects the 64-queries-per-wavefront kernel when S % 256 == 0
+_ATTN_DEFAULT_VARIANT = "v2"  # the 64-queries-per-wavefront kernel whenever S % 256 == 0

@@ -136,11 +136,16 @@ def test_attention_causality_and_sdpa_full_size_slice(K):
     B, N, S = 1, 2, 4096
     q, k, v = (torch.randn(B, N, S, 128, device=DEV).bfloat16() for _ in range(3))
     scale = 128 ** -0.5
-    out, smax, ssum = K.fused_attention(q, k, v, scale, True)
+    out, smax, ssum = K.fused_attention(q, k, v, scale, True, waves=4)
     out8, smax8, ssum8 = K.fused_attention(q, k, v, scale, True, waves=8, pingpong=False)
     assert torch.equal(out, out8) and torch.equal(smax, smax8) and torch.equal(ssum, ssum8)
     outp, smaxp, ssump = K.fused_attention(q, k, v, scale, True, waves=8, pingpong=True)
     assert torch.equal(out, outp) and torch.equal(smax, smaxp) and torch.equal(ssum, ssump)
+    # the default at this length is the 64-queries-per-wavefront kernel
+    outd, smaxd, ssumd = K.fused_attention(q, k, v, scale, True)
+    outv, smaxv, ssumv = K.fused_attention(q, k, v, scale, True, variant="v2")
+    assert torch.equal(outd, outv) and torch.equal(smaxd, smaxv) and torch.equal(ssumd, ssumv)
+    out, smax, ssum = outd, smaxd, ssumd
     for causal in (False,):
         a = K.fused_attention(q, k, v, scale, causal, waves=4)
         b = K.fused_attention(q, k, v, scale, causal, waves=8, pingpong=True)
