@@ -7,6 +7,7 @@
 // causal mask the heaviest query blocks (most key tiles) are issued first.
 #include "../mi/attention_pp.h"
 #include "../mi/attention_v2.h"
+#include "../mi/attention_v4.h"
 
 using namespace mi;
 
@@ -119,4 +120,44 @@ extern "C" __global__ __launch_bounds__(256, 1) void fused_attention_fwd_bf16_d1
     const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
     int n_heads, int S, float scale_log2e) {
   attention_entry_v2<false>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
+}
+
+// v4: 512 threads, 32 queries per wavefront, MFMA and softmax interleaved per wavefront
+// (attention_v4.h).
+template <bool CAUSAL>
+__device__ __forceinline__ void attention_entry_v4(const bf16_t* q, const bf16_t* k, const bf16_t* v,
+                                                   bf16_t* o, float* smax, float* ssum, int n_heads,
+                                                   int S, float scale_log2e) {
+  constexpr int XCDS = 8;
+  const int n_qb = S / kAttnV4BM;
+  const int id = blockIdx.x;
+  const int xcd = id % XCDS;
+  const int slot = id / XCDS;
+  if (CAUSAL) {
+    const int n_pair = (n_qb + 1) / 2;
+    const int head = (slot / n_pair) * XCDS + xcd;
+    const int lo = slot % n_pair;
+    const int hi = n_qb - 1 - lo;
+    if (head >= n_heads) return;
+    const int n_pass = lo != hi ? 2 : 1;
+#pragma nounroll
+    for (int pass = 0; pass < n_pass; ++pass)
+      attention_fwd_d128_v4<true>(q, k, v, o, smax, ssum, S, pass == 0 ? hi : lo, head, scale_log2e);
+  } else {
+    const int head = (slot / n_qb) * XCDS + xcd;
+    const int qb = slot % n_qb;
+    if (head >= n_heads) return;
+    attention_fwd_d128_v4<false>(q, k, v, o, smax, ssum, S, qb, head, scale_log2e);
+  }
+}
+
+extern "C" __global__ __launch_bounds__(512, 1) void fused_attention_fwd_bf16_d128_causal_v4(
+    const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
+    int n_heads, int S, float scale_log2e) {
+  attention_entry_v4<true>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
+}
+extern "C" __global__ __launch_bounds__(512, 1) void fused_attention_fwd_bf16_d128_full_v4(
+    const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
+    int n_heads, int S, float scale_log2e) {
+  attention_entry_v4<false>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
 }

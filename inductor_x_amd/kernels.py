@@ -447,6 +447,14 @@ def _attention_launcher() -> CachingLauncher:
             lds_bytes=_ATTN_LDS_BYTES,
         )
         for c in (1, 0)
+    ] + [
+        LaunchConfig(
+            f"fused_attention_fwd_bf16_d128_{'causal' if c else 'full'}_v4",
+            512,
+            meta={"CAUSAL": c, "WAVES": 8, "INTERLEAVED": 1},
+            lds_bytes=_ATTN_LDS_BYTES,
+        )
+        for c in (1, 0)
     ]
     return CachingLauncher(
         "fused_attention_fwd_bf16_d128",
@@ -483,11 +491,11 @@ def fused_attention(
         return out, smax, ssum
     if variant is None and waves is None and pingpong is None:
         variant = _ATTN_DEFAULT_VARIANT if S % 256 == 0 else None
-    if variant == "v2":
-        # 4 wavefronts of 64 queries: 256 queries per workgroup, causal query blocks paired
-        _require(S % 256 == 0, "the 64-queries-per-wavefront kernel needs S to be a multiple of 256")
+    if variant in ("v2", "v4"):
+        # 256 queries per workgroup (4 wavefronts of 64 or 8 of 32), causal query blocks paired
+        _require(S % 256 == 0, "the interleaved kernels need S to be a multiple of 256")
         l = _attention_launcher()
-        i = _find(l, f"fused_attention_fwd_bf16_d128_{'causal' if causal else 'full'}_v2")
+        i = _find(l, f"fused_attention_fwd_bf16_d128_{'causal' if causal else 'full'}_{variant}")
         heads = B * N
         n_qb = S // 256
         per_head = (n_qb + 1) // 2 if causal else n_qb
@@ -499,7 +507,7 @@ def fused_attention(
             _stream(),
         )
         return out, smax, ssum
-    _require(variant is None, "variant must be None or 'v2'")
+    _require(variant is None, "variant must be None, 'v2' or 'v4'")
     if waves is None:
         waves = _ATTN_DEFAULT_WAVES if S % 256 == 0 else 4
     _require(waves in (4, 8) and S % (32 * waves) == 0, "waves must be 4 or 8 and 32*waves must divide S")
@@ -526,4 +534,4 @@ def fused_attention(
 
 _ATTN_DEFAULT_WAVES = 8
 _ATTN_DEFAULT_PINGPONG = True
-_ATTN_DEFAULT_VARIANT = "v2"  # the 64-queries-per-wavefront kernel whenever S % 256 == 0
+_ATTN_DEFAULT_VARIANT = "v4"  # the interleaved 8-wavefront kernel whenever S % 256 == 0

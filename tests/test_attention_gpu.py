@@ -52,6 +52,7 @@ def test_attention_vs_oracle(K, O, B, N, S, causal, waves):
     np.testing.assert_allclose(ssum.cpu().numpy(), l_ref, rtol=2e-3)
 
 
+@pytest.mark.parametrize("variant", ["v4", "v2"])
 @pytest.mark.parametrize(
     "B,N,S,causal,qmul",
     [
@@ -64,15 +65,16 @@ def test_attention_vs_oracle(K, O, B, N, S, causal, waves):
         (1, 2, 512, False, 8.0),
     ],
 )
-def test_attention_64_queries_per_wave_vs_oracle(K, O, B, N, S, causal, qmul):
-    """The kernel with 64 queries per wavefront (inline-assembly MFMAs, lazily updated
-    reference maximum) against the oracle, to the same bars as the default kernel."""
-    announce(f"attention v2 B={B} N={N} S={S} causal={causal} qmul={qmul}")
+def test_attention_interleaved_kernels_vs_oracle(K, O, B, N, S, causal, qmul, variant):
+    """The kernels that interleave MFMAs and softmax within a wavefront (v4: 8 wavefronts of
+    32 queries, the default; v2: 4 wavefronts of 64 queries with inline-assembly MFMAs),
+    both with a lazily updated reference maximum, against the oracle."""
+    announce(f"attention {variant} B={B} N={N} S={S} causal={causal} qmul={qmul}")
     torch.manual_seed(3)
     q, k, v = (torch.randn(B, N, S, 128).bfloat16() for _ in range(3))
     q = (q.float() * qmul).bfloat16()
     scale = 128 ** -0.5
-    out, smax, ssum = K.fused_attention(q.to(DEV), k.to(DEV), v.to(DEV), scale, causal, variant="v2")
+    out, smax, ssum = K.fused_attention(q.to(DEV), k.to(DEV), v.to(DEV), scale, causal, variant=variant)
     o_ref, m_ref, l_ref = O.attention_bf16(bits(q), bits(k), bits(v), scale, causal)
     err = np.abs(O.bf16_bits_to_f32(bits(out)) - O.bf16_bits_to_f32(o_ref)).max()
     assert err <= 2e-2, err
@@ -80,28 +82,29 @@ def test_attention_64_queries_per_wave_vs_oracle(K, O, B, N, S, causal, qmul):
     np.testing.assert_allclose(ssum.cpu().numpy(), l_ref, rtol=2e-3)
 
 
-def test_attention_64_queries_per_wave_full_length(K):
-    """S = 4096: statistics equal to the default kernel's to fp32 rounding, outputs within
-    bf16 rounding of it, causal output independent of later keys."""
-    announce("attention v2 S=4096")
+@pytest.mark.parametrize("variant", ["v4", "v2"])
+def test_attention_interleaved_kernels_full_length(K, variant):
+    """S = 4096: statistics equal to the phase-separated kernel's to fp32 rounding, outputs
+    within bf16 rounding of it, causal output independent of later keys."""
+    announce(f"attention {variant} S=4096")
     torch.manual_seed(4)
     B, N, S = 1, 3, 4096
     q, k, v = (torch.randn(B, N, S, 128, device=DEV).bfloat16() for _ in range(3))
     scale = 128 ** -0.5
     for causal in (True, False):
         o1, m1, l1 = K.fused_attention(q, k, v, scale, causal, waves=8, pingpong=True)
-        o2, m2, l2 = K.fused_attention(q, k, v, scale, causal, variant="v2")
+        o2, m2, l2 = K.fused_attention(q, k, v, scale, causal, variant=variant)
         assert (o1.float() - o2.float()).abs().max().item() <= 1.6e-2
         assert torch.equal(m1, m2)
         assert torch.allclose(l1, l2, rtol=1e-5)
     k2, v2 = k.clone(), v.clone()
     k2[:, :, 2048:] = torch.randn_like(k2[:, :, 2048:])
     v2[:, :, 2048:] = torch.randn_like(v2[:, :, 2048:])
-    oa, _, _ = K.fused_attention(q, k, v, scale, True, variant="v2")
-    ob, _, _ = K.fused_attention(q, k2, v2, scale, True, variant="v2")
+    oa, _, _ = K.fused_attention(q, k, v, scale, True, variant=variant)
+    ob, _, _ = K.fused_attention(q, k2, v2, scale, True, variant=variant)
     assert torch.equal(oa[:, :, :2048], ob[:, :, :2048])
     with pytest.raises(ValueError):
-        K.fused_attention(q[:, :, :128], k[:, :, :128], v[:, :, :128], scale, True, variant="v2")
+        K.fused_attention(q[:, :, :128], k[:, :, :128], v[:, :, :128], scale, True, variant=variant)
 
 
 def test_attention_closed_forms(K):
@@ -141,9 +144,9 @@ def test_attention_causality_and_sdpa_full_size_slice(K):
     assert torch.equal(out, out8) and torch.equal(smax, smax8) and torch.equal(ssum, ssum8)
     outp, smaxp, ssump = K.fused_attention(q, k, v, scale, True, waves=8, pingpong=True)
     assert torch.equal(out, outp) and torch.equal(smax, smaxp) and torch.equal(ssum, ssump)
-    # the default at this length is the 64-queries-per-wavefront kernel
+    # the default at this length is the interleaved 8-wavefront kernel
     outd, smaxd, ssumd = K.fused_attention(q, k, v, scale, True)
-    outv, smaxv, ssumv = K.fused_attention(q, k, v, scale, True, variant="v2")
+    outv, smaxv, ssumv = K.fused_attention(q, k, v, scale, True, variant="v4")
     assert torch.equal(outd, outv) and torch.equal(smaxd, smaxv) and torch.equal(ssumd, ssumv)
     out, smax, ssum = outd, smaxd, ssumd
     for causal in (False,):
