@@ -1154,7 +1154,7 @@ class HipKernel(SIMDKernel):
         src.writeline("}")
         src.writeline("")
         # ---- pass 2
-        cpw, sl = 16, 16
+        cpw, sl = 16, 32
         src.writeline(f'extern "C" __global__ __launch_bounds__({cpw * sl}) void {kname}_final({plist}) {{')
         with src.indent():
             src.writeline("constexpr int VEC = 1;")

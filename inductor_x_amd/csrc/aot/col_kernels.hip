@@ -41,6 +41,8 @@ COL_PARTIAL_VARIANT(64, 8, 8)
   }
 
 COL_FINAL_VARIANT(16, 16)
+COL_FINAL_VARIANT(16, 32)
+COL_FINAL_VARIANT(8, 64)
 COL_FINAL_VARIANT(8, 32)
 COL_FINAL_VARIANT(4, 64)
 COL_FINAL_VARIANT(64, 4)

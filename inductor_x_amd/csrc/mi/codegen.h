@@ -712,7 +712,7 @@ __device__ __forceinline__ void col_store_partial(float* __restrict__ ws, const 
 template <class R, int CPW, int SL>
 __device__ __forceinline__ typename R::M col_final(const float* __restrict__ ws, i64 x, i64 xnumel, int nsplit,
                                                    int slot, int sl, bool live, float* lds) {
-  constexpr int BATCH = 4;
+  constexpr int BATCH = 8;  // with SL = 32 lanes per column: 256 partials in one round of loads
   const i64 plane = static_cast<i64>(nsplit) * xnumel;
   typename R::M m = R::empty();
   if (live) {

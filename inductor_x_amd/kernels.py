@@ -85,7 +85,7 @@ _COL_PARTIAL_VARIANTS = [
     (16, 32, 4),
     (64, 8, 8),
 ]
-_COL_FINAL_VARIANTS = [(16, 16), (8, 32), (4, 64), (64, 4)]
+_COL_FINAL_VARIANTS = [(16, 16), (16, 32), (8, 64), (8, 32), (4, 64), (64, 4)]
 _GATHER_VARIANTS = [(256, 128, 1), (256, 128, 2), (256, 128, 4), (256, 64, 1), (256, 64, 2), (256, 64, 4), (256, 16, 1), (256, 16, 4)]
 _PERMUTE_VARIANTS = [
     (256, 16, 32, 8),
