@@ -277,3 +277,16 @@ def test_ring_attention_forward_update():
     out, _ = compile_and_code(forward_update, *bf)
     ref = forward_update(*bf)
     assert out[0].dtype == torch.bfloat16 and (out[0].float() - ref[0].float()).abs().max().item() <= 2e-2
+    # second half of a [2S, ...] run: non-contiguous views of every operand (the strided "1S" case the
+    # reference keeps beside the contiguous one, attn_cp_test.py:113-123)
+    big = (torch.randn(2 * S, B, H, device=DEV), torch.rand(B, N, 2 * S, device=DEV).unsqueeze(3).repeat(1, 1, 1, F32_BLK),
+           torch.rand(B, N, 2 * S, device=DEV).unsqueeze(3).repeat(1, 1, 1, F32_BLK) + 0.5)
+    prev_out_s = big[0].view(2, S, B, H)[1]
+    prev_max_s = big[1].view(B, N, 2, S, F32_BLK)[:, :, 1]
+    prev_sum_s = big[2].view(B, N, 2, S, F32_BLK)[:, :, 1]
+    assert not prev_max_s.is_contiguous()
+    sargs = (prev_out_s, prev_max_s, prev_sum_s, args[3], args[4], args[5])
+    out, _ = compile_and_code(forward_update, *sargs)
+    ref = forward_update(*sargs)
+    for a, b in zip(out, ref):
+        torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-6)
