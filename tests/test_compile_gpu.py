@@ -290,3 +290,128 @@ def test_ring_attention_forward_update():
     ref = forward_update(*sargs)
     for a, b in zip(out, ref):
         torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-6)
+
+
+def test_ring_attention_lse_merge_and_copy_back():
+    """Log-sum-exp form of the ring-attention merge, functional and with the results copied
+    back into the running buffers, on whole tensors and on the second-half views
+    (reference test/npu_indexing/written/test_attn_cp.py:361-375, shapes from :403-421 scaled down)."""
+    announce("compile ring-attention LSE merge")
+
+    def forward_update_la(prev_out, prev_lse, cur_out, cur_lse):
+        lse = torch.log(torch.exp(cur_lse) + torch.exp(prev_lse))
+        out = torch.exp(prev_lse - lse) * prev_out + torch.exp(cur_lse - lse) * cur_out
+        return out, lse
+
+    def forward_update_copy(prev_out, prev_lse, cur_out, cur_lse):
+        out, lse = forward_update_la(prev_out, prev_lse, cur_out, cur_lse)
+        prev_out.copy_(out)
+        prev_lse.copy_(lse)
+
+    torch.manual_seed(0)
+    S, B, N, D = 512, 1, 12, 128
+    DS = 2 * S
+    out = torch.randn(B, N, DS, D, device=DEV)
+    lse = torch.rand(B, N, DS, 1, device=DEV)
+    cur = torch.randn(B, N, DS, D, device=DEV)
+    cur_lse = torch.rand(B, N, DS, 1, device=DEV)
+    got, _ = compile_and_code(forward_update_la, out, lse, cur, cur_lse)
+    ref = forward_update_la(out, lse, cur, cur_lse)
+    for a, b in zip(got, ref):
+        torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-6)
+    # in place, on the second half of the sequence (strided views of the running buffers)
+    out_s = out.view(B, N, 2, S, D)
+    lse_s = lse.view(B, N, 2, S, 1)
+    cur_s = torch.randn(B, N, S, D, device=DEV)
+    cur_lse_s = torch.rand(B, N, S, 1, device=DEV)
+    out_ref, lse_ref = out.clone(), lse.clone()
+    forward_update_copy(out_ref.view(B, N, 2, S, D)[:, :, 1], lse_ref.view(B, N, 2, S, 1)[:, :, 1], cur_s, cur_lse_s)
+    torch._dynamo.reset()
+    torch.compile(forward_update_copy)(out_s[:, :, 1], lse_s[:, :, 1], cur_s, cur_lse_s)
+    torch.testing.assert_close(out, out_ref, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(lse, lse_ref, rtol=1e-5, atol=1e-6)
+    assert torch.equal(out.view(B, N, 2, S, D)[:, :, 0], out_ref.view(B, N, 2, S, D)[:, :, 0])  # first half untouched
+
+
+@pytest.mark.parametrize("case", [7, 6, 5])
+def test_ring_attention_backward_update(case):
+    """Gradient accumulation step of ring attention: in-place adds into whole buffers or into
+    one half of them (reference test/npu_indexing/written/test_attn_cp.py:267-287, the three
+    cases of :329-336), bf16, shapes scaled down."""
+    announce(f"compile ring-attention backward_update case {case}")
+
+    def backward_update(dq, dk, dv, cur_dq, cur_dk, cur_dv, i, rank=1):
+        cp_size = 8
+        if i >= cp_size - rank - 1:
+            if i == cp_size - 1:
+                dq.add_(cur_dq.view(dq.shape))
+                dk.add_(cur_dk.view(dk.shape))
+                dv.add_(cur_dv.view(dv.shape))
+            else:
+                dq.add_(cur_dq.view(dq.shape))
+                dk[0].add_(cur_dk)
+                dv[0].add_(cur_dv)
+        else:
+            dq[1].add_(cur_dq)
+            dk.add_(cur_dk.view(dk.shape))
+            dv.add_(cur_dv.view(dv.shape))
+
+    torch.manual_seed(case)
+    S, B, H = 1024, 1, 1536
+    mk2 = lambda: torch.randn(2, S, B, H, device=DEV).bfloat16()  # noqa: E731
+    full = lambda: torch.randn(2 * S, B, H, device=DEV).bfloat16()  # noqa: E731
+    half = lambda: torch.randn(S, B, H, device=DEV).bfloat16()  # noqa: E731
+    dq, dk, dv = mk2(), mk2(), mk2()
+    if case == 7:
+        cur = (full(), full(), full())
+    elif case == 6:
+        cur = (full(), half(), half())
+    else:
+        cur = (half(), full(), full())
+    ref = [t.clone() for t in (dq, dk, dv)]
+    backward_update(*ref, *cur, case)
+    torch._dynamo.reset()
+    torch.compile(backward_update)(dq, dk, dv, *cur, case)
+    for a, b in zip((dq, dk, dv), ref):
+        assert torch.equal(a, b)  # one bf16 addition per element: bit-exact
+
+
+def test_mamba_split_of_permuted_input():
+    """Three-way split of a permuted tensor feeding a softplus-like tail (reference
+    test/npu_indexing/mamba_test.py:7-17; the split sizes of :10 and the shapes of :20-22 scaled down)."""
+    announce("compile mamba split")
+
+    def foo(a, b):
+        permute = a.permute(1, 0, 2).contiguous()
+        _, _, bt = torch.split(permute, [2048, 4096, 32], 2)
+        add = bt.contiguous().contiguous() + b
+        y = torch.exp(add)
+        where = torch.where(add < 20, add, torch.log1p(y))
+        return add, where, bt
+
+    torch.manual_seed(0)
+    a = torch.randn(256, 3, 6176, device=DEV)
+    b = torch.randn(32, device=DEV)
+    got, _ = compile_and_code(foo, a, b)
+    ref = foo(a, b)
+    for x, y in zip(got, ref):
+        torch.testing.assert_close(x, y, rtol=1e-5, atol=1e-6)
+
+
+def test_dynamic_shapes_reuse_one_kernel():
+    """dynamic=True: one compiled artefact serves several row counts (numel arguments are
+    passed at launch, reference inductor_x/codegen/wrapper.py:21-38)."""
+    announce("compile dynamic shapes")
+
+    def f(x, w):
+        return (torch.relu(x) * w).sum(-1), x * 2 + 1
+
+    torch._dynamo.reset()
+    cf = torch.compile(f, dynamic=True)
+    w = torch.randn(1024, device=DEV)
+    for rows in (64, 257, 1000, 3):
+        x = torch.randn(rows, 1024, device=DEV)
+        got = cf(x, w)
+        ref = f(x, w)
+        torch.testing.assert_close(got[0], ref[0], rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(got[1], ref[1])
