@@ -716,13 +716,76 @@ class HipKernel(SIMDKernel):
         if not lane_syms:
             return "uniform"
         lane = sympy.Symbol("lane_", integer=True, nonnegative=True)
-        shifted = sympy_subs(index, {s: s + lane for s in lane_syms})
-        diff = sympy.expand(shifted - index)
-        if diff == lane:
+        delta = self._lane_delta(index, lane)
+        if delta is None:
+            shifted = sympy_subs(index, {s: s + lane for s in lane_syms})
+            delta = sympy.expand(shifted - index)
+        if delta == lane:
             return "contiguous"
-        if diff == 0:
+        if delta == 0:
             return "uniform"
         return "gather"
+
+    def _lane_delta(self, expr: sympy.Expr, lane: sympy.Symbol) -> Optional[sympy.Expr]:
+        """index(lane i) - index(lane 0) as an expression in `lane`, using what symbolic
+        expansion cannot see: a lane-varying range variable is a multiple of the vector
+        width at lane 0 and 0 <= lane < width, so floor((v + lane) / d) does not depend on the
+        lane when the width divides d, and (v + lane) mod m moves with the lane when it
+        divides m.  None when the structure is not recognised."""
+        vec = self.vec
+        zero = sympy.Integer(0)
+
+        def aligned(e: sympy.Expr) -> bool:
+            base = sympy.expand(sympy_subs(e, {s: zero for s in e.free_symbols if self._is_lane_symbol(s)}))
+            if base == 0:
+                return True
+            try:
+                return bool(V.graph.sizevars.statically_known_multiple_of(base, vec))
+            except Exception:
+                return False
+
+        def rec(e: sympy.Expr) -> Optional[sympy.Expr]:
+            if e.is_Symbol:
+                return lane if self._is_lane_symbol(e) else zero
+            if e.is_number:
+                return zero
+            if isinstance(e, sympy.Add):
+                parts = [rec(a) for a in e.args]
+                return None if any(p is None for p in parts) else sympy.Add(*parts)
+            if isinstance(e, sympy.Mul):
+                consts = [a for a in e.args if a.is_number]
+                rest = [a for a in e.args if not a.is_number]
+                if len(rest) == 1:
+                    d = rec(rest[0])
+                    return None if d is None else sympy.Mul(*consts) * d
+                ds = [rec(a) for a in rest]
+                return zero if all(d == 0 for d in ds) else None
+            if isinstance(e, FloorDiv):
+                a, d = e.args
+                da = rec(a)
+                if da == 0 and rec(d) == 0:
+                    return zero
+                if da == lane and d.is_Integer and int(d) % vec == 0 and aligned(a):
+                    return zero
+                return None
+            if isinstance(e, ModularIndexing):
+                a, d, m = e.args
+                da = rec(a)
+                if da == 0 and rec(d) == 0 and rec(m) == 0:
+                    return zero
+                if da == lane and d.is_Integer and aligned(a):
+                    if int(d) % vec == 0:
+                        return zero
+                    if int(d) == 1 and m.is_Integer and int(m) % vec == 0:
+                        return lane
+                return None
+            return None
+
+        try:
+            out = rec(expr)
+        except Exception:
+            return None
+        return None if out is None else sympy.expand(out)
 
     def index_is_aligned(self, index: sympy.Expr) -> bool:
         """True when the address of lane 0 is provably a multiple of the vector

@@ -305,7 +305,7 @@ def col_mean_var_argmax(
     x: torch.Tensor,
     correction: float = 0.0,
     plan: Optional[SplitPlan] = None,
-    final_variant: tuple = (16, 16),
+    final_variant: tuple = (16, 32),
     workspace: Optional[torch.Tensor] = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Returns (mean, var, argmax) over dim 0 of a [rows, cols] fp32 matrix."""
