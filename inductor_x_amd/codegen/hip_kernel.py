@@ -446,6 +446,8 @@ class HipKernel(SIMDKernel):
         self.vec_tree_prefix = "x"
         self.lane_syms: OrderedSet[sympy.Symbol] = OrderedSet()
         self.x_entries: list[IterationRangesEntry] = []
+        # indices of the non-indirect loads that are contiguous along the vector axis (tile planning)
+        self._contiguous_load_indices: list[sympy.Expr] = []
         self.r_entries: list[IterationRangesEntry] = []
         self.r_full = False
         self.prologue = IndentedBuffer()
@@ -523,6 +525,71 @@ class HipKernel(SIMDKernel):
         # measured on MI355X (permute, gather, a*x+b at 128-512 MiB): 1 vector per
         # thread is fastest; 2 is within 1 %, 4 and 8 lose 5-10 %
         return 1
+
+    def pointwise_tile_plan(self) -> Optional[dict]:
+        """Two-dimensional workgroup tiles for a pointwise kernel that reads a tensor with
+        its two outer axes swapped relative to the output (a permuted copy).
+
+        With the linear order, a workgroup writes one long run and reads 256-byte pieces a
+        large stride apart.  When the output index decomposes as x0 + L0*(x1 + L1*(x2 + ...))
+        and some load moves faster along x2 than along x1, a workgroup instead takes T1 values
+        of x1 times T2 of x2: its reads come in runs of T2 rows and its writes in runs of T1
+        rows.  None when the kernel does not have this shape or the sizes do not divide."""
+        if self.mode != "pointwise" or self.vec <= 1 or os.environ.get("INDUCTOR_X_AMD_PW_TILE", "1") == "0":
+            return None
+        ents = sorted(
+            (e for e in self.x_entries if e.root.prefix == self.vec_tree_prefix), key=lambda e: int(e.divisor)
+            if isinstance(e.divisor, (int, sympy.Integer)) else -1
+        )
+        try:
+            ents = [e for e in ents if int(e.divisor) >= 1 and int(e.length) >= 1]
+        except (TypeError, ValueError):
+            return None
+        xnumel = self._static_numel(self.vec_tree_prefix)
+        if xnumel is None:
+            return None
+        # the variable that spans the whole range (the linear index itself) is not an axis
+        ents = [e for e in ents if not (int(e.divisor) == 1 and int(e.length) == xnumel)]
+        chain = []
+        want = 1
+        for e in ents:
+            if int(e.divisor) == want:
+                chain.append(e)
+                want *= int(e.length)
+        if len(chain) < 3 or len(chain) != len(ents):
+            return None
+        e0, e1, e2 = chain[0], chain[1], chain[2]
+        L0, L1, L2 = int(e0.length), int(e1.length), int(e2.length)
+        if L0 % self.vec != 0:
+            return None
+        cpt = L0 // self.vec  # threads per innermost row
+        if cpt > self.block or self.block % cpt != 0:
+            return None
+        s1, s2 = e1.symbol(), e2.symbol()
+        swapped = False
+        for index in self._contiguous_load_indices:
+            idx = sympy.expand(index)
+            try:
+                c1, c2 = idx.coeff(s1), idx.coeff(s2)
+                rest = sympy.expand(idx - c1 * s1 - c2 * s2)
+            except Exception:
+                return None
+            if rest.has(s1) or rest.has(s2) or not (c1.is_Integer and c2.is_Integer):
+                return None  # not affine in the two axes
+            if 0 < int(c2) < int(c1):
+                swapped = True
+        if not swapped:
+            return None
+        rows_per_iter = self.block // cpt
+        unroll = int(os.environ.get("INDUCTOR_X_AMD_PW_TILE_UNROLL", "2"))
+        t2_cap = int(os.environ.get("INDUCTOR_X_AMD_PW_TILE_T2", "4"))
+        t2 = 1
+        while t2 * 2 <= min(L2, t2_cap, rows_per_iter) and L2 % (t2 * 2) == 0:
+            t2 *= 2
+        t1 = rows_per_iter * unroll // t2
+        if t2 < 2 or L1 % t1 != 0 or xnumel % (L0 * L1 * L2) != 0:
+            return None
+        return {"L0": L0, "L1": L1, "L2": L2, "T1": t1, "T2": t2, "unroll": unroll, "cpt": cpt}
 
     def _tree(self, prefix: str):
         for t in self.range_trees:
@@ -843,6 +910,8 @@ class HipKernel(SIMDKernel):
         mask = self._load_mask_for(index)
         other = value_to_hip(self._load_other if self._load_mask else 0, dtype if dtype.is_floating_point else None)
         if kind == "contiguous":
+            if not indirect:
+                self._contiguous_load_indices.append(index)
             aligned = self.index_is_aligned(index) and self._buffer_aligned(name)
             ptr = f"{var} + ({self.index_to_str(index)})"
             if mask is None:
@@ -1119,20 +1188,40 @@ class HipKernel(SIMDKernel):
         if self.mode == "pointwise":
             plist = ", ".join(params + [f"const {idx_t} xnumel"])
             src.writeline(f'extern "C" __global__ __launch_bounds__({self.block}) void {kname}({plist}) {{')
-            unroll = self.pointwise_unroll()
+            tile = self.pointwise_tile_plan()
+            unroll = tile["unroll"] if tile else self.pointwise_unroll()
             with src.indent():
                 src.writeline(f"constexpr int VEC = {self.vec};")
                 src.writeline(f"constexpr int UNROLL = {unroll};")
-                src.writeline(
-                    f"const {idx_t} xbase = (static_cast<{idx_t}>(blockIdx.x) * UNROLL * {self.block} + threadIdx.x) * VEC;"
-                )
+                if tile:
+                    # workgroup -> (T1 x T2) tile of the two axes above the innermost one; within the
+                    # tile consecutive threads walk the innermost axis, then axis 2, then axis 1
+                    t1, t2, cpt = tile["T1"], tile["T2"], tile["cpt"]
+                    src.writeline(f"constexpr int L0 = {tile['L0']}, L1 = {tile['L1']}, L2 = {tile['L2']};")
+                    src.writeline(f"constexpr int T1 = {t1}, T2 = {t2}, CPT = {cpt};")
+                    src.writeline(f"const {idx_t} tile_ = static_cast<{idx_t}>(blockIdx.x);")
+                    src.writeline(f"const {idx_t} tile1 = tile_ % (L1 / T1);")
+                    src.writeline(f"const {idx_t} tile2 = (tile_ / (L1 / T1)) % (L2 / T2);")
+                    src.writeline(f"const {idx_t} outer_ = tile_ / ((L1 / T1) * (L2 / T2));")
+                else:
+                    src.writeline(
+                        f"const {idx_t} xbase = (static_cast<{idx_t}>(blockIdx.x) * UNROLL * {self.block} + threadIdx.x) * VEC;"
+                    )
                 # each thread handles UNROLL vectors one workgroup-width apart, so a
                 # wavefront still touches 1 KiB runs and has UNROLL loads in flight
                 src.writeline("#pragma unroll")
                 src.writeline("for (int u = 0; u < UNROLL; ++u) {")
                 with src.indent():
-                    src.writeline(f"const {idx_t} xindex = xbase + static_cast<{idx_t}>(u) * ({self.block} * VEC);")
-                    src.writeline("if (xindex >= xnumel) break;")
+                    if tile:
+                        src.writeline(f"const int e_ = u * {self.block} + static_cast<int>(threadIdx.x);")
+                        src.writeline("const int row_ = e_ / CPT;")
+                        src.writeline(
+                            f"const {idx_t} xindex = (e_ % CPT) * VEC + L0 * ((tile1 * T1 + row_ / T2) + "
+                            f"L1 * ((tile2 * T2 + row_ % T2) + static_cast<{idx_t}>(L2) * outer_));"
+                        )
+                    else:
+                        src.writeline(f"const {idx_t} xindex = xbase + static_cast<{idx_t}>(u) * ({self.block} * VEC);")
+                        src.writeline("if (xindex >= xnumel) break;")
                     src.splice(self._entry_code(self.x_entries))
                     src.splice(self.body)
                 src.writeline("}")

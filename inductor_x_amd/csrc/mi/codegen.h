@@ -306,12 +306,20 @@ __device__ __forceinline__ void vstore(T* __restrict__ p, const A& val) {
     *p = static_cast<T>(at(val, 0));
   } else {
     constexpr int PER = (16 / sizeof(T)) < N ? (16 / sizeof(T)) : N;
-#pragma unroll
-    for (int c = 0; c < N / PER; ++c) {
+    if constexpr (N == PER) {
+      // written without the chunk loop: inside it the compiler drops the non-temporal hint
       Vec<T, PER> t;
 #pragma unroll
-      for (int i = 0; i < PER; ++i) t[i] = static_cast<T>(at(val, c * PER + i));
-      store_vec<T, PER, STREAM>(p + c * PER, t);
+      for (int i = 0; i < PER; ++i) t[i] = static_cast<T>(at(val, i));
+      store_vec<T, PER, STREAM>(p, t);
+    } else {
+#pragma unroll
+      for (int c = 0; c < N / PER; ++c) {
+        Vec<T, PER> t;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) t[i] = static_cast<T>(at(val, c * PER + i));
+        store_vec<T, PER, STREAM>(p + c * PER, t);
+      }
     }
   }
 }
