@@ -1,0 +1,67 @@
+"""Backward of the fused attention forward (npu_graph::npu_fa_backward).
+
+Interim implementation: the five matrix products run as library GEMMs (torch.bmm, hipBLASLt
+underneath) on a bounded number of heads at a time, with the scores recomputed from the forward's
+saved row statistics; it is not yet a fused MFMA kernel and moves O(S^2) intermediates through HBM.
+Definitions (per head, scores scaled by `scale`, causal mask optional), with m = softmax_max and
+l = softmax_sum as saved by the forward:
+
+    S  = Q K^T * scale                      P  = exp(S - m) / l          (masked entries: 0)
+    dV = P^T dO                             dP = dO V^T
+    D  = rowsum(dO * O)                     dS = P * (dP - D) * scale
+    dQ = dS K                               dK = dS^T Q
+
+The probabilities and dS are rounded to bf16 before they enter a GEMM, as a fused kernel would do;
+all reductions and the softmax algebra are fp32.  Counterpart of the reference's call into
+torch_npu.npu_fusion_attention_grad (reference inductor_x/npu_fusion_attention_graph.py:38-42).
+"""
+from __future__ import annotations
+
+import torch
+
+# heads processed per round: bounds the fp32 [heads, S, S] intermediates (two live at a time)
+_SCORE_BYTES_BUDGET = 2 << 30
+
+
+def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale: float, causal: bool):
+    """q, k, v, out, dout: [B, N, S, D] bf16 (contiguous); softmax_max / softmax_sum: [B, N, S, 8] fp32
+    from the forward.  Returns (dq, dk, dv) in bf16."""
+    for t in (q, k, v, out, dout):
+        if not (t.is_cuda and t.dtype == torch.bfloat16 and t.dim() == 4):
+            raise ValueError("attention backward: q, k, v, out, dout must be 4-D bf16 GPU tensors")
+    if not (q.shape == k.shape == v.shape == out.shape == dout.shape):
+        raise ValueError("attention backward: q, k, v, out, dout must share one [B, N, S, D] shape")
+    B, N, S, D = q.shape
+    if softmax_max.shape != (B, N, S, 8) or softmax_sum.shape != (B, N, S, 8):
+        raise ValueError("attention backward: softmax statistics must be [B, N, S, 8]")
+    heads = B * N
+    qh, kh, vh, oh, doh = (t.contiguous().view(heads, S, D) for t in (q, k, v, out, dout))
+    m = softmax_max.reshape(heads, S, 8)[..., 0].contiguous()
+    l = softmax_sum.reshape(heads, S, 8)[..., 0].contiguous()
+    dq = torch.empty_like(qh)
+    dk = torch.empty_like(kh)
+    dv = torch.empty_like(vh)
+    if heads == 0 or S == 0:
+        return dq.view(B, N, S, D), dk.view(B, N, S, D), dv.view(B, N, S, D)
+    per_head = 2 * S * S * 4
+    chunk = max(1, min(heads, _SCORE_BYTES_BUDGET // max(per_head, 1)))
+    mask = None
+    if causal:
+        mask = torch.ones(S, S, dtype=torch.bool, device=q.device).triu_(1)
+    for h0 in range(0, heads, chunk):
+        sl = slice(h0, min(h0 + chunk, heads))
+        qc, kc, vc, oc, doc = qh[sl], kh[sl], vh[sl], oh[sl], doh[sl]
+        s = torch.bmm(qc, kc.transpose(1, 2), out_dtype=torch.float32)
+        # P = exp(S * scale - m) / l, masked entries exactly zero
+        s.mul_(scale).sub_(m[sl].unsqueeze(-1))
+        if mask is not None:
+            s.masked_fill_(mask, float("-inf"))
+        p = s.exp_().div_(l[sl].unsqueeze(-1))
+        p16 = p.to(torch.bfloat16)
+        dv[sl] = torch.bmm(p16.transpose(1, 2), doc)
+        dp = torch.bmm(doc, vc.transpose(1, 2), out_dtype=torch.float32)
+        delta = (doc.float() * oc.float()).sum(-1, keepdim=True)
+        ds16 = p.mul_(dp.sub_(delta)).mul_(scale).to(torch.bfloat16)
+        dq[sl] = torch.bmm(ds16, kc)
+        dk[sl] = torch.bmm(ds16.transpose(1, 2), qc)
+    return dq.view(B, N, S, D), dk.view(B, N, S, D), dv.view(B, N, S, D)

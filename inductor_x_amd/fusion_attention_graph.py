@@ -14,6 +14,9 @@ reference the op receives the *inverse* scale from the pattern and inverts it
 through the op's own arguments: sparse_mode 2 or 3, or next_tockens == 0 with
 pre_tockens covering the sequence.  Supported: layout "BNSD", bf16, head
 dimension 128, no pse / padding mask / dropout; anything else raises.
+The backward op recomputes the probabilities from the saved row statistics and runs its matrix
+products as library GEMMs (attention_backward.py); the training variant of the pattern is
+registered beside the inference one.
 """
 from __future__ import annotations
 
@@ -89,8 +92,30 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
 gpu_lib.impl("npu_fa", npu_fa_gpu)
 
 
-def npu_fa_backward_gpu(*args, **kwargs):
-    raise NotImplementedError("npu_fa_backward: the attention backward kernel is not part of this build")
+def npu_fa_backward_gpu(query, key, value, dy, head_num, input_layout, *, pse=None, padding_mask=None,
+                        atten_mask=None, softmax_max=None, softmax_sum=None, softmax_in=None, attention_in=None,
+                        scale_value=1.0, keep_prob=1.0, pre_tockens=TOKEN_MAX, next_tockens=TOKEN_MAX,
+                        inner_precise=0, seed=None, offset=None, numels=None, prefix=None, actual_seq_qlen=None,
+                        actual_seq_kvlen=None, sparse_mode=0, gen_mask_parallel=True, sync=False):
+    """Gradients of npu_fa (reference inductor_x/npu_fusion_attention_graph.py:38-42: like the forward,
+    the op receives the inverse scale and inverts it)."""
+    from .attention_backward import fused_attention_backward
+
+    if input_layout != "BNSD":
+        raise NotImplementedError(f"npu_fa_backward: layout {input_layout!r} (only 'BNSD')")
+    if pse is not None or padding_mask is not None or prefix or actual_seq_qlen or actual_seq_kvlen:
+        raise NotImplementedError("npu_fa_backward: pse / padding_mask / prefix / variable sequence lengths")
+    if keep_prob != 1.0:
+        raise NotImplementedError("npu_fa_backward: dropout (keep_prob != 1)")
+    if softmax_max is None or softmax_sum is None or attention_in is None:
+        raise ValueError("npu_fa_backward: needs softmax_max, softmax_sum and attention_in from the forward")
+    if scale_value == 0:
+        raise ZeroDivisionError("npu_fa_backward: the inverse scale factor is zero")
+    causal = _is_causal(query.size(2), atten_mask, pre_tockens, next_tockens, sparse_mode)
+    dq, dk, dv = fused_attention_backward(
+        query, key, value, attention_in, dy.contiguous(), softmax_max, softmax_sum, 1.0 / scale_value, causal
+    )
+    return dq, dk, dv, torch.empty([0], dtype=query.dtype, device=query.device)
 
 
 gpu_lib.impl("npu_fa_backward", npu_fa_backward_gpu)
@@ -170,7 +195,7 @@ class GraphAttentionFunction(Function):
             prefix=a["prefix"], actual_seq_qlen=a["actual_seq_qlen"], actual_seq_kvlen=a["actual_seq_kvlen"],
             sparse_mode=a["sparse_mode"], gen_mask_parallel=a["gen_mask_parallel"], sync=a["sync"],
         )
-        return (dq, dk, dv, None, None, dpse) + (None,) * 13
+        return (dq, dk, dv, None, None, dpse if pse is not None else None) + (None,) * 13
 
 
 def npu_fusion_attention_graph(query, key, value, head_num, input_layout, pse=None, padding_mask=None,

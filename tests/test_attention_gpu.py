@@ -176,3 +176,48 @@ def test_attention_rejects_bad_operands(K):
     q = torch.randn(1, 1, 128, 128, device=DEV)
     with pytest.raises(ValueError):
         K.fused_attention(q, q, q, 0.1, True)  # dtype
+
+
+@pytest.mark.parametrize("B,N,S,causal", [(1, 2, 256, True), (2, 3, 512, False), (1, 4, 1024, True), (1, 1, 128, True)])
+def test_attention_backward_vs_autograd(B, N, S, causal):
+    """npu_fa_backward through the autograd wrapper against autograd of the fp32 definition.
+    Tolerance: 1 % of the largest gradient entry (P and dS enter the GEMMs rounded to bf16)."""
+    announce(f"attention backward B={B} N={N} S={S} causal={causal}")
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
+    torch.manual_seed(5)
+    q, k, v = (torch.randn(B, N, S, 128, device=DEV).bfloat16().requires_grad_() for _ in range(3))
+    do = torch.randn(B, N, S, 128, device=DEV).bfloat16()
+    inv = 128 ** 0.5
+    out = npu_fusion_attention_graph(q, k, v, N, "BNSD", scale=inv, sparse_mode=3 if causal else 0)[0]
+    out.backward(do)
+    qf, kf, vf = (t.detach().float().requires_grad_() for t in (q, k, v))
+    s = (qf @ kf.transpose(-1, -2)) / inv
+    if causal:
+        s = s.masked_fill(torch.ones(S, S, device=DEV, dtype=torch.bool).triu(1), float("-inf"))
+    (torch.softmax(s, -1) @ vf).backward(do.float())
+    for got, ref in ((q.grad, qf.grad), (k.grad, kf.grad), (v.grad, vf.grad)):
+        assert got.dtype == torch.bfloat16 and got.shape == ref.shape
+        assert (got.float() - ref).abs().max().item() <= 1e-2 * ref.abs().max().item() + 1e-3
+
+
+def test_attention_backward_closed_forms():
+    """V gets gradient P^T dO: with dO = 1 every row of dV is the column sum of the probabilities,
+    and those sum to the number of queries over all keys; dQ and dK vanish when V is constant
+    along the sequence (the output does not depend on the probabilities)."""
+    announce("attention backward closed forms")
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
+    torch.manual_seed(6)
+    B, N, S = 1, 2, 256
+    q, k, v = (torch.randn(B, N, S, 128, device=DEV).bfloat16().requires_grad_() for _ in range(3))
+    out = npu_fusion_attention_graph(q, k, v, N, "BNSD", scale=128 ** 0.5, sparse_mode=3)[0]
+    out.backward(torch.ones_like(out))
+    col_sums = v.grad.float()[..., 0]  # identical along d
+    assert (v.grad.float() - col_sums.unsqueeze(-1)).abs().max().item() <= 2e-2
+    assert (col_sums.sum(-1) - S).abs().max().item() <= 0.02 * S
+    vc = torch.randn(B, N, 1, 128, device=DEV).bfloat16().expand(B, N, S, 128).contiguous().requires_grad_()
+    q2, k2 = (t.detach().clone().requires_grad_() for t in (q, k))
+    out = npu_fusion_attention_graph(q2, k2, vc, N, "BNSD", scale=128 ** 0.5, sparse_mode=3)[0]
+    out.backward(torch.randn_like(out))
+    assert q2.grad.float().abs().max().item() <= 2e-2 and k2.grad.float().abs().max().item() <= 2e-2
