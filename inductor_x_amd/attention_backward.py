@@ -1,9 +1,10 @@
 """Backward of the fused attention forward (npu_graph::npu_fa_backward).
 
-Interim implementation: the five matrix products run as library GEMMs (torch.bmm, hipBLASLt
-underneath) on a bounded number of heads at a time, with the scores recomputed from the forward's
-saved row statistics; it is not yet a fused MFMA kernel and moves O(S^2) intermediates through HBM.
-Definitions (per head, scores scaled by `scale`, causal mask optional), with m = softmax_max and
+Two paths.  Head dimension 128 with a sequence length that is a multiple of 128 runs the fused MFMA
+kernels (kernels.fused_attention_backward, csrc/mi/attention_bwd.h).  Other shapes run the matrix
+products as library GEMMs (torch.bmm, hipBLASLt underneath) on a bounded number of heads at a time
+and move O(S^2) intermediates through HBM.  Both recompute the probabilities from the forward's
+saved row statistics.  Definitions (per head, scores scaled by `scale`, causal mask optional), with m = softmax_max and
 l = softmax_sum as saved by the forward:
 
     S  = Q K^T * scale                      P  = exp(S - m) / l          (masked entries: 0)
@@ -23,9 +24,24 @@ import torch
 _SCORE_BYTES_BUDGET = 2 << 30
 
 
-def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale: float, causal: bool):
-    """q, k, v, out, dout: [B, N, S, D] bf16 (contiguous); softmax_max / softmax_sum: [B, N, S, 8] fp32
-    from the forward.  Returns (dq, dk, dv) in bf16."""
+def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale: float, causal: bool,
+                             use_kernels=None):
+    """q, k, v, out, dout: [B, N, S, D] bf16; softmax_max / softmax_sum: [B, N, S, 8] fp32 from the
+    forward.  Returns (dq, dk, dv) in bf16.  use_kernels: None = fused kernels where they apply."""
+    fits = q.dim() == 4 and q.size(3) == 128 and q.size(2) % 128 == 0 and q.size(2) > 0
+    if use_kernels is None:
+        use_kernels = fits
+    if use_kernels:
+        from . import kernels
+
+        return kernels.fused_attention_backward(
+            q.contiguous(), k.contiguous(), v.contiguous(), out.contiguous(), dout.contiguous(),
+            softmax_max.contiguous(), softmax_sum.contiguous(), scale, causal,
+        )
+    return _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale, causal)
+
+
+def _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale: float, causal: bool):
     for t in (q, k, v, out, dout):
         if not (t.is_cuda and t.dtype == torch.bfloat16 and t.dim() == 4):
             raise ValueError("attention backward: q, k, v, out, dout must be 4-D bf16 GPU tensors")

@@ -532,6 +532,75 @@ def fused_attention(
     return out, smax, ssum
 
 
+# ---------------------------------------------------------------------------
+# fused attention backward (bf16, head dim 128): delta, dQ and dK/dV kernels
+# ---------------------------------------------------------------------------
+_ATTN_BWD_DQ_LDS = 2 * (2 * 64 * 136 + 128 * 64) * 2
+_ATTN_BWD_DKV_LDS = 2 * ((2 * 64 * 136 + 2 * 128 * 64) * 2 + 3 * 64 * 4)
+
+
+@functools.lru_cache(maxsize=None)
+def _attention_bwd_launchers() -> dict:
+    src = codecache.aot_source("attention_bwd_kernels.hip")
+    mk = lambda name, sig, cfgs: CachingLauncher(name, src, sig, cfgs, prefer_intree=True)  # noqa: E731
+    return {
+        "delta": mk("attention_bwd_delta_bf16_d128", "PPPi", [LaunchConfig("attention_bwd_delta_bf16_d128", 256)]),
+        "dq": mk(
+            "attention_bwd_dq_bf16_d128", "PPPPPPPPiif",
+            [LaunchConfig(f"attention_bwd_dq_bf16_d128_{c}", 256, meta={"CAUSAL": c == "causal"},
+                          lds_bytes=_ATTN_BWD_DQ_LDS) for c in ("causal", "full")],
+        ),
+        "dkv": mk(
+            "attention_bwd_dkv_bf16_d128", "PPPPPPPPPiif",
+            [LaunchConfig(f"attention_bwd_dkv_bf16_d128_{c}", 256, meta={"CAUSAL": c == "causal"},
+                          lds_bytes=_ATTN_BWD_DKV_LDS) for c in ("causal", "full")],
+        ),
+    }
+
+
+def fused_attention_backward(
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, dout: torch.Tensor,
+    softmax_max: torch.Tensor, softmax_sum: torch.Tensor, scale: float, causal: bool,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Gradients (dq, dk, dv) of fused_attention for [B, N, S, 128] bf16 tensors, S a multiple of
+    128; softmax_max / softmax_sum are the forward's [B, N, S, 8] fp32 statistics."""
+    _check_cuda(q, k, v, out, dout, softmax_max, softmax_sum)
+    for t in (q, k, v, out, dout):
+        _require(t.dtype == torch.bfloat16 and t.dim() == 4 and t.shape == q.shape, "q, k, v, out, dout: one [B, N, S, D] bf16 shape")
+        _require(t.is_contiguous() and _aligned(t), "q, k, v, out, dout must be contiguous and 16-byte aligned")
+    B, N, S, D = q.shape
+    _require(D == 128, "head dimension must be 128")
+    _require(S % 128 == 0 and S > 0, "sequence length must be a positive multiple of 128")
+    for t in (softmax_max, softmax_sum):
+        _require(t.dtype == torch.float32 and t.shape == (B, N, S, 8) and t.is_contiguous(), "statistics must be contiguous fp32 [B, N, S, 8]")
+    _require(scale > 0 and math.isfinite(scale), "scale must be positive and finite")
+    _require(B * N * S * D < 2**31, "numel must fit int32 indexing")
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    heads = B * N
+    if heads == 0:
+        return dq, dk, dv
+    ls = _attention_bwd_launchers()
+    st = _stream()
+    delta = torch.empty(heads * S, dtype=torch.float32, device=q.device)
+    ls["delta"]._launch(_find(ls["delta"], "attention_bwd_delta_bf16_d128"), (out.data_ptr(), dout.data_ptr(), delta.data_ptr(), heads * S), (cdiv(heads * S * 16, 256), 1, 1), st)
+    which = "causal" if causal else "full"
+    grid = (8 * cdiv(heads, 8) * (S // 128), 1, 1)
+    ldq, ldkv = ls["dq"], ls["dkv"]
+    ldkv._launch(
+        _find(ldkv, f"attention_bwd_dkv_bf16_d128_{which}"),
+        (q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), softmax_max.data_ptr(), softmax_sum.data_ptr(),
+         delta.data_ptr(), dk.data_ptr(), dv.data_ptr(), heads, S, float(scale)),
+        grid, st,
+    )
+    ldq._launch(
+        _find(ldq, f"attention_bwd_dq_bf16_d128_{which}"),
+        (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(), softmax_max.data_ptr(),
+         softmax_sum.data_ptr(), dq.data_ptr(), heads, S, float(scale)),
+        grid, st,
+    )
+    return dq, dk, dv
+
+
 _ATTN_DEFAULT_WAVES = 8
 _ATTN_DEFAULT_PINGPONG = True
 _ATTN_DEFAULT_VARIANT = "v4"  # the interleaved 8-wavefront kernel whenever S % 256 == 0
