@@ -29,6 +29,9 @@
  *     part of the reference tree: PARITY UNPINNED against that kernel; this
  *     function restates the published definition of scaled-dot-product
  *     attention and is pinned by closed forms in tests/test_oracle.py.
+ *   - attention backward (oracle_attention_bwd): the gradients of that definition,
+ *     PARITY UNPINNED against torch_npu's npu_fusion_attention_grad for the same reason;
+ *     pinned by central differences of an independent forward and by invariants.
  *
  * Accumulations use double so the oracle is the more accurate side of every
  * comparison; element-wise math is done in float where the kernel does so.
@@ -213,4 +216,65 @@ void oracle_attention_bf16(const uint16_t* q, const uint16_t* k, const uint16_t*
   }
 }
 
-int oracle_abi_version(void) { return 1; }
+/*
+ * Attention backward, layout BNSD, Sq == Sk == S.  q, k, v, dout as bf16; dq, dk, dv out as fp64
+ * (the caller rounds as it needs).  Definition: with P = softmax(Q K^T * scale [+ causal mask]),
+ * O = P V and an upstream gradient dO,
+ *     dV = P^T dO,  dP = dO V^T,  dS = P * (dP - rowsum(P * dP)) * scale,  dQ = dS K,  dK = dS^T Q
+ * (rowsum(P * dP) = rowsum(dO * O)).  Everything in double; no intermediate rounding.
+ * The reference obtains these gradients from torch_npu.npu_fusion_attention_grad
+ * (reference inductor_x/npu_fusion_attention_graph.py:38-42), a CANN kernel outside the tree:
+ * PARITY UNPINNED against that kernel; pinned by central differences of oracle_attention's own
+ * definition in tests/test_oracle.py.
+ */
+void oracle_attention_bwd(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* dout,
+                          double* dq, double* dk, double* dv, int64_t B, int64_t N, int64_t S, int64_t D,
+                          double scale, int causal) {
+  memset(dq, 0, sizeof(double) * (size_t)(B * N * S * D));
+  memset(dk, 0, sizeof(double) * (size_t)(B * N * S * D));
+  memset(dv, 0, sizeof(double) * (size_t)(B * N * S * D));
+#pragma omp parallel for schedule(dynamic, 1)
+  for (int64_t bn = 0; bn < B * N; ++bn) {
+    const uint16_t* qb = q + bn * S * D;
+    const uint16_t* kb = k + bn * S * D;
+    const uint16_t* vb = v + bn * S * D;
+    const uint16_t* gb = dout + bn * S * D;
+    double* p = (double*)malloc(sizeof(double) * (size_t)S);
+    double* dp = (double*)malloc(sizeof(double) * (size_t)S);
+    for (int64_t i = 0; i < S; ++i) {
+      const int64_t jend = causal ? i + 1 : S;
+      double m = -INFINITY;
+      for (int64_t j = 0; j < jend; ++j) {
+        double dot = 0.0;
+        for (int64_t d = 0; d < D; ++d) dot += (double)bf16_to_f32(qb[i * D + d]) * (double)bf16_to_f32(kb[j * D + d]);
+        p[j] = dot * scale;
+        if (p[j] > m) m = p[j];
+      }
+      double l = 0.0;
+      for (int64_t j = 0; j < jend; ++j) {
+        p[j] = exp(p[j] - m);
+        l += p[j];
+      }
+      double delta = 0.0;
+      for (int64_t j = 0; j < jend; ++j) {
+        p[j] /= l;
+        double t = 0.0;
+        for (int64_t d = 0; d < D; ++d) t += (double)bf16_to_f32(gb[i * D + d]) * (double)bf16_to_f32(vb[j * D + d]);
+        dp[j] = t;
+        delta += p[j] * t;
+      }
+      for (int64_t j = 0; j < jend; ++j) {
+        const double ds = p[j] * (dp[j] - delta) * scale;
+        for (int64_t d = 0; d < D; ++d) {
+          dv[(bn * S + j) * D + d] += p[j] * (double)bf16_to_f32(gb[i * D + d]);
+          dq[(bn * S + i) * D + d] += ds * (double)bf16_to_f32(kb[j * D + d]);
+          dk[(bn * S + j) * D + d] += ds * (double)bf16_to_f32(qb[i * D + d]);
+        }
+      }
+    }
+    free(p);
+    free(dp);
+  }
+}
+
+int oracle_abi_version(void) { return 2; }

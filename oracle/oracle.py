@@ -140,3 +140,18 @@ def attention_bf16(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float, ca
     if q.size:
         lib().oracle_attention_bf16(_p(q), _p(k), _p(v), _p(out), _p(smax), _p(ssum), B, N, Sq, Sk, D, scale, int(causal))
     return out, smax, ssum
+
+
+def attention_bwd(q: np.ndarray, k: np.ndarray, v: np.ndarray, dout: np.ndarray, scale: float, causal: bool):
+    """q, k, v, dout [B,N,S,D] as bf16 bits.  Returns (dq, dk, dv) as float64 arrays."""
+    q, k, v, dout = _c(q, np.uint16), _c(k, np.uint16), _c(v, np.uint16), _c(dout, np.uint16)
+    B, N, S, D = q.shape
+    dq = np.zeros(q.shape, np.float64)
+    dk = np.zeros(q.shape, np.float64)
+    dv = np.zeros(q.shape, np.float64)
+    if q.size:
+        fn = lib().oracle_attention_bwd
+        fn.argtypes = [ctypes.c_void_p] * 7 + [ctypes.c_int64] * 4 + [ctypes.c_double, ctypes.c_int]
+        fn.restype = None
+        fn(_p(q), _p(k), _p(v), _p(dout), _p(dq), _p(dk), _p(dv), B, N, S, D, float(scale), int(causal))
+    return dq, dk, dv

@@ -265,3 +265,19 @@ def test_attention_backward_full_length_causal_independence(K):
     dq2, dk2, dv2 = K.fused_attention_backward(q, k, v, o, (do.float() * 2).bfloat16(), m, l, scale, True)
     for a, b in ((dq, dq2), (dk, dk2), (dv, dv2)):
         assert (b.float() - 2 * a.float()).abs().max().item() <= 2e-2 * max(b.float().abs().max().item(), 1.0)
+
+
+@pytest.mark.parametrize("B,N,S,causal", [(1, 2, 128, True), (1, 1, 256, False), (2, 2, 256, True)])
+def test_attention_backward_vs_oracle(K, O, B, N, S, causal):
+    """Fused backward kernels against the fp64 oracle on the same bf16 inputs (the kernels take the
+    forward kernel's output and statistics).  Bar: 1 % of the largest entry of each gradient."""
+    announce(f"attention backward vs oracle B={B} N={N} S={S} causal={causal}")
+    torch.manual_seed(9)
+    q, k, v, do = (torch.randn(B, N, S, 128).bfloat16() for _ in range(4))
+    scale = 128 ** -0.5
+    qd, kd, vd, dod = (t.to(DEV) for t in (q, k, v, do))
+    o, m, l = K.fused_attention(qd, kd, vd, scale, causal)
+    got = K.fused_attention_backward(qd, kd, vd, o, dod, m, l, scale, causal)
+    ref = O.attention_bwd(bits(q), bits(k), bits(v), bits(do), scale, causal)
+    for g, r in zip(got, ref):
+        assert np.abs(g.float().cpu().numpy() - r).max() <= 1e-2 * np.abs(r).max() + 1e-3

@@ -188,3 +188,53 @@ def test_attention_closed_forms():
     mean = v.double().mean(2, keepdim=True).expand(-1, -1, 12, -1)
     assert np.abs(O.bf16_bits_to_f32(out3) - mean.float().numpy()).max() < 1e-2  # equal keys: plain mean
     assert np.allclose(ssum3, 12.0)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_backward_vs_central_differences(causal):
+    """The backward oracle against central differences of an independent fp64 forward (numpy),
+    entry by entry: a wrong sign, a dropped rowsum term or a missing scale factor all fail."""
+    rng = np.random.default_rng(3)
+    B, N, S, D = 1, 2, 6, 4
+    mk = lambda: torch.from_numpy(rng.standard_normal((B, N, S, D)).astype(np.float32)).bfloat16()  # noqa: E731
+    q, k, v, g = mk(), mk(), mk(), mk()
+    scale = 0.37
+    dq, dk, dv = O.attention_bwd(bits(q), bits(k), bits(v), bits(g), scale, causal)
+
+    def loss(qa, ka, va):
+        s = np.einsum("bnid,bnjd->bnij", qa, ka) * scale
+        if causal:
+            s = np.where(np.triu(np.ones((S, S), bool), 1), -np.inf, s)
+        p = np.exp(s - s.max(-1, keepdims=True))
+        p /= p.sum(-1, keepdims=True)
+        return float((np.einsum("bnij,bnjd->bnid", p, va) * g.double().numpy()).sum())
+
+    base = [t.double().numpy() for t in (q, k, v)]
+    eps = 1e-5
+    for which, grad in enumerate((dq, dk, dv)):
+        fd = np.zeros_like(grad)
+        it = np.nditer(base[which], flags=["multi_index"])
+        for _ in it:
+            idx = it.multi_index
+            plus = [a.copy() for a in base]
+            minus = [a.copy() for a in base]
+            plus[which][idx] += eps
+            minus[which][idx] -= eps
+            fd[idx] = (loss(*plus) - loss(*minus)) / (2 * eps)
+        np.testing.assert_allclose(grad, fd, rtol=1e-6, atol=1e-8)
+
+
+def test_attention_backward_invariants():
+    """dV with dO = 1 holds the column sums of P (which total S per head); a V that is constant
+    along the sequence makes dQ = dK = 0; the gradients are linear in dO."""
+    torch.manual_seed(4)
+    q, k, v, g = (torch.randn(1, 2, 10, 8).bfloat16() for _ in range(4))
+    dq, dk, dv = O.attention_bwd(bits(q), bits(k), bits(v), bits(torch.ones_like(g)), 0.3, True)
+    assert np.allclose(dv, dv[..., :1]) and np.allclose(dv[..., 0].sum(-1), 10.0)
+    vc = v[:, :, :1].expand(-1, -1, 10, -1).contiguous()
+    dq, dk, _ = O.attention_bwd(bits(q), bits(k), bits(vc), bits(g), 0.3, True)
+    assert np.abs(dq).max() < 1e-12 and np.abs(dk).max() < 1e-12
+    a = O.attention_bwd(bits(q), bits(k), bits(v), bits(g), 0.3, False)
+    b = O.attention_bwd(bits(q), bits(k), bits(v), bits((g.float() * 2).bfloat16()), 0.3, False)
+    for x, y in zip(a, b):
+        assert np.allclose(2 * x, y)
