@@ -250,15 +250,15 @@ _registered = False
 
 def register_fx_pass() -> None:
     """Register the replacement with Inductor's joint-graph pattern pass
-    (reference inductor_x/npu_fusion_attention_graph.py:134-230).  Inference
-    only: the training variant needs npu_fa_backward."""
+    (reference inductor_x/npu_fusion_attention_graph.py:134-230), for inference and for
+    training graphs; patterns with dropout are not rewritten (the kernels have none)."""
     global _registered
     if _registered:
         return
     _registered = True
     from torch._inductor.fx_passes import joint_graph
     from torch._inductor.fx_passes.fuse_attention import partialize_and_update_signature
-    from torch._inductor.pattern_matcher import fwd_only, init_once_fakemode, register_replacement
+    from torch._inductor.pattern_matcher import fwd_only, init_once_fakemode, joint_fwd_bwd, register_replacement
 
     @init_once_fakemode
     def _init():
@@ -269,6 +269,13 @@ def register_fx_pass() -> None:
         replacement = partialize_and_update_signature(_attention_replacement_1, dropout_p=0.0)
         register_replacement(
             pattern, replacement, [g(), g(), g(), c()], fwd_only, joint_graph.patterns,
+            extra_check=_extra_check, scalar_workaround={},
+        )
+        # training: the same search function traced with its backward; the replacement's
+        # autograd.Function supplies npu_fa_backward (reference :196-204, without dropout)
+        gr = functools.partial(torch.empty, (2, 4, 8, 16), device=device, dtype=torch.float, requires_grad=True)
+        register_replacement(
+            pattern, replacement, [gr(), gr(), gr(), c()], joint_fwd_bwd, joint_graph.patterns,
             extra_check=_extra_check, scalar_workaround={},
         )
 

@@ -415,3 +415,36 @@ def test_dynamic_shapes_reuse_one_kernel():
         ref = f(x, w)
         torch.testing.assert_close(got[0], ref[0], rtol=1e-4, atol=1e-4)
         torch.testing.assert_close(got[1], ref[1])
+
+
+def test_attention_pattern_training():
+    """The unfused attention pattern in a graph that is differentiated: the joint-graph pass rewrites
+    it to npu_fa / npu_fa_backward (reference inductor_x/npu_fusion_attention_graph.py:196-204), and
+    the gradients agree with eager autograd to bf16 rounding."""
+    announce("compile attention pattern, training")
+    from torch._dynamo.utils import counters
+
+    torch.manual_seed(0)
+    B, S, N, D = 2, 256, 4, 128
+    qs, ks, vs = (torch.randn(B, S, N, D, device=DEV).bfloat16().requires_grad_() for _ in range(3))
+    inv = D ** 0.5
+
+    def g(q, k, v):
+        q, k, v = (t.permute(0, 2, 1, 3) for t in (q, k, v))
+        return torch.matmul(q, k.transpose(-2, -1)).div(inv).softmax(dim=-1).matmul(v)
+
+    torch._dynamo.reset()
+    counters.clear()
+    with torch._inductor.config.patch(force_disable_caches=True):
+        out = torch.compile(g)(qs, ks, vs)
+        w = torch.randn_like(out)
+        (out * w).sum().backward()
+    assert counters["inductor"]["fuse_attention"] >= 1
+    got = [t.grad.clone() for t in (qs, ks, vs)]
+    for t in (qs, ks, vs):
+        t.grad = None
+    ref = g(qs, ks, vs)
+    (ref * w).sum().backward()
+    assert (out.float() - ref.float()).abs().max().item() <= 2e-2
+    for a, t in zip(got, (qs, ks, vs)):
+        assert (a.float() - t.grad.float()).abs().max().item() <= 3e-2 * max(t.grad.float().abs().max().item(), 1.0)
