@@ -172,6 +172,13 @@ def _all_configs(K, torch) -> list:
     both("5 causal attention bf16 [4,32,4096,128]", lambda q, k, v: K.fused_attention(q, k, v, 128 ** -0.5, True),
          lambda q, k, v: npu_fusion_attention_graph(q, k, v, 32, "BNSD", scale=128 ** 0.5, sparse_mode=3)[0],
          (q, k, v), ATTN_FLOPS_CAUSAL, "mfma")
+    # Backward of the same graph (the caller next to the forward on the
+    # training path): five matrix products plus two recomputed ones, counted
+    # by the usual convention as 2.5 x the forward's algorithmic FLOPs.
+    o, m, l = K.fused_attention(q, k, v, 128 ** -0.5, True)[:3]
+    do = torch.randn_like(o)
+    add("5b causal attention backward bf16 [4,32,4096,128]", "kernel",
+        lambda: K.fused_attention_backward(q, k, v, o, do, m, l, 128 ** -0.5, True), 2.5 * ATTN_FLOPS_CAUSAL, "mfma")
     return out
 
 
