@@ -1,7 +1,7 @@
 """Backward of the fused attention forward (npu_graph::npu_fa_backward).
 
 Two paths.  Head dimension 128 with a sequence length that is a multiple of 128 runs the fused MFMA
-kernels (kernels.fused_attention_backward, csrc/mi/attention_bwd.h).  Other shapes run the matrix
+kernels (kernels.fused_attention_backward, csrc/mi/attention_bwd_w8.h).  Other shapes run the matrix
 products as library GEMMs (torch.bmm, hipBLASLt underneath) on a bounded number of heads at a time
 and move O(S^2) intermediates through HBM.  Both recompute the probabilities from the forward's
 saved row statistics.  Definitions (per head, scores scaled by `scale`, causal mask optional), with m = softmax_max and

@@ -1,0 +1,394 @@
+// Fused attention backward (bf16, head dimension 128): eight wavefronts per workgroup, two per
+// SIMD, three kernels after a small statistics pass, no atomics.
+//
+// With P = exp(S - m) / l recomputed from the forward's row statistics (S = Q K^T * scale,
+// m = row maximum, l = row sum), D = rowsum(dO * O) and dS = P * (dO V^T - D):
+//     dV = P^T dO        dK = scale * dS^T Q        dQ = scale * dS K
+// The statistics pass folds m and l into one exponent offset per row, m log2(e) + log2(l), so a
+// probability costs one fused multiply-add and one exp2.
+//
+//   dQ kernel   a wavefront owns 32 queries (lane = query), a workgroup 256; loop over 64-key tiles:
+//               S^T = K Q^T, dP^T = V dO^T (A from LDS, B = Q / dO fragments in registers),
+//               dS^T is at once the B operand of dQ^T += K^T dS^T (A = transposed K tile).
+//   dK kernel   a wavefront owns 32 keys (lane = key), loop over 64-query tiles:
+//               S = Q K^T, dP = dO V^T (A from LDS, B = K / V fragments in registers),
+//               dK^T += Q^T dS (A = transposed Q tile, query axis permuted as attn_vt_pos).
+//   dV kernel   same orientation: S = Q K^T, dV^T += dO^T P.
+//
+// dK and dV are separate kernels (the scores are recomputed three times in all, eight matrix
+// products instead of the textbook five): together their accumulators, operands and staging
+// registers need more than the 256 registers a wavefront has at two wavefronts per SIMD, and two
+// wavefronts per SIMD -- one in its MFMAs while the other recomputes probabilities -- is worth
+// more than the product saved.
+//
+// Every 64-row tile travels global -> registers -> LDS (double-buffered, one barrier per tile).
+// Sequence lengths need only be multiples of 64: rows of a last partial block are clamped for
+// loads and not stored.
+#pragma once
+
+#include "attention_v2.h"
+
+namespace mi {
+
+constexpr int kBwd8Waves = 8;
+constexpr int kBwd8Threads = 64 * kBwd8Waves;
+constexpr int kBwd8BlockRows = 32 * kBwd8Waves;  // queries (dQ) or keys (dK, dV) per workgroup
+constexpr int kBwd8RowTile = kAttnBN * kAttnKStride;  // [64][136] row-major tile, elements
+constexpr int kBwd8ColTile = kAttnD * kAttnVStride;   // [128][64] transposed tile, elements
+constexpr int kBwd8StatBytes = kAttnBN * 2 * 4;       // (exponent offset, D) of a query tile
+constexpr int kBwd8DqBufBytes = (2 * kBwd8RowTile + kBwd8ColTile) * 2;                    // K, V, K^T
+constexpr int kBwd8DkBufBytes = (2 * kBwd8RowTile + kBwd8ColTile) * 2 + kBwd8StatBytes;   // Q, dO, Q^T
+constexpr int kBwd8DvBufBytes = (kBwd8RowTile + kBwd8ColTile) * 2 + kBwd8StatBytes;       // Q, dO^T
+constexpr int kBwd8DqLdsBytes = 2 * kBwd8DqBufBytes;
+constexpr int kBwd8DkLdsBytes = 2 * kBwd8DkBufBytes;
+constexpr int kBwd8DvLdsBytes = 2 * kBwd8DvBufBytes;
+constexpr float kBwd8Log2e = 1.4426950408889634f;
+
+// stats[row] = (m log2 e + log2 l, sum_d dO[row, d] * O[row, d]); 16 lanes per row.
+__device__ __forceinline__ void attention_bwd_stats(const bf16_t* __restrict__ O, const bf16_t* __restrict__ dO,
+                                                    const float* __restrict__ softmax_max,
+                                                    const float* __restrict__ softmax_sum,
+                                                    float* __restrict__ stats, int rows) {
+  const int row = (blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+  const int part = threadIdx.x & 15;
+  float acc = 0.f;
+  if (row < rows) {
+    const bf16x8_t o = *reinterpret_cast<const bf16x8_t*>(O + static_cast<size_t>(row) * kAttnD + 8 * part);
+    const bf16x8_t d = *reinterpret_cast<const bf16x8_t*>(dO + static_cast<size_t>(row) * kAttnD + 8 * part);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc = fmaf(static_cast<float>(o[e]), static_cast<float>(d[e]), acc);
+  }
+#pragma unroll
+  for (int off = 8; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+  if (row < rows && part == 0) {
+    const float m = softmax_max[static_cast<size_t>(row) * 8];
+    const float l = softmax_sum[static_cast<size_t>(row) * 8];
+    Vec<float, 2> st;
+    st[0] = fmaf(m, kBwd8Log2e, __builtin_amdgcn_logf(l));
+    st[1] = acc;
+    store_vec<float, 2>(stats + 2 * static_cast<size_t>(row), st);
+  }
+}
+
+// Staging of a [64][128] bf16 tile by 512 threads.  Row form: 2 x 16 bytes per thread, stored
+// row-major.  Column form: 4 rows x 4 columns per thread (4 x 8 bytes), stored transposed with the
+// row index (the contraction axis of the MFMA that reads the tile) permuted, and optionally
+// row-major as well.
+struct Bwd8RowStage {
+  u32x4_t r[2];
+};
+struct Bwd8ColStage {
+  u32x2_t r[4];
+};
+__device__ __forceinline__ void bwd8_load(Bwd8RowStage& t, const bf16_t* __restrict__ src, int tid) {
+  const int row = tid >> 4, col = (tid & 15) * 8;
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+    t.r[u] = *reinterpret_cast<const u32x4_t*>(src + static_cast<size_t>(row + 32 * u) * kAttnD + col);
+}
+__device__ __forceinline__ void bwd8_store_rows(const Bwd8RowStage& t, bf16_t* dst, int tid) {
+  const int row = tid >> 4, col = (tid & 15) * 8;
+#pragma unroll
+  for (int u = 0; u < 2; ++u) *reinterpret_cast<u32x4_t*>(dst + (row + 32 * u) * kAttnKStride + col) = t.r[u];
+}
+__device__ __forceinline__ void bwd8_load(Bwd8ColStage& t, const bf16_t* __restrict__ src, int tid) {
+  const int rg = tid >> 5, cg = tid & 31;
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+    t.r[u] = *reinterpret_cast<const u32x2_t*>(src + static_cast<size_t>(4 * rg + u) * kAttnD + 4 * cg);
+}
+__device__ __forceinline__ void bwd8_store_rows(const Bwd8ColStage& t, bf16_t* dst, int tid) {
+  const int rg = tid >> 5, cg = tid & 31;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) *reinterpret_cast<u32x2_t*>(dst + (4 * rg + u) * kAttnKStride + 4 * cg) = t.r[u];
+}
+__device__ __forceinline__ void bwd8_store_cols(const Bwd8ColStage& t, bf16_t* dst, int tid) {
+  const int rg = tid >> 5, cg = tid & 31;
+  const int pos = attn_vt_pos(4 * rg);
+#pragma unroll
+  for (int e2 = 0; e2 < 2; ++e2) {
+    // dword e2 of each row holds columns 4 cg + 2 e2 (low half) and + 1 (high half)
+    const uint32_t a0 = t.r[0][e2], a1 = t.r[1][e2], a2 = t.r[2][e2], a3 = t.r[3][e2];
+    u32x2_t lo, hi;
+    lo[0] = __builtin_amdgcn_perm(a1, a0, 0x05040100u);
+    lo[1] = __builtin_amdgcn_perm(a3, a2, 0x05040100u);
+    hi[0] = __builtin_amdgcn_perm(a1, a0, 0x07060302u);
+    hi[1] = __builtin_amdgcn_perm(a3, a2, 0x07060302u);
+    *reinterpret_cast<u32x2_t*>(dst + attn_vt_offset(4 * cg + 2 * e2, pos)) = lo;
+    *reinterpret_cast<u32x2_t*>(dst + attn_vt_offset(4 * cg + 2 * e2 + 1, pos)) = hi;
+  }
+}
+__device__ __forceinline__ bf16x8_t bwd8_row_frag(const bf16_t* tile, int row, int s, int g) {
+  return *reinterpret_cast<const bf16x8_t*>(tile + row * kAttnKStride + 16 * s + 8 * g);
+}
+__device__ __forceinline__ bf16x8_t bwd8_col_frag(const bf16_t* tile, int row, int t, int g) {
+  return *reinterpret_cast<const bf16x8_t*>(tile + attn_vt_offset(row, 16 * t + 8 * g));
+}
+// accumulator (transposed: lane = row of the output, registers = head dimension) -> one output row
+__device__ __forceinline__ void bwd8_store_acc(bf16_t* __restrict__ dst_row, const f32x16_t (&acc)[4], int g,
+                                               float factor) {
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int rq = 0; rq < 4; ++rq) {
+      bf16x4_t o4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o4[e] = static_cast<bf16_t>(acc[db][4 * rq + e] * factor);
+      *reinterpret_cast<bf16x4_t*>(dst_row + 32 * db + 8 * rq + 4 * g) = o4;
+    }
+}
+__device__ __forceinline__ void bwd8_zero(f32x16_t (&acc)[4]) {
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
+}
+
+// ---------------------------------------------------------------------------------------------
+// dQ
+// ---------------------------------------------------------------------------------------------
+template <bool CAUSAL>
+__device__ __forceinline__ void attention_bwd8_dq(const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K,
+                                                  const bf16_t* __restrict__ V, const bf16_t* __restrict__ dO,
+                                                  const float* __restrict__ stats, bf16_t* __restrict__ dQ,
+                                                  int S, int q_block, int head, float scale) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char attn_lds[];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
+  const size_t head_off = static_cast<size_t>(head) * S * kAttnD;
+  const bf16_t* __restrict__ Kh = K + head_off;
+  const bf16_t* __restrict__ Vh = V + head_off;
+  const int q0 = q_block * kBwd8BlockRows;
+  const int qw = q0 + wave * 32;       // first query of this wavefront
+  const int qi = qw + li;
+  const bool valid = qi < S;
+  const int qc = valid ? qi : S - 1;   // rows past the end read the last row and are never stored
+  const size_t qrow = head_off + static_cast<size_t>(qc) * kAttnD;
+
+  bf16x8_t qf[8], dof[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    qf[s] = *reinterpret_cast<const bf16x8_t*>(Q + qrow + 16 * s + 8 * g);
+    dof[s] = *reinterpret_cast<const bf16x8_t*>(dO + qrow + 16 * s + 8 * g);
+  }
+  const Vec<float, 2> st = load_vec<float, 2>(stats + 2 * (static_cast<size_t>(head) * S + qc));
+  const float m2 = st[0], delta = st[1];
+  const float c2 = scale * kBwd8Log2e;
+
+  f32x16_t acc[4];
+  bwd8_zero(acc);
+
+  const int all_tiles = S / kAttnBN;
+  const int n_tiles = CAUSAL ? min((q0 + kBwd8BlockRows) / kAttnBN, all_tiles) : all_tiles;
+  const int wave_last_tile = (CAUSAL && qw < S) ? (qw + 31) / kAttnBN : (qw < S ? n_tiles - 1 : -1);
+
+  auto buf = [&](int b) { return reinterpret_cast<bf16_t*>(attn_lds + b * kBwd8DqBufBytes); };
+  Bwd8ColStage kt;
+  Bwd8RowStage vt;
+  auto load_tile = [&](int tile) {
+    bwd8_load(kt, Kh + static_cast<size_t>(tile) * kAttnBN * kAttnD, tid);
+    bwd8_load(vt, Vh + static_cast<size_t>(tile) * kAttnBN * kAttnD, tid);
+  };
+  auto store_tile = [&](int b) {
+    bf16_t* Ks = buf(b);
+    bwd8_store_rows(kt, Ks, tid);
+    bwd8_store_rows(vt, Ks + kBwd8RowTile, tid);
+    bwd8_store_cols(kt, Ks + 2 * kBwd8RowTile, tid);
+  };
+
+  auto compute = [&](int tile, auto mask_c) {
+    constexpr bool MASK = decltype(mask_c)::value;
+    const bf16_t* Ks = buf(tile & 1);
+    const bf16_t* Vs = Ks + kBwd8RowTile;
+    const bf16_t* Kt = Ks + 2 * kBwd8RowTile;
+    const int key0 = tile * kAttnBN;
+    bf16x8_t dsf[2][2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      f32x16_t sacc, pacc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        sacc[r] = 0.f;
+        pacc[r] = 0.f;
+      }
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bwd8_row_frag(Ks, 32 * kb + li, s, g), qf[s], sacc, 0, 0, 0);
+        pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bwd8_row_frag(Vs, 32 * kb + li, s, g), dof[s], pacc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], c2, -m2));
+        if (MASK && key0 + 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3) > qi) p = 0.f;
+        dsf[kb][r >> 3][r & 7] = static_cast<bf16_t>(p * (pacc[r] - delta));
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bwd8_col_frag(Kt, 32 * db + li, t, g), dsf[t >> 1][t & 1], acc[db], 0, 0, 0);
+  };
+
+  // Under a causal mask only the tiles that overlap the block's own queries (the last four) need
+  // the mask or are skipped by some wavefronts; they run in a loop of their own so that the loop
+  // over the tiles before them carries no masking code.
+  const int first_diag = CAUSAL ? min(q0 / kAttnBN, n_tiles) : n_tiles;
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+  for (int tile = 0; tile < first_diag; ++tile) {
+    if (tile + 1 < n_tiles) load_tile(tile + 1);
+    if (tile <= wave_last_tile) compute(tile, attn_flag<false>{});
+    if (tile + 1 < n_tiles) store_tile((tile + 1) & 1);
+    __syncthreads();
+  }
+  if constexpr (CAUSAL) {
+#pragma nounroll
+    for (int tile = first_diag; tile < n_tiles; ++tile) {
+      if (tile + 1 < n_tiles) load_tile(tile + 1);
+      if (tile <= wave_last_tile) compute(tile, attn_flag<true>{});
+      if (tile + 1 < n_tiles) store_tile((tile + 1) & 1);
+      __syncthreads();
+    }
+  }
+  if (valid) bwd8_store_acc(dQ + qrow, acc, g, scale);
+}
+
+// ---------------------------------------------------------------------------------------------
+// dK (WHICH = 0) and dV (WHICH = 1): a wavefront owns 32 keys, loop over query tiles
+// ---------------------------------------------------------------------------------------------
+template <bool CAUSAL, int WHICH>
+__device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K,
+                                                   const bf16_t* __restrict__ V, const bf16_t* __restrict__ dO,
+                                                   const float* __restrict__ stats, bf16_t* __restrict__ dKV,
+                                                   int S, int k_block, int head, float scale) {
+  constexpr bool DK = WHICH == 0;
+  constexpr int BUF = DK ? kBwd8DkBufBytes : kBwd8DvBufBytes;
+  constexpr int STAT_OFF = BUF - kBwd8StatBytes;
+  extern __shared__ __attribute__((aligned(16))) unsigned char attn_lds[];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
+  const size_t head_off = static_cast<size_t>(head) * S * kAttnD;
+  const bf16_t* __restrict__ Qh = Q + head_off;
+  const bf16_t* __restrict__ dOh = dO + head_off;
+  const int k0 = k_block * kBwd8BlockRows;
+  const int kw = k0 + wave * 32;  // first key of this wavefront
+  const int kj = kw + li;
+  const bool valid = kj < S;
+  const int kc = valid ? kj : S - 1;
+  const size_t krow = head_off + static_cast<size_t>(kc) * kAttnD;
+
+  bf16x8_t kf[8], vf[DK ? 8 : 1];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    kf[s] = *reinterpret_cast<const bf16x8_t*>(K + krow + 16 * s + 8 * g);
+    if constexpr (DK) vf[s] = *reinterpret_cast<const bf16x8_t*>(V + krow + 16 * s + 8 * g);
+  }
+  f32x16_t acc[4];
+  bwd8_zero(acc);
+  const float c2 = scale * kBwd8Log2e;
+
+  const int n_qtiles = S / kAttnBN;
+  const int first_tile = CAUSAL ? k0 / kAttnBN : 0;  // first query tile that sees a key of the block
+  const int wave_first_tile = kw < S ? (CAUSAL ? kw / kAttnBN : 0) : n_qtiles;
+
+  // DK: Q both ways + dO rows; DV: Q rows + dO transposed
+  Bwd8ColStage cst;  // DK: Q, DV: dO
+  Bwd8RowStage rst;  // DK: dO, DV: Q
+  Vec<float, 2> sst;
+  auto load_tile = [&](int tile) {
+    const bf16_t* qp = Qh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
+    const bf16_t* dp = dOh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
+    bwd8_load(cst, DK ? qp : dp, tid);
+    bwd8_load(rst, DK ? dp : qp, tid);
+    if (tid < kAttnBN) sst = load_vec<float, 2>(stats + 2 * (static_cast<size_t>(head) * S + tile * kAttnBN + tid));
+  };
+  auto store_tile = [&](int b) {
+    bf16_t* base = reinterpret_cast<bf16_t*>(attn_lds + b * BUF);
+    if constexpr (DK) {
+      bwd8_store_rows(cst, base, tid);                        // Q
+      bwd8_store_rows(rst, base + kBwd8RowTile, tid);         // dO
+      bwd8_store_cols(cst, base + 2 * kBwd8RowTile, tid);     // Q^T
+    } else {
+      bwd8_store_rows(rst, base, tid);                        // Q
+      bwd8_store_cols(cst, base + kBwd8RowTile, tid);         // dO^T
+    }
+    if (tid < kAttnBN) store_vec<float, 2>(reinterpret_cast<float*>(attn_lds + b * BUF + STAT_OFF) + 2 * tid, sst);
+  };
+
+  auto compute = [&](int tile, auto mask_c) {
+    constexpr bool MASK = decltype(mask_c)::value;
+    const bf16_t* base = reinterpret_cast<const bf16_t*>(attn_lds + (tile & 1) * BUF);
+    const bf16_t* Qs = base;
+    const bf16_t* dOs = base + kBwd8RowTile;                              // DK only
+    const bf16_t* Tt = base + (DK ? 2 * kBwd8RowTile : kBwd8RowTile);     // Q^T (DK) or dO^T (DV)
+    const float* st = reinterpret_cast<const float*>(attn_lds + (tile & 1) * BUF + STAT_OFF);
+    const int q0t = tile * kAttnBN;
+    bf16x8_t bf[2][2];  // [query block][half]: P (dV) or dS (dK) as B operands, contraction over the queries
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      f32x16_t sacc, pacc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        sacc[r] = 0.f;
+        pacc[r] = 0.f;
+      }
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bwd8_row_frag(Qs, 32 * qb + li, s, g), kf[s], sacc, 0, 0, 0);
+        if constexpr (DK)
+          pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bwd8_row_frag(dOs, 32 * qb + li, s, g), vf[s], pacc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        // rows 32 qb + 8 rq + 4 g + (0..3) of the query tile and their statistics
+        const int row0 = 32 * qb + 8 * rq + 4 * g;
+        const Vec<float, 4> sa = load_vec<float, 4>(st + 2 * row0);
+        const Vec<float, 4> sb = load_vec<float, 4>(st + 2 * row0 + 4);
+        const float mrow[4] = {sa[0], sa[2], sb[0], sb[2]};
+        const float drow[4] = {sa[1], sa[3], sb[1], sb[3]};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = 4 * rq + e;
+          float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], c2, -mrow[e]));
+          if (MASK && kj > q0t + row0 + e) p = 0.f;
+          if constexpr (DK)
+            bf[qb][r >> 3][r & 7] = static_cast<bf16_t>(p * (pacc[r] - drow[e]));
+          else
+            bf[qb][r >> 3][r & 7] = static_cast<bf16_t>(p);
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bwd8_col_frag(Tt, 32 * db + li, t, g), bf[t >> 1][t & 1], acc[db], 0, 0, 0);
+  };
+
+  if (first_tile < n_qtiles) {
+    load_tile(first_tile);
+    store_tile(first_tile & 1);
+  }
+  __syncthreads();
+  // Under a causal mask the first four query tiles overlap the block's own keys: a loop of their
+  // own with the mask (and wavefronts whose keys come later skipping), then the unmasked rest.
+  const int after_diag = CAUSAL ? min(first_tile + kBwd8BlockRows / kAttnBN, n_qtiles) : first_tile;
+  if constexpr (CAUSAL) {
+#pragma nounroll
+    for (int tile = first_tile; tile < after_diag; ++tile) {
+      if (tile + 1 < n_qtiles) load_tile(tile + 1);
+      if (tile >= wave_first_tile) compute(tile, attn_flag<true>{});
+      if (tile + 1 < n_qtiles) store_tile((tile + 1) & 1);
+      __syncthreads();
+    }
+  }
+  for (int tile = after_diag; tile < n_qtiles; ++tile) {
+    if (tile + 1 < n_qtiles) load_tile(tile + 1);
+    if (kw < S) compute(tile, attn_flag<false>{});
+    if (tile + 1 < n_qtiles) store_tile((tile + 1) & 1);
+    __syncthreads();
+  }
+  if (valid) bwd8_store_acc(dKV + krow, acc, g, DK ? scale : 1.0f);
+}
+
+}  // namespace mi

@@ -533,10 +533,13 @@ def fused_attention(
 
 
 # ---------------------------------------------------------------------------
-# fused attention backward (bf16, head dim 128): delta, dQ and dK/dV kernels
+# fused attention backward (bf16, head dim 128): row statistics, then dQ, dK and dV kernels
 # ---------------------------------------------------------------------------
 _ATTN_BWD_DQ_LDS = 2 * (2 * 64 * 136 + 128 * 64) * 2
 _ATTN_BWD_DKV_LDS = 2 * ((2 * 64 * 136 + 2 * 128 * 64) * 2 + 3 * 64 * 4)
+_ATTN_BWD8_DQ_LDS = 2 * (2 * 64 * 136 + 128 * 64) * 2
+_ATTN_BWD8_DK_LDS = 2 * ((2 * 64 * 136 + 128 * 64) * 2 + 64 * 2 * 4)
+_ATTN_BWD8_DV_LDS = 2 * ((64 * 136 + 128 * 64) * 2 + 64 * 2 * 4)
 
 
 @functools.lru_cache(maxsize=None)
@@ -555,22 +558,36 @@ def _attention_bwd_launchers() -> dict:
             [LaunchConfig(f"attention_bwd_dkv_bf16_d128_{c}", 256, meta={"CAUSAL": c == "causal"},
                           lds_bytes=_ATTN_BWD_DKV_LDS) for c in ("causal", "full")],
         ),
+        "stats": mk("attention_bwd_stats_bf16_d128", "PPPPPi", [LaunchConfig("attention_bwd_stats_bf16_d128", 256)]),
+        **{
+            which: mk(
+                f"attention_bwd8_{which[:2]}_bf16_d128", "PPPPPPiif",
+                [LaunchConfig(f"attention_bwd8_{which[:2]}_bf16_d128_{c}", 512, meta={"CAUSAL": c == "causal"}, lds_bytes=lds)
+                 for c in ("causal", "full")],
+            )
+            for which, lds in (("dq8", _ATTN_BWD8_DQ_LDS), ("dk8", _ATTN_BWD8_DK_LDS), ("dv8", _ATTN_BWD8_DV_LDS))
+        },
     }
 
 
 def fused_attention_backward(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, dout: torch.Tensor,
-    softmax_max: torch.Tensor, softmax_sum: torch.Tensor, scale: float, causal: bool,
+    softmax_max: torch.Tensor, softmax_sum: torch.Tensor, scale: float, causal: bool, variant: Optional[str] = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """Gradients (dq, dk, dv) of fused_attention for [B, N, S, 128] bf16 tensors, S a multiple of
-    128; softmax_max / softmax_sum are the forward's [B, N, S, 8] fp32 statistics."""
+    """Gradients (dq, dk, dv) of fused_attention for [B, N, S, 128] bf16 tensors; softmax_max /
+    softmax_sum are the forward's [B, N, S, 8] fp32 statistics.  variant "w8" (default): workgroups
+    of eight wavefronts on 256 rows, separate dK and dV kernels, S a multiple of 64; "w4": four
+    wavefronts on 128 rows, dK and dV in one kernel, S a multiple of 128."""
     _check_cuda(q, k, v, out, dout, softmax_max, softmax_sum)
     for t in (q, k, v, out, dout):
         _require(t.dtype == torch.bfloat16 and t.dim() == 4 and t.shape == q.shape, "q, k, v, out, dout: one [B, N, S, D] bf16 shape")
         _require(t.is_contiguous() and _aligned(t), "q, k, v, out, dout must be contiguous and 16-byte aligned")
     B, N, S, D = q.shape
     _require(D == 128, "head dimension must be 128")
-    _require(S % 128 == 0 and S > 0, "sequence length must be a positive multiple of 128")
+    variant = variant or "w8"
+    _require(variant in ("w8", "w4"), "variant must be 'w8' or 'w4'")
+    step = 64 if variant == "w8" else 128
+    _require(S % step == 0 and S > 0, f"sequence length must be a positive multiple of {step}")
     for t in (softmax_max, softmax_sum):
         _require(t.dtype == torch.float32 and t.shape == (B, N, S, 8) and t.is_contiguous(), "statistics must be contiguous fp32 [B, N, S, 8]")
     _require(scale > 0 and math.isfinite(scale), "scale must be positive and finite")
@@ -581,9 +598,26 @@ def fused_attention_backward(
         return dq, dk, dv
     ls = _attention_bwd_launchers()
     st = _stream()
+    which = "causal" if causal else "full"
+    if variant == "w8":
+        stats = torch.empty(heads * S, 2, dtype=torch.float32, device=q.device)
+        ls["stats"]._launch(
+            _find(ls["stats"], "attention_bwd_stats_bf16_d128"),
+            (out.data_ptr(), dout.data_ptr(), softmax_max.data_ptr(), softmax_sum.data_ptr(), stats.data_ptr(), heads * S),
+            (cdiv(heads * S * 16, 256), 1, 1), st,
+        )
+        blocks = cdiv(S, 256)
+        grid = (8 * cdiv(heads, 8) * (cdiv(blocks, 2) if causal else blocks), 1, 1)  # causal: pairs of blocks
+        for name, dst in (("dk8", dk), ("dv8", dv), ("dq8", dq)):
+            l = ls[name]
+            l._launch(
+                _find(l, f"attention_bwd8_{name[:2]}_bf16_d128_{which}"),
+                (q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), stats.data_ptr(), dst.data_ptr(), heads, S, float(scale)),
+                grid, st,
+            )
+        return dq, dk, dv
     delta = torch.empty(heads * S, dtype=torch.float32, device=q.device)
     ls["delta"]._launch(_find(ls["delta"], "attention_bwd_delta_bf16_d128"), (out.data_ptr(), dout.data_ptr(), delta.data_ptr(), heads * S), (cdiv(heads * S * 16, 256), 1, 1), st)
-    which = "causal" if causal else "full"
     grid = (8 * cdiv(heads, 8) * (S // 128), 1, 1)
     ldq, ldkv = ls["dq"], ls["dkv"]
     ldkv._launch(

@@ -283,3 +283,78 @@ def test_copy_probe(K):
     dst = torch.zeros_like(src)
     K.copy_bytes(dst, src)
     assert torch.equal(dst, src)
+
+
+# ------------------------------------------------- autotune cache, bandwidth print
+# counterpart of the reference's cached autotune and .best_config record
+# (inductor_x/npu_triton_heuristics.py:302-393) and of its bandwidth print
+# (NPUDebugAutotuner, :268-299)
+def _gather_family(K, tmp_path, monkeypatch, variants):
+    from inductor_x_amd import codecache
+    from inductor_x_amd.hip_heuristics import CachingLauncher, LaunchConfig
+
+    cfgs = [LaunchConfig(f"gather_rows_b16_b{b}_t{t}_r{r}", b, meta={"BLOCK": b, "TPR": t, "RPT": r}) for b, t, r in variants]
+    fam = CachingLauncher(
+        "gather_rows", codecache.aot_source("copy_kernels.hip"), "PPPiii", cfgs,
+        bytes_fn=lambda table, idx, out, n, width, nrows: 2 * n * width * 2 + 8 * n, prefer_intree=True,
+    )
+    monkeypatch.setattr(fam, "_best_path", lambda: str(tmp_path / "gather_rows.best_config"))
+    return fam
+
+
+def test_autotune_winner_is_recorded_and_reused(K, tmp_path, monkeypatch):
+    import json
+
+    from inductor_x_amd import config
+    from inductor_x_amd.hip_heuristics import cdiv
+
+    announce("autotune record")
+    monkeypatch.setattr(config, "autotune", True)
+    torch.manual_seed(5)
+    table = torch.randn(4096, 1024, device=DEV).bfloat16()
+    idx = torch.randint(0, 4096, (8192,), device=DEV)
+    out = torch.empty(8192, 1024, dtype=torch.bfloat16, device=DEV)
+    args = (table.data_ptr(), idx.data_ptr(), out.data_ptr(), 8192, 1024, 4096)
+    grid = lambda meta: (cdiv(8192, (meta["BLOCK"] // meta["TPR"]) * meta["RPT"]), 1, 1)  # noqa: E731
+    variants = [(256, 128, 1), (256, 128, 2), (256, 64, 2), (256, 16, 4)]
+    stream = torch.cuda.current_stream().cuda_stream
+
+    fam = _gather_family(K, tmp_path, monkeypatch, variants)
+    fam.run(*args, grid=grid, stream=stream)
+    torch.cuda.synchronize()
+    assert torch.equal(out, table[idx])
+    rec = json.loads((tmp_path / "gather_rows.best_config").read_text())
+    assert rec["symbol"] == fam.best_config().symbol
+    assert set(rec["timings_ms"]) == {f"gather_rows_b16_b{b}_t{t}_r{r}" for b, t, r in variants}
+    assert rec["timings_ms"][rec["symbol"]] == min(rec["timings_ms"].values())
+
+    # a second launcher object (another process would look the same) reads the record and times nothing
+    again = _gather_family(K, tmp_path, monkeypatch, variants)
+    monkeypatch.setattr(again, "bench", lambda *a, **k: pytest.fail("timed again despite a valid record"))
+    out.zero_()
+    again.run(*args, grid=grid, stream=stream)
+    torch.cuda.synchronize()
+    assert again.best_config().symbol == rec["symbol"]
+    assert torch.equal(out, table[idx])
+
+    # a record made for another configuration list is not trusted
+    other = _gather_family(K, tmp_path, monkeypatch, variants[:3])
+    other.precompile()
+    assert other._best is None
+
+
+def test_bandwidth_print(K, tmp_path, monkeypatch, capsys):
+    from inductor_x_amd import config
+
+    announce("bandwidth print")
+    monkeypatch.setattr(config, "profile_bandwidth", True)
+    table = torch.randn(1024, 1024, device=DEV).bfloat16()
+    idx = torch.arange(1024, device=DEV)
+    out = torch.empty_like(table)
+    fam = _gather_family(K, tmp_path, monkeypatch, [(256, 128, 2)])
+    fam.run(table.data_ptr(), idx.data_ptr(), out.data_ptr(), 1024, 1024, 1024, grid=(256, 1, 1),
+            stream=torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    line = [l for l in capsys.readouterr().out.splitlines() if l.startswith("gather_rows:")]
+    assert len(line) == 1 and line[0].endswith("GB/s") and " ms " in line[0]
+    assert torch.equal(out, table)
