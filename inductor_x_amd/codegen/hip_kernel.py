@@ -462,6 +462,9 @@ class HipKernel(SIMDKernel):
         self._result_defs: list[str] = []
         self._result_defs_col: list[str] = []
         self.mode_decided = False
+        # register-tile transposition of loads whose contiguous axis is not the vector axis
+        self.tplan: Optional[dict] = None
+        self.tile_decls: list[str] = []
         super().__init__(tiling, **kwargs)
         self.n_reduction_phases = self._count_reduction_phases()
 
@@ -537,6 +540,8 @@ class HipKernel(SIMDKernel):
         rows.  None when the kernel does not have this shape or the sizes do not divide."""
         if self.mode != "pointwise" or self.vec <= 1 or os.environ.get("INDUCTOR_X_AMD_PW_TILE", "1") == "0":
             return None
+        if self.tplan:
+            return None
         ents = sorted(
             (e for e in self.x_entries if e.root.prefix == self.vec_tree_prefix), key=lambda e: int(e.divisor)
             if isinstance(e.divisor, (int, sympy.Integer)) else -1
@@ -590,6 +595,114 @@ class HipKernel(SIMDKernel):
         if t2 < 2 or L1 % t1 != 0 or xnumel % (L0 * L1 * L2) != 0:
             return None
         return {"L0": L0, "L1": L1, "L2": L2, "T1": t1, "T2": t2, "unroll": unroll, "cpt": cpt}
+
+    # -- transposed operands ----------------------------------------------------
+    _TPLAN_SHAPES = ((16, 16), (8, 32), (32, 8), (4, 64), (64, 4), (8, 16), (16, 8), (8, 8))
+
+    def _affine_parts(self, index: sympy.Expr) -> Optional[dict]:
+        """{symbol: integer coefficient} when the index is an integer-affine function of range
+        variables (and nothing else that varies), else None."""
+        idx = sympy.expand(index)
+        coeffs = {}
+        rest = idx
+        for s in idx.free_symbols:
+            if s not in self.range_tree_nodes:
+                return None
+            c = idx.coeff(s)
+            if not c.is_Integer:
+                return None
+            coeffs[s] = int(c)
+            rest = rest - c * s
+        rest = sympy.expand(rest)
+        if rest.free_symbols or not rest.is_Integer:
+            return None
+        return coeffs
+
+    def _transposed_axis(self, index: sympy.Expr) -> Optional[IterationRangesEntry]:
+        """For an index that strides along the vector axis but is contiguous along another kept
+        axis: the entry of that axis.  None for every other kind of index."""
+        coeffs = self._affine_parts(index)
+        if not coeffs:
+            return None
+        lane = [s for s in coeffs if self._is_lane_symbol(s)]
+        if len(lane) != 1 or coeffs[lane[0]] <= 1 or coeffs[lane[0]] % self.vec:
+            return None
+        unit = [s for s in coeffs if coeffs[s] == 1 and not self._is_lane_symbol(s)]
+        if len(unit) != 1:
+            return None
+        entry = self.range_tree_nodes[unit[0]]
+        lane_entry = self.range_tree_nodes[lane[0]]
+        if entry.root.prefix != self.vec_tree_prefix:
+            return None
+        try:
+            dk, lk, l0 = int(entry.divisor), int(entry.length), int(lane_entry.length)
+        except (TypeError, ValueError):
+            return None
+        if lk % self.vec or dk % l0:
+            return None
+        # stepping along the axis inside one vector must move no other variable of the index
+        for s in coeffs:
+            if s in (unit[0], lane[0]):
+                continue
+            e = self.range_tree_nodes[s]
+            try:
+                d, n = int(e.divisor), int(e.length)
+            except (TypeError, ValueError):
+                return None
+            if not (d >= dk * lk or d * n <= dk):
+                return None
+        return entry
+
+    def _transpose_plan(self, prepared: Sequence[sympy.Expr]) -> Optional[dict]:
+        """Thread tiles for a pointwise kernel that reads an operand transposed (the operand's
+        contiguous axis is another kept axis xk, not the vector axis x0).
+
+        A thread then owns VEC x VEC elements: VEC consecutive x0 times VEC consecutive xk.  The
+        transposed operand is read with VEC vector loads along xk (one per x0), everything else is
+        read and written with VEC vector accesses along x0 (one per xk), and the transposition is
+        register renaming in the fully unrolled loop over xk.  A wavefront covers 8 x 8 such
+        threads, so every load and store instruction moves runs of 8 x 16 bytes.  None when no
+        load has this shape, when two loads disagree on xk, or when the extents do not divide."""
+        if self.vec <= 1 or os.environ.get("INDUCTOR_X_AMD_PW_TRANSPOSE", "1") == "0":
+            return None
+        xnumel = self._static_numel(self.vec_tree_prefix)
+        if xnumel is None:
+            return None
+        axis = None
+        for idx in prepared:
+            e = self._transposed_axis(idx)
+            if e is None:
+                continue
+            if axis is not None and e.name != axis.name:
+                return None
+            axis = e
+        if axis is None:
+            return None
+        lane_lengths = []
+        for e in self.range_tree_nodes.values():
+            if e.root.prefix == self.vec_tree_prefix and e.divisor == 1:
+                try:
+                    lane_lengths.append(int(e.length))
+                except (TypeError, ValueError):
+                    return None
+        if not lane_lengths:
+            return None
+        l0 = min(lane_lengths)
+        dk, lk = int(axis.divisor), int(axis.length)
+        if any(n % l0 for n in lane_lengths) or dk % l0 or xnumel % (dk * lk) or l0 % self.vec:
+            return None
+        n0, nk = l0 // self.vec, lk // self.vec
+        for ti, tj in self._TPLAN_SHAPES:
+            if n0 % ti == 0 and nk % tj == 0:
+                wi = min(ti, 8)
+                wj = 64 // wi
+                if wj > tj:
+                    wj = tj
+                    wi = 64 // wj
+                if wi > ti or (ti * tj) % 64:
+                    continue
+                return {"axis": axis.name, "L0": l0, "DK": dk, "LK": lk, "TI": ti, "TJ": tj, "WI": wi, "WJ": wj}
+        return None
 
     def _tree(self, prefix: str):
         for t in self.range_trees:
@@ -662,6 +775,10 @@ class HipKernel(SIMDKernel):
                 self.vec_tree_prefix = "r0_"
         self._choose_vec(prepared)
         self._choose_geometry()
+        if self.mode == "pointwise":
+            self.tplan = self._transpose_plan(prepared)
+            if self.tplan:
+                self.block = self.tplan["TI"] * self.tplan["TJ"]
         self.mode_decided = True
 
     def persistent_reduction_blocks_col(self) -> bool:
@@ -925,6 +1042,26 @@ class HipKernel(SIMDKernel):
             else:
                 line = f"mi::gather_m({var}, {self.index_to_str(index)}, {mask}, {other})"
             is_vec = False
+        elif (
+            self.tplan and not indirect and mask is None and not self._load_mask
+            and (axis := self._transposed_axis(index)) is not None and axis.name == self.tplan["axis"]
+        ):
+            # VEC loads along the operand's own contiguous axis at the first step of the tile,
+            # one column of the register tile per step
+            coeffs = self._affine_parts(index)
+            stride = next(c for s_, c in coeffs.items() if self._is_lane_symbol(s_))
+            tname = f"tile{len(self.tile_decls)}"
+            self.tile_decls.append(f"mi::Tile<{DTYPE_TO_HIP[dtype]}, VEC> {tname};")
+            # at the first step the axis variable is a multiple of the vector width, like the lane variable
+            base = sympy_subs(index, {s_: sympy.Integer(0) for s_ in coeffs if self._is_lane_symbol(s_) or s_.name == axis.name})
+            try:
+                aligned = bool(V.graph.sizevars.statically_known_multiple_of(sympy.expand(base), self.vec))
+            except Exception:
+                aligned = False
+            fill = "tile_fill" if (aligned and self._buffer_aligned(name)) else "tile_fill_u"
+            self.loads.writeline(f"if (u == 0) mi::{fill}<VEC>({tname}, {var} + ({self.index_to_str(index)}), {stride});")
+            line = f"mi::tile_col<VEC>({tname}, u)"
+            is_vec = True
         else:
             idx = self.index_to_vec_str(index)
             line = f"mi::gather({var}, {idx})" if mask is None else f"mi::gather_m({var}, {idx}, {mask}, {other})"
@@ -1189,11 +1326,33 @@ class HipKernel(SIMDKernel):
             plist = ", ".join(params + [f"const {idx_t} xnumel"])
             src.writeline(f'extern "C" __global__ __launch_bounds__({self.block}) void {kname}({plist}) {{')
             tile = self.pointwise_tile_plan()
-            unroll = tile["unroll"] if tile else self.pointwise_unroll()
+            tp = self.tplan
+            unroll = self.vec if tp else (tile["unroll"] if tile else self.pointwise_unroll())
             with src.indent():
                 src.writeline(f"constexpr int VEC = {self.vec};")
                 src.writeline(f"constexpr int UNROLL = {unroll};")
-                if tile:
+                if tp:
+                    # thread -> VEC x VEC elements (x0 times the transposed operands' contiguous axis);
+                    # wavefront -> WI x WJ threads; workgroup -> TI x TJ threads; the rest of the index
+                    # space is walked by the workgroup id
+                    src.writeline(
+                        f"constexpr int L0 = {tp['L0']}, DK = {tp['DK']}, LK = {tp['LK']}, TI = {tp['TI']}, "
+                        f"TJ = {tp['TJ']}, WI = {tp['WI']}, WJ = {tp['WJ']};"
+                    )
+                    src.writeline("const int lane_ = threadIdx.x % 64, wave_ = threadIdx.x / 64;")
+                    src.writeline("const int tj_ = lane_ % WJ + WJ * (wave_ % (TJ / WJ));")
+                    src.writeline("const int ti_ = lane_ / WJ + WI * (wave_ / (TJ / WJ));")
+                    src.writeline(f"const {idx_t} wg_ = static_cast<{idx_t}>(blockIdx.x);")
+                    src.writeline(f"const {idx_t} t0_ = wg_ % (L0 / (VEC * TI));")
+                    src.writeline(f"const {idx_t} tk_ = (wg_ / (L0 / (VEC * TI))) % (LK / (VEC * TJ));")
+                    src.writeline(f"const {idx_t} rest_ = wg_ / ((L0 / (VEC * TI)) * (LK / (VEC * TJ)));")
+                    src.writeline(
+                        f"const {idx_t} xbase = (t0_ * TI + ti_) * VEC + static_cast<{idx_t}>(DK) * ((tk_ * TJ + tj_) * VEC) + "
+                        f"(rest_ % (DK / L0)) * L0 + (rest_ / (DK / L0)) * (static_cast<{idx_t}>(DK) * LK);"
+                    )
+                    for decl in self.tile_decls:
+                        src.writeline(decl)
+                elif tile:
                     # workgroup -> (T1 x T2) tile of the two axes above the innermost one; within the
                     # tile consecutive threads walk the innermost axis, then axis 2, then axis 1
                     t1, t2, cpt = tile["T1"], tile["T2"], tile["cpt"]
@@ -1212,7 +1371,9 @@ class HipKernel(SIMDKernel):
                 src.writeline("#pragma unroll")
                 src.writeline("for (int u = 0; u < UNROLL; ++u) {")
                 with src.indent():
-                    if tile:
+                    if tp:
+                        src.writeline(f"const {idx_t} xindex = xbase + static_cast<{idx_t}>(DK) * u;")
+                    elif tile:
                         src.writeline(f"const int e_ = u * {self.block} + static_cast<int>(threadIdx.x);")
                         src.writeline("const int row_ = e_ / CPT;")
                         src.writeline(

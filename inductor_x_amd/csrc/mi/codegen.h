@@ -268,6 +268,32 @@ __device__ __forceinline__ auto vload_u(const T* __restrict__ p) {
   }
 }
 
+// Register tile for an operand whose contiguous axis is not the kernel's vector axis.  Row e
+// holds the N elements that vector lane e needs over the N steps of the (fully unrolled) loop
+// along the operand's own contiguous axis: N contiguous loads `stride` elements apart fill it at
+// the first step, and step u takes column u, which is register renaming once u is a constant.
+template <class T, int N>
+struct Tile {
+  V<T, N> row[N];
+};
+template <int N, class T, class S>
+__device__ __forceinline__ void tile_fill(Tile<T, N>& t, const T* __restrict__ p, S stride) {
+#pragma unroll
+  for (int e = 0; e < N; ++e) t.row[e] = vload<N, T>(p + e * stride);
+}
+template <int N, class T, class S>
+__device__ __forceinline__ void tile_fill_u(Tile<T, N>& t, const T* __restrict__ p, S stride) {
+#pragma unroll
+  for (int e = 0; e < N; ++e) t.row[e] = vload_u<N, T>(p + e * stride);
+}
+template <int N, class T>
+__device__ __forceinline__ V<T, N> tile_col(const Tile<T, N>& t, int u) {
+  V<T, N> r;
+#pragma unroll
+  for (int e = 0; e < N; ++e) r.v[e] = t.row[e].v[u];
+  return r;
+}
+
 // Element-wise indexed load: idx scalar -> scalar, idx vector -> vector.
 template <class T, class I>
 __device__ __forceinline__ auto gather(const T* __restrict__ p, const I& idx) {

@@ -165,3 +165,37 @@ def test_sum_broadcast_permute_matrix(dim, perm):
 
     a, b = torch.randn(8, 16, 128, 64, device=DEV), torch.randn(8, 16, 128, 64, device=DEV)
     check(f, a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.int32])
+@pytest.mark.parametrize("shape", [(512, 1024), (128, 64), (3, 256, 384), (2, 5, 64, 128)])
+def test_inner_transpose_uses_register_tiles(shape, dtype):
+    """Swapping the two innermost axes: the operand is read along its own contiguous axis into
+    VEC x VEC register tiles (no element-wise gather) and the copy is bit-exact."""
+    announce(f"compile inner transpose {shape} {dtype}")
+    t = (torch.randn(*shape, device=DEV) * 100).to(dtype)
+    code = check(lambda t: t.transpose(-1, -2).contiguous(), t, exact=True)
+    assert "mi::Tile<" in code and "mi::gather(" not in code
+
+
+def test_transposed_operand_beside_contiguous_ones():
+    """One operand transposed, one in output order, one broadcast row, two outputs."""
+    announce("compile transposed operand + contiguous operands")
+
+    def f(a, b, row):
+        y = a.transpose(1, 2) * 2 + b
+        return y + row, torch.relu(y)
+
+    a = torch.randn(6, 256, 192, device=DEV)
+    b = torch.randn(6, 192, 256, device=DEV)
+    row = torch.randn(256, device=DEV)
+    code = check(f, a, b, row)
+    assert "mi::Tile<" in code
+
+
+@pytest.mark.parametrize("shape", [(50, 526, 129), (7, 33, 20), (8, 2048, 3)])
+def test_transpose_with_extents_no_vector_divides(shape):
+    """Extents that no vector width divides fall back to element-wise accesses and stay correct."""
+    announce(f"compile transpose odd {shape}")
+    t = torch.randn(*shape, device=DEV)
+    check(lambda t: t.transpose(-1, -2).contiguous() + 1, t)
