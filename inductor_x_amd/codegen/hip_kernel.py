@@ -412,6 +412,7 @@ REDUCTION_KIND = {
     "argmax": "mi::RedArgMax",
     "argmin": "mi::RedArgMin",
     "welford_reduce": "mi::RedWelford",
+    "welford_combine": "mi::RedMoments",
 }
 REDUCTION_WORDS = {"sum": 1, "prod": 1, "max": 1, "min": 1, "any": 1, "argmax": 2, "argmin": 2, "welford_reduce": 3}
 
@@ -746,14 +747,32 @@ class HipKernel(SIMDKernel):
             self.vec_tree_prefix = "x"
         else:
             r_unit = x_unit = 0
+            lane = sympy.Symbol("lane_", integer=True, nonnegative=True)
+
+            def innermost_of(prefix):
+                def f(s):
+                    e = self.range_tree_nodes.get(s)
+                    return e is not None and e.root.prefix == prefix and e.divisor == 1
+                return f
+
             for idx in prepared:
+                found = False
                 for s in self._unit_stride_symbols(idx):
                     entry = self.range_tree_nodes[s]
                     if entry.divisor != 1:
                         continue
                     if entry.root.prefix == "r0_":
                         r_unit += 1
+                        found = True
                     elif entry.root.prefix == "x":
+                        x_unit += 1
+                        found = True
+                if not found:
+                    # the innermost variable may sit inside a division or a remainder
+                    # ((r mod 512) + 32768 * (r div 512)): contiguous in pieces all the same
+                    if self._lane_delta(idx, lane, innermost_of("r0_"), 2) == lane:
+                        r_unit += 1
+                    elif self._lane_delta(idx, lane, innermost_of("x"), 2) == lane:
                         x_unit += 1
             if (
                 r_unit == 0
@@ -910,17 +929,19 @@ class HipKernel(SIMDKernel):
             return "uniform"
         return "gather"
 
-    def _lane_delta(self, expr: sympy.Expr, lane: sympy.Symbol) -> Optional[sympy.Expr]:
+    def _lane_delta(self, expr: sympy.Expr, lane: sympy.Symbol, is_lane=None, vec: Optional[int] = None) -> Optional[sympy.Expr]:
         """index(lane i) - index(lane 0) as an expression in `lane`, using what symbolic
         expansion cannot see: a lane-varying range variable is a multiple of the vector
         width at lane 0 and 0 <= lane < width, so floor((v + lane) / d) does not depend on the
         lane when the width divides d, and (v + lane) mod m moves with the lane when it
-        divides m.  None when the structure is not recognised."""
-        vec = self.vec
+        divides m.  None when the structure is not recognised.  is_lane / vec replace the
+        kernel's own lane symbols and vector width (used before those are chosen)."""
+        vec = self.vec if vec is None else vec
+        is_lane = is_lane or self._is_lane_symbol
         zero = sympy.Integer(0)
 
         def aligned(e: sympy.Expr) -> bool:
-            base = sympy.expand(sympy_subs(e, {s: zero for s in e.free_symbols if self._is_lane_symbol(s)}))
+            base = sympy.expand(sympy_subs(e, {s: zero for s in e.free_symbols if is_lane(s)}))
             if base == 0:
                 return True
             try:
@@ -930,7 +951,7 @@ class HipKernel(SIMDKernel):
 
         def rec(e: sympy.Expr) -> Optional[sympy.Expr]:
             if e.is_Symbol:
-                return lane if self._is_lane_symbol(e) else zero
+                return lane if is_lane(e) else zero
             if e.is_number:
                 return zero
             if isinstance(e, sympy.Add):
@@ -1161,12 +1182,31 @@ class HipKernel(SIMDKernel):
             raise UnsupportedHipCodegen(f"reduction {reduction_type}")
         if reduction_type in ("sum", "prod", "max", "min") and not src_dtype.is_floating_point and src_dtype != torch.bool:
             raise UnsupportedHipCodegen(f"integer {reduction_type} reduction")
-        if isinstance(value, tuple):
+        if isinstance(value, tuple) and reduction_type != "welford_combine":
             raise UnsupportedHipCodegen(f"tuple-valued reduction input for {reduction_type}")
         kind = REDUCTION_KIND[reduction_type]
         if self._load_mask:
             raise UnsupportedHipCodegen("reduction under a load mask")
         n = next(self.acc_ids)
+        if reduction_type == "welford_combine":
+            # inputs are (mean, m2, weight) per element: the second stage of a split variance
+            if self.mode != "row":
+                raise UnsupportedHipCodegen("welford_combine outside the row shape")
+            mean, m2, weight = value
+            merged_name = f"red{n}"
+            if self.persistent_reduction:
+                self.compute.writeline(
+                    f"const auto {merged_name} = mi::group_merge<{kind}, BLOCK, TPR>("
+                    f"mi::moments_step({kind}::init(), {mean}, {m2}, {weight}, rmask), lds_red);"
+                )
+            else:
+                acc = f"acc{n}"
+                self.prologue.writeline(f"mi::Moments {acc} = {kind}::init();")
+                self.compute.writeline(f"{acc} = mi::moments_step({acc}, {mean}, {m2}, {weight}, rmask);")
+                self.row_loop_accs.append(
+                    f"const auto {merged_name} = mi::group_merge<{kind}, BLOCK, TPR>({acc}, lds_red);"
+                )
+            return self._unpack_result(merged_name, reduction_type, dtype)
         if self.mode == "row":
             if self.persistent_reduction:
                 if reduction_type == "sum":
@@ -1217,7 +1257,7 @@ class HipKernel(SIMDKernel):
     def _unpack_result(self, merged: str, reduction_type: str, dtype: torch.dtype):
         if reduction_type in ("argmax", "argmin"):
             return self._result_var(f"static_cast<mi::i64>({merged}.i)", torch.int64)
-        if reduction_type == "welford_reduce":
+        if reduction_type in ("welford_reduce", "welford_combine"):
             return (
                 self._result_var(f"{merged}.mean", torch.float32),
                 self._result_var(f"{merged}.m2", torch.float32),

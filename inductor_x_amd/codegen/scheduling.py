@@ -43,11 +43,11 @@ class HipScheduling(SIMDScheduling):
 
     @classmethod
     def get_backend_features(cls, device: torch.device) -> OrderedSet[BackendFeature]:
-        # REDUCE_TO_SINGLE_ELEMENT: long reductions are not split at the IR level;
-        # the column kernel cuts the reduced axis across workgroups itself
-        # (the reference stubs Reduction.num_splits for the same purpose,
-        # reference inductor_x/codegen/ir.py:13-24).
-        return OrderedSet([BackendFeature.REDUCE_TO_SINGLE_ELEMENT, BackendFeature.TUPLE_REDUCTION])
+        # Whether a long reduction is split at the IR level is decided by the num_splits
+        # replacement in codegen/ir.py (only for a few outputs over a long range; the column
+        # kernel cuts the reduced axis across workgroups itself), so REDUCE_TO_SINGLE_ELEMENT,
+        # which would switch the split off everywhere, is not declared.
+        return OrderedSet([BackendFeature.TUPLE_REDUCTION])
 
     @classmethod
     def get_tiling_and_scores(cls, node_schedule, numel, reduction_numel=sympy.S.One, coalesce_analysis=None):

@@ -591,6 +591,37 @@ struct RedWelford {
   }
 };
 
+// Reduction whose inputs are moments already (the second stage of a variance that was split
+// into slices): the thread state is the merged moments.
+struct RedMoments {
+  typedef Moments T;
+  typedef Moments M;
+  static constexpr int W = 3;
+  __device__ static T init() { return RedWelford::empty(); }
+  __device__ static M finish(T s) { return s; }
+  __device__ static M empty() { return RedWelford::empty(); }
+  __device__ static M merge(M a, M b) { return moments_combine(a, b); }
+  __device__ static void enc(M m, float* w) { RedWelford::enc(m, w); }
+  __device__ static M dec(const float* w) { return RedWelford::dec(w); }
+};
+template <class V1, class V2, class V3, class MT>
+__device__ __forceinline__ Moments moments_step(Moments s, const V1& mean, const V2& m2, const V3& weight,
+                                                const MT& mask) {
+  constexpr int n = MaxN<Tr<V1>::n, Tr<V2>::n, Tr<V3>::n, Tr<MT>::n>::value == 0
+                        ? 1
+                        : MaxN<Tr<V1>::n, Tr<V2>::n, Tr<V3>::n, Tr<MT>::n>::value;
+#pragma unroll
+  for (int i = 0; i < n; ++i)
+    if (static_cast<bool>(at(mask, i))) {
+      Moments m;
+      m.n = static_cast<float>(at(weight, i));
+      m.mean = static_cast<float>(at(mean, i));
+      m.m2 = static_cast<float>(at(m2, i));
+      s = moments_combine(s, m);
+    }
+  return s;
+}
+
 // ---------------------------------------------------------------------------
 // row shape: reduce a thread's vector, then the TPR threads of the row
 // ---------------------------------------------------------------------------

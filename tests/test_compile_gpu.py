@@ -448,3 +448,38 @@ def test_attention_pattern_training():
     assert (out.float() - ref.float()).abs().max().item() <= 2e-2
     for a, t in zip(got, (qs, ks, vs)):
         assert (a.float() - t.grad.float()).abs().max().item() <= 3e-2 * max(t.grad.float().abs().max().item(), 1.0)
+
+
+@pytest.mark.parametrize("case", ["all", "rows", "outer_inner", "bf16"])
+def test_few_outputs_over_a_long_range(case):
+    """Fewer outputs than compute units, each over a long range: the reduction is split into
+    slices (two kernels: partials per slice, then a short second reduction) instead of running on
+    a handful of workgroups.  The reference never splits (inductor_x/codegen/ir.py:13-24); results
+    are the same sums, so the comparison with eager is the usual one."""
+    announce(f"compile split reduction {case}")
+    torch.manual_seed(0)
+    if case == "all":
+        x = torch.randn(8 * 1024 * 1024, device=DEV)
+        f = lambda t: (t.sum(), t.mean(), t.var(), t.amax())  # noqa: E731
+    elif case == "rows":
+        x = torch.randn(16, 1024 * 1024, device=DEV)
+        f = lambda t: (t.sum(-1), torch.var_mean(t, -1), t / t.abs().sum(-1, keepdim=True))  # noqa: E731
+    elif case == "outer_inner":
+        x = torch.randn(512, 64, 512, device=DEV)
+        f = lambda t: (t.sum([0, 2]), torch.var_mean(t, [0, 2]))  # noqa: E731
+    else:
+        x = torch.randn(8, 1024 * 1024, device=DEV).bfloat16()
+        f = lambda t: (t.float().mean(-1), t.float().amin(-1))  # noqa: E731
+    got, code = compile_and_code(f, x)
+    assert code.count("generated_kernel(") >= 2
+
+    def flat(o):
+        for v in o:
+            if isinstance(v, (tuple, list)):
+                yield from flat(v)
+            else:
+                yield v
+
+    ref = f(x.double()) if case != "bf16" else f(x)
+    for g, r in zip(flat(got), flat(ref)):
+        torch.testing.assert_close(g.double(), r.double(), rtol=1e-4, atol=1e-4)
