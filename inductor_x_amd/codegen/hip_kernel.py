@@ -825,6 +825,15 @@ class HipKernel(SIMDKernel):
             vec = 1
         while vec > 1 and not self._vec_ok(vec, numel):
             vec //= 2
+        # A row held in registers by more than 512 threads pays for its workgroup barriers (16
+        # wavefronts meet twice per reduction): two 16-byte pieces per thread halve the threads.
+        if (
+            self.mode == "row" and self.persistent_reduction and self.force_vec is None and numel is not None
+            and vec * dtype_nbytes(torch.float32) >= backend_config.vector_bytes // 4
+            and numel // max(vec, 1) > 512 and self._vec_ok(vec * 2, numel)
+            and os.environ.get("INDUCTOR_X_AMD_ROW_WIDE_VEC", "1") != "0"
+        ):
+            vec *= 2
         self.vec = vec
 
     def _vec_ok(self, vec: int, numel: Optional[int]) -> bool:
@@ -1214,6 +1223,21 @@ class HipKernel(SIMDKernel):
                         self.compute, f"mi::row_sum<BLOCK, TPR>({value}, rmask, lds_red)", dtype=torch.float32
                     )
                     return self._cast_result(merged, dtype)
+                if reduction_type == "welford_reduce":
+                    # the row is in registers: mean first, then the squared distances from it (the
+                    # two-pass definition itself, reference inductor_x/lowering.py:270-293), both as
+                    # plain sums
+                    mean = self.cse.generate(
+                        self.compute, f"mi::row_sum<BLOCK, TPR>({value}, rmask, lds_red) / static_cast<float>(rnumel)",
+                        dtype=torch.float32,
+                    )
+                    m2 = self.cse.generate(
+                        self.compute,
+                        f"mi::row_sum<BLOCK, TPR>(({value} - {mean}) * ({value} - {mean}), rmask, lds_red)",
+                        dtype=torch.float32,
+                    )
+                    weight = self.cse.generate(self.compute, "static_cast<float>(rnumel)", dtype=torch.float32)
+                    return (mean, m2, weight)
                 merged_name = f"red{n}"
                 self.compute.writeline(
                     f"const auto {merged_name} = mi::group_merge<{kind}, BLOCK, TPR>({kind}::finish("
@@ -1437,18 +1461,27 @@ class HipKernel(SIMDKernel):
                 src.writeline(f"constexpr int BLOCK = {self.block};")
                 src.writeline(f"constexpr int TPR = {self.tpr};")
                 src.writeline("__shared__ float lds_red[(BLOCK / 64) * 4];")
-                src.writeline(f"const {idx_t} xrow = static_cast<{idx_t}>(blockIdx.x) * (BLOCK / TPR) + threadIdx.x / TPR;")
-                src.writeline("const bool xmask = xrow < xnumel;")
-                src.writeline(f"const {idx_t} xindex = xmask ? xrow : xnumel - 1;")
                 src.writeline("const int rlane = threadIdx.x % TPR;")
-                if self.persistent_reduction:
-                    src.writeline(f"const {idx_t} r0_index = rlane * VEC;")
-                    src.writeline("const bool rmask = r0_index < rnumel;")
-                src.splice(self._entry_code(self.x_entries))
-                if self.persistent_reduction:
-                    src.splice(self._entry_code(self.r_entries))
-                src.splice(self.prologue)
-                src.splice(self.body)
+                # a workgroup walks the rows with the stride of the grid, so the launcher can cap the
+                # grid when there are many short rows (one workgroup per 4 KiB of input would be
+                # bound by the rate at which workgroups are dispatched)
+                src.writeline(
+                    f"for ({idx_t} xrow0 = static_cast<{idx_t}>(blockIdx.x) * (BLOCK / TPR); xrow0 < xnumel; "
+                    f"xrow0 += static_cast<{idx_t}>(gridDim.x) * (BLOCK / TPR)) {{"
+                )
+                with src.indent():
+                    src.writeline(f"const {idx_t} xrow = xrow0 + threadIdx.x / TPR;")
+                    src.writeline("const bool xmask = xrow < xnumel;")
+                    src.writeline(f"const {idx_t} xindex = xmask ? xrow : xnumel - 1;")
+                    if self.persistent_reduction:
+                        src.writeline(f"const {idx_t} r0_index = rlane * VEC;")
+                        src.writeline("const bool rmask = r0_index < rnumel;")
+                    src.splice(self._entry_code(self.x_entries))
+                    if self.persistent_reduction:
+                        src.splice(self._entry_code(self.r_entries))
+                    src.splice(self.prologue)
+                    src.splice(self.body)
+                src.writeline("}")
             src.writeline("}")
             sig = codes + idx_code + idx_code
             meta.update({"tpr": self.tpr, "persistent": bool(self.persistent_reduction)})

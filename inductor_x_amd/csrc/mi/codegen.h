@@ -213,7 +213,6 @@ MI_BINARY_FN(pow, ::powf(static_cast<float>(x), static_cast<float>(y)))
 MI_BINARY_FN(atan2, ::atan2f(static_cast<float>(x), static_cast<float>(y)))
 MI_BINARY_FN(fmod, ::fmodf(static_cast<float>(x), static_cast<float>(y)))
 MI_BINARY_FN(copysign, ::copysignf(static_cast<float>(x), static_cast<float>(y)))
-MI_BINARY_FN(truediv, static_cast<float>(x) / static_cast<float>(y))
 // Python-style integer floor division and modulo
 MI_BINARY_FN(floordiv, ((x / y) - ((x % y != 0) && ((x < 0) != (y < 0)) ? 1 : 0)))
 MI_BINARY_FN(pymod, (((x % y) != 0 && ((x % y) < 0) != (y < 0)) ? (x % y) + y : (x % y)))
@@ -227,6 +226,19 @@ MI_BINARY_FN(remainder_f, (::fmodf(static_cast<float>(x), static_cast<float>(y))
                                ? ::fmodf(static_cast<float>(x), static_cast<float>(y)) + static_cast<float>(y)
                                : ::fmodf(static_cast<float>(x), static_cast<float>(y))))
 #undef MI_BINARY_FN
+
+// Division.  A vector divided by a value that is uniform for the thread (a row sum, a norm)
+// takes one correctly rounded reciprocal and a multiplication per element (within one ulp of
+// the quotient); everything else is the IEEE division.
+template <class A, class B>
+__device__ __forceinline__ auto truediv(const A& a, const B& b) {
+  if constexpr (Tr<A>::n != 0 && Tr<B>::n == 0) {
+    const float inv = 1.0f / static_cast<float>(b);
+    return apply([inv](auto x) { return static_cast<float>(x) * inv; }, a);
+  } else {
+    return apply([](auto x, auto y) { return static_cast<float>(x) / static_cast<float>(y); }, a, b);
+  }
+}
 
 template <class A, class B, class C>
 __device__ __forceinline__ auto fma(const A& a, const B& b, const C& c) {
@@ -395,6 +407,7 @@ struct RedSum {
   __device__ static M merge(M a, M b) { return a + b; }
   __device__ static void enc(M m, float* w) { w[0] = m; }
   __device__ static M dec(const float* w) { return w[0]; }
+  typedef SumOp Op;
 };
 struct RedProd {
   typedef float T;
@@ -410,36 +423,65 @@ struct RedProd {
   __device__ static M merge(M a, M b) { return a * b; }
   __device__ static void enc(M m, float* w) { w[0] = m; }
   __device__ static M dec(const float* w) { return w[0]; }
+  struct Op {
+    __device__ __forceinline__ float operator()(float a, float b) const { return a * b; }
+  };
+};
+// The thread state of a maximum / minimum keeps "a NaN was seen" beside the running extremum of
+// the numbers (three instructions per element instead of the six of a NaN-propagating
+// comparison); the two are folded into one NaN-propagating value when the thread is done.
+struct ExtremumState {
+  float m, nan;
 };
 struct RedMax {
-  typedef float T;
+  typedef ExtremumState T;
   typedef float M;
   static constexpr int W = 1;
-  __device__ static T init() { return -__builtin_inff(); }
+  __device__ static T init() {
+    T t;
+    t.m = -__builtin_inff();
+    t.nan = 0.f;
+    return t;
+  }
   __device__ static T first(float v, int) { return step(init(), v, 0); }
   __device__ static T step_fast(T s, float v, int) { return step(s, v, 0); }
   __device__ static M finish_n(T s, float) { return finish(s); }
-  __device__ static T step(T s, float v, int) { return MaxOp()(s, v); }
-  __device__ static M finish(T s) { return s; }
+  __device__ static T step(T s, float v, int) {
+    s.m = __builtin_fmaxf(s.m, v);
+    s.nan = (v != v) ? 1.f : s.nan;
+    return s;
+  }
+  __device__ static M finish(T s) { return (s.nan != 0.f) ? __builtin_nanf("") : s.m; }
   __device__ static M empty() { return -__builtin_inff(); }
   __device__ static M merge(M a, M b) { return MaxOp()(a, b); }
   __device__ static void enc(M m, float* w) { w[0] = m; }
   __device__ static M dec(const float* w) { return w[0]; }
+  typedef MaxOp Op;
 };
 struct RedMin {
-  typedef float T;
+  typedef ExtremumState T;
   typedef float M;
   static constexpr int W = 1;
-  __device__ static T init() { return __builtin_inff(); }
+  __device__ static T init() {
+    T t;
+    t.m = __builtin_inff();
+    t.nan = 0.f;
+    return t;
+  }
   __device__ static T first(float v, int) { return step(init(), v, 0); }
   __device__ static T step_fast(T s, float v, int) { return step(s, v, 0); }
   __device__ static M finish_n(T s, float) { return finish(s); }
-  __device__ static T step(T s, float v, int) { return MinOp()(s, v); }
-  __device__ static M finish(T s) { return s; }
+  __device__ static T step(T s, float v, int) {
+    s.m = __builtin_fminf(s.m, v);
+    s.nan = (v != v) ? 1.f : s.nan;
+    return s;
+  }
+  __device__ static M finish(T s) { return (s.nan != 0.f) ? __builtin_nanf("") : s.m; }
   __device__ static M empty() { return __builtin_inff(); }
   __device__ static M merge(M a, M b) { return MinOp()(a, b); }
   __device__ static void enc(M m, float* w) { w[0] = m; }
   __device__ static M dec(const float* w) { return w[0]; }
+  typedef MinOp Op;
 };
 struct RedAny {
   typedef float T;
@@ -455,6 +497,9 @@ struct RedAny {
   __device__ static M merge(M a, M b) { return (a != 0.f || b != 0.f) ? 1.f : 0.f; }
   __device__ static void enc(M m, float* w) { w[0] = m; }
   __device__ static M dec(const float* w) { return w[0]; }
+  struct Op {
+    __device__ __forceinline__ float operator()(float a, float b) const { return (a != 0.f || b != 0.f) ? 1.f : 0.f; }
+  };
 };
 template <bool IS_MAX>
 struct RedArg {
@@ -642,11 +687,61 @@ __device__ __forceinline__ typename R::M wave_merge(typename R::M m) {
   return m;
 }
 
+template <class R, class = void>
+struct HasOp : std::false_type {};
+template <class R>
+struct HasOp<R, std::void_t<typename R::Op>> : std::true_type {};
+
+// Sums of K values per thread over the TPR threads of a row at once: DPP steps per value, one
+// round through LDS for rows wider than a wavefront.  lds: at least (BLOCK / 64) * K floats.
+template <int BLOCK, int TPR, int K>
+__device__ __forceinline__ void group_sums(float (&v)[K], float* lds) {
+  if constexpr (TPR <= kWave) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = wave_reduce<TPR>(v[k], SumOp());
+  } else {
+    constexpr int WPG = TPR / kWave;
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = wave_reduce<kWave>(v[k], SumOp());
+    const int wave = threadIdx.x / kWave;
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+#pragma unroll
+      for (int k = 0; k < K; ++k) lds[wave * K + k] = v[k];
+    }
+    __syncthreads();
+    const int src = (wave / WPG) * WPG + (threadIdx.x & (WPG - 1));
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = wave_reduce<WPG>(lds[src * K + k], SumOp());
+  }
+}
+
+// Moments of the union of the threads' samples by plain sums instead of pairwise merges: the
+// total count and mean first, then every thread's M2 moved to that mean.
+template <int BLOCK, int TPR>
+__device__ __forceinline__ Moments group_moments(Moments m, float* lds) {
+  float a[2] = {m.n, m.n * m.mean};
+  group_sums<BLOCK, TPR, 2>(a, lds);
+  Moments r;
+  r.n = a[0];
+  r.mean = (a[0] > 0.f) ? a[1] / a[0] : 0.f;
+  const float d = m.mean - r.mean;
+  float b[1] = {m.m2 + m.n * d * d};
+  group_sums<BLOCK, TPR, 1>(b, lds);
+  r.m2 = b[0];
+  return r;
+}
+
 // lds: at least (BLOCK / 64) * R::W floats.  All threads of the group receive
-// the result.
+// the result.  Reductions of one float with a plain binary operation and moments take the
+// DPP paths; only states that must travel as a whole (value + index) use the butterfly.
 template <class R, int BLOCK, int TPR>
 __device__ __forceinline__ typename R::M group_merge(typename R::M m, float* lds) {
-  if constexpr (TPR <= kWave) {
+  if constexpr (HasOp<R>::value) {
+    return group_reduce<BLOCK, TPR>(m, typename R::Op(), lds);
+  } else if constexpr (std::is_same<typename R::M, Moments>::value) {
+    return group_moments<BLOCK, TPR>(m, lds);
+  } else if constexpr (TPR <= kWave) {
     return wave_merge<R, TPR>(m);
   } else {
     constexpr int WPG = TPR / kWave;
@@ -660,11 +755,8 @@ __device__ __forceinline__ typename R::M group_merge(typename R::M m, float* lds
       for (int k = 0; k < R::W; ++k) lds[wave * R::W + k] = w[k];
     }
     __syncthreads();
-    const int first = (wave / WPG) * WPG;
-    typename R::M total = R::dec(lds + first * R::W);
-#pragma unroll
-    for (int j = 1; j < WPG; ++j) total = R::merge(total, R::dec(lds + (first + j) * R::W));
-    return total;
+    const int src = (wave / WPG) * WPG + (threadIdx.x & (WPG - 1));
+    return wave_merge<R, WPG>(R::dec(lds + src * R::W));
   }
 }
 

@@ -131,12 +131,13 @@ struct SumOp {
 struct MaxOp {
   // NaN-propagating maximum, as torch.max.
   __device__ __forceinline__ float operator()(float a, float b) const {
-    return (a != a) ? a : ((b != b) ? b : (a > b ? a : b));
+    // one maximum, one unordered compare, one select
+    return __builtin_isunordered(a, b) ? __builtin_nanf("") : __builtin_fmaxf(a, b);
   }
 };
 struct MinOp {
   __device__ __forceinline__ float operator()(float a, float b) const {
-    return (a != a) ? a : ((b != b) ? b : (a < b ? a : b));
+    return __builtin_isunordered(a, b) ? __builtin_nanf("") : __builtin_fminf(a, b);
   }
 };
 
@@ -174,11 +175,11 @@ __device__ __forceinline__ float group_reduce(float v, Op op, float* lds) {
     __syncthreads();
     if ((threadIdx.x & (kWave - 1)) == 0) lds[wave] = v;
     __syncthreads();
+    // lane j of every wavefront takes the partial of wavefront j of its group; the partials
+    // then meet in log2 steps inside 16 lanes (at most 16 wavefronts per workgroup)
+    static_assert(WAVES_PER_GROUP <= 16, "a workgroup has at most 16 wavefronts");
     const int first = (wave / WAVES_PER_GROUP) * WAVES_PER_GROUP;
-    float total = lds[first];
-#pragma unroll
-    for (int w = 1; w < WAVES_PER_GROUP; ++w) total = op(total, lds[first + w]);
-    return total;
+    return wave_reduce<WAVES_PER_GROUP>(lds[first + (threadIdx.x & (WAVES_PER_GROUP - 1))], op);
   }
 }
 

@@ -425,6 +425,20 @@ def split_factor(rows: int, cols: int, ct: int, rl: int, vec: int, elem_bytes: i
 _DRYRUN = os.environ.get("INDUCTOR_X_AMD_DRYRUN", "0") == "1"
 
 
+# Row kernels walk the rows with the stride of the grid.  Up to this many workgroups each
+# takes one round of rows; beyond it the grid is capped at a few workgroups per resident slot and
+# the workgroups loop (many short rows: dispatching one workgroup per round would be the bound).
+_ROW_GRID_FREE = 16384
+_ROW_GRID_WAVES_OF_WORKGROUPS = 4
+
+
+def row_grid(rounds: int) -> int:
+    if rounds <= _ROW_GRID_FREE or os.environ.get("INDUCTOR_X_AMD_ROW_GRID_CAP", "1") == "0":
+        return max(rounds, 1)
+    hw = config.hardware()
+    return min(rounds, hw.cu_count * 8 * int(os.environ.get("INDUCTOR_X_AMD_ROW_GRID_WAVES", _ROW_GRID_WAVES_OF_WORKGROUPS)))
+
+
 class GeneratedKernel:
     """Run-time side of one generated kernel: compiles (or fetches) its code
     object on first use and launches it through the C-ABI launcher.  This is the
@@ -472,7 +486,7 @@ class GeneratedKernel:
             grid = (cdiv(xnumel, m["block"] * m["vec"] * m.get("unroll", 1)), 1, 1)
             self._fns["main"].launch(m["signature"], raw + (xnumel,), grid, (m["block"],), stream)
         elif self.mode == "row":
-            grid = (cdiv(xnumel, m["block"] // m["tpr"]), 1, 1)
+            grid = (row_grid(cdiv(xnumel, m["block"] // m["tpr"])), 1, 1)
             self._fns["main"].launch(m["signature"], raw + (xnumel, rnumel), grid, (m["block"],), stream)
         else:
             import torch
