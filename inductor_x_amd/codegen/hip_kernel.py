@@ -1500,45 +1500,75 @@ class HipKernel(SIMDKernel):
         extra = [f"float* __restrict__ ws", f"const {idx_t} xnumel", f"const {idx_t} rnumel",
                  "const int rows_per_split", "const int nsplit"]
         plist = ", ".join(params + extra)
-        # ---- pass 1
-        src.writeline(f'extern "C" __global__ __launch_bounds__({ct * rl}) void {kname}_partial({plist}) {{')
-        with src.indent():
-            src.writeline(f"constexpr int VEC = {vec};")
-            src.writeline(f"constexpr int CT = {ct};")
-            src.writeline(f"constexpr int RL = {rl};")
-            src.writeline("extern __shared__ float lds_dyn[];")
-            src.writeline("const int ct = threadIdx.x % CT;")
-            src.writeline("const int rl = threadIdx.x / CT;")
-            src.writeline(f"const {idx_t} xindex = (static_cast<{idx_t}>(blockIdx.x) * CT + ct) * VEC;")
-            src.writeline("const int split = blockIdx.y;")
-            src.writeline("const bool xmask = xindex < xnumel;")
-            src.writeline(f"const {idx_t} r_begin = static_cast<{idx_t}>(split) * rows_per_split;")
-            src.writeline(f"const {idx_t} r_end = (r_begin + rows_per_split < rnumel) ? r_begin + rows_per_split : rnumel;")
-            for c in self.col_reductions:
-                kind = REDUCTION_KIND[c.kind]
-                src.writeline(f"mi::ColAcc<{kind}, VEC> {c.acc};")
-                src.writeline(f"{c.acc}.init();")
-            src.writeline("if (xmask) {")
+        # ---- pass 1, and the same sweep finishing in place ("direct") for launches where one
+        # workgroup per column tile already fills the GPU: no workspace, no second kernel
+        def sweep(suffix: str, direct: bool) -> None:
+            src.writeline(f'extern "C" __global__ __launch_bounds__({ct * rl}) void {kname}{suffix}({plist}) {{')
             with src.indent():
-                src.splice(self._entry_code(self.x_entries))
-                src.writeline(f"#pragma unroll {int(os.environ.get('INDUCTOR_X_AMD_COL_UNROLL', '4'))}")
-                src.writeline(f"for ({idx_t} r0_index = r_begin + rl; r0_index < r_end; r0_index += RL) {{")
+                src.writeline(f"constexpr int VEC = {vec};")
+                src.writeline(f"constexpr int CT = {ct};")
+                src.writeline(f"constexpr int RL = {rl};")
+                src.writeline("extern __shared__ float lds_dyn[];")
+                src.writeline("const int ct = threadIdx.x % CT;")
+                src.writeline("const int rl = threadIdx.x / CT;")
+                src.writeline(f"const {idx_t} xindex = (static_cast<{idx_t}>(blockIdx.x) * CT + ct) * VEC;")
+                src.writeline("const int split = blockIdx.y;")
+                src.writeline("const bool xmask = xindex < xnumel;")
+                src.writeline(f"const {idx_t} r_begin = static_cast<{idx_t}>(split) * rows_per_split;")
+                src.writeline(f"const {idx_t} r_end = (r_begin + rows_per_split < rnumel) ? r_begin + rows_per_split : rnumel;")
+                for c in self.col_reductions:
+                    kind = REDUCTION_KIND[c.kind]
+                    src.writeline(f"mi::ColAcc<{kind}, VEC> {c.acc};")
+                    src.writeline(f"{c.acc}.init();")
+                src.writeline("if (xmask) {")
                 with src.indent():
-                    src.splice(self.partial_body)
+                    src.splice(self._entry_code(self.x_entries))
+                    src.writeline(f"#pragma unroll {int(os.environ.get('INDUCTOR_X_AMD_COL_UNROLL', '4'))}")
+                    src.writeline(f"for ({idx_t} r0_index = r_begin + rl; r0_index < r_end; r0_index += RL) {{")
+                    with src.indent():
+                        src.splice(self.partial_body)
+                    src.writeline("}")
                 src.writeline("}")
+                for c in self.col_reductions:
+                    kind = REDUCTION_KIND[c.kind]
+                    src.writeline(f"typename {kind}::M {c.acc}_m[VEC];")
+                    src.writeline("#pragma unroll")
+                    src.writeline(f"for (int i = 0; i < VEC; ++i) {c.acc}_m[i] = {c.acc}.finish(i);")
+                    src.writeline(f"mi::col_fold<{kind}, VEC, CT, RL>({c.acc}_m, ct, rl, lds_dyn);")
+                    if not direct:
+                        src.writeline(
+                            f"if (rl == 0) mi::col_store_partial<{kind}, VEC>(ws + {c.ws_offset_words} * "
+                            f"static_cast<mi::i64>(nsplit) * xnumel, {c.acc}_m, xindex, xnumel, split, nsplit);"
+                        )
+                if direct:
+                    # the row lane that holds the folded states finishes its VEC columns one by one
+                    # with the text of the second kernel (one column per thread there)
+                    src.writeline("if (rl == 0 && xmask) {")
+                    with src.indent():
+                        src.writeline(f"const {idx_t} xfirst_ = xindex;")
+                        src.writeline("#pragma unroll")
+                        src.writeline("for (int col_ = 0; col_ < VEC; ++col_) {")
+                        with src.indent():
+                            src.writeline(f"const {idx_t} xindex = xfirst_ + col_;")
+                            src.writeline("if (xindex < xnumel) {")
+                            with src.indent():
+                                src.writeline("constexpr int VEC = 1;")
+                                src.writeline("const bool live = true;")
+                                src.writeline("const int sl = 0;")
+                                for c in self.col_reductions:
+                                    src.writeline(f"const auto {c.result} = {c.acc}_m[col_];")
+                                for line in self._result_defs_col:
+                                    src.writeline(line)
+                                src.splice(self._final_indexing_code())
+                                src.splice(self.final_body)
+                            src.writeline("}")
+                        src.writeline("}")
+                    src.writeline("}")
             src.writeline("}")
-            for c in self.col_reductions:
-                kind = REDUCTION_KIND[c.kind]
-                src.writeline(f"typename {kind}::M {c.acc}_m[VEC];")
-                src.writeline("#pragma unroll")
-                src.writeline(f"for (int i = 0; i < VEC; ++i) {c.acc}_m[i] = {c.acc}.finish(i);")
-                src.writeline(f"mi::col_fold<{kind}, VEC, CT, RL>({c.acc}_m, ct, rl, lds_dyn);")
-                src.writeline(
-                    f"if (rl == 0) mi::col_store_partial<{kind}, VEC>(ws + {c.ws_offset_words} * "
-                    f"static_cast<mi::i64>(nsplit) * xnumel, {c.acc}_m, xindex, xnumel, split, nsplit);"
-                )
-        src.writeline("}")
-        src.writeline("")
+            src.writeline("")
+
+        sweep("_partial", False)
+        sweep("_direct", True)
         # ---- pass 2
         cpw, sl = 16, 32
         src.writeline(f'extern "C" __global__ __launch_bounds__({cpw * sl}) void {kname}_final({plist}) {{')

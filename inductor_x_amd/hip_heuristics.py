@@ -425,10 +425,12 @@ def split_factor(rows: int, cols: int, ct: int, rl: int, vec: int, elem_bytes: i
 _DRYRUN = os.environ.get("INDUCTOR_X_AMD_DRYRUN", "0") == "1"
 
 
-# Row kernels walk the rows with the stride of the grid.  Up to this many workgroups each
-# takes one round of rows; beyond it the grid is capped at a few workgroups per resident slot and
-# the workgroups loop (many short rows: dispatching one workgroup per round would be the bound).
-_ROW_GRID_FREE = 16384
+# Row kernels walk the rows with the stride of the grid, so any grid is valid.  One workgroup per
+# round of rows is the rule: measured on MI355X, capping the grid (workgroups looping over rounds
+# far apart) gains under 5 % on plain short-row reductions and loses 25-50 % where the kernel also
+# writes a permuted output, because rows written close in time are then far apart in memory.  The
+# cap only keeps the grid dimension in range.
+_ROW_GRID_FREE = 1 << 22
 _ROW_GRID_WAVES_OF_WORKGROUPS = 4
 
 
@@ -464,7 +466,8 @@ class GeneratedKernel:
         with open(path, "rb") as f:
             mod = launcher.Module(f.read(), label=self.name)
         if self.mode == "col":
-            self._fns = {"partial": mod.function(self.name + "_partial"), "final": mod.function(self.name + "_final")}
+            self._fns = {"partial": mod.function(self.name + "_partial"), "final": mod.function(self.name + "_final"),
+                         "direct": mod.function(self.name + "_direct")}
         else:
             self._fns = {"main": mod.function(self.name)}
         self._module = mod
@@ -492,6 +495,13 @@ class GeneratedKernel:
             import torch
 
             nsplit, rps = split_factor(rnumel, xnumel, m["ct"], m["rl"], m["vec"], words=m["ws_words"])
+            if nsplit == 1:
+                # one sweep that finishes in place: no workspace, no second kernel
+                self._fns["direct"].launch(
+                    m["signature"], raw + (0, xnumel, rnumel, rnumel, 1), (cdiv(xnumel, m["ct"] * m["vec"]), 1, 1),
+                    (m["block"],), stream, m["lds_partial"],
+                )
+                return
             dev = next(a.device for a in args if hasattr(a, "device"))
             ws = torch.empty(m["ws_words"] * nsplit * xnumel, dtype=torch.float32, device=dev)
             full = raw + (ws.data_ptr(), xnumel, rnumel, rps, nsplit)
