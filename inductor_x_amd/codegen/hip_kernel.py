@@ -789,6 +789,16 @@ class HipKernel(SIMDKernel):
                 for t in self.range_trees:
                     if t.is_reduction:
                         t.is_loop = True
+            elif r_unit == 0 and x_unit > 0 and os.environ.get("INDUCTOR_X_AMD_COLLOOP", "1") != "0":
+                # the reduced axis is strided and the kept axis contiguous, but the column pair does
+                # not apply (values are used again after the reduction, or the reduced axis is
+                # short): one kernel, lanes along the kept axis, a loop over the reduced axis per phase
+                self.mode = "colloop"
+                self.vec_tree_prefix = "x"
+                self.persistent_reduction = False
+                for t in self.range_trees:
+                    if t.is_reduction:
+                        t.is_loop = True
             else:
                 self.mode = "row"
                 self.vec_tree_prefix = "r0_"
@@ -875,6 +885,20 @@ class HipKernel(SIMDKernel):
             else:
                 self.tpr = min(max(next_power_of_2(vectors), 1), 256)
             self.block = max(256, self.tpr)
+        elif self.mode == "colloop":
+            xnumel = self._static_numel("x")
+            rnumel = self._static_numel("r0_")
+            groups = max(-(-(xnumel or 512) // self.vec), 1)
+            self.col_ct = min(next_power_of_2(groups), 128)
+            rl = max(512 // self.col_ct, 1)
+            if rnumel is not None:
+                # at least eight rows per row lane: a short reduced axis is cheaper walked by fewer
+                # lanes (one lane: no LDS round at all) than folded across many
+                while rl > 1 and rl * 8 > rnumel:
+                    rl //= 2
+            self.col_rl = rl
+            self.block = max(self.col_ct * self.col_rl, 64)
+            self.col_rl = self.block // self.col_ct
         elif self.mode == "col":
             xnumel = self._static_numel("x")
             groups = max(-(-(xnumel or 512) // self.vec), 1)
@@ -1139,6 +1163,9 @@ class HipKernel(SIMDKernel):
             # inside the reduction loop only live columns run; afterwards (final
             # kernel) one of the SL lanes of a column stores
             mask = None if (self.inside_reduction and not self.phase_bodies_started) else "(live && sl == 0)"
+        elif self.mode == "colloop":
+            # inside a loop every row lane owns its rows; outside, one row lane stores per column
+            mask = "xmask" if self.inside_reduction else "(xmask && rl == 0)"
         else:
             mask = None
         if kind == "contiguous":
@@ -1164,6 +1191,16 @@ class HipKernel(SIMDKernel):
         """The reduced value is uniform for the row (or column); one thread writes it."""
         var = self.args.output(name)
         index = self.prepare_indexing(index)
+        if self.mode == "colloop":
+            # one value per column: a vector along the kept axis, written by the first row lane
+            if self.classify_index(index) == "contiguous":
+                line = f"mi::vstore_m<VEC>({var} + ({self.index_to_str(index)}), {value}, (xmask && rl == 0));"
+                if not (self.index_is_aligned(index) and self._buffer_aligned(name)):
+                    line = f"mi::scatter_m<VEC>({var}, {self.index_to_vec_str(index)}, {value}, (xmask && rl == 0));"
+            else:
+                line = f"mi::scatter_m<VEC>({var}, {self.index_to_vec_str(index)}, {value}, (xmask && rl == 0));"
+            self.red_stores.writeline(DeferredLine(name, line))
+            return
         guard = "(live && sl == 0)" if self.mode == "col" else "(xmask && rlane == 0)"
         line = f"if {guard} {{ mi::vstore<1>({var} + ({self.index_to_str(index)}), {value}); }}"
         self.red_stores.writeline(DeferredLine(name, line))
@@ -1199,9 +1236,23 @@ class HipKernel(SIMDKernel):
         n = next(self.acc_ids)
         if reduction_type == "welford_combine":
             # inputs are (mean, m2, weight) per element: the second stage of a split variance
-            if self.mode != "row":
-                raise UnsupportedHipCodegen("welford_combine outside the row shape")
             mean, m2, weight = value
+            if self.mode == "colloop":
+                acc = f"acc{n}"
+                self.prologue.writeline(f"mi::ColMomentsAcc<VEC> {acc};")
+                self.prologue.writeline(f"{acc}.init();")
+                self.compute.writeline(f"{acc}.step({mean}, {m2}, {weight});")
+                self.colloop_max_words = max(getattr(self, "colloop_max_words", 1), 3)
+                self.row_loop_accs.extend([
+                    f"mi::Moments {acc}_m[VEC];",
+                    "#pragma unroll",
+                    f"for (int i = 0; i < VEC; ++i) {acc}_m[i] = {acc}.finish(i);",
+                    f"mi::col_fold<{kind}, VEC, CT, RL>({acc}_m, ct, rl, lds_dyn);",
+                    f"mi::col_share<{kind}, VEC, CT, RL>({acc}_m, ct, rl, lds_dyn);",
+                ])
+                return self._unpack_result(f"{acc}_m", "welford_reduce", dtype)
+            if self.mode != "row":
+                raise UnsupportedHipCodegen("welford_combine outside the row and column-loop shapes")
             merged_name = f"red{n}"
             if self.persistent_reduction:
                 self.compute.writeline(
@@ -1254,6 +1305,20 @@ class HipKernel(SIMDKernel):
                     f"const auto {merged_name} = mi::group_merge<{kind}, BLOCK, TPR>({kind}::finish({acc}), lds_red);"
                 )
             return self._unpack_result(merged_name, reduction_type, dtype)
+        if self.mode == "colloop":
+            acc = f"acc{n}"
+            self.prologue.writeline(f"mi::ColAcc<{kind}, VEC> {acc};")
+            self.prologue.writeline(f"{acc}.init();")
+            self.compute.writeline(f"{acc}.step({value}, r0_index, true);")
+            self.colloop_max_words = max(getattr(self, "colloop_max_words", 1), REDUCTION_WORDS[reduction_type])
+            self.row_loop_accs.extend([
+                f"typename {kind}::M {acc}_m[VEC];",
+                "#pragma unroll",
+                f"for (int i = 0; i < VEC; ++i) {acc}_m[i] = {acc}.finish(i);",
+                f"mi::col_fold<{kind}, VEC, CT, RL>({acc}_m, ct, rl, lds_dyn);",
+                f"mi::col_share<{kind}, VEC, CT, RL>({acc}_m, ct, rl, lds_dyn);",
+            ])
+            return self._unpack_result(f"{acc}_m", reduction_type, dtype)
         if self.mode == "col":
             acc = f"acc{n}"
             merged_name = f"red{n}"
@@ -1279,6 +1344,22 @@ class HipKernel(SIMDKernel):
         return var
 
     def _unpack_result(self, merged: str, reduction_type: str, dtype: torch.dtype):
+        if self.mode == "colloop":
+            # `merged` is an array of VEC states, one per column of the thread: results are vectors
+            def vec_result(getter: str, dt: torch.dtype) -> CSEVariable:
+                var = self._result_var(f"mi::col_get<VEC>({merged}, mi::{getter}())", dt)
+                if isinstance(var, HipCSEVariable):
+                    var.is_vec = True
+                return var
+
+            if reduction_type in ("argmax", "argmin"):
+                return vec_result("GetIndex", torch.int64)
+            if reduction_type == "welford_reduce":
+                return (vec_result("GetMean", torch.float32), vec_result("GetM2", torch.float32),
+                        vec_result("GetCount", torch.float32))
+            if reduction_type == "any":
+                return vec_result("GetNonzero", torch.bool)
+            return vec_result("GetSelf", torch.float32)
         if reduction_type in ("argmax", "argmin"):
             return self._result_var(f"static_cast<mi::i64>({merged}.i)", torch.int64)
         if reduction_type in ("welford_reduce", "welford_combine"):
@@ -1320,6 +1401,27 @@ class HipKernel(SIMDKernel):
                 self.final_body.splice(self.compute)
                 self.final_body.splice(self.stores)
                 self.final_body.splice(self.red_stores)
+        elif self.mode == "colloop" and self.inside_reduction:
+            # one pass over the reduced axis, row lanes RL apart; the folds that follow hold
+            # barriers, so every thread runs the loop (threads past the end on clamped columns)
+            self.body.writeline(f"for ({self.index_dtype} r0_index = rl; r0_index < rnumel; r0_index += RL) {{")
+            with self.body.indent():
+                self.body.splice(self._entry_code(self.r_entries))
+                self.body.splice(self.loads)
+                self.body.splice(self.compute)
+                self.body.splice(self.stores)
+            self.body.writeline("}")
+            for line in self.row_loop_accs:
+                self.body.writeline(line)
+            self.row_loop_accs.clear()
+            for line in self._take_result_defs():
+                self.body.writeline(line)
+            self.body.splice(self.red_stores)
+            keep = OrderedSet()
+            for item in self.cse.reduction_cache.values():
+                for v in item if isinstance(item, tuple) else (item,):
+                    keep.add(v)
+            self.cse.invalidate(keep)
         elif self.mode == "row" and self.inside_reduction and not self.persistent_reduction:
             # one pass over the reduced axis
             self.body.writeline(
@@ -1485,6 +1587,28 @@ class HipKernel(SIMDKernel):
             src.writeline("}")
             sig = codes + idx_code + idx_code
             meta.update({"tpr": self.tpr, "persistent": bool(self.persistent_reduction)})
+        elif self.mode == "colloop":
+            ct, rl = self.col_ct, self.col_rl
+            words = getattr(self, "colloop_max_words", 1)
+            plist = ", ".join(params + [f"const {idx_t} xnumel", f"const {idx_t} rnumel"])
+            src.writeline(f'extern "C" __global__ __launch_bounds__({self.block}) void {kname}({plist}) {{')
+            with src.indent():
+                src.writeline(f"constexpr int VEC = {self.vec};")
+                src.writeline(f"constexpr int CT = {ct};")
+                src.writeline(f"constexpr int RL = {rl};")
+                src.writeline("extern __shared__ float lds_dyn[];")
+                src.writeline("const int ct = threadIdx.x % CT;")
+                src.writeline("const int rl = threadIdx.x / CT;")
+                src.writeline(f"const {idx_t} xraw = (static_cast<{idx_t}>(blockIdx.x) * CT + ct) * VEC;")
+                src.writeline("const bool xmask = xraw < xnumel;")
+                src.writeline(f"const {idx_t} xindex = xmask ? xraw : 0;")
+                src.splice(self._entry_code(self.x_entries))
+                src.splice(self.prologue)
+                src.splice(self.body)
+            src.writeline("}")
+            sig = codes + idx_code + idx_code
+            meta.update({"ct": ct, "rl": rl,
+                         "lds_bytes": max((rl // 2) * ct * self.vec * words * 4, ct * self.vec * words * 4)})
         else:  # col
             sig = self._codegen_col(src, kname, params, codes, idx_t, idx_code, meta)
         meta["signature"] = sig

@@ -813,6 +813,28 @@ struct ColAcc {
   }
 };
 
+// Per-thread: N independent columns whose inputs are moments already.
+template <int N>
+struct ColMomentsAcc {
+  Moments s[N];
+  __device__ __forceinline__ void init() {
+#pragma unroll
+    for (int i = 0; i < N; ++i) s[i] = RedWelford::empty();
+  }
+  template <class V1, class V2, class V3>
+  __device__ __forceinline__ void step(const V1& mean, const V2& m2, const V3& weight) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      Moments m;
+      m.n = static_cast<float>(at(weight, i));
+      m.mean = static_cast<float>(at(mean, i));
+      m.m2 = static_cast<float>(at(m2, i));
+      s[i] = moments_combine(s[i], m);
+    }
+  }
+  __device__ __forceinline__ Moments finish(int i) const { return s[i]; }
+};
+
 // Fold the RL row lanes of a workgroup (thread = rl * CT + ct).  lds holds
 // (RL / 2) * CT * N * R::W floats.  Afterwards threads with rl == 0 own the result.
 template <class R, int N, int CT, int RL>
@@ -844,6 +866,64 @@ __device__ __forceinline__ void col_fold(typename R::M (&m)[N], int ct, int rl, 
         }
       }
     }
+  }
+}
+
+// After col_fold: hand the folded states of row lane 0 to every row lane (same LDS area).
+template <class R, int N, int CT, int RL>
+__device__ __forceinline__ void col_share(typename R::M (&m)[N], int ct, int rl, float* lds) {
+  if constexpr (RL > 1) {
+    constexpr int PLANE = CT * N;
+    __syncthreads();
+    if (rl == 0) {
+#pragma unroll
+      for (int i = 0; i < N; ++i) {
+        float w[R::W];
+        R::enc(m[i], w);
+#pragma unroll
+        for (int k = 0; k < R::W; ++k) lds[k * PLANE + ct * N + i] = w[k];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      float w[R::W];
+#pragma unroll
+      for (int k = 0; k < R::W; ++k) w[k] = lds[k * PLANE + ct * N + i];
+      m[i] = R::dec(w);
+    }
+  }
+}
+
+// One field of N per-column states as a register vector.
+struct GetSelf {
+  template <class M>
+  __device__ __forceinline__ float operator()(const M& m) const { return m; }
+};
+struct GetMean {
+  __device__ __forceinline__ float operator()(const Moments& m) const { return m.mean; }
+};
+struct GetM2 {
+  __device__ __forceinline__ float operator()(const Moments& m) const { return m.m2; }
+};
+struct GetCount {
+  __device__ __forceinline__ float operator()(const Moments& m) const { return m.n; }
+};
+struct GetIndex {
+  __device__ __forceinline__ i64 operator()(const ArgVal& m) const { return static_cast<i64>(m.i); }
+};
+struct GetNonzero {
+  __device__ __forceinline__ bool operator()(float m) const { return m != 0.f; }
+};
+template <int N, class M, class G>
+__device__ __forceinline__ auto col_get(const M (&m)[N], G get) {
+  if constexpr (N == 1) {
+    return get(m[0]);
+  } else {
+    V<decltype(get(m[0])), N> r;
+#pragma unroll
+    for (int i = 0; i < N; ++i) r.v[i] = get(m[i]);
+    return r;
   }
 }
 

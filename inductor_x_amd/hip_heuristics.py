@@ -491,6 +491,9 @@ class GeneratedKernel:
         elif self.mode == "row":
             grid = (row_grid(cdiv(xnumel, m["block"] // m["tpr"])), 1, 1)
             self._fns["main"].launch(m["signature"], raw + (xnumel, rnumel), grid, (m["block"],), stream)
+        elif self.mode == "colloop":
+            grid = (cdiv(xnumel, m["ct"] * m["vec"]), 1, 1)
+            self._fns["main"].launch(m["signature"], raw + (xnumel, rnumel), grid, (m["block"],), stream, m["lds_bytes"])
         else:
             import torch
 

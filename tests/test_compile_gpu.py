@@ -483,3 +483,28 @@ def test_few_outputs_over_a_long_range(case):
     ref = f(x.double()) if case != "bf16" else f(x)
     for g, r in zip(flat(got), flat(ref)):
         torch.testing.assert_close(g.double(), r.double(), rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("r", [4, 8, 32, 48, 100])
+def test_short_strided_axis_reductions(r):
+    """Reductions over a short axis that is not the contiguous one (the kept axis is): one kernel
+    with the lanes along the kept axis and a loop over the reduced axis, no workspace."""
+    announce(f"compile strided-axis reductions r={r}")
+    torch.manual_seed(r)
+    t = torch.randn(96, r, 320, device=DEV)
+    t[3, r // 2, 7] = float("nan")
+    t[5, :, 9] = 2.5  # ties: argmax must give the first index
+    f = lambda t: (t.sum(1), torch.var_mean(t, 1), t.amax(1), t.argmax(1), t.amin(1))  # noqa: E731
+    got, code = compile_and_code(f, t)
+    if r > 8:  # shorter reductions are unrolled into a pointwise kernel by Inductor itself
+        assert "'mode': 'colloop'" in code or "'mode': 'col'" in code
+    ref = f(t)
+    torch.testing.assert_close(got[0], ref[0], rtol=1e-5, atol=1e-5, equal_nan=True)
+    torch.testing.assert_close(got[1][0], ref[1][0], rtol=1e-4, atol=1e-5, equal_nan=True)
+    torch.testing.assert_close(got[1][1], ref[1][1], rtol=1e-5, atol=1e-5, equal_nan=True)
+    torch.testing.assert_close(got[2], ref[2], rtol=0, atol=0, equal_nan=True)
+    assert torch.equal(got[3], ref[3])
+    torch.testing.assert_close(got[4], ref[4], rtol=0, atol=0, equal_nan=True)
+    tb = torch.randn(64, r, 256, device=DEV).bfloat16()
+    gb, _ = compile_and_code(lambda t: t.float().mean(1).bfloat16(), tb)
+    torch.testing.assert_close(gb, tb.float().mean(1).bfloat16(), rtol=0, atol=1e-2)
