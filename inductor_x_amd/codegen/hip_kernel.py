@@ -3,12 +3,17 @@
 Counterpart of the reference's kernel code generator
 (reference inductor_x/codegen/triton.py): where that file prints Triton text
 with N-D block indices, this one prints C++ against the hand-written template
-library in csrc/mi/codegen.h.  Three code shapes exist:
+library in csrc/mi/codegen.h.  Four code shapes exist:
 
-  pointwise  (reference family F1/F2, triton.py:693-815)    one 16-byte vector per thread
+  pointwise  (reference family F1/F2, triton.py:693-815)    one 16-byte vector per thread; VEC x VEC
+                                                            register tiles for transposed operands
   row        (F3/F4/F6, triton.py:1103-1262)                TPR threads per row, DPP + LDS combine
   column     (F5 + the outer-reduce hint, triton.py:1003-1031,
-              split_tiling.py:159-165)                      two-pass workgroup partials
+              split_tiling.py:159-165)                      two-pass workgroup partials, or one sweep
+                                                            finishing in place when no split is needed
+  colloop    (the same strides, short reduced axis or
+              values reused after the reduction)            one kernel, lanes along the kept axis, row
+                                                            lanes loop over the reduced axis per phase
 
 The shape is chosen from the strides of the accesses (which axis is the
 contiguous one), not from tags put on the IR node.

@@ -6,7 +6,7 @@
 // accepts any mix of the two, so the generator prints one expression per
 // Inductor op and lets overload resolution widen scalars where needed.
 //
-// Three code shapes are built from these pieces (they mirror the reference's
+// Four code shapes are built from these pieces (the first three mirror the reference's
 // pointwise / row-reduction / higher-order-reduction kernel bodies,
 // reference inductor_x/codegen/triton.py:693-815, 1103-1262):
 //   pointwise  one V per thread, 128-bit loads and stores where the index
@@ -15,7 +15,10 @@
 //              the row in a loop), results meet through DPP and LDS;
 //   column     every vector lane is its own output column, row lanes of the
 //              workgroup meet through LDS, slices of the reduced axis meet
-//              through a workspace and a second kernel.
+//              through a workspace and a second kernel (or not at all when one
+//              slice is enough);
+//   colloop    the column thread mapping in one kernel: a loop over the reduced
+//              axis per phase, folded states shared with every row lane.
 #pragma once
 
 #include <type_traits>
