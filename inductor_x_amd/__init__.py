@@ -26,13 +26,47 @@ def get_current_raw_stream(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
+def _backend_fingerprint() -> str:
+    """Hash of everything that decides what this backend generates: its Python sources, the
+    device headers and ahead-of-time kernel sources, and the INDUCTOR_X_AMD_* switches."""
+    import hashlib
+    import os
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    h = hashlib.sha256()
+    for root, dirs, files in os.walk(here):
+        dirs[:] = sorted(d for d in dirs if not d.startswith(("_hsaco", "__pycache__")))
+        for name in sorted(files):
+            if name.endswith((".py", ".h", ".hip", ".cpp")):
+                path = os.path.join(root, name)
+                h.update(os.path.relpath(path, here).encode())
+                with open(path, "rb") as f:
+                    h.update(f.read())
+    for key in sorted(os.environ):
+        if key.startswith("INDUCTOR_X_AMD_") and key not in ("INDUCTOR_X_AMD_CACHE",):
+            h.update(f"{key}={os.environ[key]}".encode())
+    return h.hexdigest()
+
+
 def _inductor_register_backend_for_device() -> None:
     from torch._inductor.codegen.common import register_backend_for_device
+    from torch._inductor.custom_graph_pass import CustomGraphModulePass
 
     from .codegen.scheduling import HipScheduling
     from .codegen.wrapper import HipWrapperCodegen
 
-    register_backend_for_device(DEVICE_TYPE, HipScheduling, HipWrapperCodegen)
+    class BackendFingerprint(CustomGraphModulePass):
+        """Changes no graph.  Inductor folds the uuid of a backend's custom pass into the keys of its
+        on-disk caches (compiled graphs, AOTAutograd artefacts), so entries written by other
+        sources of this package, or under other switches, are not served."""
+
+        def __call__(self, gm) -> None:
+            return None
+
+        def uuid(self):
+            return _backend_fingerprint()
+
+    register_backend_for_device(DEVICE_TYPE, HipScheduling, HipWrapperCodegen, device_custom_pass=BackendFingerprint())
 
 
 def _inductor_register_device_op_overrides() -> None:

@@ -263,27 +263,35 @@ def register_fx_pass() -> None:
     @init_once_fakemode
     def _init():
         device = "cuda" if torch.cuda.is_available() else "cpu"
-        g = functools.partial(torch.empty, (2, 4, 8, 16), device=device, dtype=torch.float)
         c = functools.partial(torch.tensor, 2.0, device=device, dtype=torch.float)
         pattern = partialize_and_update_signature(_attention_pattern_1, dropout_p=0.0)
         replacement = partialize_and_update_signature(_attention_replacement_1, dropout_p=0.0)
-        register_replacement(
-            pattern, replacement, [g(), g(), g(), c()], fwd_only, joint_graph.patterns,
-            extra_check=_extra_check, scalar_workaround={},
-        )
-        # training: the same search function traced with its backward; the replacement's
-        # autograd.Function supplies npu_fa_backward (reference :196-204, without dropout)
-        gr = functools.partial(torch.empty, (2, 4, 8, 16), device=device, dtype=torch.float, requires_grad=True)
-        register_replacement(
-            pattern, replacement, [gr(), gr(), gr(), c()], joint_fwd_bwd, joint_graph.patterns,
-            extra_check=_extra_check, scalar_workaround={},
-        )
+        # The search function is traced once per element type: a softmax of 16-bit tensors
+        # decomposes with conversions to fp32 and back that the fp32 trace does not contain, and
+        # bf16 is the type the kernels run (the reference traces fp32 only, :218-224).
+        for dtype in (torch.float, torch.bfloat16, torch.half):
+            g = functools.partial(torch.empty, (2, 4, 8, 16), device=device, dtype=dtype)
+            register_replacement(
+                pattern, replacement, [g(), g(), g(), c()], fwd_only, joint_graph.patterns,
+                extra_check=_extra_check, scalar_workaround={},
+            )
+            # training: the same search function traced with its backward; the replacement's
+            # autograd.Function supplies npu_fa_backward (reference :196-204, without dropout)
+            gr = functools.partial(torch.empty, (2, 4, 8, 16), device=device, dtype=dtype, requires_grad=True)
+            register_replacement(
+                pattern, replacement, [gr(), gr(), gr(), c()], joint_fwd_bwd, joint_graph.patterns,
+                extra_check=_extra_check, scalar_workaround={},
+            )
 
     original_lazy_init = joint_graph.lazy_init
 
     @functools.wraps(original_lazy_init)
     def lazy_init_with_attention():
-        original_lazy_init()
+        # before Inductor's own attention patterns: a pattern pass tries the entries for a node in
+        # the order of their registration, and Inductor's first pattern (the same products without
+        # the permutes) would otherwise claim the match for scaled_dot_product_attention.  The
+        # reference gets the same order by registering at import time (:233).
         _init()
+        original_lazy_init()
 
     joint_graph.lazy_init = lazy_init_with_attention

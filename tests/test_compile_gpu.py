@@ -203,8 +203,6 @@ def test_attention_op_and_pattern():
     """The custom op under torch.compile, and the graph pattern rewriting the
     unfused matmul-softmax-matmul into it."""
     announce("compile attention op / pattern")
-    from torch._dynamo.utils import counters
-
     from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
 
     torch.manual_seed(0)
@@ -226,14 +224,25 @@ def test_attention_op_and_pattern():
         q, k, v = (t.permute(0, 2, 1, 3) for t in (q, k, v))
         return torch.matmul(q, k.transpose(-2, -1)).div(inv_scale).softmax(dim=-1).matmul(v)
 
+    from torch._inductor.utils import run_and_get_code
+
     torch._dynamo.reset()
-    counters.clear()
-    # a hit in Inductor's on-disk graph cache would skip the pattern pass being counted
-    with torch.no_grad(), torch._inductor.config.patch(force_disable_caches=True):
-        out = torch.compile(g)(qs, ks, vs)
+    with torch.no_grad():
+        out, codes = run_and_get_code(torch.compile(g), qs, ks, vs)
     ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
     assert (out.float() - ref).abs().max().item() <= 2e-2
-    assert counters["inductor"]["fuse_attention"] >= 1
+    # the compiled graph calls the fused op, not the library's scaled_dot_product_attention that
+    # Inductor's own patterns would put there (the replacement counter also ticks while patterns
+    # are traced at registration, so the generated code is what is checked)
+    code = "\n".join(codes)
+    assert "npu_graph.npu_fa" in code and "_scaled_dot_product" not in code
+
+    # what the kernel cannot run (fp32) keeps Inductor's own rewrite
+    torch._dynamo.reset()
+    with torch.no_grad():
+        out32, codes = run_and_get_code(torch.compile(g), qs.float(), ks.float(), vs.float())
+    assert "npu_graph.npu_fa" not in "\n".join(codes)
+    assert (out32 - ref).abs().max().item() <= 2e-2
 
 
 def test_ring_attention_forward_update():
@@ -422,8 +431,6 @@ def test_attention_pattern_training():
     it to npu_fa / npu_fa_backward (reference inductor_x/npu_fusion_attention_graph.py:196-204), and
     the gradients agree with eager autograd to bf16 rounding."""
     announce("compile attention pattern, training")
-    from torch._dynamo.utils import counters
-
     torch.manual_seed(0)
     B, S, N, D = 2, 256, 4, 128
     qs, ks, vs = (torch.randn(B, S, N, D, device=DEV).bfloat16().requires_grad_() for _ in range(3))
@@ -433,13 +440,19 @@ def test_attention_pattern_training():
         q, k, v = (t.permute(0, 2, 1, 3) for t in (q, k, v))
         return torch.matmul(q, k.transpose(-2, -1)).div(inv).softmax(dim=-1).matmul(v)
 
+    from torch._inductor.utils import run_and_get_code
+
     torch._dynamo.reset()
-    counters.clear()
-    with torch._inductor.config.patch(force_disable_caches=True):
+    w = torch.randn(B, N, S, D, device=DEV).bfloat16()
+
+    def step():
         out = torch.compile(g)(qs, ks, vs)
-        w = torch.randn_like(out)
         (out * w).sum().backward()
-    assert counters["inductor"]["fuse_attention"] >= 1
+        return out
+
+    out, codes = run_and_get_code(step)
+    code = "\n".join(codes)
+    assert "npu_graph.npu_fa.default" in code and "npu_graph.npu_fa_backward" in code
     got = [t.grad.clone() for t in (qs, ks, vs)]
     for t in (qs, ks, vs):
         t.grad = None

@@ -199,3 +199,20 @@ def test_import_hook_keeps_cpu_inductor_working():
     )
     proc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600)
     assert proc.returncode == 0 and "ok" in proc.stdout, proc.stderr[-2000:]
+
+
+def test_backend_fingerprint_enters_inductor_cache_keys(monkeypatch):
+    """Inductor's on-disk caches are keyed on the uuid of the backend's custom pass: it must be
+    stable for unchanged sources and switches, and move with a code-generation switch."""
+    import inductor_x_amd
+    from torch._inductor.codegen.common import custom_backend_passes
+
+    p = custom_backend_passes.get(inductor_x_amd.DEVICE_TYPE)
+    assert p is not None
+    a = p.uuid()
+    assert a == p.uuid() and len(a) == 64
+    monkeypatch.setenv("INDUCTOR_X_AMD_PW_TRANSPOSE", "0")
+    assert p.uuid() != a
+    monkeypatch.delenv("INDUCTOR_X_AMD_PW_TRANSPOSE")
+    monkeypatch.setenv("INDUCTOR_X_AMD_CACHE", "/tmp/elsewhere")  # where code objects go does not change them
+    assert p.uuid() == a
