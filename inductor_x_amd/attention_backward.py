@@ -1,6 +1,6 @@
 """Backward of the fused attention forward (npu_graph::npu_fa_backward).
 
-Two paths.  Head dimension 128 with a sequence length that is a multiple of 128 runs the fused MFMA
+Two paths.  bf16 with head dimension 128 and a sequence length that is a multiple of 128 runs the fused MFMA
 kernels (kernels.fused_attention_backward, csrc/mi/attention_bwd_w8.h).  Other shapes run the matrix
 products as library GEMMs (torch.bmm, hipBLASLt underneath) on a bounded number of heads at a time
 and move O(S^2) intermediates through HBM.  Both recompute the probabilities from the forward's
@@ -12,7 +12,7 @@ l = softmax_sum as saved by the forward:
     D  = rowsum(dO * O)                     dS = P * (dP - D) * scale
     dQ = dS K                               dK = dS^T Q
 
-The probabilities and dS are rounded to bf16 before they enter a GEMM, as a fused kernel would do;
+The probabilities and dS are rounded to the operand type before they enter a GEMM, as a fused kernel would do;
 all reductions and the softmax algebra are fp32.  Counterpart of the reference's call into
 torch_npu.npu_fusion_attention_grad (reference inductor_x/npu_fusion_attention_graph.py:38-42).
 """
@@ -22,13 +22,57 @@ import torch
 
 # heads processed per round: bounds the fp32 [heads, S, S] intermediates (two live at a time)
 _SCORE_BYTES_BUDGET = 2 << 30
+_GEMM_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
+
+
+def _bmm_f32(a, b):
+    """Batched product with an fp32 result: fp32 accumulation output for 16-bit operands."""
+    if a.dtype == torch.float32:
+        return torch.bmm(a, b)
+    return torch.bmm(a, b, out_dtype=torch.float32)
+
+
+def attention_forward_over_gemms(q, k, v, scale: float, causal: bool):
+    """softmax(q k^T * scale [+ causal mask]) v with library GEMMs for shapes and element types the
+    fused forward kernels do not cover (any head dimension and sequence length; bf16, fp16, fp32).
+    Returns (out, softmax_max, softmax_sum) like kernels.fused_attention: the row statistics are
+    fp32 [B, N, S, 8], the probabilities are rounded to the operand type before the second product
+    and O(S^2) intermediates move through HBM, a bounded number of heads at a time."""
+    for t in (q, k, v):
+        if not (t.is_cuda and t.dtype in _GEMM_DTYPES and t.dtype == q.dtype and t.dim() == 4):
+            raise ValueError("attention forward: q, k, v must be 4-D GPU tensors of one floating-point type")
+    if not (q.shape == k.shape == v.shape):
+        raise ValueError("attention forward: q, k, v must share one [B, N, S, D] shape")
+    B, N, S, D = q.shape
+    heads = B * N
+    qh, kh, vh = (t.contiguous().view(heads, S, D) for t in (q, k, v))
+    out = torch.empty_like(qh)
+    smax = torch.empty(heads, S, dtype=torch.float32, device=q.device)
+    ssum = torch.empty(heads, S, dtype=torch.float32, device=q.device)
+    if heads and S:
+        chunk = max(1, min(heads, _SCORE_BYTES_BUDGET // max(2 * S * S * 4, 1)))
+        mask = torch.ones(S, S, dtype=torch.bool, device=q.device).triu_(1) if causal else None
+        for h0 in range(0, heads, chunk):
+            sl = slice(h0, min(h0 + chunk, heads))
+            s = _bmm_f32(qh[sl], kh[sl].transpose(1, 2)).mul_(scale)
+            if mask is not None:
+                s.masked_fill_(mask, float("-inf"))
+            m = s.amax(-1)
+            p = s.sub_(m.unsqueeze(-1)).exp_()
+            l = p.sum(-1)
+            smax[sl], ssum[sl] = m, l
+            out[sl] = (_bmm_f32(p.to(q.dtype), vh[sl]) / l.unsqueeze(-1)).to(q.dtype)
+    stats = lambda t: t.view(B, N, S, 1).expand(B, N, S, 8).contiguous()  # noqa: E731
+    return out.view(B, N, S, D), stats(smax), stats(ssum)
 
 
 def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale: float, causal: bool,
                              use_kernels=None):
-    """q, k, v, out, dout: [B, N, S, D] bf16; softmax_max / softmax_sum: [B, N, S, 8] fp32 from the
-    forward.  Returns (dq, dk, dv) in bf16.  use_kernels: None = fused kernels where they apply."""
-    fits = q.dim() == 4 and q.size(3) == 128 and q.size(2) % 128 == 0 and q.size(2) > 0
+    """q, k, v, out, dout: [B, N, S, D] of one floating-point type; softmax_max / softmax_sum:
+    [B, N, S, 8] fp32 from the forward.  Returns (dq, dk, dv) in that type.  use_kernels: None = fused
+    kernels where they apply (bf16, head dimension 128, sequence a multiple of 128)."""
+    fits = (q.dim() == 4 and q.dtype == torch.bfloat16 and q.size(3) == 128 and q.size(2) % 128 == 0
+            and q.size(2) > 0)
     if use_kernels is None:
         use_kernels = fits
     if use_kernels:
@@ -43,8 +87,8 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
 
 def _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale: float, causal: bool):
     for t in (q, k, v, out, dout):
-        if not (t.is_cuda and t.dtype == torch.bfloat16 and t.dim() == 4):
-            raise ValueError("attention backward: q, k, v, out, dout must be 4-D bf16 GPU tensors")
+        if not (t.is_cuda and t.dtype in _GEMM_DTYPES and t.dtype == q.dtype and t.dim() == 4):
+            raise ValueError("attention backward: q, k, v, out, dout must be 4-D GPU tensors of one floating-point type")
     if not (q.shape == k.shape == v.shape == out.shape == dout.shape):
         raise ValueError("attention backward: q, k, v, out, dout must share one [B, N, S, D] shape")
     B, N, S, D = q.shape
@@ -67,17 +111,17 @@ def _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale: fl
     for h0 in range(0, heads, chunk):
         sl = slice(h0, min(h0 + chunk, heads))
         qc, kc, vc, oc, doc = qh[sl], kh[sl], vh[sl], oh[sl], doh[sl]
-        s = torch.bmm(qc, kc.transpose(1, 2), out_dtype=torch.float32)
+        s = _bmm_f32(qc, kc.transpose(1, 2))
         # P = exp(S * scale - m) / l, masked entries exactly zero
         s.mul_(scale).sub_(m[sl].unsqueeze(-1))
         if mask is not None:
             s.masked_fill_(mask, float("-inf"))
         p = s.exp_().div_(l[sl].unsqueeze(-1))
-        p16 = p.to(torch.bfloat16)
+        p16 = p.to(q.dtype)
         dv[sl] = torch.bmm(p16.transpose(1, 2), doc)
-        dp = torch.bmm(doc, vc.transpose(1, 2), out_dtype=torch.float32)
+        dp = _bmm_f32(doc, vc.transpose(1, 2))
         delta = (doc.float() * oc.float()).sum(-1, keepdim=True)
-        ds16 = p.mul_(dp.sub_(delta)).mul_(scale).to(torch.bfloat16)
+        ds16 = p.mul_(dp.sub_(delta)).mul_(scale).to(q.dtype)
         dq[sl] = torch.bmm(ds16, kc)
         dk[sl] = torch.bmm(ds16.transpose(1, 2), qc)
     return dq.view(B, N, S, D), dk.view(B, N, S, D), dv.view(B, N, S, D)

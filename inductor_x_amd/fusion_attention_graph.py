@@ -81,9 +81,15 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
     # the graph pattern passes the divisor of the scores; the kernel multiplies
     real_scale = 1.0 / scale
     causal = _is_causal(query.size(2), atten_mask, pre_tockens, next_tockens, sparse_mode)
-    out, smax, ssum = kernels.fused_attention(
-        query.contiguous(), key.contiguous(), value.contiguous(), real_scale, causal
-    )
+    if query.dtype == torch.bfloat16 and query.size(3) == 128 and query.size(2) % 128 == 0 and query.size(2) > 0:
+        out, smax, ssum = kernels.fused_attention(
+            query.contiguous(), key.contiguous(), value.contiguous(), real_scale, causal
+        )
+    else:
+        # shapes and element types outside the fused kernels: the same mathematics over library GEMMs
+        from .attention_backward import attention_forward_over_gemms
+
+        out, smax, ssum = attention_forward_over_gemms(query, key, value, real_scale, causal)
     softmax_out = torch.empty([0], dtype=query.dtype, device=query.device)
     zero = lambda: torch.zeros([1], dtype=torch.int64)  # noqa: E731  seed / offset / numel: no dropout
     return out, smax, ssum, softmax_out, zero(), zero(), zero()

@@ -313,3 +313,36 @@ def test_attention_backward_vs_oracle(K, O, B, N, S, causal, variant):
     ref = O.attention_bwd(bits(q), bits(k), bits(v), bits(do), scale, causal)
     for g, r in zip(got, ref):
         assert np.abs(g.float().cpu().numpy() - r).max() <= 1e-2 * np.abs(r).max() + 1e-3
+
+
+@pytest.mark.parametrize("dtype,B,N,S,D,causal", [
+    (torch.float16, 2, 3, 200, 64, True), (torch.bfloat16, 1, 4, 96, 80, False), (torch.float32, 1, 2, 130, 32, True),
+    (torch.bfloat16, 1, 2, 192, 128, True),  # head dimension 128 but a sequence the forward kernels do not take
+])
+def test_attention_op_outside_the_fused_kernels(dtype, B, N, S, D, causal):
+    """npu_fa / npu_fa_backward for shapes and element types the MFMA kernels do not cover run the same
+    mathematics over library GEMMs: outputs and gradients against fp32 autograd of the unfused graph."""
+    announce(f"attention op over GEMMs {dtype} B={B} N={N} S={S} D={D} causal={causal}")
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
+    torch.manual_seed(12)
+    q, k, v = (torch.randn(B, N, S, D, device=DEV).to(dtype).requires_grad_() for _ in range(3))
+    do = torch.randn(B, N, S, D, device=DEV).to(dtype)
+    inv = D ** 0.5
+    res = npu_fusion_attention_graph(q, k, v, N, "BNSD", scale=inv, sparse_mode=3 if causal else 0)
+    out, smax, ssum = res[0], res[1], res[2]
+    out.backward(do)
+    got = (q.grad, k.grad, v.grad)
+    qf, kf, vf = (t.detach().float().requires_grad_() for t in (q, k, v))
+    s = (qf @ kf.transpose(-1, -2)) / inv
+    if causal:
+        s = s.masked_fill(torch.ones(S, S, device=DEV, dtype=torch.bool).triu(1), float("-inf"))
+    ref = torch.softmax(s, -1) @ vf
+    ref.backward(do.float())
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert out.dtype == dtype and (out.float() - ref).abs().max().item() <= tol * max(ref.abs().max().item(), 1.0)
+    assert smax.shape == (B, N, S, 8) and ssum.dtype == torch.float32
+    torch.testing.assert_close(smax[..., 0], s.amax(-1), rtol=1e-2, atol=1e-2)
+    for g, r in zip(got, (qf.grad, kf.grad, vf.grad)):
+        assert g.dtype == dtype
+        assert (g.float() - r).abs().max().item() <= (1e-4 if dtype == torch.float32 else 3e-2) * max(r.abs().max().item(), 1.0)
