@@ -697,6 +697,10 @@ class HipKernel(SIMDKernel):
         dk, lk = int(axis.divisor), int(axis.length)
         if any(n % l0 for n in lane_lengths) or dk % l0 or xnumel % (dk * lk) or l0 % self.vec:
             return None
+        # The output is contiguous over everything below xk (x0 and the axes between), so the
+        # tile's first direction walks that whole flat range, not just x0: a short innermost
+        # output axis (16 elements) still gets full 128-byte runs on the store side.
+        l0 = dk
         n0, nk = l0 // self.vec, lk // self.vec
         for ti, tj in self._TPLAN_SHAPES:
             if n0 % ti == 0 and nk % tj == 0:

@@ -199,3 +199,16 @@ def test_transpose_with_extents_no_vector_divides(shape):
     announce(f"compile transpose odd {shape}")
     t = torch.randn(*shape, device=DEV)
     check(lambda t: t.transpose(-1, -2).contiguous() + 1, t)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("perm", [(1, 3, 2, 0), (2, 3, 1, 0), (3, 1, 2, 0), (3, 2, 1, 0), (1, 2, 3, 0), (3, 0, 1, 2), (2, 0, 3, 1)])
+def test_permutations_with_a_short_innermost_output_axis(perm, dtype):
+    """Permuted copies whose output innermost axis is short (16 elements) or whose input
+    contiguous axis lands anywhere in the output: bit-exact, and no element-wise gather for the
+    permutations that move the input's contiguous axis outward."""
+    announce(f"compile permute{perm} {dtype}")
+    t = torch.randn(16, 32, 64, 128, device=DEV).to(dtype)
+    code = check(lambda t: t.permute(*perm).contiguous(), t, exact=True)
+    if perm[-1] != 3:
+        assert "mi::Tile<" in code
