@@ -702,17 +702,29 @@ class HipKernel(SIMDKernel):
         # output axis (16 elements) still gets full 128-byte runs on the store side.
         l0 = dk
         n0, nk = l0 // self.vec, lk // self.vec
+        # Workgroup shapes in order of preference (square first); tiles may hang over the end of
+        # either direction (threads past the end do nothing): take the shape that wastes the fewest
+        # threads, and no plan when even that leaves more than half of them idle (the element-wise
+        # fallback is four to eight times slower than a full tile, so a half-empty one still wins).
+        best = None
         for ti, tj in self._TPLAN_SHAPES:
-            if n0 % ti == 0 and nk % tj == 0:
-                wi = min(ti, 8)
-                wj = 64 // wi
-                if wj > tj:
-                    wj = tj
-                    wi = 64 // wj
-                if wi > ti or (ti * tj) % 64:
-                    continue
-                return {"axis": axis.name, "L0": l0, "DK": dk, "LK": lk, "TI": ti, "TJ": tj, "WI": wi, "WJ": wj}
-        return None
+            wi = min(ti, 8)
+            wj = 64 // wi
+            if wj > tj:
+                wj = tj
+                wi = 64 // wj
+            if wi > ti or (ti * tj) % 64:
+                continue
+            tiles_i, tiles_k = -(-n0 // ti), -(-nk // tj)
+            waste = (tiles_i * ti * tiles_k * tj) / float(n0 * nk)
+            if best is None or waste < best[0] - 1e-9:
+                best = (waste, ti, tj, wi, wj, tiles_i, tiles_k)
+        if best is None or best[0] > 2.0:
+            return None
+        _, ti, tj, wi, wj, tiles_i, tiles_k = best
+        rest = xnumel // (dk * lk)
+        return {"axis": axis.name, "L0": l0, "DK": dk, "LK": lk, "TI": ti, "TJ": tj, "WI": wi, "WJ": wj,
+                "tiles_i": tiles_i, "tiles_k": tiles_k, "grid": tiles_i * tiles_k * rest}
 
     def _tree(self, prefix: str):
         for t in self.range_trees:
@@ -1517,10 +1529,13 @@ class HipKernel(SIMDKernel):
                     src.writeline("const int lane_ = threadIdx.x % 64, wave_ = threadIdx.x / 64;")
                     src.writeline("const int tj_ = lane_ % WJ + WJ * (wave_ % (TJ / WJ));")
                     src.writeline("const int ti_ = lane_ / WJ + WI * (wave_ / (TJ / WJ));")
+                    src.writeline(f"constexpr int TILES_I = {tp['tiles_i']}, TILES_K = {tp['tiles_k']};")
                     src.writeline(f"const {idx_t} wg_ = static_cast<{idx_t}>(blockIdx.x);")
-                    src.writeline(f"const {idx_t} t0_ = wg_ % (L0 / (VEC * TI));")
-                    src.writeline(f"const {idx_t} tk_ = (wg_ / (L0 / (VEC * TI))) % (LK / (VEC * TJ));")
-                    src.writeline(f"const {idx_t} rest_ = wg_ / ((L0 / (VEC * TI)) * (LK / (VEC * TJ)));")
+                    src.writeline(f"const {idx_t} t0_ = wg_ % TILES_I;")
+                    src.writeline(f"const {idx_t} tk_ = (wg_ / TILES_I) % TILES_K;")
+                    src.writeline(f"const {idx_t} rest_ = wg_ / (TILES_I * TILES_K);")
+                    # tiles may hang over the end of either direction
+                    src.writeline("if ((t0_ * TI + ti_) * VEC >= L0 || (tk_ * TJ + tj_) * VEC >= LK) return;")
                     src.writeline(
                         f"const {idx_t} xbase = (t0_ * TI + ti_) * VEC + static_cast<{idx_t}>(DK) * ((tk_ * TJ + tj_) * VEC) + "
                         f"(rest_ % (DK / L0)) * L0 + (rest_ / (DK / L0)) * (static_cast<{idx_t}>(DK) * LK);"
@@ -1564,6 +1579,8 @@ class HipKernel(SIMDKernel):
             src.writeline("}")
             sig = codes + idx_code
             meta["unroll"] = unroll
+            if tp:
+                meta["grid"] = tp["grid"]
         elif self.mode == "row":
             plist = ", ".join(params + [f"const {idx_t} xnumel", f"const {idx_t} rnumel"])
             src.writeline(f'extern "C" __global__ __launch_bounds__({self.block}) void {kname}({plist}) {{')

@@ -486,7 +486,8 @@ class GeneratedKernel:
         m = self.meta
         raw = tuple(self._raw(a) for a in args)
         if self.mode == "pointwise":
-            grid = (cdiv(xnumel, m["block"] * m["vec"] * m.get("unroll", 1)), 1, 1)
+            # a tiled kernel (static shapes) carries its own workgroup count
+            grid = (m["grid"] if "grid" in m else cdiv(xnumel, m["block"] * m["vec"] * m.get("unroll", 1)), 1, 1)
             self._fns["main"].launch(m["signature"], raw + (xnumel,), grid, (m["block"],), stream)
         elif self.mode == "row":
             grid = (row_grid(cdiv(xnumel, m["block"] // m["tpr"])), 1, 1)
