@@ -270,15 +270,26 @@ __device__ __forceinline__ auto vload(const T* __restrict__ p) {
   }
 }
 
-// Contiguous run with no alignment guarantee.
+// Contiguous run aligned to its element only.  The access is still one wide instruction per 16
+// bytes: gfx950 under ROCm runs with unaligned global access enabled, and the compiler emits
+// global_load_dwordx4 / global_store_dwordx4 for an under-aligned aggregate of that size.
+template <class T, int N>
+struct __attribute__((packed, aligned(alignof(T)))) UnalignedRun {
+  T v[N];
+};
 template <int N, class T>
 __device__ __forceinline__ auto vload_u(const T* __restrict__ p) {
   if constexpr (N == 1) {
     return *p;
   } else {
+    constexpr int PER = (16 / sizeof(T)) < N ? (16 / sizeof(T)) : N;
     V<T, N> r;
 #pragma unroll
-    for (int i = 0; i < N; ++i) r.v[i] = p[i];
+    for (int c = 0; c < N / PER; ++c) {
+      const UnalignedRun<T, PER> t = *reinterpret_cast<const UnalignedRun<T, PER>*>(p + c * PER);
+#pragma unroll
+      for (int i = 0; i < PER; ++i) r.v[c * PER + i] = t.v[i];
+    }
     return r;
   }
 }
@@ -366,8 +377,18 @@ __device__ __forceinline__ void vstore(T* __restrict__ p, const A& val) {
 }
 template <int N, class T, class A>
 __device__ __forceinline__ void vstore_u(T* __restrict__ p, const A& val) {
+  if constexpr (N <= 1) {
+    p[0] = static_cast<T>(at(val, 0));
+  } else {
+    constexpr int PER = (16 / sizeof(T)) < N ? (16 / sizeof(T)) : N;
 #pragma unroll
-  for (int i = 0; i < (N < 1 ? 1 : N); ++i) p[i] = static_cast<T>(at(val, i));
+    for (int c = 0; c < N / PER; ++c) {
+      UnalignedRun<T, PER> t;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) t.v[i] = static_cast<T>(at(val, c * PER + i));
+      *reinterpret_cast<UnalignedRun<T, PER>*>(p + c * PER) = t;
+    }
+  }
 }
 template <int N, bool STREAM = false, class T, class A, class M>
 __device__ __forceinline__ void vstore_m(T* __restrict__ p, const A& val, const M& mask) {
