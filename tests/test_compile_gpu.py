@@ -521,3 +521,19 @@ def test_short_strided_axis_reductions(r):
     tb = torch.randn(64, r, 256, device=DEV).bfloat16()
     gb, _ = compile_and_code(lambda t: t.float().mean(1).bfloat16(), tb)
     torch.testing.assert_close(gb, tb.float().mean(1).bfloat16(), rtol=0, atol=1e-2)
+
+
+def test_benchmark_helper(capsys):
+    """The compiled-versus-eager timing helper (the reference's test scripts share one,
+    test/npu_indexing/utils.py:26-65): both clocks give positive times and a line is printed."""
+    announce("benchmark helper")
+    from inductor_x_amd.testing import benchmark_test
+
+    x = torch.randn(2048, 2048, device=DEV)
+    f = lambda x: torch.relu(x) * 2 + 1  # noqa: E731
+    torch._dynamo.reset()
+    cf = torch.compile(f)
+    for graph in (False, True):
+        eager_us, compiled_us = benchmark_test(f, cf, (x,), name="relu_affine", times=5, repeat=4, graph=graph)
+        assert eager_us > 0 and compiled_us > 0
+    assert capsys.readouterr().out.count("benchmark_relu_affine") == 2
