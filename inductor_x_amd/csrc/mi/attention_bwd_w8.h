@@ -43,6 +43,19 @@ constexpr int kBwd8DqLdsBytes = 2 * kBwd8DqBufBytes;
 constexpr int kBwd8DkLdsBytes = 2 * kBwd8DkBufBytes;
 constexpr int kBwd8DvLdsBytes = 2 * kBwd8DvBufBytes;
 constexpr float kBwd8Log2e = 1.4426950408889634f;
+// LDS fragments are read this many MFMA steps ahead in the unmasked loops (0: left to the compiler)
+#ifndef BWD8_PREFETCH
+#define BWD8_PREFETCH 2
+#endif
+#ifndef BWD8_PREFETCH_DK
+#define BWD8_PREFETCH_DK 2
+#endif
+#ifndef BWD8_PREFETCH_DK_CAUSAL
+#define BWD8_PREFETCH_DK_CAUSAL 0
+#endif
+#ifndef BWD8_PREFETCH_DV
+#define BWD8_PREFETCH_DV 0
+#endif
 
 // stats[row] = (m log2 e + log2 l, sum_d dO[row, d] * O[row, d]); 16 lanes per row.
 __device__ __forceinline__ void attention_bwd_stats(const bf16_t* __restrict__ O, const bf16_t* __restrict__ dO,
@@ -202,6 +215,59 @@ __device__ __forceinline__ void attention_bwd8_dq(const bf16_t* __restrict__ Q, 
     const bf16_t* Kt = Ks + 2 * kBwd8RowTile;
     const int key0 = tile * kAttnBN;
     bf16x8_t dsf[2][2];
+#if BWD8_PREFETCH > 0
+    if constexpr (!MASK) {
+    // The 32 MFMA steps of a tile (16 score / dP pairs, then 16 dQ updates) read their LDS
+    // fragments BWD8_PREFETCH steps ahead, across the boundaries between the phases, with the
+    // order pinned by scheduling fences: the softmax arithmetic of a key block then runs while
+    // the fragments of the next steps are already in flight.
+    constexpr int PF = BWD8_PREFETCH;
+    bf16x8_t ka[16], va[16], ta[16];
+    auto issue = [&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      if constexpr (i < 16) {
+        ka[i] = bwd8_row_frag(Ks, 32 * (i >> 3) + li, i & 7, g);
+        va[i] = bwd8_row_frag(Vs, 32 * (i >> 3) + li, i & 7, g);
+      } else if constexpr (i < 32) {
+        ta[i - 16] = bwd8_col_frag(Kt, 32 * ((i - 16) & 3) + li, (i - 16) >> 2, g);
+      }
+    };
+    static_for<PF>([&](auto ic) { issue(ic); });
+    f32x16_t sacc, pacc;
+    static_for<32>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      issue(std::integral_constant<int, i + PF>{});
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (i < 16) {
+        constexpr int kb = i >> 3, s_ = i & 7;
+        if constexpr (s_ == 0) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            sacc[r] = 0.f;
+            pacc[r] = 0.f;
+          }
+        }
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[i], qf[s_], sacc, 0, 0, 0);
+        pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[i], dof[s_], pacc, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (s_ == 7) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], c2, -m2));
+            if (MASK && key0 + 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3) > qi) p = 0.f;
+            dsf[kb][r >> 3][r & 7] = static_cast<bf16_t>(p * (pacc[r] - delta));
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        constexpr int j = i - 16, t = j >> 2, db = j & 3;
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta[j], dsf[t >> 1][t & 1], acc[db], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    });
+    return;
+    }
+#endif
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       f32x16_t sacc, pacc;
@@ -324,6 +390,72 @@ __device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q,
     const float* st = reinterpret_cast<const float*>(attn_lds + (tile & 1) * BUF + STAT_OFF);
     const int q0t = tile * kAttnBN;
     bf16x8_t bf[2][2];  // [query block][half]: P (dV) or dS (dK) as B operands, contraction over the queries
+    auto probabilities = [&](auto qbc, const f32x16_t& sacc, const f32x16_t& pacc) {
+      constexpr int qb = decltype(qbc)::value;
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        // rows 32 qb + 8 rq + 4 g + (0..3) of the query tile and their statistics
+        const int row0 = 32 * qb + 8 * rq + 4 * g;
+        const Vec<float, 4> sa = load_vec<float, 4>(st + 2 * row0);
+        const Vec<float, 4> sb = load_vec<float, 4>(st + 2 * row0 + 4);
+        const float mrow[4] = {sa[0], sa[2], sb[0], sb[2]};
+        const float drow[4] = {sa[1], sa[3], sb[1], sb[3]};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = 4 * rq + e;
+          float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], c2, -mrow[e]));
+          if (MASK && kj > q0t + row0 + e) p = 0.f;
+          if constexpr (DK)
+            bf[qb][r >> 3][r & 7] = static_cast<bf16_t>(p * (pacc[r] - drow[e]));
+          else
+            bf[qb][r >> 3][r & 7] = static_cast<bf16_t>(p);
+        }
+      }
+    };
+    // the causal dK kernel has no registers to spare for fragments in flight beyond one step
+    constexpr int PF = DK ? (CAUSAL ? BWD8_PREFETCH_DK_CAUSAL : BWD8_PREFETCH_DK) : BWD8_PREFETCH_DV;
+    if constexpr (PF > 0 && !MASK) {
+      // as in the dQ kernel: LDS fragments read PF steps ahead across the phases of the tile
+      bf16x8_t qa[16], da[DK ? 16 : 1], ta[16];
+      auto issue = [&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        if constexpr (i < 16) {
+          qa[i] = bwd8_row_frag(Qs, 32 * (i >> 3) + li, i & 7, g);
+          if constexpr (DK) da[i] = bwd8_row_frag(dOs, 32 * (i >> 3) + li, i & 7, g);
+        } else if constexpr (i < 32) {
+          ta[i - 16] = bwd8_col_frag(Tt, 32 * ((i - 16) & 3) + li, (i - 16) >> 2, g);
+        }
+      };
+      static_for<PF>([&](auto ic) { issue(ic); });
+      f32x16_t sacc, pacc;
+      static_for<32>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        issue(std::integral_constant<int, i + PF>{});
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (i < 16) {
+          constexpr int qb = i >> 3, s_ = i & 7;
+          if constexpr (s_ == 0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              sacc[r] = 0.f;
+              pacc[r] = 0.f;
+            }
+          }
+          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[i], kf[s_], sacc, 0, 0, 0);
+          if constexpr (DK) pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da[i], vf[s_], pacc, 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          if constexpr (s_ == 7) {
+            probabilities(std::integral_constant<int, qb>{}, sacc, pacc);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        } else {
+          constexpr int j = i - 16, t = j >> 2, db = j & 3;
+          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta[j], bf[t >> 1][t & 1], acc[db], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      });
+      return;
+    }
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
       f32x16_t sacc, pacc;
@@ -340,7 +472,6 @@ __device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q,
       }
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
-        // rows 32 qb + 8 rq + 4 g + (0..3) of the query tile and their statistics
         const int row0 = 32 * qb + 8 * rq + 4 * g;
         const Vec<float, 4> sa = load_vec<float, 4>(st + 2 * row0);
         const Vec<float, 4> sb = load_vec<float, 4>(st + 2 * row0 + 4);
