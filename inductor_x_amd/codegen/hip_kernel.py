@@ -1726,18 +1726,24 @@ class HipKernel(SIMDKernel):
             src.writeline("constexpr int VEC = 1;")
             src.writeline(f"constexpr int CPW = {cpw};")
             src.writeline(f"constexpr int SL = {sl};")
-            src.writeline(f"__shared__ float lds_fin[CPW * SL * {max_words}];")
+            src.writeline(f"__shared__ float lds_fin[CPW * SL * {sum(REDUCTION_WORDS[c.kind] for c in self.col_reductions)}];")
             src.writeline("const int slot = threadIdx.x % CPW;")
             src.writeline("const int sl = threadIdx.x / CPW;")
             src.writeline(f"const {idx_t} xraw = static_cast<{idx_t}>(blockIdx.x) * CPW + slot;")
             src.writeline("const bool live = xraw < xnumel;")
             src.writeline(f"const {idx_t} xindex = live ? xraw : xnumel - 1;")
+            # the loads of every reduction first, then the folds (each fold holds barriers)
             for c in self.col_reductions:
                 kind = REDUCTION_KIND[c.kind]
                 src.writeline(
-                    f"const auto {c.result} = mi::col_final<{kind}, CPW, SL>(ws + {c.ws_offset_words} * "
-                    f"static_cast<mi::i64>(nsplit) * xnumel, xindex, xnumel, nsplit, slot, sl, live, lds_fin);"
+                    f"const auto {c.result}_g = mi::col_final_gather<{kind}, SL>(ws + {c.ws_offset_words} * "
+                    f"static_cast<mi::i64>(nsplit) * xnumel, xindex, xnumel, nsplit, sl, live);"
                 )
+            for c in self.col_reductions:
+                src.writeline(f"auto {c.result} = {c.result}_g;")
+            kinds = ", ".join(REDUCTION_KIND[c.kind] for c in self.col_reductions)
+            states = ", ".join(c.result for c in self.col_reductions)
+            src.writeline(f"mi::col_final_fold_all<CPW, SL, {kinds}>(lds_fin, slot, sl, {states});")
             for line in self._result_defs_col:
                 src.writeline(line)
             src.splice(self._final_indexing_code())

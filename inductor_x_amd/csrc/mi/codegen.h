@@ -967,12 +967,13 @@ __device__ __forceinline__ void col_store_partial(float* __restrict__ ws, const 
   }
 }
 
-// Second pass for one column x: thread sl of SL folds splits sl, sl+SL, ...
-// (batched loads), then the SL lanes are folded through LDS (SL * W floats per
+// Second pass for one column x, in two steps so that a kernel with several reductions can have
+// the loads of all of them in flight before the first barrier: thread sl of SL merges splits
+// sl, sl+SL, ... (batched loads), then the SL lanes are folded through LDS (SL * W floats per
 // column slot; `slot` = the column's index inside the workgroup, CPW of them).
-template <class R, int CPW, int SL>
-__device__ __forceinline__ typename R::M col_final(const float* __restrict__ ws, i64 x, i64 xnumel, int nsplit,
-                                                   int slot, int sl, bool live, float* lds) {
+template <class R, int SL>
+__device__ __forceinline__ typename R::M col_final_gather(const float* __restrict__ ws, i64 x, i64 xnumel,
+                                                          int nsplit, int sl, bool live) {
   constexpr int BATCH = 8;  // with SL = 32 lanes per column: 256 partials in one round of loads
   const i64 plane = static_cast<i64>(nsplit) * xnumel;
   typename R::M m = R::empty();
@@ -991,6 +992,10 @@ __device__ __forceinline__ typename R::M col_final(const float* __restrict__ ws,
         if (s0 + b * SL < nsplit) m = R::merge(m, R::dec(w[b]));
     }
   }
+  return m;
+}
+template <class R, int CPW, int SL>
+__device__ __forceinline__ typename R::M col_final_fold(typename R::M m, int slot, int sl, float* lds) {
   constexpr int PLANE = CPW * SL;
   const int me = sl * CPW + slot;
   __syncthreads();
@@ -1015,6 +1020,55 @@ __device__ __forceinline__ typename R::M col_final(const float* __restrict__ ws,
     __syncthreads();
   }
   return m;  // valid where sl == 0
+}
+// The same fold for several reductions at once (one tree, one set of barriers): every state
+// has its own words in LDS, CPW * SL * (sum of R::W) floats in all.
+template <class R>
+struct RedTag {
+  typedef R type;
+};
+template <int CPW, int SL, class... R>
+__device__ __forceinline__ void col_final_fold_all(float* lds, int slot, int sl, typename R::M&... m) {
+  constexpr int PLANE = CPW * SL;
+  const int me = sl * CPW + slot;
+  auto put = [&](auto tag, auto& mm, int& off) {
+    typedef typename decltype(tag)::type RR;
+    float w[RR::W];
+    RR::enc(mm, w);
+#pragma unroll
+    for (int k = 0; k < RR::W; ++k) lds[(off + k) * PLANE + me] = w[k];
+    off += RR::W;
+  };
+  auto take = [&](auto tag, auto& mm, int& off, int half) {
+    typedef typename decltype(tag)::type RR;
+    float w[RR::W];
+#pragma unroll
+    for (int k = 0; k < RR::W; ++k) w[k] = lds[(off + k) * PLANE + (sl + half) * CPW + slot];
+    mm = RR::merge(mm, RR::dec(w));
+    off += RR::W;
+  };
+  __syncthreads();
+  {
+    int off = 0;
+    (put(RedTag<R>{}, m, off), ...);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int half = SL / 2; half >= 1; half >>= 1) {
+    if (sl < half) {
+      int off = 0;
+      (take(RedTag<R>{}, m, off, half), ...);
+      off = 0;
+      (put(RedTag<R>{}, m, off), ...);
+    }
+    __syncthreads();
+  }
+}
+
+template <class R, int CPW, int SL>
+__device__ __forceinline__ typename R::M col_final(const float* __restrict__ ws, i64 x, i64 xnumel, int nsplit,
+                                                   int slot, int sl, bool live, float* lds) {
+  return col_final_fold<R, CPW, SL>(col_final_gather<R, SL>(ws, x, xnumel, nsplit, sl, live), slot, sl, lds);
 }
 
 }  // namespace mi
