@@ -23,7 +23,8 @@ DEVICE_TYPE = "cuda"  # PyTorch-ROCm exposes AMD GPUs under this device type
 def get_current_raw_stream(device) -> int:
     """Raw hipStream_t of torch's current stream as an integer
     (reference inductor_x/__init__.py:26-27)."""
-    return torch.cuda.current_stream(device).cuda_stream
+    index = device if isinstance(device, int) else torch.device(device).index
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if index is None else index)
 
 
 def _backend_fingerprint() -> str:

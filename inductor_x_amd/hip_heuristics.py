@@ -19,6 +19,7 @@ aim is enough 16-byte loads in flight per CU to cover HBM latency.
 from __future__ import annotations
 
 import dataclasses
+import functools
 import hashlib
 import json
 import logging
@@ -295,6 +296,7 @@ class RowPlan:
     rows_per_wg: int
 
 
+@functools.lru_cache(maxsize=4096)
 def row_reduction_plan(xnumel: int, rnumel: int, elem_bytes: int, persistent: bool) -> RowPlan:
     """Thread mapping for a last-dimension reduction.
 
