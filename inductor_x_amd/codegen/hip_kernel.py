@@ -196,6 +196,11 @@ class HipOverrides(OpOverrides):
     def to_dtype(x, dtype: torch.dtype, src_dtype: Optional[torch.dtype] = None, use_compute_types: bool = True) -> str:
         if dtype == torch.bool:
             return f"({x} != 0)"
+        if not use_compute_types and dtype in (torch.float16, torch.bfloat16):
+            # Asked for when eager's intermediate roundings are to be emulated
+            # (torch/_inductor/lowering.py: emulate_precision_casts): round to
+            # the 16-bit type, then carry the rounded value in fp32 as usual.
+            return f"mi::cast<float>(mi::cast<{DTYPE_TO_HIP[dtype]}>({x}))"
         return f"mi::cast<{HipOverrides._compute_type(dtype)}>({x})"
 
     @staticmethod
@@ -224,16 +229,20 @@ class HipOverrides(OpOverrides):
         return var
 
     @staticmethod
-    def masked(mask, body, other) -> str:
+    def masked(mask, body, other):
         # Evaluate the body with loads guarded by the mask, then select.
         kernel: HipKernel = V.kernel
         with kernel.mask_loads(mask, other) as new_mask:
             result = body()
-        if isinstance(result, CSEVariable) and result.dtype is not None:
-            other_s = value_to_hip(other, result.dtype)
-        else:
-            other_s = value_to_hip(other)
-        return f"mi::where({new_mask}, {result}, {other_s})"
+        dtype = result.dtype if isinstance(result, CSEVariable) else None
+        if dtype is None:
+            dtype = torch.float32 if isinstance(other, float) else (torch.bool if isinstance(other, bool) else torch.int64)
+        other_s = value_to_hip(other, dtype)
+        # The caller reads dtype off the returned value, so it has to be a
+        # variable of the kernel, not an expression string.
+        var = kernel.cse.generate(kernel.compute, f"mi::where({new_mask}, {result}, {other_s})", dtype=dtype)
+        var.is_vec = any(isinstance(v, HipCSEVariable) and v.is_vec for v in (new_mask, result))
+        return var
 
     @staticmethod
     def where(a, b, c) -> str:
