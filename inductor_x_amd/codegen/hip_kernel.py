@@ -861,7 +861,7 @@ class HipKernel(SIMDKernel):
         if self.force_vec is not None:
             vec = self.force_vec
         numel = self._static_numel(self.vec_tree_prefix)
-        if numel is None:
+        if numel is None and self.mode != "pointwise":
             vec = 1
         while vec > 1 and not self._vec_ok(vec, numel):
             vec //= 2
@@ -877,7 +877,13 @@ class HipKernel(SIMDKernel):
         self.vec = vec
 
     def _vec_ok(self, vec: int, numel: Optional[int]) -> bool:
-        if numel is None or numel % vec:
+        if numel is None:
+            # a size known only at run time (a dynamic batch of fixed-width rows, say) still
+            # takes whole vectors when it is provably a multiple of the width
+            tree = self._tree(self.vec_tree_prefix)
+            if tree is None or not self._multiple_of(tree.numel, vec):
+                return False
+        elif numel % vec:
             return False
         for entry in self.range_tree_nodes.values():
             if entry.root.prefix != self.vec_tree_prefix:
@@ -887,14 +893,21 @@ class HipKernel(SIMDKernel):
         return True
 
     @staticmethod
-    def _entry_fits_vec(entry: IterationRangesEntry, vec: int) -> bool:
-        div, length = entry.divisor, entry.length
-        if not isinstance(div, (int, sympy.Integer)) or not isinstance(length, (int, sympy.Integer)):
-            return vec == 1
-        div, length = int(div), int(length)
-        if div == 1:
-            return length % vec == 0
-        return div % vec == 0
+    def _multiple_of(expr: Any, vec: int) -> bool:
+        if isinstance(expr, (int, sympy.Integer)):
+            return int(expr) % vec == 0
+        try:
+            return bool(V.graph.sizevars.statically_known_multiple_of(expr, vec))
+        except Exception:
+            return False
+
+    @classmethod
+    def _entry_fits_vec(cls, entry: IterationRangesEntry, vec: int) -> bool:
+        if vec == 1:
+            return True
+        if isinstance(entry.divisor, (int, sympy.Integer)) and int(entry.divisor) == 1:
+            return cls._multiple_of(entry.length, vec)
+        return cls._multiple_of(entry.divisor, vec)
 
     def _choose_geometry(self) -> None:
         from ..hip_heuristics import next_power_of_2
@@ -1510,6 +1523,11 @@ class HipKernel(SIMDKernel):
 
     def codegen_kernel(self, name: Optional[str] = None) -> str:
         self.codegen_body()
+        # Size symbols in the range variables' definitions become kernel
+        # arguments the first time they are renamed: do that before the
+        # parameter list is taken.
+        for entry in (*self.x_entries, *self.r_entries):
+            self.rename_indexing(entry.expr)
         params, codes, _ = self._signature()
         idx_t = self.index_dtype
         idx_code = "i" if idx_t == "int" else "q"

@@ -102,3 +102,53 @@ def test_operator_kinds(name):
             torch.testing.assert_close(g, r, equal_nan=True, **tol)
         else:
             assert torch.equal(g, r)
+
+
+def _compare(got, ref, name=""):
+    got = got if isinstance(got, (tuple, list)) else (got,)
+    ref = ref if isinstance(ref, (tuple, list)) else (ref,)
+    assert len(got) == len(ref)
+    for g, r in zip(got, ref):
+        assert g.shape == r.shape and g.dtype == r.dtype, (name, g.shape, r.shape, g.dtype, r.dtype)
+        if r.dtype.is_floating_point:
+            torch.testing.assert_close(g, r, equal_nan=True, rtol=2e-2, atol=2e-2 * max(1.0, float(r.abs().max())))
+        else:
+            assert torch.equal(g, r), name
+
+
+@pytest.mark.parametrize("name", sorted(set(CASES) - {"dropout_eval_rand_like_shape"}))
+def test_operator_kinds_symbolic_sizes(name):
+    """The same graphs with every size symbolic: sizes reach the kernels as arguments
+    (reference inductor_x/codegen/wrapper.py:21-38 passes the numels the same way)."""
+    announce(f"compile op sweep, dynamic=True: {name}")
+    fn, make = CASES[name]
+    args = make()
+    torch._dynamo.reset()
+    got = torch.compile(fn, dynamic=True)(*args)
+    _compare(got, fn(*args), name)
+
+
+def test_dynamic_batch_keeps_vectors():
+    """Only the leading size is dynamic: rows of fixed width still move as whole vectors
+    (the symbolic element count is provably a multiple of the width), and one artefact
+    serves every batch."""
+    announce("compile dynamic batch, vector width")
+    from torch._inductor.utils import run_and_get_code
+
+    def f(a, b):
+        return torch.relu(a) * 2 + b, torch.softmax(a, -1), (a * b).permute(0, 2, 1).contiguous()
+
+    torch._dynamo.reset()
+    a, b = _t(24, 40, 256), _t(24, 40, 256, seed=1)
+    for t in (a, b):
+        torch._dynamo.mark_dynamic(t, 0)
+    cf = torch.compile(f)
+    got, codes = run_and_get_code(cf, a, b)
+    _compare(got, f(a, b))
+    import re
+
+    widths = [int(m) for m in re.findall(r"'vec': (\d+)", codes[0])]
+    assert widths and min(widths) >= 4, widths
+    for batch in (7, 100, 1):
+        a, b = _t(batch, 40, 256, seed=2), _t(batch, 40, 256, seed=3)
+        _compare(cf(a, b), f(a, b))
