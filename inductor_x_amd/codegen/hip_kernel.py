@@ -785,7 +785,17 @@ class HipKernel(SIMDKernel):
                     return e is not None and e.root.prefix == prefix and e.divisor == 1
                 return f
 
-            for idx in prepared:
+            # An index that moves along one of the two axes only (a per-row statistic in a sum
+            # over rows, a weight vector in a sum over columns) touches a sliver of what the
+            # two-axis indices touch: when both kinds occur, the two-axis ones decide.
+            def trees_of(idx):
+                return {self.range_tree_nodes[s].root.prefix for s in idx.free_symbols if s in self.range_tree_nodes}
+
+            if any(len(trees_of(idx)) > 1 for idx in prepared):
+                deciding = [idx for idx in prepared if len(trees_of(idx)) > 1]
+            else:
+                deciding = list(prepared)
+            for idx in deciding:
                 found = False
                 for s in self._unit_stride_symbols(idx):
                     entry = self.range_tree_nodes[s]

@@ -67,6 +67,11 @@ CASES = {
     "complex_broadcast_5d": (lambda a, b, c: a[:, :, None] * b[None, :, :, None, :] + c, lambda: (_t(3, 4, 5, 6), _t(4, 1, 6), _t(1, 1, 7, 5, 6))),
     "var_std_norm": (lambda a: (a.var(-1), a.std(0), a.norm(dim=-1), torch.linalg.vector_norm(a, ord=1, dim=0)), lambda: (_t(65, 130),)),
     "bf16_chain": (lambda a, b: (F.silu(a) * b + a).to(torch.bfloat16).float().sum(-1), lambda: (_t(64, 512, dtype=torch.bfloat16), _t(64, 512, dtype=torch.bfloat16))),
+    # reference test/npu_indexing/test_AddLayerNorm.py:95-100 at (64, 512, 256), scaled down
+    "add_layernorm_by_hand": (lambda a, b: (lambda x, m: (x - m) / torch.sqrt(((x - m) ** 2).mean(2, keepdim=True) + 1e-5))(a + b, (a + b).mean(2, keepdim=True)),
+                              lambda: (_t(16, 128, 256), _t(16, 128, 256, seed=1))),
+    # reference test/npu_indexing/test_sum.py:94-105: a one-row sum with a broadcast scalar operand
+    "one_row_sum_broadcast": (lambda a, b, c: (a + b + c).sum(1), lambda: (_t(1, 1024), _t(1, 1024, seed=1), _t(1, 1))),
     "logsumexp_sigmoid_bce": (lambda a, t: torch.logsumexp(a, -1).sum() + F.binary_cross_entropy_with_logits(a, torch.sigmoid(t)), lambda: (_t(32, 77), _t(32, 77))),
 }
 
@@ -152,3 +157,34 @@ def test_dynamic_batch_keeps_vectors():
     for batch in (7, 100, 1):
         a, b = _t(batch, 40, 256, seed=2), _t(batch, 40, 256, seed=3)
         _compare(cf(a, b), f(a, b))
+
+
+def test_layernorm_backward_weight_gradient_is_a_column_sweep():
+    """The weight gradient of LayerNorm sums dy * xhat over rows; xhat is rebuilt from per-row
+    statistics, whose indices move along the reduced axis only.  Those slivers must not outvote
+    the two full tensors when the code shape is chosen: the kernel walks rows with lanes along
+    the contiguous kept axis (the reference picks the tiling axis from the low dimension of the
+    dominant accesses the same way, reference inductor_x/codegen/split_tiling.py:188-239)."""
+    announce("compile layernorm backward, code shapes")
+    import re
+
+    from torch._inductor.utils import run_and_get_code
+
+    def ln_bwd(dy, x, w):
+        xf = x.float()
+        mean = xf.mean(-1, keepdim=True)
+        rstd = torch.rsqrt(xf.var(-1, keepdim=True, unbiased=False) + 1e-5)
+        return torch.ops.aten.native_layer_norm_backward(dy, x, [x.shape[-1]], mean, rstd, w, None, [True, True, False])
+
+    dy, x = _t(2048, 1024, dtype=torch.bfloat16), _t(2048, 1024, dtype=torch.bfloat16, seed=1)
+    w = _t(1024, dtype=torch.bfloat16, seed=2)
+    torch._dynamo.reset()
+    with torch.no_grad():
+        got, codes = run_and_get_code(torch.compile(ln_bwd, dynamic=False), dy, x, w)
+        ref = ln_bwd(dy, x, w)
+    modes = re.findall(r"meta=\{'mode': '(\w+)'", codes[0])
+    assert sorted(modes) == ["col", "row"], modes
+    assert "mi::gather" not in codes[0]
+    torch.testing.assert_close(got[0], ref[0], rtol=2e-2, atol=2e-2)
+    # 2048 bf16-rounded products per column: compare the sums relative to their spread
+    torch.testing.assert_close(got[1].float(), ref[1].float(), rtol=2e-2, atol=2e-2 * float(ref[1].float().abs().max()))
