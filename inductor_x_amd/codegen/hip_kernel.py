@@ -1476,18 +1476,41 @@ class HipKernel(SIMDKernel):
                     keep.add(v)
             self.cse.invalidate(keep)
         elif self.mode == "row" and self.inside_reduction and not self.persistent_reduction:
-            # one pass over the reduced axis
-            self.body.writeline(
-                f"for ({self.index_dtype} r0_base = 0; r0_base < rnumel; r0_base += TPR * VEC) {{"
-            )
-            with self.body.indent():
-                self.body.writeline(f"const {self.index_dtype} r0_index = r0_base + rlane * VEC;")
-                self.body.writeline("const bool rmask = r0_index < rnumel;")
+            # one pass over the reduced axis: whole rounds of TPR * VEC elements run unmasked (the
+            # mask is a compile-time true, so loads carry no branch and several rounds' loads can
+            # be in flight at once); the last, partial round runs the same body under the mask
+            idx_t = self.index_dtype
+            unroll = int(os.environ.get("INDUCTOR_X_AMD_ROW_LOOP_UNROLL", "4"))
+            split_tail = unroll > 0
+
+            def one_round() -> None:
                 self.body.splice(self._entry_code(self.r_entries))
                 self.body.splice(self.loads)
                 self.body.splice(self.compute)
                 self.body.splice(self.stores)
-            self.body.writeline("}")
+
+            if split_tail:
+                whole = "(rnumel - rnumel % (TPR * VEC))"
+                self.body.writeline(f"#pragma unroll {unroll}")
+                self.body.writeline(f"for ({idx_t} r0_base = 0; r0_base < {whole}; r0_base += TPR * VEC) {{")
+                with self.body.indent():
+                    self.body.writeline(f"const {idx_t} r0_index = r0_base + rlane * VEC;")
+                    self.body.writeline("constexpr bool rmask = true;")
+                    one_round()
+                self.body.writeline("}")
+                self.body.writeline(f"if ({whole} < rnumel) {{")
+                with self.body.indent():
+                    self.body.writeline(f"const {idx_t} r0_index = {whole} + rlane * VEC;")
+                    self.body.writeline("const bool rmask = r0_index < rnumel;")
+                    one_round()
+                self.body.writeline("}")
+            else:
+                self.body.writeline(f"for ({idx_t} r0_base = 0; r0_base < rnumel; r0_base += TPR * VEC) {{")
+                with self.body.indent():
+                    self.body.writeline(f"const {idx_t} r0_index = r0_base + rlane * VEC;")
+                    self.body.writeline("const bool rmask = r0_index < rnumel;")
+                    one_round()
+                self.body.writeline("}")
             for line in self.row_loop_accs:
                 self.body.writeline(line)
             self.row_loop_accs.clear()

@@ -119,7 +119,6 @@ FALLBACK_OPS = [
     aten.sort, aten.topk,
     aten.scatter, aten.scatter_add, aten.scatter_reduce, aten.index_put, aten._unsafe_index_put,
     aten.index_add, aten.bucketize, aten.searchsorted,
-    aten.gather, aten._log_softmax, aten.nll_loss_forward,
 ]
 
 FALLBACK_LIST: list = []
