@@ -427,8 +427,10 @@ REDUCTION_KIND = {
     "argmin": "mi::RedArgMin",
     "welford_reduce": "mi::RedWelford",
     "welford_combine": "mi::RedMoments",
+    "online_softmax_reduce": "mi::RedOnlineSoftmax",
 }
-REDUCTION_WORDS = {"sum": 1, "prod": 1, "max": 1, "min": 1, "any": 1, "argmax": 2, "argmin": 2, "welford_reduce": 3}
+REDUCTION_WORDS = {"sum": 1, "prod": 1, "max": 1, "min": 1, "any": 1, "argmax": 2, "argmin": 2, "welford_reduce": 3,
+                   "online_softmax_reduce": 2}
 
 
 @dataclasses.dataclass
@@ -467,6 +469,10 @@ class HipKernel(SIMDKernel):
         self.r_full = False
         self.prologue = IndentedBuffer()
         self.row_loop_accs: list[str] = []
+        # looped row kernels: contiguous loads of the reduced axis seen so far, keyed by buffer and
+        # index text; one that comes again in a later pass is served from an LDS copy of the row
+        self.row_stash: dict[tuple[str, str], dict] = {}
+        self.row_pass = 0
         self.col_reductions: list[ColReduction] = []
         self.partial_body = IndentedBuffer()
         self.final_body = IndentedBuffer()
@@ -1143,6 +1149,27 @@ class HipKernel(SIMDKernel):
             else:
                 line = f"mi::vload_m<VEC>({ptr}, {mask}, {other})"
             is_vec = True
+            if (
+                self.mode == "row" and self.inside_reduction and not self.persistent_reduction
+                and not indirect and not self._load_mask and self._index_uses_tree(index, "r0_")
+            ):
+                key = (name, self.index_to_str(index))
+                entry = self.row_stash.get(key)
+                if entry is None:
+                    entry = {"id": len(self.row_stash), "dtype": dtype, "pass": self.row_pass, "reused": False}
+                    self.row_stash[key] = entry
+                    raw = self.cse.generate(self.loads, line, dtype=dtype)
+                    if isinstance(raw, HipCSEVariable):
+                        raw.is_vec = True
+                    self.loads.writeline(f"MI_ROW_STASH_{entry['id']}({raw});")
+                    entry["raw"] = str(raw)
+                    line = str(raw)
+                elif entry["pass"] == self.row_pass:
+                    # the same load again within the pass: the value already in registers
+                    line = entry["raw"]
+                elif entry["pass"] < self.row_pass:
+                    entry["reused"] = True
+                    line = f"MI_ROW_RELOAD_{entry['id']}({line})"
         elif kind == "uniform":
             if mask is None:
                 line = f"{var}[{self.index_to_str(index)}]"
@@ -1342,6 +1369,19 @@ class HipKernel(SIMDKernel):
                     )
                     weight = self.cse.generate(self.compute, "static_cast<float>(rnumel)", dtype=torch.float32)
                     return (mean, m2, weight)
+                if reduction_type == "online_softmax_reduce":
+                    # the row is in registers: the maximum, then the sum against it
+                    top = self.cse.generate(
+                        self.compute,
+                        f"mi::group_merge<mi::RedMax, BLOCK, TPR>(mi::RedMax::finish(mi::thread_step<mi::RedMax>("
+                        f"mi::RedMax::init(), {value}, {self._r_index_str()}, rmask)), lds_red)",
+                        dtype=torch.float32,
+                    )
+                    total = self.cse.generate(
+                        self.compute, f"mi::row_sum<BLOCK, TPR>(mi::exp({value} - {top}), rmask, lds_red)",
+                        dtype=torch.float32,
+                    )
+                    return (top, total)
                 merged_name = f"red{n}"
                 self.compute.writeline(
                     f"const auto {merged_name} = mi::group_merge<{kind}, BLOCK, TPR>({kind}::finish("
@@ -1350,9 +1390,12 @@ class HipKernel(SIMDKernel):
             else:
                 acc = f"acc{n}"
                 self.prologue.writeline(f"typename {kind}::T {acc} = {kind}::init();")
-                self.compute.writeline(
-                    f"{acc} = mi::thread_step<{kind}>({acc}, {value}, {self._r_index_str()}, rmask);"
-                )
+                if reduction_type == "online_softmax_reduce":
+                    self.compute.writeline(f"{acc} = mi::softmax_step({acc}, {value}, rmask);")
+                else:
+                    self.compute.writeline(
+                        f"{acc} = mi::thread_step<{kind}>({acc}, {value}, {self._r_index_str()}, rmask);"
+                    )
                 merged_name = f"red{n}"
                 self.row_loop_accs.append(
                     f"const auto {merged_name} = mi::group_merge<{kind}, BLOCK, TPR>({kind}::finish({acc}), lds_red);"
@@ -1410,6 +1453,8 @@ class HipKernel(SIMDKernel):
             if reduction_type == "welford_reduce":
                 return (vec_result("GetMean", torch.float32), vec_result("GetM2", torch.float32),
                         vec_result("GetCount", torch.float32))
+            if reduction_type == "online_softmax_reduce":
+                return (vec_result("GetSoftmaxMax", torch.float32), vec_result("GetSoftmaxSum", torch.float32))
             if reduction_type == "any":
                 return vec_result("GetNonzero", torch.bool)
             return vec_result("GetSelf", torch.float32)
@@ -1421,6 +1466,8 @@ class HipKernel(SIMDKernel):
                 self._result_var(f"{merged}.m2", torch.float32),
                 self._result_var(f"{merged}.n", torch.float32),
             )
+        if reduction_type == "online_softmax_reduce":
+            return (self._result_var(f"{merged}.m", torch.float32), self._result_var(f"{merged}.s", torch.float32))
         if reduction_type == "any":
             return self._result_var(f"({merged} != 0.f)", torch.bool)
         return self._result_var(f"{merged}", torch.float32)
@@ -1511,6 +1558,7 @@ class HipKernel(SIMDKernel):
                     self.body.writeline("const bool rmask = r0_index < rnumel;")
                     one_round()
                 self.body.writeline("}")
+            self.row_pass += 1
             for line in self.row_loop_accs:
                 self.body.writeline(line)
             self.row_loop_accs.clear()
@@ -1554,6 +1602,47 @@ class HipKernel(SIMDKernel):
                 raise UnsupportedHipCodegen(f"kernel argument {type(arg).__name__}")
         return params, "".join(codes), [str(a) for a in call_args]
 
+    ROW_STASH_BUDGET = 144 * 1024
+
+    def _plan_row_stash(self) -> tuple[list[str], int]:
+        """A looped row kernel that reads the same piece of a row in several passes (softmax: the
+        maximum, the sum, the output) keeps the row in LDS after the first pass when it fits the
+        CU's 160 KB: later passes read LDS instead of going back to memory.  Each thread reads
+        back exactly the vectors it stored, so no barrier is involved.  One row per workgroup;
+        the workgroup grows with the row so that one or two of them still fill the CU.
+        Returns the declarations for the kernel and the dynamic LDS bytes."""
+        from ..hip_heuristics import next_power_of_2
+
+        used = [e for e in self.row_stash.values() if e["reused"]]
+        if (
+            not used or self.mode != "row" or self.persistent_reduction or self.tpr != self.block
+            or os.environ.get("INDUCTOR_X_AMD_ROW_STASH", "1") == "0"
+        ):
+            return [], 0
+        rnumel = self._static_numel("r0_")
+        if rnumel is None:
+            return [], 0
+        per_elem = sum(dtype_nbytes(e["dtype"]) for e in used)
+        vectors = -(-rnumel // self.vec)
+        raw = rnumel * per_elem
+        want = 256 if raw <= 40 * 1024 else (512 if raw <= 80 * 1024 else 1024)
+        tpr = max(min(want, next_power_of_2(vectors)), 64)
+        span = tpr * self.vec
+        padded = -(-rnumel // span) * span
+        if padded * per_elem > self.ROW_STASH_BUDGET:
+            return [], 0
+        self.tpr = self.block = tpr
+        decls = ["extern __shared__ __align__(16) unsigned char lds_rows[];"]
+        offset = 0
+        for e in used:
+            e["offset"] = offset
+            decls.append(
+                f"{DTYPE_TO_HIP[e['dtype']]}* const lds_row{e['id']} = "
+                f"reinterpret_cast<{DTYPE_TO_HIP[e['dtype']]}*>(lds_rows + {offset});"
+            )
+            offset += padded * dtype_nbytes(e["dtype"])
+        return decls, offset
+
     def codegen_kernel(self, name: Optional[str] = None) -> str:
         self.codegen_body()
         # Size symbols in the range variables' definitions become kernel
@@ -1567,6 +1656,15 @@ class HipKernel(SIMDKernel):
         kname = name or "KERNEL_NAME"
         src = IndentedBuffer()
         src.writeline('#include "mi/codegen.h"')
+        stash_decls, stash_bytes = self._plan_row_stash()
+        for entry in self.row_stash.values():
+            k = entry["id"]
+            if entry.get("offset") is not None:
+                src.writeline(f"#define MI_ROW_STASH_{k}(v) mi::vstore<VEC>(lds_row{k} + r0_index, v)")
+                src.writeline(f"#define MI_ROW_RELOAD_{k}(...) mi::vload<VEC>(lds_row{k} + r0_index)")
+            else:
+                src.writeline(f"#define MI_ROW_STASH_{k}(v)")
+                src.writeline(f"#define MI_ROW_RELOAD_{k}(...) (__VA_ARGS__)")
         src.writeline("")
         meta: dict[str, Any] = {"mode": self.mode, "vec": self.vec, "block": self.block, "index_code": idx_code}
         if self.mode == "pointwise":
@@ -1649,6 +1747,8 @@ class HipKernel(SIMDKernel):
                 src.writeline(f"constexpr int BLOCK = {self.block};")
                 src.writeline(f"constexpr int TPR = {self.tpr};")
                 src.writeline("__shared__ float lds_red[(BLOCK / 64) * 4];")
+                for line in stash_decls:
+                    src.writeline(line)
                 src.writeline("const int rlane = threadIdx.x % TPR;")
                 # a workgroup walks the rows with the stride of the grid, so the launcher can cap the
                 # grid when there are many short rows (one workgroup per 4 KiB of input would be
@@ -1672,7 +1772,8 @@ class HipKernel(SIMDKernel):
                 src.writeline("}")
             src.writeline("}")
             sig = codes + idx_code + idx_code
-            meta.update({"tpr": self.tpr, "persistent": bool(self.persistent_reduction)})
+            meta.update({"tpr": self.tpr, "persistent": bool(self.persistent_reduction), "block": self.block,
+                         "lds_bytes": stash_bytes})
         elif self.mode == "colloop":
             ct, rl = self.col_ct, self.col_rl
             words = getattr(self, "colloop_max_words", 1)

@@ -110,6 +110,3 @@ def apply_inductor_settings() -> None:
     from torch._inductor import config as inductor_config
 
     inductor_config.triton.unique_kernel_names = True
-    # softmax stays a max reduction followed by a sum reduction; the fused
-    # "online softmax" reduction type has no counterpart in the HIP generator
-    inductor_config.online_softmax = False

@@ -660,6 +660,88 @@ struct RedWelford {
   }
 };
 
+// Maximum and sum of exp(x - maximum) of a row in one sweep ("online softmax"): the state is the
+// running maximum m and the sum s of exp(x - m) over what has been seen; a larger maximum rescales
+// the sum.  While the maximum is -inf the scale is taken as 1 (exp(-inf - -inf) would be NaN), as
+// in torch/_inductor/runtime/triton_helpers.py:192-212.  NaN inputs make both results NaN.
+struct SoftmaxState {
+  float m, s;
+};
+__device__ __forceinline__ float softmax_scale(float from, float to) {
+  return (to == -__builtin_inff()) ? 1.0f : __expf(from - to);
+}
+struct RedOnlineSoftmax {
+  typedef SoftmaxState T;
+  typedef SoftmaxState M;
+  static constexpr int W = 2;
+  __device__ static T init() {
+    T t;
+    t.m = -__builtin_inff();
+    t.s = 0.f;
+    return t;
+  }
+  __device__ static M empty() { return init(); }
+  __device__ static M merge(M a, M b) {
+    M r;
+    r.m = MaxOp()(a.m, b.m);
+    r.s = a.s * softmax_scale(a.m, r.m) + b.s * softmax_scale(b.m, r.m);
+    return r;
+  }
+  __device__ static T step(T s, float v, int) {
+    T r;
+    r.m = MaxOp()(s.m, v);
+    r.s = s.s * softmax_scale(s.m, r.m) + softmax_scale(v, r.m);
+    return r;
+  }
+  __device__ static T first(float v, int) { return step(init(), v, 0); }
+  __device__ static T step_fast(T s, float v, int) { return step(s, v, 0); }
+  __device__ static M finish(T s) { return s; }
+  __device__ static M finish_n(T s, float) { return s; }
+  __device__ static void enc(M m, float* w) {
+    w[0] = m.m;
+    w[1] = m.s;
+  }
+  __device__ static M dec(const float* w) {
+    M m;
+    m.m = w[0];
+    m.s = w[1];
+    return m;
+  }
+};
+// One vector of a row at a time: the vector's own maximum first, so the running sum is rescaled
+// once per vector and every element costs one exponential.
+template <class VT, class MT>
+__device__ __forceinline__ SoftmaxState softmax_step(SoftmaxState a, const VT& val, const MT& mask) {
+  constexpr int n = Tr<VT>::n == 0 ? 1 : Tr<VT>::n;
+  float vm = -__builtin_inff();
+#pragma unroll
+  for (int i = 0; i < n; ++i)
+    if (static_cast<bool>(at(mask, i))) vm = MaxOp()(vm, static_cast<float>(at(val, i)));
+  SoftmaxState r;
+  r.m = MaxOp()(a.m, vm);
+  const float ref = (r.m == -__builtin_inff()) ? 0.f : r.m;
+  float add = 0.f;
+#pragma unroll
+  for (int i = 0; i < n; ++i)
+    if (static_cast<bool>(at(mask, i))) add += __expf(static_cast<float>(at(val, i)) - ref);
+  // with the maximum still -inf every term above is exp(-inf) = 0; count the elements instead,
+  // which is what a scale of 1 per element amounts to
+  if (r.m == -__builtin_inff()) {
+    add = 0.f;
+#pragma unroll
+    for (int i = 0; i < n; ++i)
+      if (static_cast<bool>(at(mask, i))) add += 1.f;
+  }
+  r.s = a.s * softmax_scale(a.m, r.m) + add;
+  return r;
+}
+struct GetSoftmaxMax {
+  __device__ __forceinline__ float operator()(const SoftmaxState& m) const { return m.m; }
+};
+struct GetSoftmaxSum {
+  __device__ __forceinline__ float operator()(const SoftmaxState& m) const { return m.s; }
+};
+
 // Reduction whose inputs are moments already (the second stage of a variance that was split
 // into slices): the thread state is the merged moments.
 struct RedMoments {

@@ -493,7 +493,8 @@ class GeneratedKernel:
             self._fns["main"].launch(m["signature"], raw + (xnumel,), grid, (m["block"],), stream)
         elif self.mode == "row":
             grid = (row_grid(cdiv(xnumel, m["block"] // m["tpr"])), 1, 1)
-            self._fns["main"].launch(m["signature"], raw + (xnumel, rnumel), grid, (m["block"],), stream)
+            self._fns["main"].launch(m["signature"], raw + (xnumel, rnumel), grid, (m["block"],), stream,
+                                     m.get("lds_bytes", 0))
         elif self.mode == "colloop":
             grid = (cdiv(xnumel, m["ct"] * m["vec"]), 1, 1)
             self._fns["main"].launch(m["signature"], raw + (xnumel, rnumel), grid, (m["block"],), stream, m["lds_bytes"])

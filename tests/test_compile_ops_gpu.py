@@ -188,3 +188,66 @@ def test_layernorm_backward_weight_gradient_is_a_column_sweep():
     torch.testing.assert_close(got[0], ref[0], rtol=2e-2, atol=2e-2)
     # 2048 bf16-rounded products per column: compare the sums relative to their spread
     torch.testing.assert_close(got[1].float(), ref[1].float(), rtol=2e-2, atol=2e-2 * float(ref[1].float().abs().max()))
+
+
+def _masked_logits(rows, cols, dtype=torch.float32, seed=0):
+    """Scores with -inf holes, one row of nothing but -inf and one NaN: what attention masks and
+    padded batches feed a softmax."""
+    x = _t(rows, cols, dtype=dtype, seed=seed)
+    hole = _t(rows, cols, seed=seed + 1) > 1.0
+    x = x.masked_fill(hole, float("-inf"))
+    x[1, :] = float("-inf")
+    x[2, 5] = float("nan")
+    x[3, : cols // 2] = float("-inf")
+    return x
+
+
+SOFTMAX_CASES = {
+    # rows too long for registers: maximum and sum in one sweep, the row kept in LDS for the output
+    "softmax_long_rows_bf16": (lambda x: torch.softmax(x.float(), -1).to(x.dtype), lambda: (_t(96, 50304, dtype=torch.bfloat16),)),
+    "softmax_long_rows_f32": (lambda x: torch.softmax(x, -1), lambda: (_t(64, 32768),)),
+    "log_softmax_long_rows": (lambda x: torch.log_softmax(x, -1), lambda: (_t(33, 40000),)),
+    "logsumexp_long_rows": (lambda x: torch.logsumexp(x, -1), lambda: (_t(128, 50304),)),
+    "softmax_long_rows_holes": (lambda x: torch.softmax(x, -1), lambda: (_masked_logits(16, 20000),)),
+    # rows in registers
+    "softmax_short_rows_holes": (lambda x: torch.softmax(x, -1), lambda: (_masked_logits(64, 1000),)),
+    "softmax_tiny_rows": (lambda x: torch.softmax(x, -1), lambda: (_t(4096, 8),)),
+    # the reduced axis strided
+    "softmax_dim0": (lambda x: torch.softmax(x, 0), lambda: (_t(2048, 1000),)),
+    "softmax_dim0_holes": (lambda x: torch.softmax(x, 0), lambda: (_masked_logits(300, 256).t().contiguous().t(),)),
+    "logsumexp_dim0": (lambda x: torch.logsumexp(x, 0), lambda: (_t(65536, 128),)),
+    "softmax_middle_axis": (lambda x: torch.softmax(x, 1), lambda: (_t(8, 700, 64),)),
+    "cross_entropy_rows": (lambda x, t: F.cross_entropy(x.float(), t), lambda: (_t(512, 50304, dtype=torch.bfloat16), torch.randint(0, 50304, (512,), device=DEV))),
+}
+
+
+@pytest.mark.parametrize("name", sorted(SOFTMAX_CASES))
+def test_softmax_family(name):
+    """Softmax-shaped graphs reach the generator as one reduction with two results, maximum and
+    sum of exponentials (torch/_inductor/lowering.py prepare_softmax_online); the kernels must
+    agree with eager to fp32 rounding, -inf holes, all--inf rows (NaN, as eager) and NaN included."""
+    announce(f"compile softmax family: {name}")
+    fn, make = SOFTMAX_CASES[name]
+    args = make()
+    torch._dynamo.reset()
+    with torch.no_grad():
+        got = torch.compile(fn, dynamic=False)(*args)
+        ref = fn(*args)
+    assert got.shape == ref.shape and got.dtype == ref.dtype
+    tol = dict(rtol=2e-2, atol=2e-2) if ref.dtype == torch.bfloat16 else dict(rtol=2e-5, atol=1e-6)
+    torch.testing.assert_close(got, ref, equal_nan=True, **tol)
+
+
+def test_long_softmax_is_one_sweep_plus_lds():
+    announce("compile long softmax, code shape")
+    import re
+
+    from torch._inductor.utils import run_and_get_code
+
+    x = _t(64, 50304, dtype=torch.bfloat16)
+    torch._dynamo.reset()
+    with torch.no_grad():
+        _, codes = run_and_get_code(torch.compile(lambda x: torch.softmax(x.float(), -1).to(x.dtype), dynamic=False), x)
+    code = codes[0]
+    assert "mi::softmax_step" in code and "lds_row0" in code, "expected one statistics sweep and an LDS copy of the row"
+    assert len(re.findall(r"in_ptr0 \+", code.split("group_merge")[0])) <= 2  # main rounds + the partial round
