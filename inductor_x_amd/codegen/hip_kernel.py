@@ -54,7 +54,7 @@ from torch._inductor.ops_handler import StoreMode
 from torch._inductor.utils import sympy_subs
 from torch._inductor.virtualized import V
 from torch.utils._ordered_set import OrderedSet
-from torch.utils._sympy.functions import FloorDiv, ModularIndexing
+from torch.utils._sympy.functions import FloorDiv, Identity, ModularIndexing
 from torch.utils._sympy.printers import ExprPrinter
 from torch.utils._sympy.value_ranges import ValueRanges
 
@@ -154,6 +154,15 @@ class HipExprPrinter(ExprPrinter):
 
 
 hexpr = HipExprPrinter().doprint
+
+
+def _without_identity(expr: sympy.Expr) -> sympy.Expr:
+    """Inductor wraps the shifted index of a concatenated or padded operand in Identity so that
+    it is printed as written (it may be negative where the guard is false).  For the analysis
+    of how the address moves from lane to lane the wrapper is transparent."""
+    if isinstance(expr, sympy.Expr) and expr.has(Identity):
+        return expr.replace(Identity, lambda a: a)
+    return expr
 
 
 def value_to_hip(val: Union[float, int, bool, str, CSEVariable], dtype: Optional[torch.dtype] = None) -> str:
@@ -1000,6 +1009,7 @@ class HipKernel(SIMDKernel):
         base + i) or 'gather'."""
         if self.vec == 1:
             return "uniform"
+        index = _without_identity(index)
         lane_syms = [s for s in index.free_symbols if self._is_lane_symbol(s)]
         tmp_vec = False
         for s in index.free_symbols:
@@ -1031,6 +1041,7 @@ class HipKernel(SIMDKernel):
         vec = self.vec if vec is None else vec
         is_lane = is_lane or self._is_lane_symbol
         zero = sympy.Integer(0)
+        expr = _without_identity(expr)
 
         def aligned(e: sympy.Expr) -> bool:
             base = sympy.expand(sympy_subs(e, {s: zero for s in e.free_symbols if is_lane(s)}))
@@ -1087,6 +1098,7 @@ class HipKernel(SIMDKernel):
     def index_is_aligned(self, index: sympy.Expr) -> bool:
         """True when the address of lane 0 is provably a multiple of the vector
         width (lane-varying variables are multiples of it by construction)."""
+        index = _without_identity(index)
         lane_syms = [s for s in index.free_symbols if self._is_lane_symbol(s)]
         base = sympy.expand(sympy_subs(index, {s: sympy.Integer(0) for s in lane_syms}))
         try:
@@ -1147,7 +1159,7 @@ class HipKernel(SIMDKernel):
             if mask is None:
                 line = f"mi::vload<VEC>({ptr})" if aligned else f"mi::vload_u<VEC>({ptr})"
             else:
-                line = f"mi::vload_m<VEC>({ptr}, {mask}, {other})"
+                line = f"mi::vload_m<VEC{'' if aligned else ', false'}>({ptr}, {mask}, {other})"
             is_vec = True
             if (
                 self.mode == "row" and self.inside_reduction and not self.persistent_reduction
