@@ -438,6 +438,7 @@ REDUCTION_KIND = {
     "welford_combine": "mi::RedMoments",
     "online_softmax_reduce": "mi::RedOnlineSoftmax",
 }
+INT_REDUCTION_OP = {"sum": "Sum", "prod": "Prod", "max": "Max", "min": "Min"}
 REDUCTION_WORDS = {"sum": 1, "prod": 1, "max": 1, "min": 1, "any": 1, "argmax": 2, "argmin": 2, "welford_reduce": 3,
                    "online_softmax_reduce": 2}
 
@@ -449,6 +450,8 @@ class ColReduction:
     result: str  # merged state variable in the final kernel
     value: str
     ws_offset_words: int  # offset in units of nsplit * xnumel floats
+    cxx: str = ""  # reduction class of the template library
+    words: int = 1  # floats per state
 
 
 class HipKernel(SIMDKernel):
@@ -1318,11 +1321,19 @@ class HipKernel(SIMDKernel):
         assert self.inside_reduction
         if reduction_type not in REDUCTION_KIND:
             raise UnsupportedHipCodegen(f"reduction {reduction_type}")
-        if reduction_type in ("sum", "prod", "max", "min") and not src_dtype.is_floating_point and src_dtype != torch.bool:
-            raise UnsupportedHipCodegen(f"integer {reduction_type} reduction")
         if isinstance(value, tuple) and reduction_type != "welford_combine":
             raise UnsupportedHipCodegen(f"tuple-valued reduction input for {reduction_type}")
         kind = REDUCTION_KIND[reduction_type]
+        words = REDUCTION_WORDS.get(reduction_type, 3)
+        # sums, products and extrema of integers are exact 64-bit reductions: their states travel
+        # through the same merge machinery as two 32-bit words
+        integral = (
+            reduction_type in INT_REDUCTION_OP and not src_dtype.is_floating_point
+            and (src_dtype != torch.bool or reduction_type in ("sum", "prod"))
+        )
+        if integral:
+            kind = f"mi::RedInt<mi::IntOp::{INT_REDUCTION_OP[reduction_type]}>"
+            words = 2
         if self._load_mask:
             raise UnsupportedHipCodegen("reduction under a load mask")
         n = next(self.acc_ids)
@@ -1361,7 +1372,7 @@ class HipKernel(SIMDKernel):
             return self._unpack_result(merged_name, reduction_type, dtype)
         if self.mode == "row":
             if self.persistent_reduction:
-                if reduction_type == "sum":
+                if reduction_type == "sum" and not integral:
                     merged = self.cse.generate(
                         self.compute, f"mi::row_sum<BLOCK, TPR>({value}, rmask, lds_red)", dtype=torch.float32
                     )
@@ -1412,13 +1423,13 @@ class HipKernel(SIMDKernel):
                 self.row_loop_accs.append(
                     f"const auto {merged_name} = mi::group_merge<{kind}, BLOCK, TPR>({kind}::finish({acc}), lds_red);"
                 )
-            return self._unpack_result(merged_name, reduction_type, dtype)
+            return self._unpack_result(merged_name, reduction_type, dtype, integral)
         if self.mode == "colloop":
             acc = f"acc{n}"
             self.prologue.writeline(f"mi::ColAcc<{kind}, VEC> {acc};")
             self.prologue.writeline(f"{acc}.init();")
             self.compute.writeline(f"{acc}.step({value}, r0_index, true);")
-            self.colloop_max_words = max(getattr(self, "colloop_max_words", 1), REDUCTION_WORDS[reduction_type])
+            self.colloop_max_words = max(getattr(self, "colloop_max_words", 1), words)
             self.row_loop_accs.extend([
                 f"typename {kind}::M {acc}_m[VEC];",
                 "#pragma unroll",
@@ -1426,14 +1437,16 @@ class HipKernel(SIMDKernel):
                 f"mi::col_fold<{kind}, VEC, CT, RL>({acc}_m, ct, rl, lds_dyn);",
                 f"mi::col_share<{kind}, VEC, CT, RL>({acc}_m, ct, rl, lds_dyn);",
             ])
-            return self._unpack_result(f"{acc}_m", reduction_type, dtype)
+            return self._unpack_result(f"{acc}_m", reduction_type, dtype, integral)
         if self.mode == "col":
             acc = f"acc{n}"
             merged_name = f"red{n}"
-            self.col_reductions.append(ColReduction(reduction_type, acc, merged_name, str(value), self.ws_words))
-            self.ws_words += REDUCTION_WORDS[reduction_type]
+            self.col_reductions.append(
+                ColReduction(reduction_type, acc, merged_name, str(value), self.ws_words, cxx=kind, words=words)
+            )
+            self.ws_words += words
             self.compute.writeline(f"{acc}.step({value}, r0_index, xmask);")
-            return self._unpack_result(merged_name, reduction_type, dtype)
+            return self._unpack_result(merged_name, reduction_type, dtype, integral)
         raise UnsupportedHipCodegen("reduction in a pointwise kernel")
 
     def _result_var(self, text: str, dtype: torch.dtype) -> CSEVariable:
@@ -1451,7 +1464,14 @@ class HipKernel(SIMDKernel):
     def _cast_result(self, var: CSEVariable, dtype: torch.dtype) -> CSEVariable:
         return var
 
-    def _unpack_result(self, merged: str, reduction_type: str, dtype: torch.dtype):
+    def _unpack_result(self, merged: str, reduction_type: str, dtype: torch.dtype, integral: bool = False):
+        if integral:
+            if self.mode == "colloop":
+                var = self._result_var(f"mi::col_get<VEC>({merged}, mi::GetSelfInt())", torch.int64)
+                if isinstance(var, HipCSEVariable):
+                    var.is_vec = True
+                return var
+            return self._result_var(f"{merged}", torch.int64)
         if self.mode == "colloop":
             # `merged` is an array of VEC states, one per column of the thread: results are vectors
             def vec_result(getter: str, dt: torch.dtype) -> CSEVariable:
@@ -1819,7 +1839,7 @@ class HipKernel(SIMDKernel):
         if not self.col_reductions:
             raise UnsupportedHipCodegen("column kernel without a reduction")
         ct, rl, vec = self.col_ct, self.col_rl, self.vec
-        max_words = max(REDUCTION_WORDS[c.kind] for c in self.col_reductions)
+        max_words = max(c.words for c in self.col_reductions)
         extra = [f"float* __restrict__ ws", f"const {idx_t} xnumel", f"const {idx_t} rnumel",
                  "const int rows_per_split", "const int nsplit"]
         plist = ", ".join(params + extra)
@@ -1840,7 +1860,7 @@ class HipKernel(SIMDKernel):
                 src.writeline(f"const {idx_t} r_begin = static_cast<{idx_t}>(split) * rows_per_split;")
                 src.writeline(f"const {idx_t} r_end = (r_begin + rows_per_split < rnumel) ? r_begin + rows_per_split : rnumel;")
                 for c in self.col_reductions:
-                    kind = REDUCTION_KIND[c.kind]
+                    kind = c.cxx
                     src.writeline(f"mi::ColAcc<{kind}, VEC> {c.acc};")
                     src.writeline(f"{c.acc}.init();")
                 src.writeline("if (xmask) {")
@@ -1853,7 +1873,7 @@ class HipKernel(SIMDKernel):
                     src.writeline("}")
                 src.writeline("}")
                 for c in self.col_reductions:
-                    kind = REDUCTION_KIND[c.kind]
+                    kind = c.cxx
                     src.writeline(f"typename {kind}::M {c.acc}_m[VEC];")
                     src.writeline("#pragma unroll")
                     src.writeline(f"for (int i = 0; i < VEC; ++i) {c.acc}_m[i] = {c.acc}.finish(i);")
@@ -1899,7 +1919,7 @@ class HipKernel(SIMDKernel):
             src.writeline("constexpr int VEC = 1;")
             src.writeline(f"constexpr int CPW = {cpw};")
             src.writeline(f"constexpr int SL = {sl};")
-            src.writeline(f"__shared__ float lds_fin[CPW * SL * {sum(REDUCTION_WORDS[c.kind] for c in self.col_reductions)}];")
+            src.writeline(f"__shared__ float lds_fin[CPW * SL * {sum(c.words for c in self.col_reductions)}];")
             src.writeline("const int slot = threadIdx.x % CPW;")
             src.writeline("const int sl = threadIdx.x / CPW;")
             src.writeline(f"const {idx_t} xraw = static_cast<{idx_t}>(blockIdx.x) * CPW + slot;")
@@ -1907,14 +1927,14 @@ class HipKernel(SIMDKernel):
             src.writeline(f"const {idx_t} xindex = live ? xraw : xnumel - 1;")
             # the loads of every reduction first, then the folds (each fold holds barriers)
             for c in self.col_reductions:
-                kind = REDUCTION_KIND[c.kind]
+                kind = c.cxx
                 src.writeline(
                     f"const auto {c.result}_g = mi::col_final_gather<{kind}, SL>(ws + {c.ws_offset_words} * "
                     f"static_cast<mi::i64>(nsplit) * xnumel, xindex, xnumel, nsplit, sl, live);"
                 )
             for c in self.col_reductions:
                 src.writeline(f"auto {c.result} = {c.result}_g;")
-            kinds = ", ".join(REDUCTION_KIND[c.kind] for c in self.col_reductions)
+            kinds = ", ".join(c.cxx for c in self.col_reductions)
             states = ", ".join(c.result for c in self.col_reductions)
             src.writeline(f"mi::col_final_fold_all<CPW, SL, {kinds}>(lds_fin, slot, sl, {states});")
             for line in self._result_defs_col:

@@ -705,6 +705,55 @@ struct RedWelford {
   }
 };
 
+// Exact 64-bit integer sum, product, maximum and minimum.  The state is one i64; where states
+// travel as float words (lane exchanges, LDS, the column workspace) it goes as its two 32-bit
+// halves, bit for bit: those paths only move words, they never do arithmetic on them.
+enum class IntOp { Sum, Prod, Max, Min };
+template <IntOp OP>
+struct RedInt {
+  typedef i64 V;  // the type a value is converted to before step()
+  typedef i64 T;
+  typedef i64 M;
+  static constexpr int W = 2;
+  __device__ static T init() {
+    if constexpr (OP == IntOp::Sum) return 0;
+    if constexpr (OP == IntOp::Prod) return 1;
+    if constexpr (OP == IntOp::Max) return static_cast<i64>(0x8000000000000000ull);
+    return static_cast<i64>(0x7fffffffffffffffull);
+  }
+  __device__ static M empty() { return init(); }
+  __device__ static M merge(M a, M b) {
+    if constexpr (OP == IntOp::Sum) return a + b;
+    if constexpr (OP == IntOp::Prod) return a * b;
+    if constexpr (OP == IntOp::Max) return a > b ? a : b;
+    return a < b ? a : b;
+  }
+  __device__ static T step(T s, i64 v, int) { return merge(s, v); }
+  __device__ static T first(i64 v, int) { return v; }
+  __device__ static T step_fast(T s, i64 v, int) { return merge(s, v); }
+  __device__ static M finish(T s) { return s; }
+  __device__ static M finish_n(T s, float) { return s; }
+  __device__ static void enc(M m, float* w) {
+    const unsigned long long u = static_cast<unsigned long long>(m);
+    w[0] = __builtin_bit_cast(float, static_cast<unsigned>(u & 0xffffffffull));
+    w[1] = __builtin_bit_cast(float, static_cast<unsigned>(u >> 32));
+  }
+  __device__ static M dec(const float* w) {
+    const unsigned long long lo = __builtin_bit_cast(unsigned, w[0]);
+    const unsigned long long hi = __builtin_bit_cast(unsigned, w[1]);
+    return static_cast<i64>(lo | (hi << 32));
+  }
+};
+// The type values are converted to on their way into R::step: float unless R names another.
+template <class R, class = void>
+struct ValueOf {
+  typedef float type;
+};
+template <class R>
+struct ValueOf<R, std::void_t<typename R::V>> {
+  typedef typename R::V type;
+};
+
 // Maximum and sum of exp(x - maximum) of a row in one sweep ("online softmax"): the state is the
 // running maximum m and the sum s of exp(x - m) over what has been seen; a larger maximum rescales
 // the sum.  While the maximum is -inf the scale is taken as 1 (exp(-inf - -inf) would be NaN), as
@@ -918,7 +967,8 @@ __device__ __forceinline__ typename R::T thread_step(typename R::T s, const VT& 
   constexpr int n = Tr<VT>::n == 0 ? (Tr<IT>::n == 0 ? (Tr<MT>::n == 0 ? 1 : Tr<MT>::n) : Tr<IT>::n) : Tr<VT>::n;
 #pragma unroll
   for (int i = 0; i < n; ++i)
-    if (static_cast<bool>(at(mask, i))) s = R::step(s, static_cast<float>(at(val, i)), static_cast<int>(at(idx, i)));
+    if (static_cast<bool>(at(mask, i)))
+      s = R::step(s, static_cast<typename ValueOf<R>::type>(at(val, i)), static_cast<int>(at(idx, i)));
   return s;
 }
 
@@ -952,10 +1002,10 @@ struct ColAcc {
     if (!mask) return;
     if (cnt == 0) {
 #pragma unroll
-      for (int i = 0; i < N; ++i) s[i] = R::first(static_cast<float>(at(val, i)), ridx);
+      for (int i = 0; i < N; ++i) s[i] = R::first(static_cast<typename ValueOf<R>::type>(at(val, i)), ridx);
     } else {
 #pragma unroll
-      for (int i = 0; i < N; ++i) s[i] = R::step_fast(s[i], static_cast<float>(at(val, i)), ridx);
+      for (int i = 0; i < N; ++i) s[i] = R::step_fast(s[i], static_cast<typename ValueOf<R>::type>(at(val, i)), ridx);
     }
     ++cnt;
   }
@@ -1050,6 +1100,9 @@ __device__ __forceinline__ void col_share(typename R::M (&m)[N], int ct, int rl,
 struct GetSelf {
   template <class M>
   __device__ __forceinline__ float operator()(const M& m) const { return m; }
+};
+struct GetSelfInt {
+  __device__ __forceinline__ i64 operator()(i64 m) const { return m; }
 };
 struct GetMean {
   __device__ __forceinline__ float operator()(const Moments& m) const { return m.mean; }

@@ -172,11 +172,8 @@ def _register_inductor_fallbacks() -> None:
     def sum_gpu(x, axis=None, keepdims=False, *, dtype=None):
         in_dtype = x.get_dtype()
         if (is_integer_dtype(in_dtype) or is_boolean_dtype(in_dtype)) and dtype is None:
-            # integer sums keep Inductor's lowering (int64 accumulation); the HIP
-            # generator rejects them and they never reach it
-            return fallback_handler(aten.sum.dim_IntList, add_to_fallback_set=False)(
-                x, axis, keepdims, dtype=dtype
-            )
+            # integer and boolean sums accumulate in int64, as Inductor's own lowering has them
+            return make_reduction("sum", override_return_dtype=torch.int64)(x, axis, keepdims, dtype=torch.int64)
         out_dtype = dtype or in_dtype
         if in_dtype in (torch.float16, torch.bfloat16):
             x = to_dtype(x, torch.float32)

@@ -251,3 +251,44 @@ def test_long_softmax_is_one_sweep_plus_lds():
     code = codes[0]
     assert "mi::softmax_step" in code and "lds_row0" in code, "expected one statistics sweep and an LDS copy of the row"
     assert len(re.findall(r"in_ptr0 \+", code.split("group_merge")[0])) <= 2  # main rounds + the partial round
+
+
+def _ints(*shape, lo=-(1 << 40), hi=1 << 40, dtype=torch.int64, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed + sum(shape))
+    return torch.randint(lo, hi, shape, generator=g, dtype=torch.int64).to(dtype).to(DEV)
+
+
+INTEGER_REDUCTIONS = {
+    # values far beyond 2^24: a float accumulator anywhere on the way would show
+    "rows_sum_max_min": (lambda a: (a.sum(-1), a.amax(-1), a.amin(-1)), lambda: (_ints(512, 300),)),
+    "rows_long": (lambda a: (a.sum(-1), a.amax(-1)), lambda: (_ints(8, 100000),)),
+    "columns_split": (lambda a: (a.sum(0), a.amin(0)), lambda: (_ints(70000, 64),)),
+    "columns_short": (lambda a: (a.sum(0), a.amax(0)), lambda: (_ints(40, 1000),)),
+    "middle_axis_int32": (lambda a: (a.amax(1), a.sum(1)), lambda: (_ints(16, 5000, 8, lo=-(1 << 30), hi=1 << 30, dtype=torch.int32),)),
+    "everything": (lambda a: (a.sum(), a.amax(), a.amin()), lambda: (_ints(1000, 1000),)),
+    "product_small": (lambda a: a.prod(-1), lambda: (_ints(64, 20, lo=-3, hi=4),)),
+    "uint8_int16": (lambda a, b: (a.sum(-1), a.amax(0), b.sum(0), b.amin(-1)),
+                    lambda: (_ints(300, 77, lo=0, hi=256, dtype=torch.uint8), _ints(300, 77, lo=-30000, hi=30000, dtype=torch.int16))),
+    "count_of_a_mask": (lambda a: ((a > 0).sum(), (a > 0.5).sum(-1), (a < 0).sum(0)), lambda: (_t(777, 333),)),
+    "fused_after_arithmetic": (lambda a: ((a * 3 + 7) // 2).sum(-1) - a.amax(-1), lambda: (_ints(128, 4096, lo=-(1 << 20), hi=1 << 20),)),
+}
+
+
+@pytest.mark.parametrize("name", sorted(INTEGER_REDUCTIONS))
+def test_integer_reductions_are_exact(name):
+    """Sums, products and extrema of integer tensors: 64-bit exact in every code shape (rows in
+    registers, looped rows, split and single-sweep columns, the middle axis)."""
+    announce(f"compile integer reductions: {name}")
+    from torch._inductor.utils import run_and_get_code
+
+    fn, make = INTEGER_REDUCTIONS[name]
+    args = make()
+    torch._dynamo.reset()
+    got, codes = run_and_get_code(torch.compile(fn, dynamic=False), *args)
+    ref = fn(*args)
+    got = got if isinstance(got, (tuple, list)) else (got,)
+    ref = ref if isinstance(ref, (tuple, list)) else (ref,)
+    assert "mi::RedInt" in codes[0], "expected generated integer reductions"
+    for g, r in zip(got, ref):
+        assert g.shape == r.shape and g.dtype == r.dtype, (g.shape, r.shape, g.dtype, r.dtype)
+        assert torch.equal(g, r)
