@@ -1334,6 +1334,12 @@ class HipKernel(SIMDKernel):
         if integral:
             kind = f"mi::RedInt<mi::IntOp::{INT_REDUCTION_OP[reduction_type]}>"
             words = 2
+        elif reduction_type in INT_REDUCTION_OP and src_dtype == torch.float64:
+            # fp64 tensors reduce in fp64 (moments, arg-extrema and softmax statistics of fp64
+            # tensors are still computed in fp32)
+            kind = f"mi::RedF64<mi::IntOp::{INT_REDUCTION_OP[reduction_type]}>"
+            words = 2
+            integral = "f64"
         if self._load_mask:
             raise UnsupportedHipCodegen("reduction under a load mask")
         n = next(self.acc_ids)
@@ -1466,12 +1472,13 @@ class HipKernel(SIMDKernel):
 
     def _unpack_result(self, merged: str, reduction_type: str, dtype: torch.dtype, integral: bool = False):
         if integral:
+            wide_dtype, getter = (torch.float64, "GetSelfF64") if integral == "f64" else (torch.int64, "GetSelfInt")
             if self.mode == "colloop":
-                var = self._result_var(f"mi::col_get<VEC>({merged}, mi::GetSelfInt())", torch.int64)
+                var = self._result_var(f"mi::col_get<VEC>({merged}, mi::{getter}())", wide_dtype)
                 if isinstance(var, HipCSEVariable):
                     var.is_vec = True
                 return var
-            return self._result_var(f"{merged}", torch.int64)
+            return self._result_var(f"{merged}", wide_dtype)
         if self.mode == "colloop":
             # `merged` is an array of VEC states, one per column of the thread: results are vectors
             def vec_result(getter: str, dt: torch.dtype) -> CSEVariable:

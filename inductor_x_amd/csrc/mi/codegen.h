@@ -199,45 +199,55 @@ __device__ __forceinline__ float erf_f32(float x) {
   return (p * x) * __builtin_amdgcn_rcpf(q);
 }
 
-#define MI_UNARY_FN(NAME, EXPR)                                   \
+// Float and double forms: fp64 tensors are computed in fp64 (x is the element, already of its
+// own type); everything narrower has been widened to fp32 by the load.
+#define MI_UNARY_FN(NAME, FEXPR, DEXPR)                           \
   template <class A>                                              \
   __device__ __forceinline__ auto NAME(const A& a) {              \
-    return apply([](auto x) { return EXPR; }, a);                 \
+    return apply(                                                 \
+        [](auto x) {                                              \
+          if constexpr (std::is_same<decltype(x), double>::value) { \
+            return DEXPR;                                         \
+          } else {                                                \
+            return FEXPR;                                         \
+          }                                                       \
+        },                                                        \
+        a);                                                       \
   }
-MI_UNARY_FN(exp, __expf(static_cast<float>(x)))
-MI_UNARY_FN(exp2, __builtin_amdgcn_exp2f(static_cast<float>(x)))
-MI_UNARY_FN(expm1, ::expm1f(static_cast<float>(x)))
-MI_UNARY_FN(log, ::logf(static_cast<float>(x)))
-MI_UNARY_FN(log2, ::log2f(static_cast<float>(x)))
-MI_UNARY_FN(log10, ::log10f(static_cast<float>(x)))
-MI_UNARY_FN(log1p, ::log1pf(static_cast<float>(x)))
-MI_UNARY_FN(sqrt, ::sqrtf(static_cast<float>(x)))
-MI_UNARY_FN(rsqrt, ::rsqrtf(static_cast<float>(x)))
-MI_UNARY_FN(sin, ::sinf(static_cast<float>(x)))
-MI_UNARY_FN(cos, ::cosf(static_cast<float>(x)))
-MI_UNARY_FN(tan, ::tanf(static_cast<float>(x)))
-MI_UNARY_FN(tanh, tanh_f32(static_cast<float>(x)))
-MI_UNARY_FN(sinh, ::sinhf(static_cast<float>(x)))
-MI_UNARY_FN(cosh, ::coshf(static_cast<float>(x)))
-MI_UNARY_FN(asin, ::asinf(static_cast<float>(x)))
-MI_UNARY_FN(acos, ::acosf(static_cast<float>(x)))
-MI_UNARY_FN(atan, ::atanf(static_cast<float>(x)))
-MI_UNARY_FN(erf, erf_f32(static_cast<float>(x)))
-MI_UNARY_FN(erfc, ::erfcf(static_cast<float>(x)))
-MI_UNARY_FN(lgamma, ::lgammaf(static_cast<float>(x)))
-MI_UNARY_FN(floor, ::floorf(static_cast<float>(x)))
-MI_UNARY_FN(ceil, ::ceilf(static_cast<float>(x)))
-MI_UNARY_FN(trunc, ::truncf(static_cast<float>(x)))
-MI_UNARY_FN(round, ::nearbyintf(static_cast<float>(x)))
-MI_UNARY_FN(reciprocal, 1.0f / static_cast<float>(x))
-MI_UNARY_FN(sigmoid, __builtin_amdgcn_rcpf(1.0f + __expf(-static_cast<float>(x))))
-MI_UNARY_FN(isnan, (x != x))
-MI_UNARY_FN(isinf, (::isinf(static_cast<float>(x)) != 0))
-MI_UNARY_FN(signbit, (::signbit(static_cast<float>(x)) != 0))
-MI_UNARY_FN(abs, (x < 0 ? -x : x))
-MI_UNARY_FN(logical_not, (!x))
+MI_UNARY_FN(exp, __expf(static_cast<float>(x)), ::exp(x))
+MI_UNARY_FN(exp2, __builtin_amdgcn_exp2f(static_cast<float>(x)), ::exp2(x))
+MI_UNARY_FN(expm1, ::expm1f(static_cast<float>(x)), ::expm1(x))
+MI_UNARY_FN(log, ::logf(static_cast<float>(x)), ::log(x))
+MI_UNARY_FN(log2, ::log2f(static_cast<float>(x)), ::log2(x))
+MI_UNARY_FN(log10, ::log10f(static_cast<float>(x)), ::log10(x))
+MI_UNARY_FN(log1p, ::log1pf(static_cast<float>(x)), ::log1p(x))
+MI_UNARY_FN(sqrt, ::sqrtf(static_cast<float>(x)), ::sqrt(x))
+MI_UNARY_FN(rsqrt, ::rsqrtf(static_cast<float>(x)), 1.0 / ::sqrt(x))
+MI_UNARY_FN(sin, ::sinf(static_cast<float>(x)), ::sin(x))
+MI_UNARY_FN(cos, ::cosf(static_cast<float>(x)), ::cos(x))
+MI_UNARY_FN(tan, ::tanf(static_cast<float>(x)), ::tan(x))
+MI_UNARY_FN(tanh, tanh_f32(static_cast<float>(x)), ::tanh(x))
+MI_UNARY_FN(sinh, ::sinhf(static_cast<float>(x)), ::sinh(x))
+MI_UNARY_FN(cosh, ::coshf(static_cast<float>(x)), ::cosh(x))
+MI_UNARY_FN(asin, ::asinf(static_cast<float>(x)), ::asin(x))
+MI_UNARY_FN(acos, ::acosf(static_cast<float>(x)), ::acos(x))
+MI_UNARY_FN(atan, ::atanf(static_cast<float>(x)), ::atan(x))
+MI_UNARY_FN(erf, erf_f32(static_cast<float>(x)), ::erf(x))
+MI_UNARY_FN(erfc, ::erfcf(static_cast<float>(x)), ::erfc(x))
+MI_UNARY_FN(lgamma, ::lgammaf(static_cast<float>(x)), ::lgamma(x))
+MI_UNARY_FN(floor, ::floorf(static_cast<float>(x)), ::floor(x))
+MI_UNARY_FN(ceil, ::ceilf(static_cast<float>(x)), ::ceil(x))
+MI_UNARY_FN(trunc, ::truncf(static_cast<float>(x)), ::trunc(x))
+MI_UNARY_FN(round, ::nearbyintf(static_cast<float>(x)), ::nearbyint(x))
+MI_UNARY_FN(reciprocal, 1.0f / static_cast<float>(x), 1.0 / x)
+MI_UNARY_FN(sigmoid, __builtin_amdgcn_rcpf(1.0f + __expf(-static_cast<float>(x))), 1.0 / (1.0 + ::exp(-x)))
+MI_UNARY_FN(isnan, (x != x), (x != x))
+MI_UNARY_FN(isinf, (::isinf(static_cast<float>(x)) != 0), (::isinf(x) != 0))
+MI_UNARY_FN(signbit, (::signbit(static_cast<float>(x)) != 0), (::signbit(x) != 0))
+MI_UNARY_FN(abs, (x < 0 ? -x : x), ::fabs(x))
+MI_UNARY_FN(logical_not, (!x), (!x))
 // relu keeps NaN (a plain fmaxf would drop it)
-MI_UNARY_FN(relu, (x != x ? x : (x > 0 ? x : static_cast<decltype(x)>(0))))
+MI_UNARY_FN(relu, (x != x ? x : (x > 0 ? x : static_cast<decltype(x)>(0))), (x != x ? x : (x > 0 ? x : 0.0)))
 #undef MI_UNARY_FN
 
 template <class A>
@@ -253,10 +263,30 @@ __device__ __forceinline__ auto sign(const A& a) {
 // NaN-propagating, as torch.maximum / torch.minimum
 MI_BINARY_FN(maximum, (x != x ? x : (y != y ? static_cast<decltype(x)>(y) : (x > y ? x : static_cast<decltype(x)>(y)))))
 MI_BINARY_FN(minimum, (x != x ? x : (y != y ? static_cast<decltype(x)>(y) : (x < y ? x : static_cast<decltype(x)>(y)))))
-MI_BINARY_FN(pow, ::powf(static_cast<float>(x), static_cast<float>(y)))
-MI_BINARY_FN(atan2, ::atan2f(static_cast<float>(x), static_cast<float>(y)))
-MI_BINARY_FN(fmod, ::fmodf(static_cast<float>(x), static_cast<float>(y)))
-MI_BINARY_FN(copysign, ::copysignf(static_cast<float>(x), static_cast<float>(y)))
+#undef MI_BINARY_FN
+#define MI_BINARY_MATH(NAME, FFN, DFN)                                                         \
+  template <class A, class B>                                                                  \
+  __device__ __forceinline__ auto NAME(const A& a, const B& b) {                               \
+    return apply(                                                                              \
+        [](auto x, auto y) {                                                                   \
+          if constexpr (std::is_same<decltype(x), double>::value || std::is_same<decltype(y), double>::value) { \
+            return DFN(static_cast<double>(x), static_cast<double>(y));                        \
+          } else {                                                                             \
+            return FFN(static_cast<float>(x), static_cast<float>(y));                          \
+          }                                                                                    \
+        },                                                                                     \
+        a, b);                                                                                 \
+  }
+MI_BINARY_MATH(pow, ::powf, ::pow)
+MI_BINARY_MATH(atan2, ::atan2f, ::atan2)
+MI_BINARY_MATH(fmod, ::fmodf, ::fmod)
+MI_BINARY_MATH(copysign, ::copysignf, ::copysign)
+#undef MI_BINARY_MATH
+#define MI_BINARY_FN(NAME, EXPR)                                   \
+  template <class A, class B>                                      \
+  __device__ __forceinline__ auto NAME(const A& a, const B& b) {   \
+    return apply([](auto x, auto y) { return EXPR; }, a, b);       \
+  }
 // Python-style integer floor division and modulo
 MI_BINARY_FN(floordiv, ((x / y) - ((x % y != 0) && ((x < 0) != (y < 0)) ? 1 : 0)))
 MI_BINARY_FN(pymod, (((x % y) != 0 && ((x % y) < 0) != (y < 0)) ? (x % y) + y : (x % y)))
@@ -276,11 +306,20 @@ MI_BINARY_FN(remainder_f, (::fmodf(static_cast<float>(x), static_cast<float>(y))
 // the quotient); everything else is the IEEE division.
 template <class A, class B>
 __device__ __forceinline__ auto truediv(const A& a, const B& b) {
-  if constexpr (Tr<A>::n != 0 && Tr<B>::n == 0) {
+  if constexpr (Tr<A>::n != 0 && Tr<B>::n == 0 && !std::is_same<B, double>::value &&
+                !std::is_same<typename Tr<A>::elem, double>::value) {
     const float inv = 1.0f / static_cast<float>(b);
     return apply([inv](auto x) { return static_cast<float>(x) * inv; }, a);
   } else {
-    return apply([](auto x, auto y) { return static_cast<float>(x) / static_cast<float>(y); }, a, b);
+    return apply(
+        [](auto x, auto y) {
+          if constexpr (std::is_same<decltype(x), double>::value || std::is_same<decltype(y), double>::value) {
+            return static_cast<double>(x) / static_cast<double>(y);
+          } else {
+            return static_cast<float>(x) / static_cast<float>(y);
+          }
+        },
+        a, b);
   }
 }
 
@@ -705,45 +744,58 @@ struct RedWelford {
   }
 };
 
-// Exact 64-bit integer sum, product, maximum and minimum.  The state is one i64; where states
-// travel as float words (lane exchanges, LDS, the column workspace) it goes as its two 32-bit
-// halves, bit for bit: those paths only move words, they never do arithmetic on them.
+// Sum, product, maximum and minimum of 64-bit values, integer (exact) or double.  The state is
+// one 64-bit value; where states travel as float words (lane exchanges, LDS, the column
+// workspace) it goes as its two 32-bit halves, bit for bit: those paths only move words, they
+// never do arithmetic on them.  Extrema of doubles propagate NaN, as torch does.
 enum class IntOp { Sum, Prod, Max, Min };
-template <IntOp OP>
-struct RedInt {
-  typedef i64 V;  // the type a value is converted to before step()
-  typedef i64 T;
-  typedef i64 M;
+template <class VAL, IntOp OP>
+struct RedWide {
+  typedef VAL V;  // the type a value is converted to before step()
+  typedef VAL T;
+  typedef VAL M;
   static constexpr int W = 2;
+  static constexpr bool kFloat = std::is_same<VAL, double>::value;
   __device__ static T init() {
-    if constexpr (OP == IntOp::Sum) return 0;
-    if constexpr (OP == IntOp::Prod) return 1;
-    if constexpr (OP == IntOp::Max) return static_cast<i64>(0x8000000000000000ull);
-    return static_cast<i64>(0x7fffffffffffffffull);
+    if constexpr (OP == IntOp::Sum) return static_cast<VAL>(0);
+    if constexpr (OP == IntOp::Prod) return static_cast<VAL>(1);
+    if constexpr (kFloat) {
+      return OP == IntOp::Max ? -__builtin_inf() : __builtin_inf();
+    } else {
+      return OP == IntOp::Max ? static_cast<VAL>(0x8000000000000000ull) : static_cast<VAL>(0x7fffffffffffffffull);
+    }
   }
   __device__ static M empty() { return init(); }
   __device__ static M merge(M a, M b) {
     if constexpr (OP == IntOp::Sum) return a + b;
     if constexpr (OP == IntOp::Prod) return a * b;
+    if constexpr (kFloat) {
+      if (a != a) return a;
+      if (b != b) return b;
+    }
     if constexpr (OP == IntOp::Max) return a > b ? a : b;
     return a < b ? a : b;
   }
-  __device__ static T step(T s, i64 v, int) { return merge(s, v); }
-  __device__ static T first(i64 v, int) { return v; }
-  __device__ static T step_fast(T s, i64 v, int) { return merge(s, v); }
+  __device__ static T step(T s, VAL v, int) { return merge(s, v); }
+  __device__ static T first(VAL v, int) { return v; }
+  __device__ static T step_fast(T s, VAL v, int) { return merge(s, v); }
   __device__ static M finish(T s) { return s; }
   __device__ static M finish_n(T s, float) { return s; }
   __device__ static void enc(M m, float* w) {
-    const unsigned long long u = static_cast<unsigned long long>(m);
+    const unsigned long long u = __builtin_bit_cast(unsigned long long, m);
     w[0] = __builtin_bit_cast(float, static_cast<unsigned>(u & 0xffffffffull));
     w[1] = __builtin_bit_cast(float, static_cast<unsigned>(u >> 32));
   }
   __device__ static M dec(const float* w) {
     const unsigned long long lo = __builtin_bit_cast(unsigned, w[0]);
     const unsigned long long hi = __builtin_bit_cast(unsigned, w[1]);
-    return static_cast<i64>(lo | (hi << 32));
+    return __builtin_bit_cast(VAL, lo | (hi << 32));
   }
 };
+template <IntOp OP>
+using RedInt = RedWide<i64, OP>;
+template <IntOp OP>
+using RedF64 = RedWide<double, OP>;
 // The type values are converted to on their way into R::step: float unless R names another.
 template <class R, class = void>
 struct ValueOf {
@@ -1103,6 +1155,9 @@ struct GetSelf {
 };
 struct GetSelfInt {
   __device__ __forceinline__ i64 operator()(i64 m) const { return m; }
+};
+struct GetSelfF64 {
+  __device__ __forceinline__ double operator()(double m) const { return m; }
 };
 struct GetMean {
   __device__ __forceinline__ float operator()(const Moments& m) const { return m.mean; }

@@ -292,3 +292,31 @@ def test_integer_reductions_are_exact(name):
     for g, r in zip(got, ref):
         assert g.shape == r.shape and g.dtype == r.dtype, (g.shape, r.shape, g.dtype, r.dtype)
         assert torch.equal(g, r)
+
+
+FLOAT64_CASES = {
+    "elementwise": (lambda a: torch.exp(a) / (1 + a * a) + torch.tanh(a) + torch.erf(a) + torch.sqrt(a.abs())
+                    + torch.log1p(a.abs()) + a.pow(3) + torch.sigmoid(a) * torch.sin(a) + torch.atan2(a, a + 2),
+                    lambda: (_t(300, 1000, dtype=torch.float64),)),
+    "rounding_beyond_2_24": (lambda a: torch.floor(a * 1e9) + torch.round(a * 3e8) + torch.trunc(a * 7e10), lambda: (_t(64, 512, dtype=torch.float64),)),
+    "row_and_column_sums": (lambda a: (a.sum(-1), a.sum(0), a.mean(), a.amax(-1), a.amin(0)), lambda: (_t(300, 1000, dtype=torch.float64),)),
+    "long_rows_and_split_columns": (lambda a: (a.sum(-1), a.sum(0)), lambda: (_t(16, 70000, dtype=torch.float64),)),
+    "mixed_with_fp32": (lambda a, b: (a * b.double() + 1e-9).sum(-1) / b.double().abs().sum(-1), lambda: (_t(128, 2048, dtype=torch.float64), _t(128, 2048, seed=1))),
+}
+
+
+@pytest.mark.parametrize("name", sorted(FLOAT64_CASES))
+def test_float64_is_computed_in_float64(name):
+    """fp64 tensors keep fp64 arithmetic through generated kernels: elementwise functions and
+    sums / extrema agree with eager to 1e-12, far inside what an fp32 detour would give."""
+    announce(f"compile float64: {name}")
+    fn, make = FLOAT64_CASES[name]
+    args = make()
+    torch._dynamo.reset()
+    got = torch.compile(fn, dynamic=False)(*args)
+    ref = fn(*args)
+    got = got if isinstance(got, (tuple, list)) else (got,)
+    ref = ref if isinstance(ref, (tuple, list)) else (ref,)
+    for g, r in zip(got, ref):
+        assert g.dtype == torch.float64 and g.shape == r.shape
+        torch.testing.assert_close(g, r, rtol=1e-12, atol=1e-12 * max(1.0, float(r.abs().max())))
