@@ -1246,7 +1246,7 @@ class HipKernel(SIMDKernel):
     def store(self, name: str, index: sympy.Expr, value: CSEVariable, mode: StoreMode = None) -> None:
         var = self.args.output(name)
         index = self.prepare_indexing(index)
-        if mode is not None:
+        if mode not in (None, "atomic_add"):
             raise UnsupportedHipCodegen(f"store mode {mode}")
         kind = self.classify_index(index)
         if self.mode == "row":
@@ -1263,6 +1263,15 @@ class HipKernel(SIMDKernel):
             mask = "xmask" if self.inside_reduction else "(xmask && rl == 0)"
         else:
             mask = None
+        if mode == "atomic_add":
+            # accumulating scatter: several elements may land on one address, each adds atomically
+            if self.vec > 1 and kind != "uniform":
+                idx = self.index_to_vec_str(index)
+                line = f"mi::scatter_add_m<VEC>({var}, {idx}, {value}, {mask or 'true'});"
+            else:
+                line = f"mi::scatter_add_m<1>({var}, {self.index_to_str(index)}, {value}, {mask or 'true'});"
+            self.stores.writeline(DeferredLine(name, line))
+            return
         if kind == "contiguous":
             aligned = self.index_is_aligned(index) and self._buffer_aligned(name)
             ptr = f"{var} + ({self.index_to_str(index)})"

@@ -495,6 +495,50 @@ __device__ __forceinline__ void scatter_m(T* __restrict__ p, const I& idx, const
     if (static_cast<bool>(at(mask, i))) p[at(idx, i)] = static_cast<T>(at(val, i));
 }
 
+// Accumulating scatter (index_put / scatter_add / embedding gradients): one atomic per element.
+// 32- and 64-bit types use the memory atomics; narrower ones (bf16, fp16, 8- and 16-bit
+// integers) update their slice of the enclosing aligned 32-bit word in a compare-and-swap loop.
+template <class T, class A>
+__device__ __forceinline__ void atomic_accumulate(T* p, A v) {
+  if constexpr (std::is_same<T, float>::value || std::is_same<T, double>::value || std::is_same<T, int>::value ||
+                std::is_same<T, unsigned>::value) {
+    atomicAdd(p, static_cast<T>(v));
+  } else if constexpr (sizeof(T) == 8) {
+    atomicAdd(reinterpret_cast<unsigned long long*>(p), static_cast<unsigned long long>(static_cast<T>(v)));
+  } else {
+    static_assert(sizeof(T) < 4, "unexpected element size");
+    typedef typename RawBits<sizeof(T)>::type bits_t;
+    const unsigned long long a = reinterpret_cast<unsigned long long>(p);
+    unsigned* word = reinterpret_cast<unsigned*>(a & ~3ull);
+    const unsigned shift = static_cast<unsigned>(a & 3ull) * 8u;
+    const unsigned field = ((1u << (8 * sizeof(T))) - 1u) << shift;
+    unsigned seen = *word;
+    while (true) {
+      const bits_t cur_bits = static_cast<bits_t>((seen & field) >> shift);
+      T cur;
+      __builtin_memcpy(&cur, &cur_bits, sizeof(T));
+      T next;
+      if constexpr (std::is_integral<T>::value) {
+        next = static_cast<T>(cur + static_cast<T>(v));
+      } else {
+        next = from_f32<T>(to_f32(cur) + static_cast<float>(v));
+      }
+      bits_t next_bits;
+      __builtin_memcpy(&next_bits, &next, sizeof(T));
+      const unsigned want = (seen & ~field) | (static_cast<unsigned>(next_bits) << shift);
+      const unsigned was = atomicCAS(word, seen, want);
+      if (was == seen) break;
+      seen = was;
+    }
+  }
+}
+template <int N, class T, class I, class A, class M>
+__device__ __forceinline__ void scatter_add_m(T* __restrict__ p, const I& idx, const A& val, const M& mask) {
+#pragma unroll
+  for (int i = 0; i < (N < 1 ? 1 : N); ++i)
+    if (static_cast<bool>(at(mask, i))) atomic_accumulate(p + at(idx, i), at(val, i));
+}
+
 // ---------------------------------------------------------------------------
 // reduction kinds.  Thread-level state T (cheap per-element step), merge-level
 // state M (what travels between threads), W floats per M on the wire.
