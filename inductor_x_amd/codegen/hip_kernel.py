@@ -1265,11 +1265,9 @@ class HipKernel(SIMDKernel):
             mask = None
         if mode == "atomic_add":
             # accumulating scatter: several elements may land on one address, each adds atomically
-            if self.vec > 1 and kind != "uniform":
-                idx = self.index_to_vec_str(index)
-                line = f"mi::scatter_add_m<VEC>({var}, {idx}, {value}, {mask or 'true'});"
-            else:
-                line = f"mi::scatter_add_m<1>({var}, {self.index_to_str(index)}, {value}, {mask or 'true'});"
+            # (every one of the thread's VEC elements contributes, also when they share an address)
+            idx = self.index_to_str(index) if kind == "uniform" else self.index_to_vec_str(index)
+            line = f"mi::scatter_add_m<VEC>({var}, {idx}, {value}, {mask or 'true'});"
             self.stores.writeline(DeferredLine(name, line))
             return
         if kind == "contiguous":

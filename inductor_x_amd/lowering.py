@@ -112,13 +112,14 @@ GENERATE_LIST = [
     prims.maximum,
 ]
 
-# Ops whose Inductor lowering needs scans, sorts, atomics or device-side random
-# numbers: on GPU tensors they run as eager kernels.
+# Ops whose Inductor lowering needs scans, sorts or device-side random numbers: on GPU tensors
+# they run as eager kernels.  Scatters and index_put are generated (plain or atomic stores
+# through an indirect index); Inductor itself sends the reducing scatters it cannot express
+# (amax / amin / prod, 64-bit and boolean accumulation) to eager.
 FALLBACK_OPS = [
     aten.cumsum, aten.cumprod, aten.cummax, aten.cummin, aten.logcumsumexp,
     aten.sort, aten.topk,
-    aten.scatter, aten.scatter_add, aten.scatter_reduce, aten.index_put, aten._unsafe_index_put,
-    aten.index_add, aten.bucketize, aten.searchsorted,
+    aten.bucketize, aten.searchsorted,
 ]
 
 FALLBACK_LIST: list = []

@@ -148,3 +148,60 @@ def test_dropout_in_training_keeps_its_rate():
     torch._dynamo.reset()
     kept = torch.compile(lambda a: (F.dropout(a, 0.5, training=True) != 0).float().mean(), dynamic=False)(t(512, 512))
     assert abs(kept.item() - 0.5) < 0.02
+
+
+def _setitem(a, p, v):
+    b = a.clone()
+    b[p[:10]] = v[:10]
+    b[:, 3] = 7.0
+    b[p[10:20], 5] += 1.0
+    return b
+
+
+def _scatter_inputs():
+    g = torch.Generator(device="cpu").manual_seed(11)
+    a = torch.randn(1000, 64, generator=g).to(DEV)
+    i = torch.randint(0, 1000, (5000,), generator=g).to(DEV)
+    v = torch.randn(5000, 64, generator=g).to(DEV)
+    perm = torch.randperm(1000, generator=g).to(DEV)
+    return a, i, v, perm
+
+
+SCATTERS = {
+    # accumulate=True / *_add: memory atomics, any number of sources per destination
+    "index_put_accumulate": lambda a, i, v, p: a.index_put((i,), v * 2, accumulate=True),
+    "index_put_two_axes_accumulate": lambda a, i, v, p: a.index_put((i[:300] % 1000, i[300:600] % 64), v[:300, 0], accumulate=True),
+    "index_add_after_relu": lambda a, i, v, p: a.index_add(0, i, v.relu()),
+    "scatter_add_sixteen_sources_per_address": lambda a, i, v, p: a.scatter_add(1, (i[:1000].view(1000, 1) % 64).expand(1000, 16).contiguous(), v[:1000, :16]),
+    "scatter_reduce_sum": lambda a, i, v, p: a.scatter_reduce(0, i.view(5000, 1).expand(5000, 64).contiguous(), v, "sum"),
+    "scatter_reduce_amax": lambda a, i, v, p: a.scatter_reduce(0, i.view(5000, 1).expand(5000, 64).contiguous(), v, "amax"),
+    "histogram": lambda a, i, v, p: torch.zeros(1000, device=DEV).index_put((i,), torch.ones(5000, device=DEV), accumulate=True),
+    "int32_scatter_add": lambda a, i, v, p: torch.zeros(1000, 64, dtype=torch.int32, device=DEV).scatter_add(0, i.view(5000, 1).expand(5000, 64).contiguous(), (v * 4).to(torch.int32)),
+    "int64_scatter_add": lambda a, i, v, p: torch.zeros(1000, 64, dtype=torch.int64, device=DEV).scatter_add(0, i.view(5000, 1).expand(5000, 64).contiguous(), (v * 4).to(torch.int64)),
+    "bf16_index_add": lambda a, i, v, p: a.bfloat16().index_add(0, i[:200], v[:200].bfloat16()),
+    # one source per destination: plain stores through the index, bit-exact
+    "index_put_permutation": lambda a, i, v, p: a.index_put((p,), v[:1000] + 1),
+    "scatter_value": lambda a, i, v, p: a.scatter(0, p.view(1000, 1).expand(1000, 64).contiguous(), 3.0),
+    "scatter_source_permutation": lambda a, i, v, p: a.scatter(0, p.view(1000, 1).expand(1000, 64).contiguous(), v[:1000]),
+    "setitem_rows_column_and_increment": lambda a, i, v, p: _setitem(a, p, v),
+}
+
+
+@pytest.mark.parametrize("name", sorted(SCATTERS))
+def test_scatters_are_generated(name):
+    """index_put / index_add / scatter / scatter_add / scatter_reduce through torch.compile.  The
+    reference leaves all of them to eager (reference inductor_x/lowering.py:173-339); here they
+    are stores through an indirect index, atomic where sources can collide."""
+    announce(f"compile scatter: {name}")
+    fn = SCATTERS[name]
+    torch._dynamo.reset()
+    got = torch.compile(fn, dynamic=False)(*_scatter_inputs())
+    ref = fn(*_scatter_inputs())
+    assert got.shape == ref.shape and got.dtype == ref.dtype
+    if not ref.dtype.is_floating_point or name in ("index_put_permutation", "scatter_value", "scatter_source_permutation"):
+        assert torch.equal(got, ref)
+    elif ref.dtype == torch.bfloat16:
+        # the order of the additions differs: one bf16 ulp at the largest magnitudes
+        torch.testing.assert_close(got.float(), ref.float(), rtol=2e-2, atol=4e-2)
+    else:
+        torch.testing.assert_close(got, ref, rtol=1e-4, atol=1e-4)
