@@ -110,3 +110,8 @@ def apply_inductor_settings() -> None:
     from torch._inductor import config as inductor_config
 
     inductor_config.triton.unique_kernel_names = True
+    # one kernel that reduces the same tile along rows and along columns at once is a Triton
+    # code shape (torch/_inductor/codegen/simd.py codegen_mix_order_reduction); here the row
+    # reduction and the column reduction stay two kernels
+    if hasattr(inductor_config.triton, "mix_order_reduction"):
+        inductor_config.triton.mix_order_reduction = False

@@ -89,3 +89,29 @@ def test_transformer_block_training_step(dtype, dim):
         scale = max(q.grad.float().abs().max().item(), 1e-6)
         err = (p.grad.float() - q.grad.float()).abs().max().item()
         assert err <= (2e-3 if dtype == torch.float32 else 5e-2) * scale + 1e-6, f"{name}: {err} vs scale {scale}"
+
+
+def test_layernorm_training_at_a_size_where_inductor_would_mix_reduction_orders():
+    """From 5 M elements on, Inductor fuses a row reduction and a column reduction over the same
+    tile into one Triton-shaped kernel (torch/_inductor/scheduler.py MixOrderReduction.can_fuse);
+    this backend keeps them as a row kernel and a column sweep, and the step must compile and
+    agree with eager (input, weight and bias gradients of LayerNorm on [8192, 1024])."""
+    announce("compile layernorm forward+backward [8192,1024]")
+    torch.manual_seed(0)
+    x = torch.randn(8192, 1024, device=DEV, requires_grad=True)
+    w = torch.randn(1024, device=DEV, requires_grad=True)
+    b = torch.randn(1024, device=DEV, requires_grad=True)
+    dy = torch.randn(8192, 1024, device=DEV)
+
+    def step(x, w, b):
+        for t_ in (x, w, b):
+            t_.grad = None
+        y = F.layer_norm(x, (1024,), w, b)
+        y.backward(dy)
+        return y.detach(), x.grad.clone(), w.grad.clone(), b.grad.clone()
+
+    ref = step(x, w, b)
+    torch._dynamo.reset()
+    got = torch.compile(step, dynamic=False)(x, w, b)
+    for g, r in zip(got, ref):
+        torch.testing.assert_close(g, r, rtol=1e-4, atol=1e-4 * float(r.abs().max()))
