@@ -530,6 +530,11 @@ class HipKernel(SIMDKernel):
                 continue
             if getattr(n, "is_reduction", lambda: False)():
                 seen_reduction = True
+                # merging moments of slices (the second stage of a split variance) exists in the
+                # row and column-loop shapes only
+                data = getattr(getattr(n, "node", None), "data", None)
+                if getattr(data, "reduction_type", None) == "welford_combine":
+                    return False
                 continue
             if seen_reduction:
                 try:

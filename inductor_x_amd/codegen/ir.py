@@ -7,8 +7,8 @@ reference inductor_x/codegen/__init__.py:23); cutting a long reduced axis is lef
 to the kernel.  Here the replacement does the same for most reductions (scans keep
 Inductor's behaviour), with one exception the reference does not make: a reduction
 with fewer outputs than the GPU has compute units over a long range keeps
-Inductor's two-stage split, because a single kernel would occupy a handful of
-workgroups.  It only acts for GPU devices, so CPU compilation in the same process
+Inductor's two-stage split (whether the range is contiguous or strided), because a
+single kernel would occupy a handful of workgroups.  It only acts for GPU devices, so CPU compilation in the same process
 is untouched.
 """
 from __future__ import annotations
@@ -26,9 +26,12 @@ def num_splits(device, dst_dtype, src_dtype, inner_fn, ranges, reduction_ranges,
         hint, split = _original_num_splits(
             device, dst_dtype, src_dtype, inner_fn, ranges, reduction_ranges, reduction_type, reduction_numel, input_node
         )
-        # only rows that are contiguous along the reduced range: strided ones go to the column
-        # kernel, which cuts the range across workgroups itself
-        return (hint, split) if hint == ReductionHint.INNER else (ReductionHint.DEFAULT, 1)
+        # contiguous rows and strided ones alike: a strided range whose values are used again
+        # after the reduction (batch statistics of a channels-last tensor) becomes one
+        # column-loop kernel, which does not cut the range across workgroups
+        if __import__("os").environ.get("INDUCTOR_X_AMD_SPLIT_OUTER", "1") == "0" and hint != ReductionHint.INNER:
+            return ReductionHint.DEFAULT, 1
+        return hint, split
     return _original_num_splits(
         device, dst_dtype, src_dtype, inner_fn, ranges, reduction_ranges, reduction_type, reduction_numel, input_node
     )
