@@ -443,6 +443,19 @@ def row_grid(rounds: int) -> int:
     return min(rounds, hw.cu_count * 8 * int(os.environ.get("INDUCTOR_X_AMD_ROW_GRID_WAVES", _ROW_GRID_WAVES_OF_WORKGROUPS)))
 
 
+_pool = None
+
+
+def _compile_pool():
+    global _pool
+    if _pool is None:
+        from concurrent.futures import ThreadPoolExecutor
+
+        workers = int(os.environ.get("INDUCTOR_X_AMD_COMPILE_THREADS", "0")) or min(16, os.cpu_count() or 4)
+        _pool = ThreadPoolExecutor(max_workers=workers, thread_name_prefix="mi-hipcc")
+    return _pool
+
+
 class GeneratedKernel:
     """Run-time side of one generated kernel: compiles (or fetches) its code
     object on first use and launches it through the C-ABI launcher.  This is the
@@ -456,11 +469,17 @@ class GeneratedKernel:
         self.source = source
         self.mode = meta["mode"]
         self._fns: Optional[dict] = None
+        # hipcc starts as soon as the wrapper module defines the kernel, in a worker thread (the
+        # compiler is a subprocess), so the kernels of a graph build side by side instead of one
+        # after the other at their first launches (the reference compiles inside precompile(),
+        # reference inductor_x/npu_triton_heuristics.py:71-109, which Inductor's AsyncCompile
+        # calls from its worker pool)
+        self._pending = _compile_pool().submit(codecache.compile_source, source, label=name)
 
     def precompile(self) -> None:
         if self._fns is not None:
             return
-        path = codecache.compile_source(self.source, label=self.name)
+        path = self._pending.result()
         self.hsaco_path = path
         if _DRYRUN:
             self._fns = {}
