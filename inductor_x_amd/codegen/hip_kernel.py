@@ -54,6 +54,7 @@ from torch._inductor.ops_handler import StoreMode
 from torch._inductor.utils import sympy_subs
 from torch._inductor.virtualized import V
 from torch.utils._ordered_set import OrderedSet
+from torch._inductor.codegen.triton_utils import should_unwrap_unspec_arg
 from torch.utils._sympy.functions import FloorDiv, Identity, ModularIndexing
 from torch.utils._sympy.printers import ExprPrinter
 from torch.utils._sympy.value_ranges import ValueRanges
@@ -425,6 +426,13 @@ class HipCSEVariable(CSEVariable):
         if any_vec(args) or any_vec(list(kwargs.values())):
             self.is_vec = True
 
+
+# C type and struct code of a scalar kernel argument that stands for a 0-d CPU tensor
+SCALAR_ARG = {
+    torch.float16: ("float", "f"), torch.bfloat16: ("float", "f"), torch.float32: ("float", "f"),
+    torch.float64: ("double", "d"), torch.int64: ("mi::i64", "q"), torch.int32: ("int", "i"),
+    torch.int16: ("int", "i"), torch.int8: ("int", "i"), torch.uint8: ("int", "i"), torch.bool: ("int", "i"),
+}
 
 REDUCTION_KIND = {
     "sum": "mi::RedSum",
@@ -1156,6 +1164,12 @@ class HipKernel(SIMDKernel):
         indirect = self.is_indirect_indexing(index)
         index = self.prepare_indexing(index)
         dtype = V.graph.get_dtype(name)
+        if should_unwrap_unspec_arg(name):
+            # the value itself is the kernel argument
+            if dtype in (torch.float16, torch.bfloat16):
+                dtype = torch.float32
+            text = f"({var} != 0)" if dtype == torch.bool else str(var)
+            return self.cse.generate(self.loads, text, dtype=dtype)
         kind = self.classify_index(index)
         mask = self._load_mask_for(index)
         other = value_to_hip(self._load_other if self._load_mask else 0, dtype if dtype.is_floating_point else None)
@@ -1638,9 +1652,18 @@ class HipKernel(SIMDKernel):
     def _signature(self):
         """C parameter list, struct codes for packing, python call arguments."""
         _, call_args, signature, _ = self.args.python_argdefs()
+        call_args = [str(a) for a in call_args]
         params, codes = [], []
-        for arg in signature:
-            if isinstance(arg, TensorArg):
+        for pos, arg in enumerate(signature):
+            if isinstance(arg, TensorArg) and should_unwrap_unspec_arg(arg.buffer):
+                # a zero-dimensional CPU tensor among GPU operands (a Python number dynamo chose not
+                # to bake in, or a CPU scalar tensor): its value is a kernel argument, read on the
+                # host at launch (torch/_inductor/codegen/triton_utils.py:24-33, wrapper.py:2743-2747)
+                ctype, code = SCALAR_ARG[arg.dtype]
+                params.append(f"const {ctype} {arg.name}")
+                codes.append(code)
+                call_args[pos] = f"{call_args[pos]}.item()"
+            elif isinstance(arg, TensorArg):
                 const = "" if (arg.name.startswith("out_ptr") or arg.name.startswith("in_out_ptr")) else "const "
                 params.append(f"{const}{DTYPE_TO_HIP[arg.dtype]}* __restrict__ {arg.name}")
                 codes.append("P")
@@ -1651,7 +1674,7 @@ class HipKernel(SIMDKernel):
                 raise UnsupportedHipCodegen("Inductor-managed workspace arguments")
             else:
                 raise UnsupportedHipCodegen(f"kernel argument {type(arg).__name__}")
-        return params, "".join(codes), [str(a) for a in call_args]
+        return params, "".join(codes), call_args
 
     ROW_STASH_BUDGET = 144 * 1024
 

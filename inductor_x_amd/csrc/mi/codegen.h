@@ -137,9 +137,27 @@ __device__ __forceinline__ auto iota() {
   }
 }
 
+// A float that the target integer type cannot hold (a negative number to uint8) is undefined
+// in a direct conversion, and the optimiser may then garble neighbouring lanes of the vector as
+// well.  Narrow and unsigned integer targets are reached through a wider signed integer, which
+// wraps the way ATen's own conversion does (c10 static_cast_with_inter_type: uint8 via int64).
 template <class T, class A>
 __device__ __forceinline__ auto cast(const A& a) {
-  return apply([](auto x) { return static_cast<T>(x); }, a);
+  return apply(
+      [](auto x) {
+        typedef decltype(x) X;
+        if constexpr (std::is_floating_point<X>::value && std::is_integral<T>::value &&
+                      !std::is_same<T, bool>::value && (sizeof(T) < 4 || std::is_unsigned<T>::value)) {
+          if constexpr (sizeof(T) < 4) {
+            return static_cast<T>(static_cast<int>(x));
+          } else {
+            return static_cast<T>(static_cast<long long>(x));
+          }
+        } else {
+          return static_cast<T>(x);
+        }
+      },
+      a);
 }
 template <class T, class A>
 __device__ __forceinline__ auto bitcast(const A& a) {

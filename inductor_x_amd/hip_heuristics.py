@@ -495,7 +495,10 @@ class GeneratedKernel:
 
     @staticmethod
     def _raw(a):
-        return a.data_ptr() if hasattr(a, "data_ptr") else int(a)
+        if hasattr(a, "data_ptr"):
+            return a.data_ptr()
+        # numbers that are kernel arguments themselves (sizes, values of 0-d CPU tensors)
+        return a if isinstance(a, float) else int(a)
 
     def run(self, *args, xnumel: int, r0_numel: int = 1, stream: int = 0) -> None:
         self.precompile()

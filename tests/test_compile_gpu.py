@@ -537,3 +537,39 @@ def test_benchmark_helper(capsys):
         eager_us, compiled_us = benchmark_test(f, cf, (x,), name="relu_affine", times=5, repeat=4, graph=graph)
         assert eager_us > 0 and compiled_us > 0
     assert capsys.readouterr().out.count("benchmark_relu_affine") == 2
+
+
+@pytest.mark.parametrize("mode", ["reduce-overhead", "max-autotune-no-cudagraphs", "max-autotune"])
+def test_compile_modes(mode):
+    """torch.compile's other modes over the same backend: HIP-graph capture of the generated
+    launches (reduce-overhead) and autotuned library GEMMs around generated kernels, forward and
+    one training step."""
+    announce(f"compile mode {mode}")
+    torch.manual_seed(0)
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.l1 = torch.nn.Linear(512, 1024)
+            self.ln = torch.nn.LayerNorm(1024)
+            self.l2 = torch.nn.Linear(1024, 512)
+
+        def forward(self, x):
+            return x + self.l2(torch.nn.functional.gelu(self.ln(self.l1(x)))).softmax(-1)
+
+    net = Net().to(DEV)
+    x = torch.randn(256, 512, device=DEV)
+    ref = net(x)
+    torch._dynamo.reset()
+    compiled = torch.compile(net, mode=mode, dynamic=False)
+    with torch.no_grad():
+        for _ in range(4):  # graph capture happens after the warm-up calls
+            out = compiled(x).clone()
+    torch.testing.assert_close(out, ref, rtol=1e-5, atol=1e-6)
+    for _ in range(3):
+        net.zero_grad()
+        compiled(x).pow(2).mean().backward()
+    got = net.l1.weight.grad.clone()
+    net.zero_grad()
+    net(x).pow(2).mean().backward()
+    torch.testing.assert_close(got, net.l1.weight.grad, rtol=1e-4, atol=1e-7)

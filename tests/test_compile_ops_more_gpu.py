@@ -205,3 +205,64 @@ def test_scatters_are_generated(name):
         torch.testing.assert_close(got.float(), ref.float(), rtol=2e-2, atol=4e-2)
     else:
         torch.testing.assert_close(got, ref, rtol=1e-4, atol=1e-4)
+
+
+def _edge_inputs():
+    base = t(4097 * 33 + 7)
+    return {
+        "storage_offset_elementwise": (lambda a: a * 2 + 1, (base[3:3 + 4096 * 33].view(4096, 33),)),
+        "storage_offset_softmax": (lambda a: torch.softmax(a, -1), (base[1:1 + 4096 * 33].view(4096, 33),)),
+        # a zero-dimensional CPU tensor among GPU operands is a kernel argument, not a pointer
+        "cpu_scalar_tensors": (lambda a, s, h, i, b: (a * s + s + h).float() * i + b,
+                               (t(64, 64), torch.tensor(2.5), torch.tensor(1.5).bfloat16(), torch.tensor(3), torch.tensor(True))),
+        "python_numbers": (lambda a, s, k: a * s + k, (t(64, 64), 2.5, 3)),
+        "views_of_inputs_returned": (lambda a: (a.t(), a[::2], a + 1, a), (t(64, 48),)),
+        "channels_last_in_and_out": (lambda a: F.relu(a) * 2, (t(4, 8, 16, 16).to(memory_format=torch.channels_last),)),
+        "view_of_input_mutated": (lambda a: a[:, :8].mul_(3).sum() + a.sum(), (t(32, 32),)),
+        "integer_float_promotion": (lambda a, b: a + b * 1.5, (ti(64, 64), ti(64, 64, seed=1).int())),
+        "uint8_wraps": (lambda a: a + 200, (ti(64, 64, hi=255).to(torch.uint8),)),
+        "int8_wraps": (lambda a: a * 3, (ti(64, 64, lo=-128, hi=127).to(torch.int8),)),
+        "strided_slice_of_three_million": (lambda a: a.view(-1)[::3].sum(), (t(3, 1 << 20),)),
+        "expanded_input": (lambda a: a * 2 + 1, (t(1, 64).expand(128, 64),)),
+        "flipped_input": (lambda a: a.flip(1) + 1, (t(32, 48),)),
+        "no_rows": (lambda a: (a.sum(0), a.sum(1)), (torch.zeros(0, 16, device=DEV),)),
+        "nan_and_infinities_in_extrema": (lambda a: (a.amax(-1), a.amin(0), a.argmax(-1), torch.maximum(a, a.t())),
+                                          (torch.tensor([[1.0, float("nan"), 3], [float("inf"), 2, -float("inf")], [0, 0, 0]], device=DEV),)),
+        # negative and out-of-range floats to narrow integers wrap as ATen's conversion does
+        "float_to_integer_casts": (lambda a: (a.to(torch.int32), a.to(torch.int64), a.to(torch.uint8), a.to(torch.int8), a.bool(), a.to(torch.int16)),
+                                   (t(64, 64) * 100,)),
+    }
+
+
+EDGE_NAMES = ["storage_offset_elementwise", "storage_offset_softmax", "cpu_scalar_tensors", "python_numbers", "views_of_inputs_returned", "channels_last_in_and_out", "view_of_input_mutated", "integer_float_promotion", "uint8_wraps", "int8_wraps", "strided_slice_of_three_million", "expanded_input", "flipped_input", "no_rows", "nan_and_infinities_in_extrema", "float_to_integer_casts"]
+
+
+@pytest.mark.parametrize("name", EDGE_NAMES)
+def test_edge_inputs(name):
+    announce(f"compile edge inputs: {name}")
+    fn, args = _edge_inputs()[name]
+    args2 = tuple(a.clone() if isinstance(a, torch.Tensor) else a for a in args)
+    torch._dynamo.reset()
+    got = torch.compile(fn, dynamic=False)(*args)
+    ref = fn(*args2)
+    got = got if isinstance(got, (tuple, list)) else (got,)
+    ref = ref if isinstance(ref, (tuple, list)) else (ref,)
+    for g, r in zip(got, ref):
+        assert g.shape == r.shape and g.dtype == r.dtype and g.stride() == r.stride(), (g.shape, g.stride(), r.stride())
+        if r.dtype.is_floating_point:
+            torch.testing.assert_close(g, r, rtol=1e-5, atol=1e-5 * max(1.0, float(r[r.isfinite()].abs().max()) if r.isfinite().any() else 1.0), equal_nan=True)
+        else:
+            assert torch.equal(g, r)
+    for a, b in zip(args, args2):
+        if isinstance(a, torch.Tensor) and a.device.type == "cuda":
+            torch.testing.assert_close(a, b, rtol=1e-6, atol=1e-6, equal_nan=True)
+
+
+def test_more_than_two_to_the_31_elements():
+    """Indices and element counts switch to 64 bits."""
+    announce("compile 2^31 + 1024 int8 elements")
+    a = torch.ones((1 << 31) + 1024, device=DEV, dtype=torch.int8)
+    torch._dynamo.reset()
+    total, doubled = torch.compile(lambda a: ((a + 1).sum(dtype=torch.float32), a * 2), dynamic=False)(a)
+    assert total.item() == 2.0 * ((1 << 31) + 1024)
+    assert doubled[-1].item() == 2 and doubled[1 << 31].item() == 2 and int(doubled[:: 1 << 20].sum()) == 2 * 2049
