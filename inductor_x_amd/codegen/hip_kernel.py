@@ -56,6 +56,7 @@ from torch._inductor.virtualized import V
 from torch.utils._ordered_set import OrderedSet
 from torch._inductor.codegen.triton_utils import should_unwrap_unspec_arg
 from torch.utils._sympy.functions import FloorDiv, Identity, ModularIndexing
+from torch.utils._sympy.symbol import SymT, symbol_is_type
 from torch.utils._sympy.printers import ExprPrinter
 from torch.utils._sympy.value_ranges import ValueRanges
 
@@ -147,8 +148,34 @@ class HipExprPrinter(ExprPrinter):
         a, b = expr.args
         return f"mi::truediv({self.doprint(a)}, {self.doprint(b)})"
 
+    def _print_PythonMod(self, expr: sympy.Expr) -> str:
+        # the sign of the result follows the divisor (sizes that are only known at run time keep
+        # expressions like (x + s - 3) mod s in this form)
+        a, b = expr.args
+        return f"mi::pymod({self.doprint(a)}, {self.doprint(b)})"
+
     def _print_FloorToInt(self, expr: sympy.Expr) -> str:
         return f"mi::cast<mi::i64>(mi::floor({self.doprint(expr.args[0])}))"
+
+    _print_floor = _print_FloorToInt
+
+    def _print_CeilToInt(self, expr: sympy.Expr) -> str:
+        return f"mi::cast<mi::i64>(mi::ceil({self.doprint(expr.args[0])}))"
+
+    _print_ceiling = _print_CeilToInt
+
+    def _print_RoundToInt(self, expr: sympy.Expr) -> str:
+        return f"mi::cast<mi::i64>(mi::round({self.doprint(expr.args[0])}))"
+
+    def _print_TruncToFloat(self, expr: sympy.Expr) -> str:
+        return f"mi::trunc({self.doprint(expr.args[0])})"
+
+    def _print_FloatPow(self, expr: sympy.Expr) -> str:
+        x, y = expr.args
+        return f"mi::pow({self.doprint(x)}, {self.doprint(y)})"
+
+    def _print_Rational(self, expr: sympy.Expr) -> str:
+        return f"({float(expr.p)!r} / {float(expr.q)!r})"
 
     def _print_TruncToInt(self, expr: sympy.Expr) -> str:
         return f"mi::cast<mi::i64>(mi::trunc({self.doprint(expr.args[0])}))"
@@ -1668,8 +1695,16 @@ class HipKernel(SIMDKernel):
                 params.append(f"{const}{DTYPE_TO_HIP[arg.dtype]}* __restrict__ {arg.name}")
                 codes.append("P")
             elif isinstance(arg, SizeArg):
-                params.append(f"const mi::i64 {arg.name}")
-                codes.append("q")
+                expr = getattr(arg, "expr", None)
+                is_float = isinstance(expr, (float, sympy.Float)) or (
+                    isinstance(expr, sympy.Symbol) and symbol_is_type(expr, (SymT.FLOAT, SymT.UNBACKED_FLOAT))
+                )
+                if is_float:
+                    params.append(f"const double {arg.name}")
+                    codes.append("d")
+                else:
+                    params.append(f"const mi::i64 {arg.name}")
+                    codes.append("q")
             elif isinstance(arg, WorkspaceArg):
                 raise UnsupportedHipCodegen("Inductor-managed workspace arguments")
             else:

@@ -266,3 +266,24 @@ def test_more_than_two_to_the_31_elements():
     total, doubled = torch.compile(lambda a: ((a + 1).sum(dtype=torch.float32), a * 2), dynamic=False)(a)
     assert total.item() == 2.0 * ((1 << 31) + 1024)
     assert doubled[-1].item() == 2 and doubled[1 << 31].item() == 2 and int(doubled[:: 1 << 20].sum()) == 2 * 2049
+
+
+@pytest.mark.parametrize("name", sorted(set(CASES) - {"data_dependent_sizes"}))
+def test_more_operator_kinds_symbolic_sizes(name):
+    """The same graphs with every size symbolic (index expressions keep PythonMod, floor and
+    ceiling forms that static shapes fold away)."""
+    announce(f"compile op sweep 2, dynamic=True: {name}")
+    fn, make = CASES[name]
+    torch._dynamo.reset()
+    got = torch.compile(fn, dynamic=True)(*make())
+    _compare(got, fn(*make()), name)
+
+
+def test_roll_and_flip_one_artefact_for_several_shapes():
+    announce("compile roll/flip, dynamic shapes")
+    fn = lambda a: torch.flip(a, [1]) + torch.roll(a, 3, 0) + torch.flip(a, [0, 1]) + torch.roll(a, (-2, 5), (0, 1))  # noqa: E731
+    torch._dynamo.reset()
+    compiled = torch.compile(fn, dynamic=True)
+    for shape in ((33, 70), (17, 40), (64, 64)):
+        a = t(*shape)
+        assert torch.equal(compiled(a), fn(a))
