@@ -1395,6 +1395,13 @@ class HipKernel(SIMDKernel):
             integral = "f64"
         if self._load_mask:
             raise UnsupportedHipCodegen("reduction under a load mask")
+        if self.mode == "row" and self.vec > 1:
+            # a value that does not vary over the thread's VEC elements (it was computed from
+            # indices a whole vector shares) still counts once per element
+            def lanes(v):
+                return v if (isinstance(v, HipCSEVariable) and v.is_vec) else f"mi::splat<VEC>({v})"
+
+            value = tuple(lanes(v) for v in value) if isinstance(value, tuple) else lanes(value)
         n = next(self.acc_ids)
         if reduction_type == "welford_combine":
             # inputs are (mean, m2, weight) per element: the second stage of a split variance

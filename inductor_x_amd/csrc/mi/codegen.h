@@ -59,6 +59,20 @@ __device__ __forceinline__ auto at(const A& a, int i) {
   }
 }
 
+// A value that is the same for all N elements of a thread, as N lanes (no-op for vectors): a
+// reduction must count it once per element.
+template <int N, class A>
+__device__ __forceinline__ auto splat(const A& a) {
+  if constexpr (Tr<A>::n != 0 || N <= 1) {
+    return a;
+  } else {
+    V<A, N> r;
+#pragma unroll
+    for (int i = 0; i < N; ++i) r.v[i] = a;
+    return r;
+  }
+}
+
 template <int... Ns>
 struct MaxN;
 template <int A>

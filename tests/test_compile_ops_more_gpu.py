@@ -287,3 +287,97 @@ def test_roll_and_flip_one_artefact_for_several_shapes():
     for shape in ((33, 70), (17, 40), (64, 64)):
         a = t(*shape)
         assert torch.equal(compiled(a), fn(a))
+
+
+REPEATED_VALUES = {
+    # the reduced value is the same for a whole vector of reduced positions (it depends on
+    # r // 8 only): it must still be counted once per position
+    "gather_of_expanded_index": (lambda a, i: torch.gather(a, 1, i[:, None].expand(-1, 8) % a.shape[1]).sum(), lambda: (t(100, 16), ti(100, hi=100))),
+    "sum_of_repeat_interleave": (lambda a: a.repeat_interleave(8, 1).sum(-1), lambda: (t(64, 32),)),
+    "max_and_mean_of_expanded": (lambda a: (a[:, :, None].expand(32, 16, 16).reshape(32, 256).amax(-1), a[:, :, None].expand(32, 16, 16).reshape(32, 256).mean(-1)), lambda: (t(32, 16),)),
+    "softmax_over_repeated_columns": (lambda a: torch.softmax(a.repeat_interleave(4, 1), -1), lambda: (t(16, 12000),)),
+    "variance_of_repeated_columns": (lambda a: a.repeat_interleave(16, 1).var(-1), lambda: (t(64, 64),)),
+}
+
+
+@pytest.mark.parametrize("name", sorted(REPEATED_VALUES))
+def test_row_reductions_of_values_shared_by_a_vector(name):
+    announce(f"compile reductions of repeated values: {name}")
+    fn, make = REPEATED_VALUES[name]
+    torch._dynamo.reset()
+    got = torch.compile(fn, dynamic=False)(*make())
+    ref = fn(*make())
+    got = got if isinstance(got, (tuple, list)) else (got,)
+    ref = ref if isinstance(ref, (tuple, list)) else (ref,)
+    for g, r in zip(got, ref):
+        torch.testing.assert_close(g, r, rtol=1e-4, atol=1e-4 * max(1.0, float(r.abs().max())))
+
+
+def _custom_square(a):
+    class Square(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x):
+            ctx.save_for_backward(x)
+            return x * x
+
+        @staticmethod
+        def backward(ctx, g):
+            (x,) = ctx.saved_tensors
+            return 2 * x * g
+
+    return Square.apply(a).sin()
+
+
+def _with_graph_break(a):
+    b = a * 2
+    print("", end="")  # forces a graph break
+    return (b.relu() + 1).sum(-1)
+
+
+BACKWARD_CASES = {
+    "softmax": (lambda a: torch.softmax(a, -1) * a, lambda: (t(128, 1000),), False, 1e-4),
+    "softmax_long_rows": (lambda a: torch.softmax(a, -1) * a, lambda: (t(16, 40000),), False, 1e-4),
+    "log_softmax_dim0": (lambda a: torch.log_softmax(a, 0) * a, lambda: (t(1000, 128),), False, 1e-4),
+    "logsumexp_var_std": (lambda a: torch.logsumexp(a, -1) + a.var(-1) + a.std(0).sum(), lambda: (t(256, 300),), False, 1e-4),
+    "layernorm_symbolic_sizes": (lambda a, w, b: F.layer_norm(a, (a.shape[-1],), w, b), lambda: (t(64, 100, 256), t(256, seed=1), t(256, seed=2)), True, 1e-4),
+    "rmsnorm_bf16": (lambda a, w: (a.float() * torch.rsqrt(a.float().pow(2).mean(-1, keepdim=True) + 1e-6)).to(a.dtype) * w,
+                     lambda: (t(512, 2048, dtype=torch.bfloat16), t(2048, dtype=torch.bfloat16, seed=1)), False, 3e-2),
+    "gelu_mlp_symbolic_sizes": (lambda a, w1, w2: F.gelu(a @ w1) @ w2, lambda: (t(100, 64), t(64, 256, seed=1), t(256, 64, seed=2)), True, 1e-3),
+    "extrema": (lambda a: a.amax(-1).sum() + a.amin(0).sum() + a.max(), lambda: (t(100, 200),), False, 1e-4),
+    "cumsum": (lambda a: a.cumsum(-1) * a, lambda: (t(64, 128),), False, 1e-4),
+    "index_and_gather": (lambda a, i: a[i].pow(2) + torch.gather(a, 1, i[:, None].expand(-1, 8) % a.shape[1]).sum(), lambda: (t(100, 16), ti(100, hi=100)), False, 1e-4),
+    "embedding_mean": (lambda w, i: F.embedding(i, w).mean(1), lambda: (t(1000, 64), ti(32, 20, hi=1000)), False, 1e-4),
+    "where_clamp_sqrt": (lambda a, b: torch.where(a > 0, a * b, b.clamp(-1, 1)) + a.abs().sqrt(), lambda: (t(128, 128), t(128, 128, seed=1)), False, 1e-4),
+    "conv_batchnorm_relu": (lambda a, w, g, b: F.relu(F.batch_norm(F.conv2d(a, w, padding=1), None, None, g, b, training=True)),
+                            lambda: (t(8, 16, 32, 32), t(16, 16, 3, 3, seed=1), t(16, seed=2), t(16, seed=3)), False, 1e-3),
+    "six_axes_permuted": (lambda a: a.permute(5, 3, 1, 4, 2, 0).contiguous() * 2 + a.permute(5, 3, 1, 4, 2, 0).sum((0, 2), keepdim=True), lambda: (t(2, 3, 4, 5, 6, 7),), False, 1e-4),
+    "broadcast_over_four_axes": (lambda a, b, c: (a[:, None, :, None] * b[None, :, None, :] + c).sum((1, 3)), lambda: (t(8, 16), t(12, 20), t(8, 12, 16, 20)), False, 1e-4),
+    "autocast_bf16": (lambda a, w: torch.autocast("cuda", dtype=torch.bfloat16)(lambda: F.layer_norm(F.gelu(a @ w), (256,)).float())(), lambda: (t(128, 64), t(64, 256, seed=1)), False, 3e-2),
+    "custom_autograd_function": (_custom_square, lambda: (t(64, 64),), False, 1e-4),
+    "graph_break": (_with_graph_break, lambda: (t(64, 64),), False, 1e-4),
+    "one_element": (lambda a: a.sum() * a.mean() + a[0, 0], lambda: (t(1, 1),), False, 1e-4),
+    "sixteen_million_wide_rows": (lambda a: a.sum(-1) + a.amax(-1), lambda: (t(2, (1 << 24) + 5),), False, 1e-3),
+}
+
+
+@pytest.mark.parametrize("name", sorted(BACKWARD_CASES))
+def test_forward_and_backward(name):
+    """Forward value and every input gradient through torch.compile against eager autograd."""
+    announce(f"compile forward+backward: {name}")
+    fn, make, dynamic, tol = BACKWARD_CASES[name]
+    a1 = [a.clone().requires_grad_() if a.is_floating_point() else a for a in make()]
+    a2 = [a.clone().requires_grad_() if a.is_floating_point() else a for a in make()]
+    torch._dynamo.reset()
+
+    def total(out):
+        return sum(o.float().sum() for o in (out if isinstance(out, (tuple, list)) else (out,)))
+
+    got = total(torch.compile(fn, dynamic=dynamic)(*a1))
+    ref = total(fn(*a2))
+    got.backward()
+    ref.backward()
+    torch.testing.assert_close(got, ref, rtol=tol, atol=tol * max(1.0, abs(ref.item())))
+    for x, y in zip(a1, a2):
+        if x.is_floating_point():
+            scale = max(1.0, float(y.grad.float().abs().max()))
+            torch.testing.assert_close(x.grad.float(), y.grad.float(), rtol=10 * tol, atol=10 * tol * scale)
