@@ -1264,6 +1264,10 @@ class HipKernel(SIMDKernel):
         if dtype in (torch.float16, torch.bfloat16):
             line = f"mi::cast<float>({line})"
             dtype = torch.float32
+        # under a guard that differs between the thread's elements the result differs too, also
+        # when every element reads the same address
+        if isinstance(self._load_mask, HipCSEVariable) and self._load_mask.is_vec:
+            is_vec = True
         # a load whose address or guard is itself computed must follow that computation
         buf = self.compute if (indirect or self._load_mask) else self.loads
         out = self.cse.generate(buf, line, dtype=dtype)

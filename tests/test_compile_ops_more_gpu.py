@@ -381,3 +381,21 @@ def test_forward_and_backward(name):
         if x.is_floating_point():
             scale = max(1.0, float(y.grad.float().abs().max()))
             torch.testing.assert_close(x.grad.float(), y.grad.float(), rtol=10 * tol, atol=10 * tol * scale)
+
+
+def test_guarded_load_of_a_shared_address_is_lane_varying():
+    """Inside a concatenation the guard differs between the elements of a thread's vector while
+    the guarded index load reads one address for all of them: the loaded index is then
+    lane-varying, and what it addresses is gathered (this graph did not compile)."""
+    announce("compile index_select -> cat -> where -> prod over the leading axis")
+
+    def fn(x, idx):
+        y = x.index_select(1, idx)
+        y = torch.cat([y, y * 0.5 + 1], 2)
+        y = torch.where(y > -0.45, y, -y * 0.5)
+        return y.clamp(-1.1, 1.1).prod(0)
+
+    x, idx = t(33, 16, 512), ti(40, hi=16)
+    torch._dynamo.reset()
+    got = torch.compile(fn, dynamic=False)(x, idx)
+    torch.testing.assert_close(got, fn(x, idx), rtol=1e-4, atol=1e-5)
