@@ -1928,8 +1928,9 @@ class HipKernel(SIMDKernel):
             raise UnsupportedHipCodegen("column kernel without a reduction")
         ct, rl, vec = self.col_ct, self.col_rl, self.vec
         max_words = max(c.words for c in self.col_reductions)
-        extra = [f"float* __restrict__ ws", f"const {idx_t} xnumel", f"const {idx_t} rnumel",
-                 "const int rows_per_split", "const int nsplit"]
+        extra = [f"float* __restrict__ ws", f"const {idx_t} xnumel", f"const {idx_t} rnumel", "const int nsplit"]
+        # rows handed to a thread between two looks at the loop counter
+        unroll = int(os.environ.get("INDUCTOR_X_AMD_COL_UNROLL", "4"))
         plist = ", ".join(params + extra)
         # ---- pass 1, and the same sweep finishing in place ("direct") for launches where one
         # workgroup per column tile already fills the GPU: no workspace, no second kernel
@@ -1945,8 +1946,12 @@ class HipKernel(SIMDKernel):
                 src.writeline(f"const {idx_t} xindex = (static_cast<{idx_t}>(blockIdx.x) * CT + ct) * VEC;")
                 src.writeline("const int split = blockIdx.y;")
                 src.writeline("const bool xmask = xindex < xnumel;")
-                src.writeline(f"const {idx_t} r_begin = static_cast<{idx_t}>(split) * rows_per_split;")
-                src.writeline(f"const {idx_t} r_end = (r_begin + rows_per_split < rnumel) ? r_begin + rows_per_split : rnumel;")
+                # The reduced axis is dealt out in batches of RL * UNR consecutive rows, batch b
+                # to split b % nsplit: the workgroups of a column tile read one contiguous
+                # stretch between them at any moment, and any split count is valid.
+                src.writeline(f"constexpr int UNR = {unroll};")
+                src.writeline(f"const {idx_t} batch_ = RL * UNR;")
+                src.writeline(f"const {idx_t} full_ = rnumel / batch_;")
                 for c in self.col_reductions:
                     kind = c.cxx
                     src.writeline(f"mi::ColAcc<{kind}, VEC> {c.acc};")
@@ -1954,10 +1959,23 @@ class HipKernel(SIMDKernel):
                 src.writeline("if (xmask) {")
                 with src.indent():
                     src.splice(self._entry_code(self.x_entries))
-                    src.writeline(f"#pragma unroll {int(os.environ.get('INDUCTOR_X_AMD_COL_UNROLL', '4'))}")
-                    src.writeline(f"for ({idx_t} r0_index = r_begin + rl; r0_index < r_end; r0_index += RL) {{")
+                    src.writeline(f"{idx_t} b_ = split;")
+                    src.writeline("for (; b_ < full_; b_ += nsplit) {")
                     with src.indent():
-                        src.splice(self.partial_body)
+                        src.writeline("#pragma unroll")
+                        src.writeline("for (int u_ = 0; u_ < UNR; ++u_) {")
+                        with src.indent():
+                            src.writeline(f"const {idx_t} r0_index = b_ * batch_ + u_ * RL + rl;")
+                            src.splice(self.partial_body)
+                        src.writeline("}")
+                    src.writeline("}")
+                    # the last, partly filled batch
+                    src.writeline("if (b_ == full_) {")
+                    with src.indent():
+                        src.writeline(f"for ({idx_t} r0_index = full_ * batch_ + rl; r0_index < rnumel; r0_index += RL) {{")
+                        with src.indent():
+                            src.splice(self.partial_body)
+                        src.writeline("}")
                     src.writeline("}")
                 src.writeline("}")
                 for c in self.col_reductions:
@@ -2030,9 +2048,9 @@ class HipKernel(SIMDKernel):
             src.splice(self._final_indexing_code())
             src.splice(self.final_body)
         src.writeline("}")
-        meta.update({"ct": ct, "rl": rl, "cpw": cpw, "sl": sl, "ws_words": self.ws_words,
+        meta.update({"ct": ct, "rl": rl, "cpw": cpw, "sl": sl, "ws_words": self.ws_words, "col_unroll": unroll,
                      "lds_partial": (rl // 2) * ct * vec * max_words * 4})
-        return codes + "P" + idx_code + idx_code + "ii"
+        return codes + "P" + idx_code + idx_code + "i"
 
     def _final_indexing_code(self) -> IndentedBuffer:
         """Range variables of the kept axis for the final kernel (one column per

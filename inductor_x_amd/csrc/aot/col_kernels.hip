@@ -9,8 +9,8 @@ using namespace mi;
 #define COL_PARTIAL_VARIANT(CT, RL, UNROLL)                                                   \
   extern "C" __global__ __launch_bounds__(CT* RL) void                                        \
       col_mean_var_argmax_partial_f32_c##CT##_r##RL##_u##UNROLL(                              \
-          const float* x, float* part, int rows, int cols, int rows_per_split, int nsplit) {  \
-    col_stats_partial<CT, RL, UNROLL>(x, part, rows, cols, rows_per_split, nsplit);           \
+          const float* x, float* part, int rows, int cols, int nsplit) {                      \
+    col_stats_partial<CT, RL, UNROLL>(x, part, rows, cols, nsplit);                           \
   }
 
 COL_PARTIAL_VARIANT(128, 2, 4)

@@ -345,7 +345,7 @@ def split_reduction_plan(
     cols: int,
     elem_bytes: int = 4,
     vgprs: int = 48,
-    unroll: int = 4,
+    unroll: int = 8,
     hw: Optional[config.Hardware] = None,
     max_workspace_frac: float = 0.05,
 ) -> SplitPlan:
@@ -357,7 +357,10 @@ def split_reduction_plan(
     inductor_x/codegen/split_tiling.py:159-182).  Here:
       1. the number of wavefronts wanted per CU comes from the in-flight-bytes
          target and the kernel's register budget (waves_per_cu_target); measured
-         on MI355X at [65536, 512]: 8 wavefronts per CU (22.5 us) beat 16 (25.3 us);
+         on MI355X at [65536, 512], first pass alone: the same bytes in flight from
+         half as many wavefronts with twice the unrolled batch (4 per CU, 2 x 8
+         loads each: 22.3 us) do as well as 8 per CU with 2 x 4 loads (22.3 us) and
+         better than 16 per CU (25.3 us), and fewer wavefronts mean fewer partials;
       2. a workgroup spans up to 512 kept elements (128 threads x float4) and
          as many row lanes as make up that many wavefronts - big workgroups mean
          few partials, so little workspace traffic;
@@ -523,17 +526,18 @@ class GeneratedKernel:
         else:
             import torch
 
-            nsplit, rps = split_factor(rnumel, xnumel, m["ct"], m["rl"], m["vec"], words=m["ws_words"])
+            nsplit, _ = split_factor(rnumel, xnumel, m["ct"], m["rl"], m["vec"], unroll=m.get("col_unroll", 4),
+                                     words=m["ws_words"])
             if nsplit == 1:
                 # one sweep that finishes in place: no workspace, no second kernel
                 self._fns["direct"].launch(
-                    m["signature"], raw + (0, xnumel, rnumel, rnumel, 1), (cdiv(xnumel, m["ct"] * m["vec"]), 1, 1),
+                    m["signature"], raw + (0, xnumel, rnumel, 1), (cdiv(xnumel, m["ct"] * m["vec"]), 1, 1),
                     (m["block"],), stream, m["lds_partial"],
                 )
                 return
             dev = next(a.device for a in args if hasattr(a, "device"))
             ws = torch.empty(m["ws_words"] * nsplit * xnumel, dtype=torch.float32, device=dev)
-            full = raw + (ws.data_ptr(), xnumel, rnumel, rps, nsplit)
+            full = raw + (ws.data_ptr(), xnumel, rnumel, nsplit)
             self._fns["partial"].launch(
                 m["signature"], full, (cdiv(xnumel, m["ct"] * m["vec"]), nsplit, 1), (m["block"],), stream,
                 m["lds_partial"],

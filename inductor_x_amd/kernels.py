@@ -143,7 +143,7 @@ def _col_partial_launcher() -> CachingLauncher:
         for ct, rl, u in _COL_PARTIAL_VARIANTS
     ]
     return CachingLauncher(
-        "col_mean_var_argmax_partial_f32", codecache.aot_source("col_kernels.hip"), "PPiiii", cfgs, prefer_intree=True
+        "col_mean_var_argmax_partial_f32", codecache.aot_source("col_kernels.hip"), "PPiii", cfgs, prefer_intree=True
     )
 
 
@@ -342,7 +342,7 @@ def col_mean_var_argmax(
     st = _stream()
     lp._launch(
         ip,
-        (x.data_ptr(), workspace.data_ptr(), rows, cols, plan.rows_per_split, plan.nsplit),
+        (x.data_ptr(), workspace.data_ptr(), rows, cols, plan.nsplit),
         (plan.col_tiles, plan.nsplit, 1),
         st,
     )
