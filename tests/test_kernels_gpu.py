@@ -194,6 +194,40 @@ def test_col_stats_variants(K, O, ct, rl, u):
         _check_col(K, O, x, plan=plan, final_variant=fv)
 
 
+@pytest.mark.parametrize("rows", [1, 7, 16, 17, 64, 65, 4099])
+@pytest.mark.parametrize("nsplit", [1, 7, 64])
+def test_col_stats_batch_cyclic_row_order(K, O, rows, nsplit):
+    """Rows go to the splits in batches of RL * UNROLL, batch b to split b % nsplit: fewer rows than
+    one batch, a partly filled last batch, whole batches only, and more splits than batches (splits
+    without any row), with NaNs and ties planted so the rare re-walk of a column runs too."""
+    from inductor_x_amd.hip_heuristics import SplitPlan, cdiv
+
+    announce(f"col stats cyclic rows={rows} nsplit={nsplit}")
+    torch.manual_seed(rows * 100 + nsplit)
+    cols = 64
+    x = torch.randn(rows, cols)
+    if rows > 16:
+        x[rows - 1, 3] = float("nan")
+        x[5, 3] = float("nan")  # first NaN wins -> 5
+        x[rows - 2, 4] = 9.0
+        x[2, 4] = 9.0  # tie -> 2
+        x[1, 5] = float("inf")
+        x[9, 5] = float("-inf")  # inf - inf makes the shifted sum NaN without a NaN sample
+    for ct, rl, u in [(128, 2, 8), (128, 4, 4), (64, 8, 4), (16, 16, 4)]:
+        plan = SplitPlan(ct, rl, u, nsplit, cdiv(rows, nsplit), cdiv(cols, ct * 4))
+        mean, var, arg = K.col_mean_var_argmax(x.to(DEV), 0.0, plan=plan)
+        assert np.array_equal(arg.cpu().numpy(), torch.argmax(x, 0).numpy()), (ct, rl, u)
+        assert np.array_equal(arg.cpu().numpy(), O.col_mean_var_argmax(x.numpy(), 0.0)[2])
+        v_ref, m_ref = torch.var_mean(x.double(), 0, unbiased=False)
+        ok = torch.isfinite(m_ref)
+        # same bar as _check_col: 1e-5 of the column's scale for the (near-zero) means, 1e-5 relative for var
+        scale = v_ref[ok].sqrt().clamp_min(1e-15)
+        assert ((mean.cpu().double()[ok] - m_ref[ok]).abs() <= 1e-5 * torch.maximum(m_ref[ok].abs(), scale) + 1e-12).all()
+        assert torch.allclose(var.cpu().double()[ok], v_ref[ok], rtol=1e-5, atol=1e-12)
+        if rows > 16:
+            assert torch.isnan(mean.cpu()[3]) and torch.isnan(var.cpu()[3])
+
+
 def test_col_stats_invariants_full_size(K):
     """BASELINE shape: var(x + c) == var(x), var(k x) == k^2 var(x), argmax unchanged."""
     announce("col stats invariants 65536x512")
