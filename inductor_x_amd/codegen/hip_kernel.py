@@ -29,6 +29,7 @@ import dataclasses
 import itertools
 import math
 import os
+import re
 from typing import Any, Optional, Sequence, Union
 
 import sympy
@@ -1581,6 +1582,27 @@ class HipKernel(SIMDKernel):
         self._result_defs = []
         return defs
 
+    def _plan_col_pipeline(self) -> Optional[tuple[str, list[str], str]]:
+        """(entry text, loaded variable names, loads text, rest text) when the loop body of a column
+        sweep starts with nothing but plain vector loads: those can be issued one batch ahead of
+        the folds that use them.  Anything else in the loads (guards, stashes, a load through a
+        loaded index) keeps the plain loop."""
+        if os.environ.get("INDUCTOR_X_AMD_COL_PIPELINE", "1") == "0":
+            return None
+        lines = [l.strip() for l in self.loads.getvalue().splitlines() if l.strip()]
+        names = []
+        for line in lines:
+            m = re.fullmatch(r"auto (tmp\d+) = mi::vload(?:_u)?<[^;]*\);", line)
+            if m is None or re.search(r"\btmp\d+\b", line.split("=", 1)[1]):
+                return None
+            names.append(m.group(1))
+        if not 1 <= len(names) <= 4:
+            return None
+        rest = IndentedBuffer()
+        rest.splice(self.compute)
+        rest.splice(self.stores)
+        return (self._entry_code(self.r_entries).getvalue(), names, self.loads.getvalue(), rest.getvalue())
+
     def codegen_body(self) -> None:
         if not (self.loads or self.compute or self.stores or self.row_loop_accs or self._result_defs or self.red_stores):
             return
@@ -1591,6 +1613,7 @@ class HipKernel(SIMDKernel):
                 self.partial_body.splice(self.loads)
                 self.partial_body.splice(self.compute)
                 self.partial_body.splice(self.stores)
+                self._col_pipeline = self._plan_col_pipeline()
                 self.phase_bodies_started = True
                 self._result_defs_col = self._take_result_defs()
                 self.final_body.splice(self.red_stores)
@@ -1960,15 +1983,54 @@ class HipKernel(SIMDKernel):
                 with src.indent():
                     src.splice(self._entry_code(self.x_entries))
                     src.writeline(f"{idx_t} b_ = split;")
-                    src.writeline("for (; b_ < full_; b_ += nsplit) {")
-                    with src.indent():
-                        src.writeline("#pragma unroll")
-                        src.writeline("for (int u_ = 0; u_ < UNR; ++u_) {")
+                    pipe = getattr(self, "_col_pipeline", None)
+                    if pipe is not None:
+                        # the loads of batch b + nsplit are in flight while batch b is folded
+                        entry_text, names, loads_text, rest_text = pipe
+                        src.writeline(f"auto ld_ = [&](const {idx_t} r0_index) {{")
                         with src.indent():
-                            src.writeline(f"const {idx_t} r0_index = b_ * batch_ + u_ * RL + rl;")
-                            src.splice(self.partial_body)
+                            src.splice(entry_text)
+                            src.splice(loads_text)
+                            src.writeline(f"return mi::pack({', '.join(names)});")
+                        src.writeline("};")
+                        src.writeline(f"using L_ = decltype(ld_({idx_t}(0)));")
+                        src.writeline("L_ cur_[UNR];")
+                        src.writeline("if (b_ < full_) {")
+                        with src.indent():
+                            src.writeline("#pragma unroll")
+                            src.writeline("for (int u_ = 0; u_ < UNR; ++u_) cur_[u_] = ld_(b_ * batch_ + u_ * RL + rl);")
                         src.writeline("}")
-                    src.writeline("}")
+                        src.writeline("while (b_ < full_) {")
+                        with src.indent():
+                            src.writeline(f"const {idx_t} bn_ = b_ + nsplit;")
+                            src.writeline("L_ nxt_[UNR];")
+                            src.writeline("if (bn_ < full_) {")
+                            with src.indent():
+                                src.writeline("#pragma unroll")
+                                src.writeline("for (int u_ = 0; u_ < UNR; ++u_) nxt_[u_] = ld_(bn_ * batch_ + u_ * RL + rl);")
+                            src.writeline("}")
+                            src.writeline("#pragma unroll")
+                            src.writeline("for (int u_ = 0; u_ < UNR; ++u_) {")
+                            with src.indent():
+                                src.writeline(f"const {idx_t} r0_index = b_ * batch_ + u_ * RL + rl;")
+                                src.splice(entry_text)
+                                src.writeline(f"auto [{', '.join(names)}] = cur_[u_];")
+                                src.splice(rest_text)
+                            src.writeline("}")
+                            src.writeline("b_ = bn_;")
+                            src.writeline("#pragma unroll")
+                            src.writeline("for (int u_ = 0; u_ < UNR; ++u_) cur_[u_] = nxt_[u_];")
+                        src.writeline("}")
+                    else:
+                        src.writeline("for (; b_ < full_; b_ += nsplit) {")
+                        with src.indent():
+                            src.writeline("#pragma unroll")
+                            src.writeline("for (int u_ = 0; u_ < UNR; ++u_) {")
+                            with src.indent():
+                                src.writeline(f"const {idx_t} r0_index = b_ * batch_ + u_ * RL + rl;")
+                                src.splice(self.partial_body)
+                            src.writeline("}")
+                        src.writeline("}")
                     # the last, partly filled batch
                     src.writeline("if (b_ == full_) {")
                     with src.indent():

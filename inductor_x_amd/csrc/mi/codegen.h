@@ -1262,6 +1262,19 @@ __device__ __forceinline__ auto col_get(const M (&m)[N], G get) {
   }
 }
 
+// The values one row's loads of a column sweep deliver, kept together so a whole batch of rows
+// can be in flight while the previous batch is folded (unpacked with a structured binding).
+template <class A> struct Pack1 { A a; };
+template <class A, class B> struct Pack2 { A a; B b; };
+template <class A, class B, class C> struct Pack3 { A a; B b; C c; };
+template <class A, class B, class C, class D> struct Pack4 { A a; B b; C c; D d; };
+template <class A> __device__ __forceinline__ Pack1<A> pack(const A& a) { return {a}; }
+template <class A, class B> __device__ __forceinline__ Pack2<A, B> pack(const A& a, const B& b) { return {a, b}; }
+template <class A, class B, class C>
+__device__ __forceinline__ Pack3<A, B, C> pack(const A& a, const B& b, const C& c) { return {a, b, c}; }
+template <class A, class B, class C, class D>
+__device__ __forceinline__ Pack4<A, B, C, D> pack(const A& a, const B& b, const C& c, const D& d) { return {a, b, c, d}; }
+
 // Workspace layout for one reduction: [R::W][nsplit][xnumel] floats.
 template <class R, int N>
 __device__ __forceinline__ void col_store_partial(float* __restrict__ ws, const typename R::M (&m)[N], i64 x0,
