@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define MI355_ABI_VERSION 1
+#define MI355_ABI_VERSION 2
 
 /* Hardware numbers the split/tiling heuristics consume.  Replaces the
  * reference's num_aicore / num_vector_core / npu_block knobs
@@ -49,6 +49,9 @@ typedef struct mi_device_props {
   int32_t mem_bus_bits;      /* memory bus width                                */
   int64_t l2_bytes;          /* L2 size as reported by the runtime              */
   int64_t hbm_bytes;         /* total device memory                             */
+  int64_t mall_bytes;        /* memory-side cache (Infinity Cache) in front of
+                                HBM: summed level-3 entries of the device's KFD
+                                topology node, 0 when the topology is unreadable */
   char    arch[64];          /* gcnArchName, e.g. "gfx950:sramecc+:xnack-"      */
 } mi_device_props;
 
@@ -92,6 +95,32 @@ int mi_launch_packed(void* function,
                      uint32_t block_x, uint32_t block_y, uint32_t block_z,
                      uint32_t dynamic_lds_bytes, void* hip_stream,
                      const void* arg_segment, size_t arg_segment_bytes);
+
+/* No counterpart in the reference.  For callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc): mi_launch_packed for a kernel that takes a workspace
+ * pointer among its parameters, with that workspace supplied by the library.
+ * The 8-byte pointer parameter at byte `scratch_arg_offset` of the argument
+ * segment (whatever the caller put there is ignored) is replaced by the address
+ * of a fixed MI355_SCRATCH_BYTES array in device memory that the library holds,
+ * one copy per GPU, until the process ends; the kernel must need no more than
+ * `scratch_bytes_needed` bytes of it.  The call allocates and frees nothing.
+ *   - scratch_bytes_needed > MI355_SCRATCH_BYTES returns
+ *     MI_ERROR_SCRATCH_TOO_LARGE and launches nothing.
+ *   - The array keeps the previous call's contents: a kernel that needs zeroed
+ *     workspace must clear it itself.  Launches that share the array must be
+ *     ordered on one stream; calls that overlap on one GPU race.
+ *   - The device is the calling thread's current device, which must be the
+ *     stream's device. */
+#define MI355_SCRATCH_BYTES (8u << 20)
+#define MI_ERROR_SCRATCH_TOO_LARGE 100001
+int mi_launch_packed_scratch(void* function,
+                             uint32_t grid_x, uint32_t grid_y, uint32_t grid_z,
+                             uint32_t block_x, uint32_t block_y, uint32_t block_z,
+                             uint32_t dynamic_lds_bytes, void* hip_stream,
+                             const void* arg_segment, size_t arg_segment_bytes,
+                             size_t scratch_arg_offset, size_t scratch_bytes_needed);
+int mi_scratch_capacity(size_t* bytes_out);
 
 /* Hardware query used where the reference reads the Triton driver's device
  * properties (reference inductor_x/config.py:15-20). */

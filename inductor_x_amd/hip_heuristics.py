@@ -201,6 +201,13 @@ class CachingLauncher:
         g = grid_arg(cfg.meta) if callable(grid_arg) else grid_arg
         fn.launch(self.signature, args, g, (cfg.block,), stream, cfg.lds_bytes)
 
+    def _launch_on_library_scratch(self, idx: int, args, scratch_arg: int, scratch_bytes: int, grid_arg, stream: int) -> None:
+        """_launch with pointer parameter `scratch_arg` supplied by the launcher library's fixed
+        per-GPU scratch array (nothing is allocated)."""
+        cfg, fn = self.launchers[idx]
+        g = grid_arg(cfg.meta) if callable(grid_arg) else grid_arg
+        fn.launch_with_library_scratch(self.signature, args, scratch_arg, scratch_bytes, g, (cfg.block,), stream, cfg.lds_bytes)
+
     def bench(self, idx: int, args, grid_arg, stream: int, warmup: int = 3, rep: int = 10) -> float:
         """Average milliseconds per launch of configuration idx, timed with
         events on torch's current stream (which must be `stream`)."""

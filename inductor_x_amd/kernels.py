@@ -312,17 +312,30 @@ def col_mean_var_argmax(
     correction: float = 0.0,
     plan: Optional[SplitPlan] = None,
     final_variant: tuple = (16, 32),
-    workspace: Optional[torch.Tensor] = None,
+    workspace=None,
+    out: Optional[tuple] = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """Returns (mean, var, argmax) over dim 0 of a [rows, cols] fp32 matrix."""
+    """Returns (mean, var, argmax) over dim 0 of a [rows, cols] fp32 matrix.
+
+    workspace: a fp32 tensor for the per-split partials (allocated when None), or the string
+    "library": both kernels then run on the launcher library's fixed per-GPU scratch array
+    (mi_launch_packed_scratch), and with `out=(mean, var, argmax)` given the call allocates no
+    device memory at all.  Calls on the library scratch must not overlap on one GPU."""
     _check_cuda(x)
     _require(x.dtype == torch.float32 and x.dim() == 2, "x must be a 2-D fp32 matrix")
     _require(x.is_contiguous(), "x must be contiguous")
     rows, cols = x.shape
     _require(rows > 0, "argmax over an empty axis is undefined")
-    mean = torch.empty(cols, dtype=torch.float32, device=x.device)
-    var = torch.empty(cols, dtype=torch.float32, device=x.device)
-    arg = torch.empty(cols, dtype=torch.int64, device=x.device)
+    if out is not None:
+        mean, var, arg = out
+        _check_cuda(x, mean, var, arg)
+        _require(mean.dtype == var.dtype == torch.float32 and arg.dtype == torch.int64, "out must be (fp32, fp32, int64)")
+        _require(mean.shape == var.shape == arg.shape == (cols,), "out tensors must have one element per column")
+        _require(mean.is_contiguous() and var.is_contiguous() and arg.is_contiguous(), "out tensors must be contiguous")
+    else:
+        mean = torch.empty(cols, dtype=torch.float32, device=x.device)
+        var = torch.empty(cols, dtype=torch.float32, device=x.device)
+        arg = torch.empty(cols, dtype=torch.int64, device=x.device)
     if cols == 0:
         return mean, var, arg
     _require(cols % 4 == 0 and _aligned(x), "cols must be a multiple of 4 and x 16-byte aligned")
@@ -332,14 +345,25 @@ def col_mean_var_argmax(
     _require(plan.rows_per_split * plan.nsplit >= rows, "split plan does not cover all rows")
     _require(plan.col_tiles * plan.ct * 4 >= cols, "split plan does not cover all columns")
     need = plan.workspace_floats(cols)
-    if workspace is None:
-        workspace = torch.empty(need, dtype=torch.float32, device=x.device)
-    _require(workspace.numel() >= need and workspace.dtype == torch.float32, "workspace too small")
     lp, lf = _col_partial_launcher(), _col_final_launcher()
     ip = _find(lp, f"col_mean_var_argmax_partial_f32_c{plan.ct}_r{plan.rl}_u{plan.unroll}")
     cpw, sl = final_variant
     jf = _find(lf, f"col_mean_var_argmax_final_f32_c{cpw}_s{sl}")
     st = _stream()
+    if isinstance(workspace, str):
+        _require(workspace == "library", "workspace must be a tensor, None or 'library'")
+        # every partial word the second kernel reads is written by the first: nothing to clear
+        lp._launch_on_library_scratch(
+            ip, (x.data_ptr(), 0, rows, cols, plan.nsplit), 1, need * 4, (plan.col_tiles, plan.nsplit, 1), st
+        )
+        lf._launch_on_library_scratch(
+            jf, (0, mean.data_ptr(), var.data_ptr(), arg.data_ptr(), cols, plan.nsplit, float(correction)), 0,
+            need * 4, (cdiv(cols, cpw), 1, 1), st,
+        )
+        return mean, var, arg
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.float32, device=x.device)
+    _require(workspace.numel() >= need and workspace.dtype == torch.float32, "workspace too small")
     lp._launch(
         ip,
         (x.data_ptr(), workspace.data_ptr(), rows, cols, plan.nsplit),

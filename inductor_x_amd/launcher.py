@@ -25,6 +25,8 @@ EXPORTS = (
     "mi_function_get_attrs",
     "mi_launch",
     "mi_launch_packed",
+    "mi_launch_packed_scratch",
+    "mi_scratch_capacity",
     "mi_device_props_get",
     "mi_device_count",
     "mi_error_string",
@@ -45,6 +47,7 @@ class DeviceProps(ctypes.Structure):
         ("mem_bus_bits", ctypes.c_int32),
         ("l2_bytes", ctypes.c_int64),
         ("hbm_bytes", ctypes.c_int64),
+        ("mall_bytes", ctypes.c_int64),
         ("arch", ctypes.c_char * 64),
     ]
 
@@ -57,6 +60,9 @@ class FunctionAttrs(ctypes.Structure):
         ("max_threads_per_block", ctypes.c_int32),
     ]
 
+
+ABI_VERSION = 2
+SCRATCH_TOO_LARGE = 100001  # MI_ERROR_SCRATCH_TOO_LARGE
 
 _lib_lock = threading.Lock()
 _lib: Optional[ctypes.CDLL] = None
@@ -92,13 +98,17 @@ def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
         lib.mi_launch.argtypes = [vp, u32, u32, u32, u32, u32, u32, u32, vp, ctypes.POINTER(vp)]
         lib.mi_launch_packed.restype = ctypes.c_int
         lib.mi_launch_packed.argtypes = [vp, u32, u32, u32, u32, u32, u32, u32, vp, ctypes.c_char_p, sz]
+        lib.mi_launch_packed_scratch.restype = ctypes.c_int
+        lib.mi_launch_packed_scratch.argtypes = [vp, u32, u32, u32, u32, u32, u32, u32, vp, ctypes.c_char_p, sz, sz, sz]
+        lib.mi_scratch_capacity.restype = ctypes.c_int
+        lib.mi_scratch_capacity.argtypes = [ctypes.POINTER(sz)]
         lib.mi_device_props_get.restype = ctypes.c_int
         lib.mi_device_props_get.argtypes = [ctypes.c_int, ctypes.POINTER(DeviceProps)]
         lib.mi_device_count.restype = ctypes.c_int
         lib.mi_device_count.argtypes = [ctypes.POINTER(ctypes.c_int)]
         lib.mi_error_string.restype = ctypes.c_char_p
         lib.mi_error_string.argtypes = [ctypes.c_int]
-        if lib.mi_abi_version() != 1:
+        if lib.mi_abi_version() != ABI_VERSION:
             raise LauncherError(f"{path}: unexpected ABI version {lib.mi_abi_version()}")
         _lib = lib
         return lib
@@ -209,6 +219,37 @@ class Function:
                 f"launch of {self.name} grid=({gx},{gy},{gz}) block=({bx},{by},{bz}) lds={lds_bytes} failed: "
                 f"HIP error {err} ({error_string(err)})"
             )
+
+    def launch_with_library_scratch(
+        self,
+        signature: str,
+        args: Sequence,
+        scratch_arg: int,
+        scratch_bytes: int,
+        grid: Sequence[int],
+        block: Sequence[int],
+        stream: int,
+        lds_bytes: int = 0,
+    ) -> None:
+        """Enqueue through mi_launch_packed_scratch: parameter number `scratch_arg` (a pointer) is
+        filled in by the library with its fixed per-GPU scratch array, of which the kernel uses
+        `scratch_bytes`.  Nothing is allocated on the way."""
+        if signature[scratch_arg] != "P":
+            raise LauncherError(f"{self.name}: parameter {scratch_arg} is not a pointer")
+        packer = self._packers.get(signature)
+        if packer is None:
+            packer = struct.Struct("@" + signature)
+            self._packers[signature] = packer
+        seg = packer.pack(*args)
+        offset = struct.calcsize("@" + signature[:scratch_arg] + "P") - 8
+        gx, gy, gz = (tuple(grid) + (1, 1))[:3]
+        bx, by, bz = (tuple(block) + (1, 1))[:3]
+        err = self._lib.mi_launch_packed_scratch(
+            self._handle, gx, gy, gz, bx, by, bz, lds_bytes, ctypes.c_void_p(stream), seg, len(seg), offset,
+            scratch_bytes,
+        )
+        if err != 0:
+            raise LauncherError(f"launch of {self.name} on the library scratch failed: error {err} ({error_string(err)})")
 
     def launch_pointers(self, ctypes_values: Sequence, grid, block, stream: int, lds_bytes: int = 0) -> None:
         """Enqueue through mi_launch (array of pointers to ctypes values)."""

@@ -33,7 +33,34 @@ def test_header_symbols_are_exported(built):
     lib = ctypes.CDLL(built.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in the header but not exported"
-    assert built.load_library().mi_abi_version() == 1
+    assert built.load_library().mi_abi_version() == 2
+
+
+def test_scratch_array_is_resolvable_by_the_runtime(built, tmp_path):
+    """The HIP runtime finds a registered device variable by name in the library's gfx950 code
+    object; a symbol with local binding there aborts the process at hipGetSymbolAddress."""
+    import subprocess
+
+    llvm = "/opt/rocm/llvm/bin"
+    if not os.path.exists(os.path.join(llvm, "clang-offload-bundler")):
+        pytest.skip("ROCm LLVM tools not installed")
+    fat, co = str(tmp_path / "fat.bin"), str(tmp_path / "dev.co")
+    subprocess.run(["objcopy", "-O", "binary", "--only-section=.hip_fatbin", built.LIB_PATH, fat], check=True)
+    subprocess.run([os.path.join(llvm, "clang-offload-bundler"), "--type=o", "--unbundle", f"--input={fat}",
+                    "--targets=hipv4-amdgcn-amd-amdhsa--gfx950", f"--output={co}"], check=True)
+    syms = subprocess.run([os.path.join(llvm, "llvm-readelf"), "-sW", co], check=True, capture_output=True, text=True).stdout
+    rows = [ln.split() for ln in syms.splitlines() if ln.strip().endswith("scratch")]
+    assert rows, "no scratch array in the device code object"
+    assert all(r[4] == "GLOBAL" and int(r[2]) == 8 << 20 for r in rows), rows
+    # nothing above the capacity is accepted, and the refusal has a text of its own
+    assert lib_refuses_oversize(built)
+
+
+def lib_refuses_oversize(built) -> bool:
+    lib = built.load_library()
+    seg = bytes(16)
+    err = lib.mi_launch_packed_scratch(ctypes.c_void_p(1), 1, 1, 1, 64, 1, 1, 0, None, seg, len(seg), 0, (8 << 20) + 1)
+    return err == built.SCRATCH_TOO_LARGE and "scratch" in built.error_string(err)
 
 
 def test_launcher_error_paths_without_gpu(built):
