@@ -5,7 +5,7 @@
 
 using namespace mi;
 
-// Dynamic LDS for pass 1: (RL / 2) * CT * 4 * 5 floats (0 when RL == 1).
+// Dynamic LDS for pass 1: col_fold_planes(CT, RL) * CT * 4 * 5 floats.
 #define COL_PARTIAL_VARIANT(CT, RL, UNROLL)                                                   \
   extern "C" __global__ __launch_bounds__(CT* RL) void                                        \
       col_mean_var_argmax_partial_f32_c##CT##_r##RL##_u##UNROLL(                              \
@@ -31,13 +31,24 @@ COL_PARTIAL_VARIANT(32, 32, 4)
 COL_PARTIAL_VARIANT(32, 16, 4)
 COL_PARTIAL_VARIANT(16, 32, 4)
 COL_PARTIAL_VARIANT(64, 8, 8)
+COL_PARTIAL_VARIANT(32, 8, 4)
+COL_PARTIAL_VARIANT(32, 8, 8)
+COL_PARTIAL_VARIANT(32, 16, 8)
+COL_PARTIAL_VARIANT(64, 16, 8)
+COL_PARTIAL_VARIANT(64, 4, 16)
+COL_PARTIAL_VARIANT(32, 8, 16)
+COL_PARTIAL_VARIANT(128, 4, 16)
+COL_PARTIAL_VARIANT(128, 2, 16)
+COL_PARTIAL_VARIANT(16, 16, 8)
 
 #define COL_FINAL_VARIANT(CPW, SL)                                                            \
   extern "C" __global__ __launch_bounds__(CPW* SL) void                                       \
       col_mean_var_argmax_final_f32_c##CPW##_s##SL(const float* part, float* mean_out,        \
                                                    float* var_out, long long* argmax_out,     \
-                                                   int cols, int nsplit, float correction) {  \
-    col_stats_final<CPW, SL>(part, mean_out, var_out, argmax_out, cols, nsplit, correction);  \
+                                                   int cols, int nsplit, int rows, int batch, \
+                                                   float correction) {                        \
+    col_stats_final<CPW, SL>(part, mean_out, var_out, argmax_out, cols, nsplit, rows, batch,  \
+                             correction);                                                     \
   }
 
 COL_FINAL_VARIANT(16, 16)
@@ -46,3 +57,11 @@ COL_FINAL_VARIANT(8, 64)
 COL_FINAL_VARIANT(8, 32)
 COL_FINAL_VARIANT(4, 64)
 COL_FINAL_VARIANT(64, 4)
+COL_FINAL_VARIANT(4, 16)
+COL_FINAL_VARIANT(4, 32)
+COL_FINAL_VARIANT(2, 64)
+COL_FINAL_VARIANT(2, 32)
+COL_FINAL_VARIANT(8, 16)
+COL_FINAL_VARIANT(8, 8)
+COL_FINAL_VARIANT(16, 4)
+COL_FINAL_VARIANT(16, 8)

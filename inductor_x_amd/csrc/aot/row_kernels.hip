@@ -18,7 +18,7 @@ struct ReluSigmoidRowSum {
   __device__ __forceinline__ float identity() const { return 0.f; }
   __device__ __forceinline__ float combine(float a, float b) const { return a + b; }
   __device__ __forceinline__ float partial(int row, int r) const {
-    const Vec<float, 4> v = load_vec<float, 4, true>(x + static_cast<size_t>(row) * rnumel + r);
+    const Vec<float, 4> v = load_vec_readonly<float, 4>(x + static_cast<size_t>(row) * rnumel + r);
     float s = 0.f;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
@@ -100,6 +100,12 @@ ROWSUM_VARIANT(256, 128, 8)
 ROWSUM_VARIANT(256, 64, 8)
 ROWSUM_VARIANT(512, 512, 2)
 ROWSUM_VARIANT(1024, 1024, 1)
+ROWSUM_VARIANT(512, 256, 4)
+ROWSUM_VARIANT(512, 128, 8)
+ROWSUM_VARIANT(128, 128, 8)
+ROWSUM_VARIANT(64, 64, 16)
+ROWSUM_VARIANT(128, 64, 16)
+ROWSUM_VARIANT(512, 64, 16)
 
 #define RMSNORM_VARIANT(BLOCK, TPR, ITERS)                                                      \
   extern "C" __global__ __launch_bounds__(BLOCK) void                                           \

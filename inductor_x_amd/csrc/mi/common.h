@@ -77,6 +77,30 @@ __device__ __forceinline__ Vec<T, N> load_vec(const T* __restrict__ p) {
   return out;
 }
 
+// Load for kernels that only read (a reduction's sweep over its input), with a hint switch of
+// its own.  Measured on MI355X with a plain summing kernel: 1 GiB streams at 7.2-7.3 TB/s with
+// the non-temporal hint against 6.5-6.7 TB/s without, 128 MiB takes 17.9 us against 19.0 us.
+// The hint also keeps the data out of the memory-side cache: a 16 MiB row sum that is launched
+// again on the same input goes from 3.4 to 4.4 us with it, and the column statistics sweep of
+// 128 MiB is 0.2 us slower, so it is off by default.
+#ifndef MI_NT_READONLY
+#define MI_NT_READONLY 0
+#endif
+template <typename T, int N>
+__device__ __forceinline__ Vec<T, N> load_vec_readonly(const T* __restrict__ p) {
+  constexpr int B = sizeof(T) * N;
+  typedef typename RawBits<B>::type raw_t;
+  raw_t r;
+  if constexpr (MI_NT_READONLY) {
+    r = __builtin_nontemporal_load(reinterpret_cast<const raw_t*>(p));
+  } else {
+    r = *reinterpret_cast<const raw_t*>(p);
+  }
+  Vec<T, N> out;
+  __builtin_memcpy(&out, &r, B);
+  return out;
+}
+
 template <typename T, int N, bool STREAM = false>
 __device__ __forceinline__ void store_vec(T* __restrict__ p, const Vec<T, N>& val) {
   constexpr int B = sizeof(T) * N;

@@ -326,6 +326,20 @@ def row_reduction_plan(xnumel: int, rnumel: int, elem_bytes: int, persistent: bo
     return RowPlan(block=block, tpr=tpr, vec=vec, iters=iters, rows_per_wg=block // tpr)
 
 
+def col_fold_lds_bytes(ct: int, rl: int, wave: int = 64) -> int:
+    """Dynamic LDS of the hand-written column sweep's fold over row lanes: row lanes that share a
+    wavefront meet through lane exchanges, the remaining groups are halved through LDS while more than
+    four are left and then collected in one round (the device side computes the same number,
+    col_fold_planes in csrc/mi/col.h)."""
+    in_wave = min(wave // ct, rl) if ct < wave else 1
+    groups = rl // max(in_wave, 1)
+    if groups <= 1:
+        return 0
+    tree = groups // 2 if groups > 4 else 0
+    last = min(groups, 4) - 1
+    return max(tree, last) * ct * 4 * 5 * 4
+
+
 @dataclasses.dataclass(frozen=True)
 class SplitPlan:
     ct: int  # threads across the kept (contiguous) axis, 4 elements each
@@ -341,10 +355,11 @@ class SplitPlan:
 
     @property
     def lds_bytes(self) -> int:
-        return (self.rl // 2) * self.ct * 4 * 5 * 4
+        return col_fold_lds_bytes(self.ct, self.rl)
 
     def workspace_floats(self, cols: int) -> int:
-        return 5 * self.nsplit * cols
+        # mean, M2, best value, best row per (split, column); the row count is implied by the geometry
+        return 4 * self.nsplit * cols
 
 
 def split_reduction_plan(
@@ -368,9 +383,14 @@ def split_reduction_plan(
          half as many wavefronts with twice the unrolled batch (4 per CU, 2 x 8
          loads each: 22.3 us) do as well as 8 per CU with 2 x 4 loads (22.3 us) and
          better than 16 per CU (25.3 us), and fewer wavefronts mean fewer partials;
-      2. a workgroup spans up to 512 kept elements (128 threads x float4) and
-         as many row lanes as make up that many wavefronts - big workgroups mean
-         few partials, so little workspace traffic;
+      2. a workgroup spans only 128 kept elements (32 threads x float4, runs of
+         512 bytes per row) and as many row lanes as make up those wavefronts, so
+         the kept axis is cut into many column tiles and the reduced axis into few
+         splits: the partials a column has are what the second pass must fold, and
+         their number is the workgroup count divided by the column tiles.  Measured
+         at [65536, 512], both passes: 32 x 8 threads in 4 tiles x 64 splits 25.3 us,
+         64 x 4 in 2 x 128 26.0 us, 128 x 2 in 1 x 256 27.1 us (at 2 KiB rows the
+         narrower tiles cost the sweep nothing);
       3. nsplit is the smallest count that gives every CU that many wavefronts,
          rounded to a multiple of the CU count so the last round of workgroups
          is full, then capped so that writing and re-reading the partials stays
@@ -380,7 +400,7 @@ def split_reduction_plan(
     """
     hw = hw or config.hardware()
     vec = 4
-    ct = min(next_power_of_2(cdiv(cols, vec)), 128)
+    ct = min(next_power_of_2(cdiv(cols, vec)), 32)
     col_tiles = cdiv(cols, ct * vec)
     # the kernel keeps two batches of `unroll` loads in flight (software pipeline)
     waves_cu = waves_per_cu_target(2 * unroll, vgprs, hw)
@@ -392,8 +412,8 @@ def split_reduction_plan(
     if nsplit * col_tiles > hw.cu_count:
         per = max(hw.cu_count // col_tiles, 1)
         nsplit = cdiv(nsplit, per) * per
-    # workspace traffic cap: 2 * nsplit * cols * 20 B <= frac * rows * cols * elem_bytes
-    cap_ws = int(max_workspace_frac * rows * elem_bytes / 40)
+    # workspace traffic cap: 2 * nsplit * cols * 16 B <= frac * rows * cols * elem_bytes
+    cap_ws = int(max_workspace_frac * rows * elem_bytes / 32)
     # every thread should own at least one unrolled batch
     cap_rows = rows // (rl * unroll)
     nsplit = max(min(nsplit, max(cap_ws, 1), max(cap_rows, 1)), 1)

@@ -22,6 +22,7 @@ from .hip_heuristics import (
     CachingLauncher,
     LaunchConfig,
     cdiv,
+    col_fold_lds_bytes,
     next_power_of_2,
     row_reduction_plan,
     split_reduction_plan,
@@ -53,7 +54,8 @@ def _check_cuda(*tensors: torch.Tensor) -> None:
 # ---------------------------------------------------------------------------
 # code objects (one per aot file), loaded lazily
 # ---------------------------------------------------------------------------
-_ROWSUM_VARIANTS = [(256, 256), (256, 128), (256, 64), (512, 512), (1024, 1024)]
+_ROWSUM_VARIANTS = [(256, 256), (256, 128), (256, 64), (512, 512), (1024, 1024), (512, 256), (512, 128), (128, 128),
+                    (64, 64), (128, 64), (512, 64)]
 _RMSNORM_VARIANTS = [
     (256, 256, 2),
     (256, 128, 4),
@@ -86,8 +88,18 @@ _COL_PARTIAL_VARIANTS = [
     (32, 16, 4),
     (16, 32, 4),
     (64, 8, 8),
+    (32, 8, 4),
+    (32, 8, 8),
+    (32, 16, 8),
+    (64, 16, 8),
+    (64, 4, 16),
+    (32, 8, 16),
+    (128, 4, 16),
+    (128, 2, 16),
+    (16, 16, 8),
 ]
-_COL_FINAL_VARIANTS = [(16, 16), (16, 32), (8, 64), (8, 32), (4, 64), (64, 4)]
+_COL_FINAL_VARIANTS = [(16, 16), (16, 32), (8, 64), (8, 32), (4, 64), (64, 4), (4, 16), (4, 32), (2, 64), (2, 32),
+                       (8, 16), (8, 8), (16, 4), (16, 8)]
 _GATHER_VARIANTS = [(256, 128, 1), (256, 128, 2), (256, 128, 4), (256, 64, 1), (256, 64, 2), (256, 64, 4), (256, 16, 1), (256, 16, 4)]
 _PERMUTE_VARIANTS = [
     (256, 16, 32, 8),
@@ -138,7 +150,7 @@ def _col_partial_launcher() -> CachingLauncher:
             f"col_mean_var_argmax_partial_f32_c{ct}_r{rl}_u{u}",
             ct * rl,
             meta={"CT": ct, "RL": rl, "UNROLL": u},
-            lds_bytes=(rl // 2) * ct * 4 * 5 * 4,
+            lds_bytes=col_fold_lds_bytes(ct, rl),
         )
         for ct, rl, u in _COL_PARTIAL_VARIANTS
     ]
@@ -154,7 +166,7 @@ def _col_final_launcher() -> CachingLauncher:
         for c, s in _COL_FINAL_VARIANTS
     ]
     return CachingLauncher(
-        "col_mean_var_argmax_final_f32", codecache.aot_source("col_kernels.hip"), "PPPPiif", cfgs, prefer_intree=True
+        "col_mean_var_argmax_final_f32", codecache.aot_source("col_kernels.hip"), "PPPPiiiif", cfgs, prefer_intree=True
     )
 
 
@@ -311,7 +323,7 @@ def col_mean_var_argmax(
     x: torch.Tensor,
     correction: float = 0.0,
     plan: Optional[SplitPlan] = None,
-    final_variant: tuple = (16, 32),
+    final_variant: Optional[tuple] = None,
     workspace=None,
     out: Optional[tuple] = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
@@ -347,6 +359,11 @@ def col_mean_var_argmax(
     need = plan.workspace_floats(cols)
     lp, lf = _col_partial_launcher(), _col_final_launcher()
     ip = _find(lp, f"col_mean_var_argmax_partial_f32_c{plan.ct}_r{plan.rl}_u{plan.unroll}")
+    if final_variant is None:
+        # few columns per workgroup so that the second pass has hundreds of workgroups, and as many
+        # split lanes as there are splits up to 16 (measured at 512 columns x 64 splits: (4, 16) 25.3 us
+        # for both passes, (16, 16) 25.6, (16, 32) 26.1, (64, 4) 28.1)
+        final_variant = (4, 16) if cols >= 256 else (8, 8)
     cpw, sl = final_variant
     jf = _find(lf, f"col_mean_var_argmax_final_f32_c{cpw}_s{sl}")
     st = _stream()
@@ -357,7 +374,8 @@ def col_mean_var_argmax(
             ip, (x.data_ptr(), 0, rows, cols, plan.nsplit), 1, need * 4, (plan.col_tiles, plan.nsplit, 1), st
         )
         lf._launch_on_library_scratch(
-            jf, (0, mean.data_ptr(), var.data_ptr(), arg.data_ptr(), cols, plan.nsplit, float(correction)), 0,
+            jf, (0, mean.data_ptr(), var.data_ptr(), arg.data_ptr(), cols, plan.nsplit, rows, plan.rl * plan.unroll,
+                 float(correction)), 0,
             need * 4, (cdiv(cols, cpw), 1, 1), st,
         )
         return mean, var, arg
@@ -372,7 +390,8 @@ def col_mean_var_argmax(
     )
     lf._launch(
         jf,
-        (workspace.data_ptr(), mean.data_ptr(), var.data_ptr(), arg.data_ptr(), cols, plan.nsplit, float(correction)),
+        (workspace.data_ptr(), mean.data_ptr(), var.data_ptr(), arg.data_ptr(), cols, plan.nsplit, rows,
+         plan.rl * plan.unroll, float(correction)),
         (cdiv(cols, cpw), 1, 1),
         st,
     )

@@ -116,7 +116,8 @@ def test_split_heuristic_properties():
         if rows * cols * 4 >= 1 << 20:
             assert 2 * p.workspace_floats(cols) * 4 <= 0.06 * rows * cols * 4 + 40 * cols  # partial traffic cap
     big = split_reduction_plan(65536, 512, hw=hw)
-    assert big.nsplit == 256 and big.rows_per_split == 256 and big.block == 256 and big.unroll == 8
+    assert (big.ct, big.rl, big.col_tiles) == (32, 8, 4)  # narrow column tiles: few partials per column
+    assert big.nsplit == 64 and big.rows_per_split == 1024 and big.block == 256 and big.unroll == 8
     # more CUs never means fewer splits
     import dataclasses
 
