@@ -31,11 +31,34 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
 
-# HBM bytes per launch of add_rmsnorm_bf16 at [8192, 4096], from rocprofv3 --pmc
-# FETCH_SIZE and WRITE_SIZE runs scaled by the same counters on a plain copy
-# kernel of known size (scale factors 1.99984 and 0.99922); summary in
-# profiles/add_rmsnorm_bf16_8192x4096_pmc.txt.
-MEASURED_TRAFFIC_BYTES = {"add_rmsnorm": 268_550_300}
+# HBM-side bytes per call, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
+# `bench.py --pmc-config <n>`, each scaled by what the same counter reads for a plain
+# copy kernel of known size in the same run.  Keyed by (configuration, path); an entry
+# applies only while the call still launches exactly the symbols that were profiled.
+MEASURED_TRAFFIC: dict = {
+    ('1', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_817_884, "write_bytes": 32_742,
+        "profile": "profiles/rowsum_f32_1024x4096_warm_pmc.txt"},
+    ('1', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 16_805_597, "write_bytes": 32_742,
+        "profile": "profiles/rowsum_f32_1024x4096_warm_pmc.txt"},
+    ('1cold', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_819_024, "write_bytes": 32_740,
+        "profile": "profiles/rowsum_f32_1024x4096_cold_pmc.txt"},
+    ('2', 'kernel'): {"symbols": ["add_rmsnorm_bf16_b512_t512_i1"], "fetch_bytes": 134_289_498, "write_bytes": 134_240_626,
+        "profile": "profiles/add_rmsnorm_bf16_8192x4096_pmc.txt"},
+    ('2', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 134_297_689, "write_bytes": 134_277_240,
+        "profile": "profiles/add_rmsnorm_bf16_8192x4096_pmc.txt"},
+    ('3', 'kernel'): {"symbols": ["col_mean_var_argmax_partial_f32_c32_r8_u8", "col_mean_var_argmax_final_f32_c4_s16"], "fetch_bytes": 138_611_172, "write_bytes": 536_141,
+        "profile": "profiles/col_mean_var_argmax_f32_65536x512_pmc.txt"},
+    ('3', 'torch.compile'): {"symbols": ["hip_col_0_partial", "hip_col_0_final"], "fetch_bytes": 147_016_534, "write_bytes": 1_583_867,
+        "profile": "profiles/col_mean_var_argmax_f32_65536x512_pmc.txt"},
+    ('4a', 'kernel'): {"symbols": ["gather_rows_b16_b256_t128_r2"], "fetch_bytes": 66_447_574, "write_bytes": 67_213_165,
+        "profile": "profiles/gather_rows_bf16_50304x1024_32768_pmc.txt"},
+    ('4a', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 67_434_256, "write_bytes": 67_096_785,
+        "profile": "profiles/gather_rows_bf16_50304x1024_32768_pmc.txt"},
+    ('4b', 'kernel'): {"symbols": ["permute_copy_b16_b256_p16_t32x4"], "fetch_bytes": 268_466_890, "write_bytes": 268_421_811,
+        "profile": "profiles/permute_0213_bf16_16x2048x32x128_pmc.txt"},
+    ('4b', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 268_441_292, "write_bytes": 268_519_390,
+        "profile": "profiles/permute_0213_bf16_16x2048x32x128_pmc.txt"},
+}
 
 ALGO_BYTES = {
     "rowsum": 16_781_312,
@@ -90,6 +113,94 @@ def _graph_time_ms(fn, launches_per_graph: int = 20, replays: int = 5) -> float:
     return start.elapsed_time(end) / (replays * launches_per_graph)
 
 
+def _config_table(K, torch, only=None):
+    """name -> builder of (direct call, graph function, arguments, algorithmic work, bound) for every graph
+    of the benchmark definition.  Builders allocate their seeded inputs when called and not before."""
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
+    dev = "cuda:0"
+
+    def c1():
+        torch.manual_seed(0)
+        x = torch.randn(1024, 4096).to(dev)
+        return (K.fused_relu_sigmoid_rowsum, lambda x: (torch.relu(2 * x + 1) * torch.sigmoid(x)).sum(-1), (x,),
+                ALGO_BYTES["rowsum"], "hbm")
+
+    def c2():
+        torch.manual_seed(0)
+        h = torch.randn(8192, 4096).bfloat16().to(dev)
+        r = torch.randn(8192, 4096).bfloat16().to(dev)
+        w = (1 + 0.02 * torch.randn(4096)).bfloat16().to(dev)
+
+        def rms(h, r, w):
+            s = h + r
+            sf = s.float()
+            return (sf * torch.rsqrt(sf.pow(2).mean(-1, keepdim=True) + 1e-6) * w.float()).to(torch.bfloat16), s
+
+        return (lambda h, r, w: K.add_rmsnorm(h, r, w, 1e-6), rms, (h, r, w), ALGO_BYTES["add_rmsnorm"], "hbm")
+
+    def c3():
+        torch.manual_seed(0)
+        x = torch.randn(65536, 512).to(dev)
+        return (K.col_mean_var_argmax, lambda x: (x.mean(0), x.var(0, unbiased=False), x.argmax(0)), (x,),
+                ALGO_BYTES["col_mean_var_argmax"], "hbm")
+
+    def c4a():
+        torch.manual_seed(0)
+        table = (0.02 * torch.randn(50304, 1024)).bfloat16().to(dev)
+        idx = torch.randint(0, 50304, (32768,), dtype=torch.int64).to(dev)
+        return (K.gather_rows, lambda t, i: t[i], (table, idx), ALGO_BYTES["gather"], "hbm")
+
+    def c4b():
+        torch.manual_seed(0)
+        t = torch.randn(16, 2048, 32, 128).bfloat16().to(dev)
+        return (K.permute_0213_contiguous, lambda t: t.permute(0, 2, 1, 3).contiguous(), (t,), ALGO_BYTES["permute"], "hbm")
+
+    def c5():
+        torch.manual_seed(0)
+        q = torch.randn(4, 32, 4096, 128).bfloat16().to(dev)
+        k = torch.randn(4, 32, 4096, 128).bfloat16().to(dev)
+        v = torch.randn(4, 32, 4096, 128).bfloat16().to(dev)
+        return (lambda q, k, v: K.fused_attention(q, k, v, 128 ** -0.5, True),
+                lambda q, k, v: npu_fusion_attention_graph(q, k, v, 32, "BNSD", scale=128 ** 0.5, sparse_mode=3)[0],
+                (q, k, v), ATTN_FLOPS_CAUSAL, "mfma")
+
+    table = {
+        "1 pointwise+rowsum fp32 [1024,4096] (cache-warm)": c1,
+        "2 add+rmsnorm bf16 [8192,4096]": c2,
+        "3 col mean/var/argmax fp32 [65536,512]": c3,
+        "4a gather bf16 [50304,1024][32768]": c4a,
+        "4b permute(0,2,1,3) bf16 [16,2048,32,128]": c4b,
+        "5 causal attention bf16 [4,32,4096,128]": c5,
+    }
+    if only is not None:
+        table = {k: v for k, v in table.items() if k.split()[0] == only}
+    return table
+
+
+def _launched_symbols(fn) -> list:
+    """Kernel symbols one call of fn enqueues through the C-ABI launcher, in order."""
+    from inductor_x_amd import launcher
+
+    launcher.launch_log = []
+    try:
+        fn()
+    finally:
+        log, launcher.launch_log = launcher.launch_log, None
+    return log
+
+
+def _traffic_for(config: str, path: str, symbols: list, work):
+    """HBM-side bytes per call from the committed counter profiles, or None when a launched symbol
+    is not the one that was profiled (the table then no longer describes what ran)."""
+    rec = MEASURED_TRAFFIC.get((config.split()[0], path))
+    if rec is None or list(rec["symbols"]) != list(symbols):
+        return None
+    total = rec["fetch_bytes"] + rec["write_bytes"]
+    return {"bytes": total, "fetch_bytes": rec["fetch_bytes"], "write_bytes": rec["write_bytes"],
+            "over_algorithmic": round(total / work, 4), "profile": rec["profile"]}
+
+
 def _all_configs(K, torch) -> list:
     """Every graph of the benchmark definition, two ways: the hand-written kernel
     family called directly through the launcher ("kernel"), and the same graph
@@ -97,12 +208,16 @@ def _all_configs(K, torch) -> list:
     ("torch.compile": generated HIP kernels; the attention graph reaches the
     MFMA kernel through the custom op)."""
     import inductor_x_amd  # noqa: F401  registers the Inductor backend
-    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
 
     dev = "cuda:0"
     out = []
 
     def add(name, path, fn, work, bound):
+        try:
+            symbols = _launched_symbols(fn)
+        except Exception as e:
+            out.append({"config": name, "path": path, "error": f"{type(e).__name__}: {e}"[:200]})
+            return
         try:
             ms = _graph_time_ms(fn)
             how = "hip-graph replay"
@@ -113,14 +228,15 @@ def _all_configs(K, torch) -> list:
             except Exception as e2:
                 out.append({"config": name, "path": path, "error": f"{type(e2).__name__}: {e2}"[:200]})
                 return
+        rec = {"config": name, "path": path, "ms": round(ms, 5), "bound": bound, "kernels": symbols, "timing": how}
         if bound == "hbm":
             ach = work / ms / 1e6
-            out.append({"config": name, "path": path, "ms": round(ms, 5), "bound": "hbm", "achieved": round(ach, 1),
-                        "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "timing": how})
+            rec.update({"achieved": round(ach, 1), "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
+                        "traffic": _traffic_for(name, path, symbols, work)})
         else:
             ach = work / ms / 1e9
-            out.append({"config": name, "path": path, "ms": round(ms, 5), "bound": "mfma", "achieved": round(ach, 1),
-                        "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4), "timing": how})
+            rec.update({"achieved": round(ach, 1), "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TFLOPS, 4)})
+        out.append(rec)
 
     def both(name, direct, graph_fn, args, work, bound):
         add(name, "kernel", lambda: direct(*args), work, bound)
@@ -132,72 +248,82 @@ def _all_configs(K, torch) -> list:
         except Exception as e:
             out.append({"config": name, "path": "torch.compile", "error": f"{type(e).__name__}: {e}"[:200]})
 
-    torch.manual_seed(0)
-    x = torch.randn(1024, 4096).to(dev)
-    both("1 pointwise+rowsum fp32 [1024,4096] (cache-warm)", K.fused_relu_sigmoid_rowsum,
-         lambda x: (torch.relu(2 * x + 1) * torch.sigmoid(x)).sum(-1), (x,), ALGO_BYTES["rowsum"], "hbm")
-    # The same kernel on inputs that cannot be cache-resident: 72 distinct 16 MiB
-    # inputs (1.1 GiB, several times the 256 MB memory-side cache) visited in
-    # turn, one pass over all of them per graph replay.
-    xs = [x] + [torch.randn(1024, 4096, device=dev) for _ in range(71)]
-    turn = [0]
+    for name, build in _config_table(K, torch).items():
+        direct, graph_fn, args, work, bound = build()
+        both(name, direct, graph_fn, args, work, bound)
+        if name.startswith("1 "):
+            # The same kernel on inputs that cannot be cache-resident: 72 distinct 16 MiB
+            # inputs (1.1 GiB, several times the 256 MB memory-side cache) visited in
+            # turn, one pass over all of them per graph replay.
+            xs = [args[0]] + [torch.randn(1024, 4096, device=dev) for _ in range(71)]
+            turn = [0]
 
-    def cold():
-        turn[0] = (turn[0] + 1) % len(xs)
-        return K.fused_relu_sigmoid_rowsum(xs[turn[0]])
+            def cold():
+                turn[0] = (turn[0] + 1) % len(xs)
+                return K.fused_relu_sigmoid_rowsum(xs[turn[0]])
 
-    try:
-        ms = _graph_time_ms(cold, launches_per_graph=len(xs))
-        ach = ALGO_BYTES["rowsum"] / ms / 1e6
-        out.append({"config": "1 pointwise+rowsum fp32 [1024,4096] (cold: 72 inputs in turn)", "path": "kernel",
-                    "ms": round(ms, 5), "bound": "hbm", "achieved": round(ach, 1), "unit": "GB/s",
-                    "frac": round(ach / HBM_PEAK_GBS, 4), "timing": "hip-graph replay"})
-    except Exception as e:
-        out.append({"config": "1 cold", "path": "kernel", "error": f"{type(e).__name__}: {e}"[:200]})
-    del x, xs
-    torch.manual_seed(0)
-    h = torch.randn(8192, 4096).bfloat16().to(dev)
-    r = torch.randn(8192, 4096).bfloat16().to(dev)
-    w = (1 + 0.02 * torch.randn(4096)).bfloat16().to(dev)
-
-    def rms(h, r, w):
-        s = h + r
-        sf = s.float()
-        return (sf * torch.rsqrt(sf.pow(2).mean(-1, keepdim=True) + 1e-6) * w.float()).to(torch.bfloat16), s
-
-    both("2 add+rmsnorm bf16 [8192,4096]", lambda h, r, w: K.add_rmsnorm(h, r, w, 1e-6), rms, (h, r, w),
-         ALGO_BYTES["add_rmsnorm"], "hbm")
-    del h, r, w
-    torch.manual_seed(0)
-    x = torch.randn(65536, 512).to(dev)
-    both("3 col mean/var/argmax fp32 [65536,512]", K.col_mean_var_argmax,
-         lambda x: (x.mean(0), x.var(0, unbiased=False), x.argmax(0)), (x,), ALGO_BYTES["col_mean_var_argmax"], "hbm")
-    del x
-    torch.manual_seed(0)
-    table = (0.02 * torch.randn(50304, 1024)).bfloat16().to(dev)
-    idx = torch.randint(0, 50304, (32768,), dtype=torch.int64).to(dev)
-    both("4a gather bf16 [50304,1024][32768]", K.gather_rows, lambda t, i: t[i], (table, idx), ALGO_BYTES["gather"], "hbm")
-    del table, idx
-    torch.manual_seed(0)
-    t = torch.randn(16, 2048, 32, 128).bfloat16().to(dev)
-    both("4b permute(0,2,1,3) bf16 [16,2048,32,128]", K.permute_0213_contiguous,
-         lambda t: t.permute(0, 2, 1, 3).contiguous(), (t,), ALGO_BYTES["permute"], "hbm")
-    del t
-    torch.manual_seed(0)
-    q = torch.randn(4, 32, 4096, 128).bfloat16().to(dev)
-    k = torch.randn(4, 32, 4096, 128).bfloat16().to(dev)
-    v = torch.randn(4, 32, 4096, 128).bfloat16().to(dev)
-    both("5 causal attention bf16 [4,32,4096,128]", lambda q, k, v: K.fused_attention(q, k, v, 128 ** -0.5, True),
-         lambda q, k, v: npu_fusion_attention_graph(q, k, v, 32, "BNSD", scale=128 ** 0.5, sparse_mode=3)[0],
-         (q, k, v), ATTN_FLOPS_CAUSAL, "mfma")
-    # Backward of the same graph (the caller next to the forward on the
-    # training path): five matrix products plus two recomputed ones, counted
-    # by the usual convention as 2.5 x the forward's algorithmic FLOPs.
-    o, m, l = K.fused_attention(q, k, v, 128 ** -0.5, True)[:3]
-    do = torch.randn_like(o)
-    add("5b causal attention backward bf16 [4,32,4096,128]", "kernel",
-        lambda: K.fused_attention_backward(q, k, v, o, do, m, l, 128 ** -0.5, True), 2.5 * ATTN_FLOPS_CAUSAL, "mfma")
+            cname = "1cold pointwise+rowsum fp32 [1024,4096] (cold: 72 inputs in turn)"
+            try:
+                ms = _graph_time_ms(cold, launches_per_graph=len(xs))
+                ach = ALGO_BYTES["rowsum"] / ms / 1e6
+                syms = _launched_symbols(cold)
+                out.append({"config": cname, "path": "kernel", "ms": round(ms, 5), "bound": "hbm", "kernels": syms,
+                            "achieved": round(ach, 1), "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
+                            "timing": "hip-graph replay",
+                            "traffic": _traffic_for(cname, "kernel", syms, ALGO_BYTES["rowsum"])})
+            except Exception as e:
+                out.append({"config": cname, "path": "kernel", "error": f"{type(e).__name__}: {e}"[:200]})
+            del xs
+        if name.startswith("5 "):
+            # Backward of the same graph (the caller next to the forward on the
+            # training path): five matrix products plus two recomputed ones, counted
+            # by the usual convention as 2.5 x the forward's algorithmic FLOPs.
+            q, k, v = args
+            o, m, l = K.fused_attention(q, k, v, 128 ** -0.5, True)[:3]
+            do = torch.randn_like(o)
+            add("5b causal attention backward bf16 [4,32,4096,128]", "kernel",
+                lambda: K.fused_attention_backward(q, k, v, o, do, m, l, 128 ** -0.5, True), 2.5 * ATTN_FLOPS_CAUSAL, "mfma")
+            del o, m, l, do
+        del direct, graph_fn, args
     return out
+
+
+def _pmc_run(K, torch, which: str, steps: int, warmup: int) -> dict:
+    """Plain (ungraphed) launches of one configuration, both paths, plus the copy probe: the
+    program a counter collection run (rocprofv3 --pmc) wraps.  Counters come back per dispatch
+    and per kernel name, so the two paths and the probe separate in the output."""
+    import inductor_x_amd  # noqa: F401
+
+    dev = "cuda:0"
+    res = {"pmc_config": which, "steps": steps}
+    cold = which == "1cold"
+    table = _config_table(K, torch, only="1" if cold else which)
+    if not table:
+        raise SystemExit(f"bench.py: no configuration {which!r} (1, 1cold, 2, 3, 4a, 4b, 5)")
+    (name, build), = table.items()
+    direct, graph_fn, args, work, bound = build()
+    if cold:
+        xs = [args[0]] + [torch.randn(1024, 4096, device=dev) for _ in range(71)]
+        for i in range(warmup + steps):
+            K.fused_relu_sigmoid_rowsum(xs[i % len(xs)])
+        res["kernels"] = _launched_symbols(lambda: K.fused_relu_sigmoid_rowsum(xs[0]))
+    else:
+        for _ in range(warmup + steps):
+            direct(*args)
+        res["kernels"] = _launched_symbols(lambda: direct(*args))
+        torch._dynamo.reset()
+        cf = torch.compile(graph_fn)
+        for _ in range(warmup + steps):
+            cf(*args)
+        res["compiled_kernels"] = _launched_symbols(lambda: cf(*args))
+    torch.cuda.synchronize()
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(10):
+        K.copy_bytes(dst, src)
+    torch.cuda.synchronize()
+    res["copy_probe"] = {"kernel": "copy_b128", "bytes_read": 256 << 20, "bytes_written": 256 << 20, "launches": 10}
+    return res
 
 
 # --------------------------------------------------------------------------
@@ -355,6 +481,9 @@ def main() -> None:
     ap.add_argument("--no-all-configs", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB copy kernel 10 times (calibrates HBM byte counters under rocprofv3 --pmc)")
+    ap.add_argument("--pmc-config", default=None,
+                    help="run only plain launches of one configuration (1, 1cold, 2, 3, 4a, 4b, 5), both paths, and the "
+                         "copy probe: the program for a rocprofv3 --pmc counter run")
     ap.add_argument("--cpu-baseline-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
 
@@ -373,6 +502,9 @@ def main() -> None:
         sys.exit(1)
     from inductor_x_amd import kernels as K
 
+    if args.pmc_config is not None:
+        print(json.dumps(_pmc_run(K, torch, args.pmc_config, args.steps, args.warmup)))
+        return
     dev = "cuda:0"
     torch.manual_seed(0)
     rows, cols = 8192, 4096
@@ -415,16 +547,22 @@ def main() -> None:
         "dtype": "bf16",
         "data": "synthetic (seed 0, N(0,1) h and r, N(1,0.02) weight), resident in HBM before timing",
         "config": {"workload": "residual-add + RMSNorm, bf16, h,r [8192,4096], w [4096], eps 1e-6, returns (norm, h+r)",
-                   "kernel": K._rmsnorm_launcher().name, "algorithmic_bytes_per_step": ALGO_BYTES["add_rmsnorm"]},
+                   "algorithmic_bytes_per_step": ALGO_BYTES["add_rmsnorm"]},
         "roofline": {
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES["add_rmsnorm"],
+            "traffic": None,
         },
     }
+    step_symbols = _launched_symbols(step)
+    line["config"]["kernel"] = step_symbols
+    tr = _traffic_for("2 add+rmsnorm", "kernel", step_symbols, ALGO_BYTES["add_rmsnorm"])
+    if tr is not None:
+        line["roofline"]["traffic"] = tr["bytes"]
+        line["roofline"]["traffic_profile"] = tr["profile"]
     del h, r, w
     if args.copy_probe:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
