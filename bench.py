@@ -212,7 +212,10 @@ def _all_configs(K, torch) -> list:
     dev = "cuda:0"
     out = []
 
-    def add(name, path, fn, work, bound):
+    def add(name, path, fn, work, bound, error=None):
+        if error is not None:
+            out.append({"config": name, "path": path, "error": error})
+            return
         try:
             symbols = _launched_symbols(fn)
         except Exception as e:
@@ -285,7 +288,67 @@ def _all_configs(K, torch) -> list:
                 lambda: K.fused_attention_backward(q, k, v, o, do, m, l, 128 ** -0.5, True), 2.5 * ATTN_FLOPS_CAUSAL, "mfma")
             del o, m, l, do
         del direct, graph_fn, args
+    _ring_merge_configs(torch, add)
     return out
+
+
+def _ring_merge_configs(torch, add) -> None:
+    """The merge steps of ring attention at the reference's shapes (the callers next to the fused
+    attention op on a sequence-parallel path), compiled through the backend; HBM-bound.  Algorithmic
+    bytes: every operand read once, every result written once.  `add` records one measurement."""
+    dev = "cuda:0"
+
+    def trans(x):
+        b, n, s, d = x.shape
+        return x.permute(2, 0, 1, 3).reshape(s, b, n * d)
+
+    def bcast(x, h):
+        n = x.shape[1]
+        return trans(x[..., 0].unsqueeze(3).repeat(1, 1, 1, h // n))
+
+    def forward_update(po, pm, ps, co, cm, cs):
+        m = torch.maximum(pm, cm)
+        a, b = ps * torch.exp(pm - m), cs * torch.exp(cm - m)
+        tot = a + b
+        return (po * bcast(a / tot, po.shape[-1]) + co * bcast(b / tot, po.shape[-1])).to(po.dtype), m, tot
+
+    def forward_update_la(po, pl, co, cl):
+        lse = torch.log(torch.exp(cl) + torch.exp(pl))
+        return torch.exp(pl - lse) * po + torch.exp(cl - lse) * co, lse
+
+    def backward_update(dq, dk, dv, cdq, cdk, cdv):
+        dq.add_(cdq.view(dq.shape))
+        dk.add_(cdk.view(dk.shape))
+        dv.add_(cdv.view(dv.shape))
+
+    def one(name, fn, args, work):
+        try:
+            torch._dynamo.reset()
+            cf = torch.compile(fn)
+            cf(*args)
+        except Exception as e:
+            add(name, "torch.compile", None, work, "hbm", error=f"{type(e).__name__}: {e}"[:200])
+            return
+        add(name, "torch.compile", lambda: cf(*args), work, "hbm")
+
+    torch.manual_seed(0)
+    DS, B, H, N = 8192, 1, 6144, 48
+    st = lambda off: (torch.rand(B, N, DS, device=dev) + off).unsqueeze(3).repeat(1, 1, 1, 8).contiguous()  # noqa: E731
+    args = (torch.randn(DS, B, H, device=dev).bfloat16(), st(0.0), st(0.5), torch.randn(DS, B, H, device=dev).bfloat16(),
+            st(0.0), st(0.5))
+    one("f1a ring forward_update bf16 [8192,1,6144] N=48", forward_update, args, 3 * DS * B * H * 2 + 6 * B * N * DS * 8 * 4)
+    del args
+    B, N, DS, D = 1, 48, 8192, 128
+    args = (torch.randn(B, N, DS, D, device=dev), torch.rand(B, N, DS, 1, device=dev), torch.randn(B, N, DS, D, device=dev),
+            torch.rand(B, N, DS, 1, device=dev))
+    one("f1b ring forward_update (log-sum-exp) fp32 [1,48,8192,128]", forward_update_la, args,
+        3 * B * N * DS * D * 4 + 3 * B * N * DS * 4)
+    del args
+    S, B, H = 16384, 1, 1536
+    args = tuple(torch.randn(2, S, B, H, device=dev).bfloat16() for _ in range(3)) + tuple(
+        torch.randn(2 * S, B, H, device=dev).bfloat16() for _ in range(3))
+    one("f1c ring backward_update bf16 3 x [2,16384,1,1536]", backward_update, args, 3 * 3 * 2 * S * B * H * 2)
+    del args
 
 
 def _pmc_run(K, torch, which: str, steps: int, warmup: int) -> dict:

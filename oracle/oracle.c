@@ -32,6 +32,12 @@
  *   - attention backward (oracle_attention_bwd): the gradients of that definition,
  *     PARITY UNPINNED against torch_npu's npu_fusion_attention_grad for the same reason;
  *     pinned by central differences of an independent forward and by invariants.
+ *   - ring-attention merge steps (oracle_forward_update, oracle_forward_update_lse,
+ *     oracle_add_bf16): the test scenarios the reference compiles through its backend
+ *       (reference test/npu_indexing/attn_cp_test.py:36-59,
+ *        reference test/npu_indexing/written/test_attn_cp.py:267-287,361-367);
+ *     pinned by the identity "merging the softmax partials of two key ranges equals the
+ *     softmax over their union", evaluated independently in tests/test_oracle.py.
  *
  * Accumulations use double so the oracle is the more accurate side of every
  * comparison; element-wise math is done in float where the kernel does so.
@@ -277,4 +283,72 @@ void oracle_attention_bwd(const uint16_t* q, const uint16_t* k, const uint16_t* 
   }
 }
 
-int oracle_abi_version(void) { return 2; }
+/* Merge step of ring attention, statistics in (max, sum) form
+ * (reference test/npu_indexing/attn_cp_test.py:36-59).
+ *   prev_out, cur_out : [S, B, H] floats, H = N * D
+ *   *_max, *_sum      : [B, N, S, 8] floats; the output scales come from element 0 of the trailing
+ *                       axis (the reference's x[..., 0]), max and sum are merged element by element
+ *   out               : [S, B, H] doubles (the caller rounds to the tensor's type)
+ *   max_out, sum_out  : [B, N, S, 8] doubles
+ * prev_* may be strided views: element strides are passed for the sequence axis of prev_out
+ * (p_out_s, the B and H axes being dense below it) and for the N and S axes of the prev statistics. */
+void oracle_forward_update(const float* prev_out, const float* prev_max, const float* prev_sum,
+                           const float* cur_out, const float* cur_max, const float* cur_sum,
+                           double* out, double* max_out, double* sum_out, int64_t S, int64_t B,
+                           int64_t N, int64_t D, int64_t p_out_s, int64_t p_st_b, int64_t p_st_n,
+                           int64_t p_st_s) {
+  const int64_t H = N * D;
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int64_t b = 0; b < B; ++b) {
+    for (int64_t n = 0; n < N; ++n) {
+      for (int64_t s = 0; s < S; ++s) {
+        const float* pm = prev_max + b * p_st_b + n * p_st_n + s * p_st_s;
+        const float* ps = prev_sum + b * p_st_b + n * p_st_n + s * p_st_s;
+        const int64_t c = ((b * N + n) * S + s) * 8;
+        double scale_prev = 0.0, scale_cur = 0.0;
+        for (int e = 0; e < 8; ++e) {
+          const double m = fmax((double)pm[e], (double)cur_max[c + e]);
+          const double a = (double)ps[e] * exp((double)pm[e] - m);
+          const double bb = (double)cur_sum[c + e] * exp((double)cur_max[c + e] - m);
+          max_out[c + e] = m;
+          sum_out[c + e] = a + bb;
+          if (e == 0) {
+            scale_prev = a / (a + bb);
+            scale_cur = bb / (a + bb);
+          }
+        }
+        const float* po = prev_out + s * p_out_s + b * H + n * D;
+        const float* co = cur_out + (s * B + b) * H + n * D;
+        double* o = out + (s * B + b) * H + n * D;
+        for (int64_t d = 0; d < D; ++d) o[d] = (double)po[d] * scale_prev + (double)co[d] * scale_cur;
+      }
+    }
+  }
+}
+
+/* Merge step in log-sum-exp form (reference test/npu_indexing/written/test_attn_cp.py:361-367):
+ * rows of D values with one statistic each.
+ *   lse  = log(exp(cur_lse) + exp(prev_lse))
+ *   out  = exp(prev_lse - lse) * prev_out + exp(cur_lse - lse) * cur_out */
+void oracle_forward_update_lse(const float* prev_out, const float* prev_lse, const float* cur_out,
+                               const float* cur_lse, double* out, double* lse_out, int64_t rows,
+                               int64_t D) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    const double a = (double)prev_lse[r], b = (double)cur_lse[r];
+    const double l = log(exp(b) + exp(a));
+    lse_out[r] = l;
+    const double wa = exp(a - l), wb = exp(b - l);
+    for (int64_t d = 0; d < D; ++d)
+      out[r * D + d] = wa * (double)prev_out[r * D + d] + wb * (double)cur_out[r * D + d];
+  }
+}
+
+/* dst = bf16(float(dst) + float(src)), the in-place accumulation of the gradient merge
+ * (reference test/npu_indexing/written/test_attn_cp.py:267-287): one rounding per element. */
+void oracle_add_bf16(uint16_t* dst, const uint16_t* src, int64_t n) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; ++i) dst[i] = f32_to_bf16(bf16_to_f32(dst[i]) + bf16_to_f32(src[i]));
+}
+
+int oracle_abi_version(void) { return 3; }

@@ -155,3 +155,52 @@ def attention_bwd(q: np.ndarray, k: np.ndarray, v: np.ndarray, dout: np.ndarray,
         fn.restype = None
         fn(_p(q), _p(k), _p(v), _p(dout), _p(dq), _p(dk), _p(dv), B, N, S, D, float(scale), int(causal))
     return dq, dk, dv
+
+
+def forward_update(prev_out, prev_max, prev_sum, cur_out, cur_max, cur_sum):
+    """Ring-attention merge, (max, sum) statistics.  prev_out / cur_out [S, B, H] float32, statistics
+    [B, N, S, 8] float32 (all contiguous).  Returns (out, max, sum) as float64 arrays."""
+    prev_out, cur_out = _c(prev_out, np.float32), _c(cur_out, np.float32)
+    prev_max, prev_sum = _c(prev_max, np.float32), _c(prev_sum, np.float32)
+    cur_max, cur_sum = _c(cur_max, np.float32), _c(cur_sum, np.float32)
+    S, B, H = prev_out.shape
+    Bs, N, Ss, E = prev_max.shape
+    assert (Bs, Ss, E) == (B, S, 8) and H % N == 0 and cur_out.shape == prev_out.shape
+    assert prev_sum.shape == cur_max.shape == cur_sum.shape == prev_max.shape
+    out = np.zeros(prev_out.shape, np.float64)
+    mx = np.zeros(prev_max.shape, np.float64)
+    sm = np.zeros(prev_max.shape, np.float64)
+    fn = lib().oracle_forward_update
+    fn.argtypes = [ctypes.c_void_p] * 9 + [ctypes.c_int64] * 8
+    fn.restype = None
+    fn(_p(prev_out), _p(prev_max), _p(prev_sum), _p(cur_out), _p(cur_max), _p(cur_sum), _p(out), _p(mx), _p(sm),
+       S, B, N, H // N, B * H, N * S * 8, S * 8, 8)
+    return out, mx, sm
+
+
+def forward_update_lse(prev_out, prev_lse, cur_out, cur_lse):
+    """Ring-attention merge, log-sum-exp statistics.  prev_out / cur_out [..., D] float32, lse [..., 1]
+    float32.  Returns (out, lse) as float64 arrays."""
+    prev_out, cur_out = _c(prev_out, np.float32), _c(cur_out, np.float32)
+    prev_lse, cur_lse = _c(prev_lse, np.float32), _c(cur_lse, np.float32)
+    D = prev_out.shape[-1]
+    rows = prev_out.size // D
+    assert prev_lse.size == rows and cur_lse.size == rows and cur_out.shape == prev_out.shape
+    out = np.zeros(prev_out.shape, np.float64)
+    lse = np.zeros(prev_lse.shape, np.float64)
+    fn = lib().oracle_forward_update_lse
+    fn.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int64] * 2
+    fn.restype = None
+    fn(_p(prev_out), _p(prev_lse), _p(cur_out), _p(cur_lse), _p(out), _p(lse), rows, D)
+    return out, lse
+
+
+def add_bf16(dst: np.ndarray, src: np.ndarray) -> np.ndarray:
+    """bf16(float(dst) + float(src)) element by element, on raw bf16 bits; returns a new array."""
+    dst, src = _c(dst, np.uint16).copy(), _c(src, np.uint16)
+    assert dst.shape == src.shape
+    fn = lib().oracle_add_bf16
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
+    fn.restype = None
+    fn(_p(dst), _p(src), dst.size)
+    return dst

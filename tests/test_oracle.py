@@ -238,3 +238,96 @@ def test_attention_backward_invariants():
     b = O.attention_bwd(bits(q), bits(k), bits(v), bits((g.float() * 2).bfloat16()), 0.3, False)
     for x, y in zip(a, b):
         assert np.allclose(2 * x, y)
+
+
+# ---------------------------------------------------------------- ring-attention merges
+def _softmax_partials(scores, v):
+    """Attention over one key range in float64 with numpy: (out, row max, row sum of exp(s - max))."""
+    m = scores.max(-1, keepdims=True)
+    p = np.exp(scores - m)
+    l = p.sum(-1, keepdims=True)
+    return (p / l) @ v, m[..., 0], l[..., 0]
+
+
+def test_forward_update_equals_softmax_over_the_union():
+    """Merging the partial results of two key ranges must give the softmax attention over their
+    union: out, row maximum and row sum (reference test/npu_indexing/attn_cp_test.py:36-59).
+    A swapped weight, a missing rescale or statistics read from the wrong row fails this."""
+    rng = np.random.default_rng(0)
+    B, N, S, D, K1, K2 = 2, 3, 5, 4, 7, 6
+    q = rng.standard_normal((B, N, S, D))
+    k = rng.standard_normal((B, N, K1 + K2, D)) * 2.0
+    v = rng.standard_normal((B, N, K1 + K2, D))
+    s = q @ k.transpose(0, 1, 3, 2)
+    o1, m1, l1 = _softmax_partials(s[..., :K1], v[:, :, :K1])
+    o2, m2, l2 = _softmax_partials(s[..., K1:], v[:, :, K1:])
+    o, m, l = _softmax_partials(s, v)
+    sbh = lambda t: np.ascontiguousarray(t.transpose(2, 0, 1, 3).reshape(S, B, N * D)).astype(np.float32)  # noqa: E731
+    st8 = lambda t: np.ascontiguousarray(np.repeat(t[..., None], 8, -1)).astype(np.float32)  # noqa: E731
+    out, mx, sm = O.forward_update(sbh(o1), st8(m1), st8(l1), sbh(o2), st8(m2), st8(l2))
+    np.testing.assert_allclose(out, sbh(o).astype(np.float64), rtol=2e-6, atol=2e-6)
+    np.testing.assert_allclose(mx[..., 0], m, rtol=1e-6)
+    np.testing.assert_allclose(sm[..., 0], l, rtol=2e-6)
+    assert (mx == mx[..., :1]).all() and (sm == sm[..., :1]).all()
+    # the order of the two partials does not matter
+    out_b, mx_b, sm_b = O.forward_update(sbh(o2), st8(m2), st8(l2), sbh(o1), st8(m1), st8(l1))
+    np.testing.assert_allclose(out_b, out, rtol=1e-12, atol=1e-12)
+    assert np.array_equal(mx_b, mx)
+    # a partner whose sum is zero leaves the other side unchanged
+    zero = np.zeros_like(st8(l2))
+    out_z, mx_z, sm_z = O.forward_update(sbh(o1), st8(m1), st8(l1), sbh(o2), st8(m1) - 1.0, zero)
+    np.testing.assert_allclose(out_z, sbh(o1).astype(np.float64), rtol=0, atol=0)
+    np.testing.assert_allclose(sm_z, st8(l1).astype(np.float64))
+
+
+def test_forward_update_scales_come_from_the_first_statistic_lane():
+    """The output weights read element 0 of the trailing axis of 8 (reference
+    attn_cp_test.py:24-32, `x[..., 0]`), while max and sum merge element by element."""
+    rng = np.random.default_rng(1)
+    S, B, N, D = 3, 1, 2, 2
+    po, co = rng.standard_normal((S, B, N * D)).astype(np.float32), rng.standard_normal((S, B, N * D)).astype(np.float32)
+    pm, cm = rng.random((B, N, S, 8)).astype(np.float32), rng.random((B, N, S, 8)).astype(np.float32)
+    ps, cs = rng.random((B, N, S, 8)).astype(np.float32) + 0.5, rng.random((B, N, S, 8)).astype(np.float32) + 0.5
+    out, mx, sm = O.forward_update(po, pm, ps, co, cm, cs)
+    m = np.maximum(pm.astype(np.float64), cm)
+    a, b = ps * np.exp(pm - m), cs * np.exp(cm - m)
+    np.testing.assert_allclose(mx, m)
+    np.testing.assert_allclose(sm, a + b, rtol=1e-12)
+    wa = (a / (a + b))[..., 0].transpose(2, 0, 1)[..., None].repeat(D, -1).reshape(S, B, N * D)
+    np.testing.assert_allclose(out, po * wa + co * (1 - wa), rtol=1e-12, atol=1e-12)
+
+
+def test_forward_update_lse_equals_softmax_over_the_union():
+    """Same identity in log-sum-exp form, lse = max + log(sum)
+    (reference test/npu_indexing/written/test_attn_cp.py:361-367)."""
+    rng = np.random.default_rng(2)
+    R, D, K1, K2 = 11, 8, 5, 9
+    q = rng.standard_normal((R, D))
+    k = rng.standard_normal((K1 + K2, D)) * 1.5
+    v = rng.standard_normal((K1 + K2, D))
+    s = q @ k.T
+    o1, m1, l1 = _softmax_partials(s[:, :K1], v[:K1])
+    o2, m2, l2 = _softmax_partials(s[:, K1:], v[K1:])
+    o, m, l = _softmax_partials(s, v)
+    f = lambda t: np.ascontiguousarray(t).astype(np.float32)  # noqa: E731
+    out, lse = O.forward_update_lse(f(o1), f((m1 + np.log(l1))[:, None]), f(o2), f((m2 + np.log(l2))[:, None]))
+    np.testing.assert_allclose(out, f(o).astype(np.float64), rtol=3e-6, atol=3e-6)
+    np.testing.assert_allclose(lse[:, 0], m + np.log(l), rtol=2e-6, atol=2e-6)
+    # merging a result with itself doubles the weight sum and keeps the output
+    out2, lse2 = O.forward_update_lse(f(o1), f((m1 + np.log(l1))[:, None]), f(o1), f((m1 + np.log(l1))[:, None]))
+    np.testing.assert_allclose(out2, f(o1).astype(np.float64), rtol=1e-12)
+    np.testing.assert_allclose(lse2[:, 0], f(m1 + np.log(l1)).astype(np.float64) + np.log(2.0), rtol=1e-12)
+
+
+def test_add_bf16_rounds_once_to_nearest_even():
+    """1 + 2^-8 is a tie between two bf16 values and goes to the even one; 1 + 3 * 2^-9 rounds up;
+    the sum is formed in fp32 before the single rounding."""
+    one = O.f32_to_bf16_bits(np.array([1.0, 1.0, 256.0, -3.0], np.float32))
+    add = O.f32_to_bf16_bits(np.array([2.0 ** -8, 3 * 2.0 ** -9, 1.0, 3.0], np.float32))
+    got = O.bf16_bits_to_f32(O.add_bf16(one, add))
+    assert list(got) == [1.0, 1.0078125, 256.0, 0.0]  # 257 is a tie between 256 and 258 -> even mantissa (256)
+    rng = np.random.default_rng(3)
+    a = O.f32_to_bf16_bits(rng.standard_normal(1000).astype(np.float32))
+    b = O.f32_to_bf16_bits(rng.standard_normal(1000).astype(np.float32))
+    ref = torch.from_numpy(O.bf16_bits_to_f32(a)).bfloat16() + torch.from_numpy(O.bf16_bits_to_f32(b)).bfloat16()
+    assert np.array_equal(O.bf16_bits_to_f32(O.add_bf16(a, b)), ref.float().numpy())
