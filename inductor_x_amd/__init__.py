@@ -107,6 +107,59 @@ def _register_device_interface() -> None:
     register_interface_for_device(DEVICE_TYPE, HipInterface)
 
 
+def _find_unsupported(exc: BaseException):
+    """The UnsupportedHipCodegen in the cause / context chain of `exc`, if any."""
+    from .codegen.hip_kernel import UnsupportedHipCodegen
+
+    seen = set()
+    while exc is not None and id(exc) not in seen:
+        seen.add(id(exc))
+        if isinstance(exc, UnsupportedHipCodegen):
+            return exc
+        inner = getattr(exc, "inner_exception", None)
+        exc = inner or exc.__cause__ or exc.__context__
+    return None
+
+
+def install_unsupported_retry() -> None:
+    """Wrap Inductor's in-process graph compile: when the HIP generator refuses a fused node, the ATen
+    ops that node came from are sent to their eager kernels (lowering.add_runtime_fallback) and the
+    graph is lowered again, instead of torch.compile failing.  When nothing is left to fall back on,
+    the generator's error, which names the node and the ops, ends the compilation.  Switch:
+    config.retry_unsupported_with_eager."""
+    import copy
+    import logging
+
+    from torch._inductor import compile_fx as cfx
+
+    cls = getattr(cfx, "_InProcessFxCompile", None)
+    if cls is None or getattr(cls.codegen_and_compile, "_inductor_x_amd", False):
+        return
+    original = cls.codegen_and_compile
+    log = logging.getLogger(__name__)
+
+    def codegen_and_compile(self, gm, example_inputs, inputs_to_check, graph_kwargs):
+        from .lowering import add_runtime_fallback
+
+        if not config.retry_unsupported_with_eager:
+            return original(self, gm, example_inputs, inputs_to_check, graph_kwargs)
+        pristine = copy.deepcopy(gm)  # the post-grad passes rewrite gm in place
+        for _ in range(4):
+            try:
+                return original(self, gm, example_inputs, inputs_to_check, graph_kwargs)
+            except Exception as e:
+                unsupported = _find_unsupported(e)
+                changed = [op for op in getattr(unsupported, "ops", ()) if add_runtime_fallback(op)]
+                if unsupported is None or not changed:
+                    raise
+                log.warning("%s; compiling again with %s as eager kernels", unsupported, ", ".join(map(str, changed)))
+                gm = copy.deepcopy(pristine)
+        return original(self, gm, example_inputs, inputs_to_check, graph_kwargs)
+
+    codegen_and_compile._inductor_x_amd = True
+    cls.codegen_and_compile = codegen_and_compile
+
+
 _registered = False
 
 
@@ -130,6 +183,7 @@ def _register() -> None:
     inductor_lowering.make_reduction = make_reduction
     _register_inductor_fallbacks()
     _register_inductor_decompositions()
+    install_unsupported_retry()
     from . import fusion_attention_graph
 
     fusion_attention_graph.register_fx_pass()

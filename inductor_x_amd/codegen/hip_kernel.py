@@ -520,6 +520,8 @@ class HipKernel(SIMDKernel):
         # looped row kernels: contiguous loads of the reduced axis seen so far, keyed by buffer and
         # index text; one that comes again in a later pass is served from an LDS copy of the row
         self.row_stash: dict[tuple[str, str], dict] = {}
+        # bounds-checked indirect index variable -> (its clamped copy, its in-range predicate)
+        self._indirect_bounds: dict[str, tuple] = {}
         self.row_pass = 0
         self.col_reductions: list[ColReduction] = []
         self.partial_body = IndentedBuffer()
@@ -1194,6 +1196,7 @@ class HipKernel(SIMDKernel):
     # -- loads / stores ------------------------------------------------------
     def load(self, name: str, index: sympy.Expr) -> CSEVariable:
         var = self.args.input(name)
+        index, _ = self._bounded_index(index)
         indirect = self.is_indirect_indexing(index)
         index = self.prepare_indexing(index)
         dtype = V.graph.get_dtype(name)
@@ -1301,10 +1304,13 @@ class HipKernel(SIMDKernel):
 
     def store(self, name: str, index: sympy.Expr, value: CSEVariable, mode: StoreMode = None) -> None:
         var = self.args.output(name)
+        index, in_range = self._bounded_index(index)
         index = self.prepare_indexing(index)
         if mode not in (None, "atomic_add"):
             raise UnsupportedHipCodegen(f"store mode {mode}")
         kind = self.classify_index(index)
+        if in_range is not None and kind == "contiguous":
+            kind = "gather"  # per-element guard: the masked element-wise form
         if self.mode == "row":
             if self.inside_reduction:
                 mask = "xmask" if self.r_full else "(rmask && xmask)"
@@ -1319,6 +1325,8 @@ class HipKernel(SIMDKernel):
             mask = "xmask" if self.inside_reduction else "(xmask && rl == 0)"
         else:
             mask = None
+        if in_range is not None:
+            mask = in_range if mask is None else f"mi::logical_and({mask}, {in_range})"
         if mode == "atomic_add":
             # accumulating scatter: several elements may land on one address, each adds atomically
             # (every one of the thread's VEC elements contributes, also when they share an address)
@@ -1364,9 +1372,38 @@ class HipKernel(SIMDKernel):
         self.red_stores.writeline(DeferredLine(name, line))
 
     def check_bounds(self, expr: sympy.Expr, size: sympy.Expr, lower: bool, upper: bool) -> None:
-        # Out-of-range indices are undefined behaviour in the source program; no
-        # device-side assert is generated.
-        return
+        """Inductor calls this for every indirect index it would assert on (reference
+        inductor_x/npu_triton_heuristics.py:131-133 passes the same switch to Triton as `debug`).
+        No device-side assert is generated here; instead (config.indirect_bounds == "clamp") a
+        clamped copy of the index is computed next to it, loads through the index use the copy, and
+        stores / atomics through it are dropped for elements whose index is out of range."""
+        if backend_config.indirect_bounds != "clamp" or not isinstance(expr, sympy.Symbol) or not (lower or upper):
+            return
+        name = str(expr)
+        if name in self._indirect_bounds:
+            return
+        var = self.cse.varname_map.get(name)
+        if var is None:
+            return
+        size_str = self.index_to_str(size)
+        clamped = self.cse.generate(self.compute, f"mi::clamp_index({name}, {size_str})", dtype=getattr(var, "dtype", None))
+        inside = self.cse.generate(self.compute, f"mi::index_in_range({name}, {size_str})", dtype=torch.bool)
+        for v in (clamped, inside):
+            if isinstance(v, HipCSEVariable):
+                v.is_vec = bool(getattr(var, "is_vec", False))
+        self._indirect_bounds[name] = (sympy.Symbol(str(clamped), integer=True), str(inside))
+
+    def _bounded_index(self, index: sympy.Expr) -> tuple:
+        """(index with every bounds-checked indirect symbol replaced by its clamped copy, conjunction
+        of their in-range predicates or None)."""
+        hits = {s: self._indirect_bounds[str(s)] for s in index.free_symbols if str(s) in self._indirect_bounds}
+        if not hits:
+            return index, None
+        preds = [p for _, p in hits.values()]
+        guard = preds[0]
+        for p in preds[1:]:
+            guard = f"mi::logical_and({guard}, {p})"
+        return sympy_subs(index, {s: c for s, (c, _) in hits.items()}), guard
 
     # -- reductions -----------------------------------------------------------
     def reduction(self, dtype, src_dtype, reduction_type, value):

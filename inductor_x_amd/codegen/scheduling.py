@@ -24,7 +24,7 @@ from torch._inductor.utils import get_kernel_metadata
 from torch._inductor.virtualized import V
 from torch.utils._ordered_set import OrderedSet
 
-from .hip_kernel import HipKernel, VecConstraintError
+from .hip_kernel import HipKernel, UnsupportedHipCodegen, VecConstraintError
 
 log = logging.getLogger(__name__)
 
@@ -66,6 +66,41 @@ class HipScheduling(SIMDScheduling):
             tiling = kernel.tiling
             kernel.__init__(tiling, force_vec=1, features=features)
             return super().codegen_node_schedule_with_kernel(node_schedule, kernel)
+
+    def codegen_node(self, node):
+        """A fused node the generator cannot express ends compilation with ONE error that names the
+        node, the ATen ops it came from and the reason; the ops travel on the exception so that the
+        compile wrapper (inductor_x_amd.install_unsupported_retry) can send them to their eager kernels
+        and compile the graph again.  The reference drops a failing configuration and goes on
+        (reference inductor_x/npu_triton_heuristics.py:87-106,194-198)."""
+        try:
+            return super().codegen_node(node)
+        except UnsupportedHipCodegen as e:
+            if getattr(e, "node_names", None):
+                raise
+            nodes = list(node.get_nodes()) if hasattr(node, "get_nodes") else [node]
+            culprits = [n for n in nodes if n.is_reduction()] or nodes
+            ops: list = []
+            for n in culprits:
+                for fx in getattr(n.node, "origins", ()) or ():
+                    tgt = getattr(fx, "target", None)
+                    if isinstance(tgt, torch._ops.OpOverload) and tgt not in ops:
+                        ops.append(tgt)
+            # ops the generator is exercised on every day (pointwise arithmetic fused into the node)
+            # are not what it refused: keep them generated unless they are all there is
+            from ..lowering import GENERATE_LIST, REDUCING_OPS
+
+            everyday = {p for p in GENERATE_LIST if p not in REDUCING_OPS}
+            narrowed = [o for o in ops if getattr(o, "overloadpacket", None) not in everyday]
+            ops = narrowed or ops
+            names = [n.get_name() for n in nodes]
+            err = UnsupportedHipCodegen(
+                f"inductor_x_amd cannot generate a HIP kernel for fused node {'+'.join(names)} "
+                f"(from {', '.join(str(o) for o in ops) or 'unknown ops'}): {e}"
+            )
+            err.node_names = names
+            err.ops = ops
+            raise err from e
 
     def define_kernel(self, src_code: str, node_schedule, kernel: HipKernel) -> str:
         wrapper = V.graph.wrapper_code

@@ -29,6 +29,21 @@ autotune = os.environ.get("INDUCTOR_X_AMD_AUTOTUNE", "0") == "1"
 # reference's NPUDebugAutotuner, reference inductor_x/npu_triton_heuristics.py:268-299).
 profile_bandwidth = os.environ.get("INDUCTOR_X_AMD_PROFILE_BANDWIDTH", "0") == "1"
 
+# A fused node the HIP generator cannot express: send the ATen ops it came from to their eager
+# kernels and lower the graph again (True), or end compilation with the generator's error (False).
+retry_unsupported_with_eager = os.environ.get("INDUCTOR_X_AMD_RETRY_UNSUPPORTED", "1") == "1"
+
+# sum of a 16-bit floating-point tensor: accumulate in fp32 and round the result back to the input
+# type, which is the type eager PyTorch returns (False), or return the fp32 sum itself as the
+# reference's lowering does (True; reference inductor_x/lowering.py:204-215).
+sum_returns_fp32 = os.environ.get("INDUCTOR_X_AMD_SUM_FP32", "0") == "1"
+
+# Generated indirect accesses (embedding, index, gather, index_put, scatter): "clamp" keeps every
+# index inside its buffer (loads read the nearest valid element, stores and atomics outside the
+# range are dropped), "none" uses the index as it comes, as the reference's generated code does
+# unless assert_indirect_indexing is on.
+indirect_bounds = os.environ.get("INDUCTOR_X_AMD_INDIRECT_BOUNDS", "clamp")
+
 # Persistent (row held in registers) reductions are used up to this many
 # elements per row (the reference's limit is 1024,
 # reference inductor_x/codegen/triton.py:401-424; registers allow more here).
@@ -56,6 +71,7 @@ class Hardware:
     simds_per_cu: int = 4
     clock_khz: int = 2400000
     l2_bytes: int = 4 * 1024 * 1024
+    mall_bytes: int = 256 * 1024 * 1024
     hbm_bytes: int = 288 * 1024**3
     arch: str = "gfx950"
     probed: bool = False
@@ -86,6 +102,7 @@ def hardware(device: int = 0) -> Hardware:
                 max_threads_per_cu=p.max_threads_per_cu or hw.max_threads_per_cu,
                 clock_khz=p.clock_khz or hw.clock_khz,
                 l2_bytes=p.l2_bytes or hw.l2_bytes,
+                mall_bytes=p.mall_bytes or hw.mall_bytes,
                 hbm_bytes=p.hbm_bytes or hw.hbm_bytes,
                 arch=p.arch.decode() or hw.arch,
                 probed=True,

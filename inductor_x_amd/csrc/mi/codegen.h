@@ -433,6 +433,25 @@ __device__ __forceinline__ V<T, N> tile_col(const Tile<T, N>& t, int u) {
 }
 
 // Element-wise indexed load: idx scalar -> scalar, idx vector -> vector.
+// Indirect indices: the index a generated indirect load reads with when the one it was given lies
+// outside [0, size) (the nearest valid one), and whether an index is inside (stores and atomics
+// through an index outside the buffer are dropped).  Out-of-range indices are an error of the
+// program being compiled; this keeps that error from touching memory the kernel does not own.
+template <class A, class S>
+__device__ __forceinline__ auto clamp_index(const A& a, S size) {
+  return apply(
+      [size](auto x) {
+        typedef decltype(x) T;
+        const T hi = static_cast<T>(size) - 1;
+        return x < 0 ? static_cast<T>(0) : (x > hi ? hi : x);
+      },
+      a);
+}
+template <class A, class S>
+__device__ __forceinline__ auto index_in_range(const A& a, S size) {
+  return apply([size](auto x) { return x >= 0 && static_cast<long long>(x) < static_cast<long long>(size); }, a);
+}
+
 template <class T, class I>
 __device__ __forceinline__ auto gather(const T* __restrict__ p, const I& idx) {
   return apply([p](auto i) { return p[i]; }, idx);

@@ -14,9 +14,10 @@ reference the op receives the *inverse* scale from the pattern and inverts it
 through the op's own arguments: sparse_mode 2 or 3, or next_tockens == 0 with
 pre_tockens covering the sequence.  Supported: layout "BNSD", bf16, head
 dimension 128, no pse / padding mask / dropout; anything else raises.
-The backward op recomputes the probabilities from the saved row statistics and runs its matrix
-products as library GEMMs (attention_backward.py); the training variant of the pattern is
-registered beside the inference one.
+The backward op recomputes the probabilities from the saved row statistics inside fused
+gradient kernels (head dimension 128; kernels.fused_attention_backward) and falls back to the
+same mathematics over library GEMMs for other head dimensions (attention_backward.py); the
+training variant of the pattern is registered beside the inference one.
 """
 from __future__ import annotations
 
@@ -240,15 +241,27 @@ def _attention_replacement_1(query, key, value, inv_scale_factor, dropout_p):
 
 
 def _extra_check(match) -> bool:
-    """Only rewrite what the kernel can run: bf16 GPU tensors with head dim 128."""
+    """Only rewrite what the op can run: bf16 GPU tensors with head dim 128, query, key and value of
+    one shape and type (no cross attention: the kernels take one sequence length), and a positive
+    divisor of the scores when it is a constant.  Anything else stays on Inductor's own path."""
     try:
         q = match.kwargs["query"].meta["val"]
+        k = match.kwargs["key"].meta["val"]
+        v = match.kwargs["value"].meta["val"]
     except Exception:
         return False
-    return (
+    if not (
         q.device.type == "cuda" and q.dtype == torch.bfloat16 and q.dim() == 4 and q.size(3) == 128
         and q.size(1) % 128 == 0
-    )
+    ):
+        return False
+    for t in (k, v):
+        if tuple(t.shape) != tuple(q.shape) or t.dtype != q.dtype or t.device != q.device:
+            return False
+    divisor = match.kwargs.get("inv_scale_factor")
+    if isinstance(divisor, (int, float)) and not (divisor > 0 and divisor == divisor and divisor != float("inf")):
+        return False
+    return True
 
 
 _registered = False

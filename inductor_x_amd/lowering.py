@@ -16,8 +16,9 @@ What differs, on purpose:
     indexing and embedding - which the reference leaves unfused - stay fused;
   - var / var_mean keep Inductor's single-pass Welford form: it computes the same
     two-pass definition (:270-293) to fp32 accuracy while reading the input once;
-  - sum of a 16-bit tensor is rounded back to that type at the end (the
-    reference returns fp32), which keeps the output type PyTorch promises;
+  - sum of a 16-bit tensor is rounded back to that type at the end, which keeps
+    the output type PyTorch promises; config.sum_returns_fp32 switches to the
+    reference's behaviour (the fp32 sum itself is the result);
   - every patch only acts on GPU tensors; CPU compilation in the same process
     keeps Inductor's own lowerings.
 """
@@ -41,6 +42,8 @@ from torch._inductor.lowering import (
 )
 from torch._inductor.utils import sympy_product
 from torch._prims_common import is_boolean_dtype, is_integer_dtype
+
+from . import config as backend_config
 
 log = logging.getLogger(__name__)
 aten = torch.ops.aten
@@ -78,7 +81,7 @@ def make_reduction(reduction_type: str, override_return_dtype=None):
         )
         result = Reduction.create(reduction_type=reduction_type, input_node=x, **kwargs)
         data = getattr(getattr(result, "data", None), "data", None)
-        if isinstance(data, Reduction):
+        if isinstance(data, Reduction) and _is_gpu(x):  # CPU graphs keep Inductor's own (lazy) node
             reduced = set(_validate_reduction_axis(x, axis))
             ndim = len(x.get_size())
             # IR nodes are frozen dataclasses: annotate past the freeze
@@ -112,6 +115,10 @@ GENERATE_LIST = [
     prims.maximum,
 ]
 
+# The members of GENERATE_LIST that lower to a reduction (the rest is pointwise arithmetic, views and indexing).
+REDUCING_OPS = [aten.sum, aten.mean, aten.var, aten.var_mean, aten.amax, aten.amin, aten.min, aten.max, aten.argmax,
+                aten.argmin]
+
 # Ops whose Inductor lowering needs scans, sorts or device-side random numbers: on GPU tensors
 # they run as eager kernels.  Scatters and index_put are generated (plain or atomic stores
 # through an indirect index); Inductor itself sends the reducing scatters it cannot express
@@ -123,6 +130,9 @@ FALLBACK_OPS = [
 ]
 
 FALLBACK_LIST: list = []
+# Ops sent to eager kernels after the code generator refused a fused node that came from them
+# (filled at compile time by add_runtime_fallback; process-wide, so later graphs skip the retry).
+RUNTIME_FALLBACKS: list = []
 _registered = False
 
 
@@ -137,6 +147,25 @@ def _device_aware(op, original, replacement):
 
     wrapper._inductor_x_amd = True
     return wrapper
+
+
+def add_runtime_fallback(op) -> bool:
+    """Send `op` (an OpOverload with a lowering) to its eager kernel for GPU tensors from now on.
+    Returns True when the lowering table changed.  Counterpart of the reference dropping a
+    configuration that fails to compile and going on with what is left
+    (reference inductor_x/npu_triton_heuristics.py:87-106,194-198): here the unit that is
+    dropped is the op's generated lowering, and what is left is its library kernel."""
+    if not isinstance(op, torch._ops.OpOverload) or op not in lowerings or op in RUNTIME_FALLBACKS:
+        return False
+    original = lowerings[op]
+    try:
+        handler = fallback_handler(op, add_to_fallback_set=False)
+    except Exception as e:
+        log.debug("no eager fallback for %s: %s", op, e)
+        return False
+    lowerings[op] = _device_aware(op, original, handler)
+    RUNTIME_FALLBACKS.append(op)
+    return True
 
 
 def _register_inductor_fallbacks() -> None:
@@ -179,6 +208,8 @@ def _register_inductor_fallbacks() -> None:
         if in_dtype in (torch.float16, torch.bfloat16):
             x = to_dtype(x, torch.float32)
         result = tagged_sum(x, axis, keepdims, dtype=torch.float32 if out_dtype != torch.float64 else None)
+        if backend_config.sum_returns_fp32 and dtype is None and in_dtype in (torch.float16, torch.bfloat16):
+            return result  # the reference's result type: the fp32 sum, not rounded back
         return to_dtype(result, out_dtype)
 
     def mean_gpu(x, axis=None, keepdim=False, *, dtype=None):

@@ -245,6 +245,35 @@ def test_attention_op_and_pattern():
     assert (out32 - ref).abs().max().item() <= 2e-2
 
 
+def test_attention_pattern_leaves_cross_attention_and_negative_divisors_alone():
+    """Query and key of different sequence lengths, or a negative divisor of the scores, are not
+    what the fused op runs: the pattern must not fire and the compiled result equals eager."""
+    announce("compile attention pattern: cross attention / negative divisor")
+    from torch._inductor.utils import run_and_get_code
+
+    torch.manual_seed(1)
+    B, Sq, Sk, N, D = 2, 256, 384, 4, 128
+    q = torch.randn(B, Sq, N, D, device=DEV).bfloat16()
+    k = torch.randn(B, Sk, N, D, device=DEV).bfloat16()
+    v = torch.randn(B, Sk, N, D, device=DEV).bfloat16()
+
+    def make(div):
+        def g(q, k, v):
+            q, k, v = (t.permute(0, 2, 1, 3) for t in (q, k, v))
+            return torch.matmul(q, k.transpose(-2, -1)).div(div).softmax(dim=-1).matmul(v)
+
+        return g
+
+    for args, div in (((q, k, v), D ** 0.5), ((q, q.clone(), q.clone()), -(D ** 0.5))):
+        g = make(div)
+        torch._dynamo.reset()
+        with torch.no_grad():
+            out, codes = run_and_get_code(torch.compile(g), *args)
+            ref = g(*(t.float() for t in args))
+        assert "npu_graph.npu_fa" not in "\n".join(codes)
+        assert (out.float() - ref).abs().max().item() <= 3e-2
+
+
 def test_ring_attention_forward_update():
     """Merge step of ring attention: online-softmax rescale of two partial
     attention outputs (reference test/npu_indexing/attn_cp_test.py:19-59, shapes

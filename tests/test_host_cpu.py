@@ -211,6 +211,94 @@ def test_codegen_dry_run(tmp_path, built):
     assert len(built_objs) >= len(got)
 
 
+DRY_HEAD = r'''
+import os, sys
+os.environ["INDUCTOR_X_AMD_DRYRUN"] = "1"
+os.environ["INDUCTOR_X_AMD_CACHE"] = sys.argv[1]
+sys.path.insert(0, sys.argv[2])
+import torch
+import inductor_x_amd
+from inductor_x_amd import lowering, config
+from inductor_x_amd.codegen import hip_kernel
+lowering.GPU_DEVICE_TYPE = "cpu"  # the device-aware patches then act on the CPU tensors of the dry run
+from torch._inductor.codegen.common import register_backend_for_device
+from torch._inductor.codegen.wrapper import PythonWrapperCodegen
+from inductor_x_amd.codegen.scheduling import HipScheduling
+from torch._inductor.utils import run_and_get_code
+register_backend_for_device("cpu", HipScheduling, PythonWrapperCodegen)
+'''
+
+DRY_UNSUPPORTED = DRY_HEAD + r'''
+hip_kernel.REDUCTION_KIND.pop("prod")  # force the generator to refuse a product reduction
+x = torch.rand(8, 256) + 0.5
+_, codes = run_and_get_code(torch.compile(lambda x: (x * 2).prod(-1) + 1), x)
+code = "\n".join(codes)
+print("RETRY", "aten.prod" in code, "generated_kernel(" in code, ",".join(str(o) for o in lowering.RUNTIME_FALLBACKS))
+config.retry_unsupported_with_eager = False
+hip_kernel.REDUCTION_KIND.pop("max")
+torch._dynamo.reset()
+try:
+    torch.compile(lambda x: x.amax(-1))(x)
+    print("ERROR none")
+except Exception as e:
+    msg = str(e)
+    print("ERROR", "cannot generate a HIP kernel for fused node" in msg, "aten.amax" in msg, "reduction max" in msg)
+'''
+
+DRY_BOUNDS = DRY_HEAD + r'''
+cases = {
+  "embedding": (lambda t, i: torch.nn.functional.embedding(i, t) * 2, (torch.randn(100, 1024).bfloat16(), torch.randint(0, 100, (64,)))),
+  "index": (lambda t, i: t[i], (torch.randn(100, 64), torch.randint(0, 100, (7, 5)))),
+  "index_put": (lambda t, i, v: t.index_put((i,), v, accumulate=True), (torch.zeros(100, 64), torch.randint(0, 100, (32,)), torch.randn(32, 64))),
+  "scatter": (lambda t, i, v: t.scatter(1, i, v), (torch.zeros(16, 64), torch.randint(0, 64, (16, 8)), torch.randn(16, 8))),
+  "gather": (lambda t, i: torch.gather(t, 1, i), (torch.randn(16, 64), torch.randint(0, 64, (16, 8)))),
+}
+import re
+for name, (fn, args) in cases.items():
+    torch._dynamo.reset()
+    _, codes = run_and_get_code(torch.compile(fn), *args)
+    code = "\n".join(codes)
+    clamp = re.search(r"auto (tmp\d+) = mi::clamp_index\((tmp\d+), (\d+)\)", code)
+    inside = re.search(r"auto (tmp\d+) = mi::index_in_range\((tmp\d+), (\d+)\)", code)
+    raw, safe, ok = clamp.group(2), clamp.group(1), inside.group(1)
+    accesses = [l for l in code.splitlines() if re.search(r"mi::(gather|vload|scatter)", l) and (raw in re.findall(r"tmp\d+", l) or safe in l)]
+    uses_raw = any(raw in re.findall(r"tmp\d+", l.split("=", 1)[-1]) for l in accesses)
+    guarded = all(ok in l for l in accesses if "scatter" in l)
+    print("CASE", name, clamp.group(3), bool(accesses), uses_raw, guarded)
+'''
+
+
+def _run_dry(tmp_path, text):
+    script = tmp_path / "dry_case.py"
+    script.write_text(text)
+    proc = subprocess.run([sys.executable, str(script), str(tmp_path / "cache"), ROOT], capture_output=True, text=True,
+                          timeout=900)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    return proc.stdout
+
+
+def test_unsupported_node_falls_back_to_eager_or_names_the_node(tmp_path, built):
+    """A fused node the generator refuses: by default its ops are sent to their eager kernels and the
+    graph compiles on the second attempt; with the retry off compilation ends with one error naming
+    the node, the ATen op and the reason (reference inductor_x/npu_triton_heuristics.py:87-106)."""
+    out = _run_dry(tmp_path, DRY_UNSUPPORTED)
+    retry = next(l.split() for l in out.splitlines() if l.startswith("RETRY"))
+    assert retry[1:3] == ["True", "True"] and "aten.prod" in retry[3] and "aten.mul" not in retry[3]
+    assert next(l for l in out.splitlines() if l.startswith("ERROR")).split()[1:] == ["True", "True", "True"]
+
+
+def test_indirect_accesses_stay_inside_their_buffer(tmp_path, built):
+    """Generated embedding / index / gather loads read through a clamped copy of the index, and
+    index_put / scatter stores carry the in-range predicate, so an out-of-range index cannot touch
+    memory outside the buffer (the emitted source is checked; nothing is launched)."""
+    out = _run_dry(tmp_path, DRY_BOUNDS)
+    got = {l.split()[1]: l.split()[2:] for l in out.splitlines() if l.startswith("CASE")}
+    assert set(got) == {"embedding", "index", "index_put", "scatter", "gather"}
+    assert got["embedding"][0] == "100" and got["scatter"][0] == "64"
+    for name, (size, found, uses_raw, guarded) in got.items():
+        assert found == "True" and uses_raw == "False" and guarded == "True", (name, got[name])
+
+
 def test_import_hook_keeps_cpu_inductor_working():
     """The table patches only act on GPU tensors: CPU compilation in the same
     process still goes through Inductor's C++ backend and matches eager."""
