@@ -258,9 +258,15 @@ def _extra_check(match) -> bool:
     for t in (k, v):
         if tuple(t.shape) != tuple(q.shape) or t.dtype != q.dtype or t.device != q.device:
             return False
-    divisor = match.kwargs.get("inv_scale_factor")
-    if isinstance(divisor, (int, float)) and not (divisor > 0 and divisor == divisor and divisor != float("inf")):
-        return False
+    # the divisor of the scores: a keyword of the match when the pattern captured it, otherwise the
+    # second operand of the division node that was matched
+    divisors = [match.kwargs.get("inv_scale_factor")]
+    for node in getattr(match, "nodes", ()):
+        if getattr(node, "target", None) in (torch.ops.aten.div.Tensor, torch.ops.aten.div.Scalar) and len(node.args) > 1:
+            divisors.append(node.args[1])
+    for divisor in divisors:
+        if isinstance(divisor, (int, float)) and not (divisor > 0 and divisor != float("inf")):
+            return False
     return True
 
 

@@ -486,12 +486,34 @@ def _compile_pool():
     return _pool
 
 
+class LaunchPlan:
+    """Everything one (kernel, extents) pair needs at launch, computed once: which entry points,
+    their grids, the split of a column reduction and its workspace size."""
+
+    __slots__ = ("steps", "ws_floats", "candidate")
+
+    def __init__(self, steps, ws_floats: int, candidate: dict):
+        self.steps = steps  # [(function key, grid, block, lds bytes, tail of scalar arguments, takes workspace)]
+        self.ws_floats = ws_floats
+        self.candidate = candidate
+
+
 class GeneratedKernel:
     """Run-time side of one generated kernel: compiles (or fetches) its code
     object on first use and launches it through the C-ABI launcher.  This is the
     object the generated wrapper calls, in the place of the reference's
     `kernel.run(*args, grid=grid(...), stream=stream0)`
-    (reference test/npu_indexing/issue61_test.py:62)."""
+    (reference test/npu_indexing/issue61_test.py:62).
+
+    Per extents the launch geometry is planned once and kept (grids, the split of a column
+    reduction, its workspace).  Where the geometry is a run-time choice there are a few candidates
+    (the grid of a row kernel, which walks its rows with the stride of the grid; the split count of
+    a column pair): the first is the heuristic's, and with config.autotune on all are timed on the
+    first call and the winner is written next to the code object as
+    `<code object>.<xnumel>x<rnumel>.best_config`, which later objects and processes read instead
+    of timing again (reference inductor_x/npu_triton_heuristics.py:302-435).  With
+    config.profile_bandwidth on, every planned launch is timed once more and
+    `name: ms  GB  GB/s` is printed (reference :268-299)."""
 
     def __init__(self, name: str, meta: dict, source: str):
         self.name = name
@@ -499,6 +521,8 @@ class GeneratedKernel:
         self.source = source
         self.mode = meta["mode"]
         self._fns: Optional[dict] = None
+        self._plans: dict = {}
+        self.hsaco_path: Optional[str] = None
         # hipcc starts as soon as the wrapper module defines the kernel, in a worker thread (the
         # compiler is a subprocess), so the kernels of a graph build side by side instead of one
         # after the other at their first launches (the reference compiles inside precompile(),
@@ -530,6 +554,132 @@ class GeneratedKernel:
         # numbers that are kernel arguments themselves (sizes, values of 0-d CPU tensors)
         return a if isinstance(a, float) else int(a)
 
+    # -- launch geometry ------------------------------------------------------
+    def candidates(self, xnumel: int, rnumel: int) -> list:
+        """Run-time choices for these extents, the heuristic's first."""
+        m = self.mode
+        if m == "row":
+            rounds = cdiv(xnumel, self.meta["block"] // self.meta["tpr"])
+            cu = config.hardware().cu_count
+            caps = [None] + [c for c in (cu * 16, cu * 8) if c < rounds]
+            return [{"grid_cap": c} for c in caps]
+        if m == "col":
+            mm = self.meta
+            base, _ = split_factor(rnumel, xnumel, mm["ct"], mm["rl"], mm["vec"], unroll=mm.get("col_unroll", 4),
+                                   words=mm["ws_words"])
+            out = []
+            for n in (base, max(base // 2, 1), base * 2):
+                n = min(n, max(rnumel // (mm["rl"] * mm.get("col_unroll", 4)), 1))
+                if n >= 1 and {"nsplit": n} not in out:
+                    out.append({"nsplit": n})
+            return out
+        return [{}]
+
+    def _plan(self, xnumel: int, rnumel: int, cand: dict) -> LaunchPlan:
+        m = self.meta
+        if self.mode == "pointwise":
+            # a tiled kernel (static shapes) carries its own workgroup count
+            grid = (m["grid"] if "grid" in m else cdiv(xnumel, m["block"] * m["vec"] * m.get("unroll", 1)), 1, 1)
+            return LaunchPlan([("main", grid, (m["block"],), 0, (xnumel,), False)], 0, cand)
+        if self.mode == "row":
+            rounds = cdiv(xnumel, m["block"] // m["tpr"])
+            g = row_grid(rounds)
+            if cand.get("grid_cap"):
+                g = min(g, int(cand["grid_cap"]))
+            return LaunchPlan([("main", (g, 1, 1), (m["block"],), m.get("lds_bytes", 0), (xnumel, rnumel), False)], 0, cand)
+        if self.mode == "colloop":
+            grid = (cdiv(xnumel, m["ct"] * m["vec"]), 1, 1)
+            return LaunchPlan([("main", grid, (m["block"],), m["lds_bytes"], (xnumel, rnumel), False)], 0, cand)
+        nsplit = int(cand["nsplit"])
+        tiles = cdiv(xnumel, m["ct"] * m["vec"])
+        if nsplit == 1:
+            # one sweep that finishes in place: no workspace, no second kernel
+            return LaunchPlan([("direct", (tiles, 1, 1), (m["block"],), m["lds_partial"], (0, xnumel, rnumel, 1), False)], 0, cand)
+        tail = (xnumel, rnumel, nsplit)
+        return LaunchPlan(
+            [("partial", (tiles, nsplit, 1), (m["block"],), m["lds_partial"], tail, True),
+             ("final", (cdiv(xnumel, m["cpw"]), 1, 1), (m["cpw"] * m["sl"],), 0, tail, True)],
+            m["ws_words"] * nsplit * xnumel, cand,
+        )
+
+    def _workspace(self, args, floats: int):
+        """fp32 workspace of a column pair, from torch's caching allocator on every call (a block
+        handed back by the previous call as a rule).  A buffer kept across calls would outlive the
+        memory pools that HIP-graph capture of a compiled module (mode="reduce-overhead") checks for
+        stray live storage."""
+        import torch
+
+        dev = next(a.device for a in args if hasattr(a, "device"))
+        return torch.empty(floats, dtype=torch.float32, device=dev)
+
+    def _launch_plan(self, plan: LaunchPlan, args, raw, stream: int) -> None:
+        sig = self.meta["signature"]
+        ws = self._workspace(args, plan.ws_floats) if plan.ws_floats else None
+        ws_ptr = ws.data_ptr() if ws is not None else None
+        for key, grid, block, lds, tail, takes_ws in plan.steps:
+            full = raw + ((ws_ptr,) if takes_ws else ()) + tail
+            self._fns[key].launch(sig, full, grid, block, stream, lds)
+
+    # -- best-configuration record ------------------------------------------
+    def _best_path(self, xnumel: int, rnumel: int) -> Optional[str]:
+        if not self.hsaco_path:
+            return None
+        return f"{self.hsaco_path[:-len('.hsaco')]}.{xnumel}x{rnumel}.best_config"
+
+    def _load_best(self, xnumel: int, rnumel: int, cands: list) -> Optional[dict]:
+        p = self._best_path(xnumel, rnumel)
+        if not p or not os.path.exists(p):
+            return None
+        try:
+            with open(p) as f:
+                rec = json.load(f)
+        except (OSError, ValueError):
+            return None
+        if rec.get("candidates") != cands or rec.get("best") not in cands:
+            return None
+        return rec["best"]
+
+    def _autotune(self, xnumel: int, rnumel: int, cands: list, args, raw, stream: int) -> dict:
+        timings = []
+        for cand in cands:
+            plan = self._plan(xnumel, rnumel, cand)
+            try:
+                timings.append(self._time(plan, args, raw, stream, warmup=2, rep=5))
+            except launcher.LauncherError as e:
+                log.debug("candidate %s of %s failed to launch: %s", cand, self.name, e)
+                timings.append(float("inf"))
+        best = cands[timings.index(min(timings))]
+        p = self._best_path(xnumel, rnumel)
+        if p:
+            try:
+                with open(p, "w") as f:
+                    json.dump({"kernel": self.name, "mode": self.mode, "xnumel": xnumel, "rnumel": rnumel,
+                               "candidates": cands, "timings_ms": timings, "best": best}, f)
+            except OSError:
+                pass
+        return best
+
+    def _time(self, plan: LaunchPlan, args, raw, stream: int, warmup: int, rep: int) -> float:
+        """Milliseconds per call of the plan, with events on torch's current stream (which the
+        wrapper's raw stream is)."""
+        import torch
+
+        for _ in range(warmup):
+            self._launch_plan(plan, args, raw, stream)
+        start = torch.cuda.Event(enable_timing=True)
+        end = torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(rep):
+            self._launch_plan(plan, args, raw, stream)
+        end.record()
+        end.synchronize()
+        return start.elapsed_time(end) / rep
+
+    def num_bytes(self, args) -> int:
+        """Bytes of every tensor argument, read or written once: the figure the reference's
+        bandwidth print divides by (reference inductor_x/npu_triton_heuristics.py:282-299)."""
+        return sum(a.numel() * a.element_size() for a in args if hasattr(a, "data_ptr"))
+
     def run(self, *args, xnumel: int, r0_numel: int = 1, stream: int = 0) -> None:
         self.precompile()
         if _DRYRUN:
@@ -537,41 +687,26 @@ class GeneratedKernel:
         xnumel, rnumel = int(xnumel), int(r0_numel)
         if xnumel == 0:
             return
-        m = self.meta
         raw = tuple(self._raw(a) for a in args)
-        if self.mode == "pointwise":
-            # a tiled kernel (static shapes) carries its own workgroup count
-            grid = (m["grid"] if "grid" in m else cdiv(xnumel, m["block"] * m["vec"] * m.get("unroll", 1)), 1, 1)
-            self._fns["main"].launch(m["signature"], raw + (xnumel,), grid, (m["block"],), stream)
-        elif self.mode == "row":
-            grid = (row_grid(cdiv(xnumel, m["block"] // m["tpr"])), 1, 1)
-            self._fns["main"].launch(m["signature"], raw + (xnumel, rnumel), grid, (m["block"],), stream,
-                                     m.get("lds_bytes", 0))
-        elif self.mode == "colloop":
-            grid = (cdiv(xnumel, m["ct"] * m["vec"]), 1, 1)
-            self._fns["main"].launch(m["signature"], raw + (xnumel, rnumel), grid, (m["block"],), stream, m["lds_bytes"])
-        else:
+        key = (xnumel, rnumel)
+        plan = self._plans.get(key)
+        if plan is None:
             import torch
 
-            nsplit, _ = split_factor(rnumel, xnumel, m["ct"], m["rl"], m["vec"], unroll=m.get("col_unroll", 4),
-                                     words=m["ws_words"])
-            if nsplit == 1:
-                # one sweep that finishes in place: no workspace, no second kernel
-                self._fns["direct"].launch(
-                    m["signature"], raw + (0, xnumel, rnumel, 1), (cdiv(xnumel, m["ct"] * m["vec"]), 1, 1),
-                    (m["block"],), stream, m["lds_partial"],
-                )
-                return
-            dev = next(a.device for a in args if hasattr(a, "device"))
-            ws = torch.empty(m["ws_words"] * nsplit * xnumel, dtype=torch.float32, device=dev)
-            full = raw + (ws.data_ptr(), xnumel, rnumel, nsplit)
-            self._fns["partial"].launch(
-                m["signature"], full, (cdiv(xnumel, m["ct"] * m["vec"]), nsplit, 1), (m["block"],), stream,
-                m["lds_partial"],
-            )
-            self._fns["final"].launch(
-                m["signature"], full, (cdiv(xnumel, m["cpw"]), 1, 1), (m["cpw"] * m["sl"],), stream
-            )
+            cands = self.candidates(xnumel, rnumel)
+            best = cands[0]
+            if len(cands) > 1:
+                best = self._load_best(xnumel, rnumel, cands) or best
+                if config.autotune and best is cands[0] and not torch.cuda.is_current_stream_capturing() \
+                        and self._load_best(xnumel, rnumel, cands) is None:
+                    best = self._autotune(xnumel, rnumel, cands, args, raw, stream)
+            plan = self._plan(xnumel, rnumel, best)
+            self._plans[key] = plan
+            if config.profile_bandwidth and not torch.cuda.is_current_stream_capturing():
+                ms = self._time(plan, args, raw, stream, warmup=1, rep=5)
+                nbytes = self.num_bytes(args)
+                print(f"{self.name}: {ms:.4f} ms  {nbytes / 1e9:.4f} GB  {nbytes / 1e6 / ms:.1f} GB/s")
+        self._launch_plan(plan, args, raw, stream)
 
 
 def generated_kernel(name: str, meta: dict, source: str) -> GeneratedKernel:

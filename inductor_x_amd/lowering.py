@@ -81,13 +81,14 @@ def make_reduction(reduction_type: str, override_return_dtype=None):
         )
         result = Reduction.create(reduction_type=reduction_type, input_node=x, **kwargs)
         data = getattr(getattr(result, "data", None), "data", None)
-        if isinstance(data, Reduction) and _is_gpu(x):  # CPU graphs keep Inductor's own (lazy) node
-            reduced = set(_validate_reduction_axis(x, axis))
-            ndim = len(x.get_size())
-            # IR nodes are frozen dataclasses: annotate past the freeze
-            object.__setattr__(data, "kept_idx", [i for i in range(ndim) if i not in reduced])
-            object.__setattr__(data, "reduced_idx", [i for i in range(ndim) if i in reduced])
-            result.realize()
+        if isinstance(data, Reduction):
+            if _is_gpu(x):
+                reduced = set(_validate_reduction_axis(x, axis))
+                ndim = len(x.get_size())
+                # IR nodes are frozen dataclasses: annotate past the freeze
+                object.__setattr__(data, "kept_idx", [i for i in range(ndim) if i not in reduced])
+                object.__setattr__(data, "reduced_idx", [i for i in range(ndim) if i in reduced])
+            result.realize()  # as Inductor's own make_reduction does, for every device
         return result
 
     return inner
