@@ -111,7 +111,34 @@ def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
         if lib.mi_abi_version() != ABI_VERSION:
             raise LauncherError(f"{path}: unexpected ABI version {lib.mi_abi_version()}")
         _lib = lib
+        _load_fastcall(lib)
         return lib
+
+
+FASTCALL_PATH = os.path.join(_HERE, "_mi_fastcall.so")
+_fast = None
+
+
+def _load_fastcall(lib: ctypes.CDLL):
+    """The vectorcall entry to mi_launch_packed (csrc/mi_fastcall.c), bound to the loaded library.
+    Optional: without it every launch goes through ctypes, which is the same C ABI call with more
+    Python objects on the way."""
+    global _fast
+    if _fast is not None or not os.path.exists(FASTCALL_PATH):
+        return _fast
+    import importlib.machinery
+    import importlib.util
+
+    try:
+        loader = importlib.machinery.ExtensionFileLoader("_mi_fastcall", FASTCALL_PATH)
+        spec = importlib.util.spec_from_loader("_mi_fastcall", loader)
+        mod = importlib.util.module_from_spec(spec)
+        loader.exec_module(mod)
+        mod.bind(ctypes.cast(lib.mi_launch_packed, ctypes.c_void_p).value)
+        _fast = mod
+    except Exception:  # built for another interpreter: ctypes carries on
+        _fast = None
+    return _fast
 
 
 def error_string(err: int) -> str:
@@ -185,6 +212,8 @@ class Function:
         self.name = name
         self._handle = handle
         self._lib = load_library()
+        self._fast = _fast
+        self._raw_handle = handle.value
         self._packers: dict[str, struct.Struct] = {}
 
     def attrs(self) -> FunctionAttrs:
@@ -218,9 +247,12 @@ class Function:
         bx, by, bz = (tuple(block) + (1, 1))[:3]
         if launch_log is not None:
             launch_log.append(self.name)
-        err = self._lib.mi_launch_packed(
-            self._handle, gx, gy, gz, bx, by, bz, lds_bytes, ctypes.c_void_p(stream), seg, len(seg)
-        )
+        if self._fast is not None:
+            err = self._fast.launch(self._raw_handle, gx, gy, gz, bx, by, bz, lds_bytes, stream, seg)
+        else:
+            err = self._lib.mi_launch_packed(
+                self._handle, gx, gy, gz, bx, by, bz, lds_bytes, ctypes.c_void_p(stream), seg, len(seg)
+            )
         if err != 0:
             raise LauncherError(
                 f"launch of {self.name} grid=({gx},{gy},{gz}) block=({bx},{by},{bz}) lds={lds_bytes} failed: "

@@ -63,6 +63,26 @@ def lib_refuses_oversize(built) -> bool:
     return err == built.SCRATCH_TOO_LARGE and "scratch" in built.error_string(err)
 
 
+def test_fastcall_entry_reaches_the_same_c_abi(built):
+    """The vectorcall entry hands its arguments to mi_launch_packed unchanged: the library's own
+    argument checks answer (no GPU needed), and wrong Python types are refused before the call."""
+    if not os.path.exists(built.FASTCALL_PATH):
+        import __graft_entry__
+
+        __graft_entry__.build_fastcall()
+    built.load_library()
+    fast = built._load_fastcall(built.load_library())
+    assert fast is not None
+    assert fast.launch(0, 1, 1, 1, 64, 1, 1, 0, 0, b"") != 0  # null function handle: hipErrorInvalidValue
+    assert fast.launch(1, 0, 1, 1, 64, 1, 1, 0, 0, b"") != 0  # empty grid: hipErrorInvalidConfiguration
+    with pytest.raises(TypeError):
+        fast.launch(1, 1, 1, 1, 64, 1, 1, 0, 0, "not bytes")
+    with pytest.raises(TypeError):
+        fast.launch(1, 1, 1)
+    with pytest.raises(OverflowError):
+        fast.launch(1, 1 << 40, 1, 1, 64, 1, 1, 0, 0, b"")
+
+
 def test_launcher_error_paths_without_gpu(built):
     lib = built.load_library()
     assert lib.mi_module_load(None, 0, None) != 0  # invalid arguments never crash
