@@ -8,6 +8,7 @@
 #include "../mi/attention_pp.h"
 #include "../mi/attention_v2.h"
 #include "../mi/attention_v4.h"
+#include "../mi/attention_v5.h"
 
 using namespace mi;
 
@@ -160,4 +161,44 @@ extern "C" __global__ __launch_bounds__(512, 1) void fused_attention_fwd_bf16_d1
     const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
     int n_heads, int S, float scale_log2e) {
   attention_entry_v4<false>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
+}
+
+// v5: the v4 schedule with K and V tiles loaded straight into LDS and V read back transposed
+// (attention_v5.h).  Same workgroup shape and grid as v4; 64 KiB of LDS.
+template <bool CAUSAL>
+__device__ __forceinline__ void attention_entry_v5(const bf16_t* q, const bf16_t* k, const bf16_t* v,
+                                                   bf16_t* o, float* smax, float* ssum, int n_heads,
+                                                   int S, float scale_log2e) {
+  constexpr int XCDS = 8;
+  const int n_qb = S / kAttnV5BM;
+  const int id = blockIdx.x;
+  const int xcd = id % XCDS;
+  const int slot = id / XCDS;
+  if (CAUSAL) {
+    const int n_pair = (n_qb + 1) / 2;
+    const int head = (slot / n_pair) * XCDS + xcd;
+    const int lo = slot % n_pair;
+    const int hi = n_qb - 1 - lo;
+    if (head >= n_heads) return;
+    const int n_pass = lo != hi ? 2 : 1;
+#pragma nounroll
+    for (int pass = 0; pass < n_pass; ++pass)
+      attention_fwd_d128_v5<true>(q, k, v, o, smax, ssum, S, pass == 0 ? hi : lo, head, scale_log2e);
+  } else {
+    const int head = (slot / n_qb) * XCDS + xcd;
+    const int qb = slot % n_qb;
+    if (head >= n_heads) return;
+    attention_fwd_d128_v5<false>(q, k, v, o, smax, ssum, S, qb, head, scale_log2e);
+  }
+}
+
+extern "C" __global__ __launch_bounds__(512, 1) void fused_attention_fwd_bf16_d128_causal_v5(
+    const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
+    int n_heads, int S, float scale_log2e) {
+  attention_entry_v5<true>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
+}
+extern "C" __global__ __launch_bounds__(512, 1) void fused_attention_fwd_bf16_d128_full_v5(
+    const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
+    int n_heads, int S, float scale_log2e) {
+  attention_entry_v5<false>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
 }

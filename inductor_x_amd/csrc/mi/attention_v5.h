@@ -1,0 +1,337 @@
+// Fused attention forward, 32 queries per wavefront, two wavefronts per SIMD, K and V tiles brought
+// into LDS by direct global -> LDS loads and V read back transposed.
+//
+// Same mathematics, operand layouts and software pipeline as attention_v4.h (its results are
+// bit-identical); what changes is how a tile travels:
+//   - K and V tiles go memory -> LDS with 16-byte `global_load_lds` (gfx950): no staging registers, no
+//     LDS store instructions, no byte permutes.  One wavefront instruction fills a 1 KiB block (four
+//     256-byte rows); which global 16-byte chunk a lane fetches is free, so the chunks of a row are
+//     XOR-swizzled on the way in (K by row mod 16; V by a 4-entry table that keeps the transposing
+//     reads of 16- and 32-lane groups on distinct banks).  The loads of iteration t are issued in its
+//     first two chunks into the buffers iteration t - 1 released, and must only have landed by the
+//     barrier that ends the iteration.
+//   - V stays [key][d] in LDS; the V^T operand of O^T += V^T P^T is read with two
+//     `ds_read_b64_tr_b16` per fragment: in every group of 16 lanes, lane s points at four consecutive
+//     d of key 4 g + s / 4 and receives, for its own d, the four keys of the group -- which is the
+//     key order P arrives in from the first product's accumulator layout.
+// Measured on MI355X at [4,32,4096,128] (HIP events, same process): 0.576 / 0.996 ms causal / full
+// against 0.587 / 1.010 ms for attention_v4.h: the tile traffic it removes (0.116 -> 0.068 ms by
+// ablation) is partly paid back by the second LDS read per V fragment (fragment reads 0.25 -> 0.30 ms).
+#pragma once
+
+#include "attention_v2.h"
+
+
+namespace mi {
+
+constexpr int kAttnV5Waves = 8;
+constexpr int kAttnV5BM = kAttnV5Waves * 32;
+
+template <bool CAUSAL>
+__device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__ Q,
+                                                      const bf16_t* __restrict__ K,
+                                                      const bf16_t* __restrict__ V,
+                                                      bf16_t* __restrict__ O,
+                                                      float* __restrict__ softmax_max,
+                                                      float* __restrict__ softmax_sum, int S,
+                                                      int q_block, int head, float scale_log2e) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char attn_lds[];
+  // K and V tiles as they come from memory, [64 rows][128] bf16 without padding, 16-byte chunks of a
+  // row XOR-swizzled; written by direct global -> LDS loads (one 1 KiB block = four rows per
+  // wavefront instruction), two buffers each
+  constexpr int kTileElems = 64 * 128;
+  bf16_t* Kbuf = reinterpret_cast<bf16_t*>(attn_lds);
+  bf16_t* Vbuf = Kbuf + 2 * kTileElems;
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int li = lane & 31;
+  const int g = lane >> 5;
+
+  const size_t head_off = static_cast<size_t>(head) * S * kAttnD;
+  const bf16_t* __restrict__ Qh = Q + head_off;
+  const bf16_t* __restrict__ Kh = K + head_off;
+  const bf16_t* __restrict__ Vh = V + head_off;
+
+  const int q0 = q_block * kAttnV5BM;
+  const int qi = q0 + wave * 32 + li;
+
+  bf16x8_t qf[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s)
+    qf[s] = *reinterpret_cast<const bf16x8_t*>(Qh + static_cast<size_t>(qi) * kAttnD + 16 * s + 8 * g);
+
+  f32x16_t oacc[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+  float m_run = -__builtin_inff(), m_true = -__builtin_inff(), l_run = 0.f, alpha = 1.f;
+
+  const int n_tiles = CAUSAL ? (q0 + kAttnV5BM) / kAttnBN : S / kAttnBN;
+  const int first_masked = CAUSAL ? n_tiles - kAttnV5BM / kAttnBN : n_tiles;
+
+  // direct global -> LDS copies: block b of a tile (rows 4 b .. 4 b + 3) is written by one wavefront
+  // instruction, lane l filling LDS chunk l of the block (row 4 b + l / 16, chunk position l % 16)
+  // with the global chunk that the swizzle puts there
+  const int blk_row = lane >> 4;
+  const int blk_pos = lane & 15;
+  auto issue_tile = [&](const bf16_t* __restrict__ src, bf16_t* dst, int tile, auto swz) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int b = 2 * wave + u;
+      const int row = 4 * b + blk_row;
+      const int gchunk = blk_pos ^ swz(row);
+      const bf16_t* gp = src + (static_cast<size_t>(tile) * kAttnBN + row) * kAttnD + 8 * gchunk;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gp),
+                                       (__attribute__((address_space(3))) void*)(dst + b * 512), 16, 0, 0);
+    }
+  };
+  auto swz_k = [](int row) { return row & 15; };
+  auto swz_v = [](int row) { return (0xE4A0 >> (4 * (row & 3))) & 15; };  // 0, 10, 4, 14
+  auto issue_k = [&](int tile, int buf) { issue_tile(Kh, Kbuf + buf * kTileElems, tile, swz_k); };
+  auto issue_v = [&](int tile, int buf) { issue_tile(Vh, Vbuf + buf * kTileElems, tile, swz_v); };
+
+  f32x16_t sacc[2];  // [key block]
+  u32x4_t pw[4];     // P of the current tile: [key slice of 16] x four 32-bit words
+
+  // K fragment of chunk i of phase B (key block i / 8, d slice i % 8): row 32 kb + li, chunk 2 ks + g
+  int k_off[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) k_off[ks] = li * kAttnD + 8 * ((2 * ks + g) ^ (li & 15));
+  auto k_frag = [&](const bf16_t* Ks, int i) {
+    return *reinterpret_cast<const bf16x8_t*>(Ks + 32 * (i >> 3) * kAttnD + k_off[i & 7]);
+  };
+  // V^T fragment of chunk i of phase A (key slice t4 = i / 4, d block db = i % 4) by two transposing
+  // LDS reads: in each group of 16 lanes, lane s points at four consecutive d of key
+  // 4 g + s / 4 (+ 8 for the second read) and receives, for its own d, the four keys of the group
+  int v_off[4];
+  {
+    const int sl16 = lane & 15, grp = lane >> 4;
+    const int key_l = 4 * (grp >> 1) + (sl16 >> 2);
+    const int f = (0xE4A0 >> (4 * (key_l & 3))) & 15;
+    const int c_l = 2 * (grp & 1) + ((sl16 & 3) >> 1);
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+      v_off[db] = key_l * kAttnD + 8 * (((4 * db) ^ (f & 12)) + (c_l ^ (f & 2))) + 4 * (sl16 & 1);
+  }
+  typedef __bf16 bf16x4v_t __attribute__((__vector_size__(4 * sizeof(__bf16))));
+  auto v_frag = [&](const bf16_t* Vt, int i) {
+    const int t4 = i >> 2, db = i & 3;
+    const bf16_t* p0 = Vt + 16 * t4 * kAttnD + v_off[db];
+    const bf16x4v_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4v_t*)(p0));
+    const bf16x4v_t hi =
+        __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4v_t*)(p0 + 8 * kAttnD));
+    bf16x8_t r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      r[e] = lo[e];
+      r[4 + e] = hi[e];
+    }
+    return r;
+  };
+
+  auto apply_mask = [&](int tile) {
+    const int d = qi - (tile * kAttnBN + 4 * g);  // keys with local offset > d are masked
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (32 * kb + 8 * (r >> 2) + (r & 3) > d) sacc[kb][r] = -__builtin_inff();
+  };
+  float mpart, mx, m_new, psum;
+  auto softmax_rowmax = [&](auto kb_c) {
+    constexpr int kb = decltype(kb_c)::value;
+    float a = sacc[kb][0];
+#pragma unroll
+    for (int r = 1; r < 16; ++r) a = fmaxf(a, sacc[kb][r]);
+    if constexpr (kb == 0) {
+      mpart = a;
+    } else {
+      a = fmaxf(a, mpart);
+      const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(a), false, false);
+      mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+    }
+  };
+  auto softmax_ref = [&]() {
+    m_true = fmaxf(m_true, mx * scale_log2e);
+    m_new = m_true > m_run + kAttnV2Slack ? m_true : m_run;
+    alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    m_run = m_new;
+    psum = 0.f;
+  };
+  auto softmax_word = [&](auto t4_c, auto j_c) {  // word j of key slice t4
+    constexpr int t4 = decltype(t4_c)::value, j = decltype(j_c)::value;
+    constexpr int kb = t4 >> 1;
+    constexpr int r = 8 * (t4 & 1) + 2 * j;
+    const float p0 = __builtin_amdgcn_exp2f(fmaf(sacc[kb][r], scale_log2e, -m_new));
+    const float p1 = __builtin_amdgcn_exp2f(fmaf(sacc[kb][r + 1], scale_log2e, -m_new));
+    psum += p0 + p1;
+    bf16x2_t pk;
+    pk[0] = static_cast<bf16_t>(p0);
+    pk[1] = static_cast<bf16_t>(p1);
+    uint32_t word = __builtin_bit_cast(uint32_t, pk);
+    asm volatile("" : "+v"(word), "+v"(psum));  // keep the work in this slot of the schedule
+    pw[t4][j] = word;
+  };
+
+  // ---- phase A: O += V^T(tile-1) P(tile-1) beside the first part of the softmax step on S(tile) ----
+  auto phase_a = [&](auto pv_c, auto odd_c, int k_tile, int v_tile) {
+    constexpr bool DO_PV = decltype(pv_c)::value;
+    constexpr int ODD = decltype(odd_c)::value ? 1 : 0;
+    const bf16_t* Vt = Vbuf + (1 - ODD) * kTileElems;
+    bf16x8_t f[16];
+    if constexpr (DO_PV) {
+      f[0] = v_frag(Vt, 0);
+      f[1] = v_frag(Vt, 1);
+    }
+    static_for<16>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      constexpr int t4 = i >> 2, db = i & 3;
+      if constexpr (DO_PV) {
+        if constexpr (i + 2 < 16) f[i + 2] = v_frag(Vt, i + 2);
+        oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], attn_as_bf16x8(pw[t4]), oacc[db], 0, 0, 0);
+      }
+      if constexpr (i == 0) issue_k(k_tile, ODD);
+      if constexpr (i == 1) issue_v(v_tile, ODD);
+      if constexpr (i == 0) softmax_rowmax(std::integral_constant<int, 0>());
+      if constexpr (i == 1) softmax_rowmax(std::integral_constant<int, 1>());
+      if constexpr (i == 2) softmax_ref();
+      // key slice j of P may be rewritten once chunk 4 j + 3 has issued its MFMA
+      if constexpr (i >= 4 && i < 12)
+        softmax_word(std::integral_constant<int, (i >= 4 && i < 12) ? (i >> 2) - 1 : 0>(), std::integral_constant<int, (i & 3)>());
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  auto rescale = [&]() {
+    if (__any(alpha != 1.0f)) {
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+    }
+  };
+  // ---- phase B: S(tile+1) = K(tile+1) Q^T beside the rest of P(tile) and the LDS writes ----
+  auto phase_b = [&](auto qk_c, auto odd_c) {
+    constexpr bool DO_QK = decltype(qk_c)::value;
+    constexpr int ODD = decltype(odd_c)::value ? 1 : 0;
+    const bf16_t* Ks = Kbuf + (1 - ODD) * kTileElems;
+    bf16x8_t f[16];
+    if constexpr (DO_QK) {
+      f[0] = k_frag(Ks, 0);
+      f[1] = k_frag(Ks, 1);
+    }
+    static_for<16>([&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      constexpr int kb = i >> 3, ks = i & 7;
+      if constexpr (DO_QK) {
+        if constexpr (i + 2 < 16) f[i + 2] = k_frag(Ks, i + 2);
+        if constexpr (ks == 0) {
+          f32x16_t z;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) z[r] = 0.f;
+          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], qf[ks], z, 0, 0, 0);
+        } else {
+          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], qf[ks], sacc[kb], 0, 0, 0);
+        }
+      }
+      // key slices 2 and 3 of P read S's second key block, which chunk 8 starts to overwrite
+      if constexpr (i < 8) softmax_word(std::integral_constant<int, 2 + (i >> 2)>(), std::integral_constant<int, (i & 3)>());
+      if constexpr (i == 7) l_run = fmaf(l_run, alpha, psum);
+      if constexpr (i == 15) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this iteration's tiles have landed
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+
+  // ---- prologue: K(0), K(1) in LDS, S(0) ----
+  issue_k(0, 0);
+  issue_k(1, 1);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): Q fragments and the tiles above have landed
+  __syncthreads();
+  {
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      sacc[i >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag(Kbuf, i), qf[i & 7], sacc[i >> 3], 0, 0, 0);
+  }
+  __syncthreads();  // K buffer 0 is rewritten in iteration 0
+
+  using T = std::true_type;
+  using F = std::false_type;
+  if (CAUSAL && 0 >= first_masked) apply_mask(0);
+  phase_a(F(), F(), 2, 0);
+  phase_b(T(), F());
+  __syncthreads();
+
+  auto pair = [&](int t, auto mask_c) {
+    constexpr bool MASK = decltype(mask_c)::value;
+    {
+      if constexpr (MASK) apply_mask(t);
+      phase_a(T(), T(), min(t + 2, n_tiles - 1), t);  // K past the end: a harmless reload
+      rescale();
+      phase_b(T(), T());
+      __syncthreads();
+    }
+    {
+      const int u = t + 1;
+      if constexpr (MASK) apply_mask(u);
+      phase_a(T(), F(), min(u + 2, n_tiles - 1), u);
+      rescale();
+      phase_b(T(), F());
+      __syncthreads();
+    }
+  };
+  int t = 1;
+  for (; t + 1 < first_masked; t += 2) pair(t, F());
+  if constexpr (CAUSAL) {
+    for (; t < n_tiles - 1; t += 2) pair(t, T());
+  }
+  {
+    t = n_tiles - 1;
+    if (CAUSAL) apply_mask(t);
+    phase_a(T(), T(), t, t);
+    rescale();
+    phase_b(F(), T());
+    __syncthreads();
+    const bf16_t* Vt = Vbuf + kTileElems;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(Vt, i), attn_as_bf16x8(pw[i >> 2]), oacc[i & 3], 0, 0, 0);
+  }
+
+  // ---- epilogue ----
+  const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
+  const float l_tot = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+  const float inv_l = 1.0f / l_tot;
+  const float l_true = l_tot * __builtin_amdgcn_exp2f(m_run - m_true);
+  bf16_t* __restrict__ orow = O + head_off + static_cast<size_t>(qi) * kAttnD;
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int rq = 0; rq < 4; ++rq) {
+      bf16x4_t o4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o4[e] = static_cast<bf16_t>(oacc[db][4 * rq + e] * inv_l);
+      *reinterpret_cast<bf16x4_t*>(orow + 32 * db + 8 * rq + 4 * g) = o4;
+    }
+  if (g == 0) {
+    const size_t so = (static_cast<size_t>(head) * S + qi) * 8;
+    const float m_nat = m_true * 0.69314718055994530942f;
+    Vec<float, 4> mv, lv;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      mv[e] = m_nat;
+      lv[e] = l_true;
+    }
+    store_vec<float, 4>(softmax_max + so, mv);
+    store_vec<float, 4>(softmax_max + so + 4, mv);
+    store_vec<float, 4>(softmax_sum + so, lv);
+    store_vec<float, 4>(softmax_sum + so + 4, lv);
+  }
+}
+
+}  // namespace mi

@@ -504,6 +504,14 @@ def _attention_launcher() -> CachingLauncher:
             lds_bytes=_ATTN_LDS_BYTES,
         )
         for c in (1, 0)
+    ] + [
+        LaunchConfig(
+            f"fused_attention_fwd_bf16_d128_{'causal' if c else 'full'}_v5",
+            512,
+            meta={"CAUSAL": c, "WAVES": 8, "INTERLEAVED": 1, "DIRECT_LDS": 1},
+            lds_bytes=4 * 64 * 128 * 2,  # two K and two V tiles of [64, 128] bf16
+        )
+        for c in (1, 0)
     ]
     return CachingLauncher(
         "fused_attention_fwd_bf16_d128",
@@ -540,7 +548,7 @@ def fused_attention(
         return out, smax, ssum
     if variant is None and waves is None and pingpong is None:
         variant = _ATTN_DEFAULT_VARIANT if S % 256 == 0 else None
-    if variant in ("v2", "v4"):
+    if variant in ("v2", "v4", "v5"):
         # 256 queries per workgroup (4 wavefronts of 64 or 8 of 32), causal query blocks paired
         _require(S % 256 == 0, "the interleaved kernels need S to be a multiple of 256")
         l = _attention_launcher()
@@ -556,7 +564,7 @@ def fused_attention(
             _stream(),
         )
         return out, smax, ssum
-    _require(variant is None, "variant must be None, 'v2' or 'v4'")
+    _require(variant is None, "variant must be None, 'v2', 'v4' or 'v5'")
     if waves is None:
         waves = _ATTN_DEFAULT_WAVES if S % 256 == 0 else 4
     _require(waves in (4, 8) and S % (32 * waves) == 0, "waves must be 4 or 8 and 32*waves must divide S")
@@ -686,4 +694,5 @@ def fused_attention_backward(
 
 _ATTN_DEFAULT_WAVES = 8
 _ATTN_DEFAULT_PINGPONG = True
-_ATTN_DEFAULT_VARIANT = "v4"  # the interleaved 8-wavefront kernel whenever S % 256 == 0
+# the interleaved 8-wavefront kernel with direct global -> LDS tile loads whenever S % 256 == 0
+_ATTN_DEFAULT_VARIANT = "v5"

@@ -52,7 +52,7 @@ def test_attention_vs_oracle(K, O, B, N, S, causal, waves):
     np.testing.assert_allclose(ssum.cpu().numpy(), l_ref, rtol=2e-3)
 
 
-@pytest.mark.parametrize("variant", ["v4", "v2"])
+@pytest.mark.parametrize("variant", ["v5", "v4", "v2"])
 @pytest.mark.parametrize(
     "B,N,S,causal,qmul",
     [
@@ -82,7 +82,7 @@ def test_attention_interleaved_kernels_vs_oracle(K, O, B, N, S, causal, qmul, va
     np.testing.assert_allclose(ssum.cpu().numpy(), l_ref, rtol=2e-3)
 
 
-@pytest.mark.parametrize("variant", ["v4", "v2"])
+@pytest.mark.parametrize("variant", ["v5", "v4", "v2"])
 def test_attention_interleaved_kernels_full_length(K, variant):
     """S = 4096: statistics equal to the phase-separated kernel's to fp32 rounding, outputs
     within bf16 rounding of it, causal output independent of later keys."""
@@ -146,8 +146,11 @@ def test_attention_causality_and_sdpa_full_size_slice(K):
     assert torch.equal(out, outp) and torch.equal(smax, smaxp) and torch.equal(ssum, ssump)
     # the default at this length is the interleaved 8-wavefront kernel
     outd, smaxd, ssumd = K.fused_attention(q, k, v, scale, True)
-    outv, smaxv, ssumv = K.fused_attention(q, k, v, scale, True, variant="v4")
+    outv, smaxv, ssumv = K.fused_attention(q, k, v, scale, True, variant="v5")
     assert torch.equal(outd, outv) and torch.equal(smaxd, smaxv) and torch.equal(ssumd, ssumv)
+    # the direct-to-LDS kernel computes what the register-staged one does, bit for bit
+    out4, smax4, ssum4 = K.fused_attention(q, k, v, scale, True, variant="v4")
+    assert torch.equal(outd, out4) and torch.equal(smaxd, smax4) and torch.equal(ssumd, ssum4)
     out, smax, ssum = outd, smaxd, ssumd
     for causal in (False,):
         a = K.fused_attention(q, k, v, scale, causal, waves=4)
