@@ -55,7 +55,15 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
   const bf16_t* __restrict__ Vh = V + head_off;
 
   const int q0 = q_block * kAttnV5BM;
-  const int qi = q0 + wave * 32 + li;
+  // Wavefronts 4..7 take the 32-query sub-blocks in reverse order: with a causal mask a sub-block
+  // needs 1 + sub / 2 of the four diagonal tiles, and the two wavefronts that share a SIMD
+  // (w and w + 4) then have five tiles of diagonal work between them on every SIMD instead of
+  // four to six.
+#ifndef MI_ATTN_V5_BALANCE
+#define MI_ATTN_V5_BALANCE 1
+#endif
+  const int sub = (CAUSAL && MI_ATTN_V5_BALANCE && wave >= 4) ? 11 - wave : wave;
+  const int qi = q0 + sub * 32 + li;
 
   bf16x8_t qf[8];
 #pragma unroll
@@ -177,30 +185,40 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
   };
 
   // ---- phase A: O += V^T(tile-1) P(tile-1) beside the first part of the softmax step on S(tile) ----
-  auto phase_a = [&](auto pv_c, auto odd_c, int k_tile, int v_tile) {
+  // GUARD: the wavefront-uniform flags do_pv / do_sm switch the matrix and the softmax work of the
+  // phase off (diagonal tiles that lie wholly above this wavefront's queries); without GUARD they
+  // are ignored and the phase is straight-line code.
+  auto phase_a = [&](auto pv_c, auto odd_c, int k_tile, int v_tile, auto guard_c, bool do_pv, bool do_sm) {
     constexpr bool DO_PV = decltype(pv_c)::value;
+    constexpr bool GUARD = decltype(guard_c)::value;
     constexpr int ODD = decltype(odd_c)::value ? 1 : 0;
     const bf16_t* Vt = Vbuf + (1 - ODD) * kTileElems;
     bf16x8_t f[16];
     if constexpr (DO_PV) {
-      f[0] = v_frag(Vt, 0);
-      f[1] = v_frag(Vt, 1);
+      if (!GUARD || do_pv) {
+        f[0] = v_frag(Vt, 0);
+        f[1] = v_frag(Vt, 1);
+      }
     }
     static_for<16>([&](auto ic) {
       constexpr int i = decltype(ic)::value;
       constexpr int t4 = i >> 2, db = i & 3;
       if constexpr (DO_PV) {
-        if constexpr (i + 2 < 16) f[i + 2] = v_frag(Vt, i + 2);
-        oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], attn_as_bf16x8(pw[t4]), oacc[db], 0, 0, 0);
+        if (!GUARD || do_pv) {
+          if constexpr (i + 2 < 16) f[i + 2] = v_frag(Vt, i + 2);
+          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], attn_as_bf16x8(pw[t4]), oacc[db], 0, 0, 0);
+        }
       }
       if constexpr (i == 0) issue_k(k_tile, ODD);
       if constexpr (i == 1) issue_v(v_tile, ODD);
-      if constexpr (i == 0) softmax_rowmax(std::integral_constant<int, 0>());
-      if constexpr (i == 1) softmax_rowmax(std::integral_constant<int, 1>());
-      if constexpr (i == 2) softmax_ref();
-      // key slice j of P may be rewritten once chunk 4 j + 3 has issued its MFMA
-      if constexpr (i >= 4 && i < 12)
-        softmax_word(std::integral_constant<int, (i >= 4 && i < 12) ? (i >> 2) - 1 : 0>(), std::integral_constant<int, (i & 3)>());
+      if (!GUARD || do_sm) {
+        if constexpr (i == 0) softmax_rowmax(std::integral_constant<int, 0>());
+        if constexpr (i == 1) softmax_rowmax(std::integral_constant<int, 1>());
+        if constexpr (i == 2) softmax_ref();
+        // key slice j of P may be rewritten once chunk 4 j + 3 has issued its MFMA
+        if constexpr (i >= 4 && i < 12)
+          softmax_word(std::integral_constant<int, (i >= 4 && i < 12) ? (i >> 2) - 1 : 0>(), std::integral_constant<int, (i & 3)>());
+      }
       __builtin_amdgcn_sched_barrier(0);
     });
   };
@@ -213,32 +231,39 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
     }
   };
   // ---- phase B: S(tile+1) = K(tile+1) Q^T beside the rest of P(tile) and the LDS writes ----
-  auto phase_b = [&](auto qk_c, auto odd_c) {
+  auto phase_b = [&](auto qk_c, auto odd_c, auto guard_c, bool do_qk, bool do_sm) {
     constexpr bool DO_QK = decltype(qk_c)::value;
+    constexpr bool GUARD = decltype(guard_c)::value;
     constexpr int ODD = decltype(odd_c)::value ? 1 : 0;
     const bf16_t* Ks = Kbuf + (1 - ODD) * kTileElems;
     bf16x8_t f[16];
     if constexpr (DO_QK) {
-      f[0] = k_frag(Ks, 0);
-      f[1] = k_frag(Ks, 1);
+      if (!GUARD || do_qk) {
+        f[0] = k_frag(Ks, 0);
+        f[1] = k_frag(Ks, 1);
+      }
     }
     static_for<16>([&](auto ic) {
       constexpr int i = decltype(ic)::value;
       constexpr int kb = i >> 3, ks = i & 7;
       if constexpr (DO_QK) {
-        if constexpr (i + 2 < 16) f[i + 2] = k_frag(Ks, i + 2);
-        if constexpr (ks == 0) {
-          f32x16_t z;
+        if (!GUARD || do_qk) {
+          if constexpr (i + 2 < 16) f[i + 2] = k_frag(Ks, i + 2);
+          if constexpr (ks == 0) {
+            f32x16_t z;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) z[r] = 0.f;
-          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], qf[ks], z, 0, 0, 0);
-        } else {
-          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], qf[ks], sacc[kb], 0, 0, 0);
+            for (int r = 0; r < 16; ++r) z[r] = 0.f;
+            sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], qf[ks], z, 0, 0, 0);
+          } else {
+            sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], qf[ks], sacc[kb], 0, 0, 0);
+          }
         }
       }
-      // key slices 2 and 3 of P read S's second key block, which chunk 8 starts to overwrite
-      if constexpr (i < 8) softmax_word(std::integral_constant<int, 2 + (i >> 2)>(), std::integral_constant<int, (i & 3)>());
-      if constexpr (i == 7) l_run = fmaf(l_run, alpha, psum);
+      if (!GUARD || do_sm) {
+        // key slices 2 and 3 of P read S's second key block, which chunk 8 starts to overwrite
+        if constexpr (i < 8) softmax_word(std::integral_constant<int, 2 + (i >> 2)>(), std::integral_constant<int, (i & 3)>());
+        if constexpr (i == 7) l_run = fmaf(l_run, alpha, psum);
+      }
       if constexpr (i == 15) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this iteration's tiles have landed
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -262,26 +287,34 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
 
   using T = std::true_type;
   using F = std::false_type;
-  if (CAUSAL && 0 >= first_masked) apply_mask(0);
-  phase_a(F(), F(), 2, 0);
-  phase_b(T(), F());
+  // last key tile this wavefront's queries can see (only the diagonal tiles differ between wavefronts)
+  const int last_tile = CAUSAL ? first_masked + (sub >> 1) : n_tiles - 1;
+  if (CAUSAL && 0 == last_tile) apply_mask(0);
+  phase_a(F(), F(), 2, 0, F(), true, true);
+  phase_b(T(), F(), F(), true, true);
   __syncthreads();
 
   auto pair = [&](int t, auto mask_c) {
     constexpr bool MASK = decltype(mask_c)::value;
     {
-      if constexpr (MASK) apply_mask(t);
-      phase_a(T(), T(), min(t + 2, n_tiles - 1), t);  // K past the end: a harmless reload
-      rescale();
-      phase_b(T(), T());
+      if constexpr (MASK) {
+        if (t == last_tile) apply_mask(t);
+      }
+      const bool sm = !MASK || t <= last_tile;
+      phase_a(T(), T(), min(t + 2, n_tiles - 1), t, mask_c, t - 1 <= last_tile, sm);  // K past the end: a harmless reload
+      if (sm) rescale();
+      phase_b(T(), T(), mask_c, t + 1 <= last_tile, sm);
       __syncthreads();
     }
     {
       const int u = t + 1;
-      if constexpr (MASK) apply_mask(u);
-      phase_a(T(), F(), min(u + 2, n_tiles - 1), u);
-      rescale();
-      phase_b(T(), F());
+      if constexpr (MASK) {
+        if (u == last_tile) apply_mask(u);
+      }
+      const bool sm = !MASK || u <= last_tile;
+      phase_a(T(), F(), min(u + 2, n_tiles - 1), u, mask_c, u - 1 <= last_tile, sm);
+      if (sm) rescale();
+      phase_b(T(), F(), mask_c, u + 1 <= last_tile, sm);
       __syncthreads();
     }
   };
@@ -292,15 +325,18 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
   }
   {
     t = n_tiles - 1;
-    if (CAUSAL) apply_mask(t);
-    phase_a(T(), T(), t, t);
-    rescale();
-    phase_b(F(), T());
+    const bool sm = t <= last_tile;
+    if (CAUSAL && t == last_tile) apply_mask(t);
+    phase_a(T(), T(), t, t, std::integral_constant<bool, CAUSAL>(), t - 1 <= last_tile, sm);
+    if (sm) rescale();
+    phase_b(F(), T(), std::integral_constant<bool, CAUSAL>(), false, sm);
     __syncthreads();
-    const bf16_t* Vt = Vbuf + kTileElems;
+    if (sm) {
+      const bf16_t* Vt = Vbuf + kTileElems;
 #pragma unroll
-    for (int i = 0; i < 16; ++i)
-      oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(Vt, i), attn_as_bf16x8(pw[i >> 2]), oacc[i & 3], 0, 0, 0);
+      for (int i = 0; i < 16; ++i)
+        oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(Vt, i), attn_as_bf16x8(pw[i >> 2]), oacc[i & 3], 0, 0, 0);
+    }
   }
 
   // ---- epilogue ----
