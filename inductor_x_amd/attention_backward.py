@@ -32,12 +32,35 @@ def _bmm_f32(a, b):
     return torch.bmm(a, b, out_dtype=torch.float32)
 
 
-def attention_forward_over_gemms(q, k, v, scale: float, causal: bool):
+def _heads_per_round(heads: int, S: int) -> int:
+    return max(1, min(heads, _SCORE_BYTES_BUDGET // max(2 * S * S * 4, 1)))
+
+
+def dropout_keep_mask(seed: int, first_head: int, heads: int, S: int, keep_prob: float, device):
+    """The [heads, S, S] mask of kept probabilities for heads first_head .. first_head + heads - 1 of
+    a call whose dropout seed is `seed`: a uniform draw per entry from a generator seeded with
+    seed + first_head, kept where it is below keep_prob.  Forward and backward walk the heads in the
+    same rounds (_heads_per_round) and so regenerate identical masks from the seed alone."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed((int(seed) + int(first_head)) & ((1 << 63) - 1))
+    return torch.rand(heads, S, S, device=device, generator=gen) < keep_prob
+
+
+def _check_keep_prob(keep_prob: float) -> float:
+    if not (0.0 <= keep_prob <= 1.0):
+        raise ValueError(f"attention: keep_prob must lie in [0, 1], got {keep_prob}")
+    return 0.0 if keep_prob == 0.0 else 1.0 / keep_prob
+
+
+def attention_forward_over_gemms(q, k, v, scale: float, causal: bool, keep_prob: float = 1.0, seed: int = 0):
     """softmax(q k^T * scale [+ causal mask]) v with library GEMMs for shapes and element types the
     fused forward kernels do not cover (any head dimension and sequence length; bf16, fp16, fp32).
     Returns (out, softmax_max, softmax_sum) like kernels.fused_attention: the row statistics are
     fp32 [B, N, S, 8], the probabilities are rounded to the operand type before the second product
-    and O(S^2) intermediates move through HBM, a bounded number of heads at a time."""
+    and O(S^2) intermediates move through HBM, a bounded number of heads at a time.
+    keep_prob < 1 drops probabilities after the softmax (dropout_keep_mask) and scales the kept ones
+    by 1 / keep_prob; the row statistics are those of the undropped softmax."""
+    inv_keep = _check_keep_prob(keep_prob)
     for t in (q, k, v):
         if not (t.is_cuda and t.dtype in _GEMM_DTYPES and t.dtype == q.dtype and t.dim() == 4):
             raise ValueError("attention forward: q, k, v must be 4-D GPU tensors of one floating-point type")
@@ -50,7 +73,7 @@ def attention_forward_over_gemms(q, k, v, scale: float, causal: bool):
     smax = torch.empty(heads, S, dtype=torch.float32, device=q.device)
     ssum = torch.empty(heads, S, dtype=torch.float32, device=q.device)
     if heads and S:
-        chunk = max(1, min(heads, _SCORE_BYTES_BUDGET // max(2 * S * S * 4, 1)))
+        chunk = _heads_per_round(heads, S)
         mask = torch.ones(S, S, dtype=torch.bool, device=q.device).triu_(1) if causal else None
         for h0 in range(0, heads, chunk):
             sl = slice(h0, min(h0 + chunk, heads))
@@ -61,31 +84,40 @@ def attention_forward_over_gemms(q, k, v, scale: float, causal: bool):
             p = s.sub_(m.unsqueeze(-1)).exp_()
             l = p.sum(-1)
             smax[sl], ssum[sl] = m, l
+            if keep_prob < 1.0:
+                p.mul_(dropout_keep_mask(seed, h0, sl.stop - h0, S, keep_prob, q.device)).mul_(inv_keep)
             out[sl] = (_bmm_f32(p.to(q.dtype), vh[sl]) / l.unsqueeze(-1)).to(q.dtype)
     stats = lambda t: t.view(B, N, S, 1).expand(B, N, S, 8).contiguous()  # noqa: E731
     return out.view(B, N, S, D), stats(smax), stats(ssum)
 
 
 def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale: float, causal: bool,
-                             use_kernels=None):
+                             use_kernels=None, keep_prob: float = 1.0, seed: int = 0):
     """q, k, v, out, dout: [B, N, S, D] of one floating-point type; softmax_max / softmax_sum:
     [B, N, S, 8] fp32 from the forward.  Returns (dq, dk, dv) in that type.  use_kernels: None = fused
-    kernels where they apply (bf16, head dimension 128, sequence a multiple of 128)."""
+    kernels where they apply (bf16, head dimension 128, sequence a multiple of 128, no dropout).
+    keep_prob < 1 with the forward's seed regenerates the forward's dropout mask (GEMM path only)."""
     fits = (q.dim() == 4 and q.dtype == torch.bfloat16 and q.size(3) == 128 and q.size(2) % 128 == 0
-            and q.size(2) > 0)
+            and q.size(2) > 0 and keep_prob == 1.0)
     if use_kernels is None:
         use_kernels = fits
     if use_kernels:
+        if keep_prob != 1.0:
+            raise NotImplementedError("attention backward: the fused kernels have no dropout")
         from . import kernels
 
         return kernels.fused_attention_backward(
             q.contiguous(), k.contiguous(), v.contiguous(), out.contiguous(), dout.contiguous(),
             softmax_max.contiguous(), softmax_sum.contiguous(), scale, causal,
         )
-    return _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale, causal)
+    return _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale, causal, keep_prob, seed)
 
 
-def _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale: float, causal: bool):
+def _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale: float, causal: bool,
+                         keep_prob: float = 1.0, seed: int = 0):
+    # With dropout, Pd = P * keep / keep_prob takes P's place in dV = Pd^T dO, and dP = (dO V^T) * keep /
+    # keep_prob; D = rowsum(dO * O) = rowsum(P * dP) still holds because O = Pd V.
+    inv_keep = _check_keep_prob(keep_prob)
     for t in (q, k, v, out, dout):
         if not (t.is_cuda and t.dtype in _GEMM_DTYPES and t.dtype == q.dtype and t.dim() == 4):
             raise ValueError("attention backward: q, k, v, out, dout must be 4-D GPU tensors of one floating-point type")
@@ -103,8 +135,7 @@ def _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale: fl
     dv = torch.empty_like(vh)
     if heads == 0 or S == 0:
         return dq.view(B, N, S, D), dk.view(B, N, S, D), dv.view(B, N, S, D)
-    per_head = 2 * S * S * 4
-    chunk = max(1, min(heads, _SCORE_BYTES_BUDGET // max(per_head, 1)))
+    chunk = _heads_per_round(heads, S)
     mask = None
     if causal:
         mask = torch.ones(S, S, dtype=torch.bool, device=q.device).triu_(1)
@@ -117,9 +148,14 @@ def _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale: fl
         if mask is not None:
             s.masked_fill_(mask, float("-inf"))
         p = s.exp_().div_(l[sl].unsqueeze(-1))
-        p16 = p.to(q.dtype)
-        dv[sl] = torch.bmm(p16.transpose(1, 2), doc)
         dp = _bmm_f32(doc, vc.transpose(1, 2))
+        if keep_prob < 1.0:
+            keep = dropout_keep_mask(seed, h0, sl.stop - h0, S, keep_prob, q.device)
+            dv[sl] = torch.bmm((p * keep).mul_(inv_keep).to(q.dtype).transpose(1, 2), doc)
+            dp.mul_(keep).mul_(inv_keep)
+            del keep
+        else:
+            dv[sl] = torch.bmm(p.to(q.dtype).transpose(1, 2), doc)
         delta = (doc.float() * oc.float()).sum(-1, keepdim=True)
         ds16 = p.mul_(dp.sub_(delta)).mul_(scale).to(q.dtype)
         dq[sl] = torch.bmm(ds16, kc)

@@ -12,8 +12,10 @@ The device implementation runs the MFMA kernel of this package.  As in the
 reference the op receives the *inverse* scale from the pattern and inverts it
 (:20-35, :162).  The reference's pattern carries no mask; a causal mask enters
 through the op's own arguments: sparse_mode 2 or 3, or next_tockens == 0 with
-pre_tockens covering the sequence.  Supported: layout "BNSD", bf16, head
-dimension 128, no pse / padding mask / dropout; anything else raises.
+pre_tockens covering the sequence.  Supported: layouts "BNSD", "BSH", "SBH"; the fused kernels take bf16, head
+dimension 128, no pse / padding mask; dropout (keep_prob < 1) runs the GEMM path; anything else raises.  Layouts
+"BSH" and "SBH" are viewed as [B, N, S, D], copied once into that order for the
+kernels and copied back.
 The backward op recomputes the probabilities from the saved row statistics inside fused
 gradient kernels (head dimension 128; kernels.fused_attention_backward) and falls back to the
 same mathematics over library GEMMs for other head dimensions (attention_backward.py); the
@@ -51,6 +53,38 @@ npu_def.define(
 )
 
 
+LAYOUTS = ("BNSD", "BSH", "SBH")
+
+
+def _to_bnsd(t, head_num: int, layout: str):
+    """View a tensor given in `layout` as [B, N, S, D] (reference
+    inductor_x/npu_fusion_attention_graph.py:49-61 reads B and S out of the same three layouts)."""
+    if layout == "BNSD":
+        return t
+    if t.dim() != 3 or t.size(2) % head_num:
+        raise ValueError(f"npu_fa: layout {layout} needs a 3-d tensor whose hidden size is a multiple of "
+                         f"head_num {head_num}, got {tuple(t.shape)}")
+    d = t.size(2) // head_num
+    if layout == "BSH":
+        return t.view(t.size(0), t.size(1), head_num, d).permute(0, 2, 1, 3)
+    return t.view(t.size(0), t.size(1), head_num, d).permute(1, 2, 0, 3)  # SBH
+
+
+def _from_bnsd(t, layout: str):
+    """[B, N, S, D] back to `layout`, contiguous."""
+    if layout == "BNSD":
+        return t
+    b, n, s, d = t.shape
+    if layout == "BSH":
+        return t.permute(0, 2, 1, 3).reshape(b, s, n * d)
+    return t.permute(2, 0, 1, 3).reshape(s, b, n * d)  # SBH
+
+
+def _check_layout(op: str, layout: str):
+    if layout not in LAYOUTS:
+        raise NotImplementedError(f"{op}: layout {layout!r} (supported: {', '.join(LAYOUTS)})")
+
+
 def _is_causal(seq_len: int, atten_mask, pre_tockens: int, next_tockens: int, sparse_mode: int) -> bool:
     if sparse_mode in (2, 3):
         return True
@@ -69,12 +103,13 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
                actual_seq_qlen=None, actual_seq_kvlen=None, sparse_mode=0, gen_mask_parallel=True, sync=False):
     from . import kernels
 
-    if input_layout != "BNSD":
-        raise NotImplementedError(f"npu_fa: layout {input_layout!r} (only 'BNSD')")
+    _check_layout("npu_fa", input_layout)
+    layout = input_layout
+    query, key, value = (_to_bnsd(t, head_num, layout) for t in (query, key, value))
     if pse is not None or padding_mask is not None or prefix or actual_seq_qlen or actual_seq_kvlen:
         raise NotImplementedError("npu_fa: pse / padding_mask / prefix / variable sequence lengths")
-    if keep_prob != 1.0:
-        raise NotImplementedError("npu_fa: dropout (keep_prob != 1)")
+    if not (0.0 <= keep_prob <= 1.0):
+        raise ValueError(f"npu_fa: keep_prob {keep_prob} outside [0, 1]")
     if query.size(1) != head_num:
         raise ValueError(f"npu_fa: head_num {head_num} does not match query of shape {tuple(query.shape)}")
     if scale == 0:
@@ -82,18 +117,25 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
     # the graph pattern passes the divisor of the scores; the kernel multiplies
     real_scale = 1.0 / scale
     causal = _is_causal(query.size(2), atten_mask, pre_tockens, next_tockens, sparse_mode)
-    if query.dtype == torch.bfloat16 and query.size(3) == 128 and query.size(2) % 128 == 0 and query.size(2) > 0:
+    seed = numels = 0
+    if (keep_prob == 1.0 and query.dtype == torch.bfloat16 and query.size(3) == 128 and query.size(2) % 128 == 0
+            and query.size(2) > 0):
         out, smax, ssum = kernels.fused_attention(
             query.contiguous(), key.contiguous(), value.contiguous(), real_scale, causal
         )
     else:
-        # shapes and element types outside the fused kernels: the same mathematics over library GEMMs
+        # shapes and element types outside the fused kernels, and dropout: the same mathematics over
+        # library GEMMs.  The dropout seed comes from torch's CPU generator (torch.manual_seed makes a
+        # run repeatable) and travels to the backward in the op's seed output, as in the reference's op.
         from .attention_backward import attention_forward_over_gemms
 
-        out, smax, ssum = attention_forward_over_gemms(query, key, value, real_scale, causal)
+        if keep_prob < 1.0:
+            seed = int(torch.randint(0, 1 << 62, (1,), dtype=torch.int64).item())
+            numels = query.size(0) * query.size(1) * query.size(2) * key.size(2)
+        out, smax, ssum = attention_forward_over_gemms(query, key, value, real_scale, causal, keep_prob, seed)
     softmax_out = torch.empty([0], dtype=query.dtype, device=query.device)
-    zero = lambda: torch.zeros([1], dtype=torch.int64)  # noqa: E731  seed / offset / numel: no dropout
-    return out, smax, ssum, softmax_out, zero(), zero(), zero()
+    word = lambda v: torch.tensor([v], dtype=torch.int64)  # noqa: E731  seed / offset / numels live on the host
+    return _from_bnsd(out, layout), smax, ssum, softmax_out, word(seed), word(0), word(numels)
 
 
 gpu_lib.impl("npu_fa", npu_fa_gpu)
@@ -108,20 +150,27 @@ def npu_fa_backward_gpu(query, key, value, dy, head_num, input_layout, *, pse=No
     the op receives the inverse scale and inverts it)."""
     from .attention_backward import fused_attention_backward
 
-    if input_layout != "BNSD":
-        raise NotImplementedError(f"npu_fa_backward: layout {input_layout!r} (only 'BNSD')")
+    _check_layout("npu_fa_backward", input_layout)
+    layout = input_layout
     if pse is not None or padding_mask is not None or prefix or actual_seq_qlen or actual_seq_kvlen:
         raise NotImplementedError("npu_fa_backward: pse / padding_mask / prefix / variable sequence lengths")
-    if keep_prob != 1.0:
-        raise NotImplementedError("npu_fa_backward: dropout (keep_prob != 1)")
+    if not (0.0 <= keep_prob <= 1.0):
+        raise ValueError(f"npu_fa_backward: keep_prob {keep_prob} outside [0, 1]")
+    if keep_prob < 1.0 and seed is None:
+        raise ValueError("npu_fa_backward: dropout needs the forward's seed")
     if softmax_max is None or softmax_sum is None or attention_in is None:
         raise ValueError("npu_fa_backward: needs softmax_max, softmax_sum and attention_in from the forward")
     if scale_value == 0:
         raise ZeroDivisionError("npu_fa_backward: the inverse scale factor is zero")
+    query, key, value, attention_in, dy = (
+        _to_bnsd(t, head_num, layout).contiguous() for t in (query, key, value, attention_in, dy)
+    )
     causal = _is_causal(query.size(2), atten_mask, pre_tockens, next_tockens, sparse_mode)
     dq, dk, dv = fused_attention_backward(
-        query, key, value, attention_in, dy.contiguous(), softmax_max, softmax_sum, 1.0 / scale_value, causal
+        query, key, value, attention_in, dy, softmax_max, softmax_sum, 1.0 / scale_value, causal,
+        keep_prob=keep_prob, seed=int(seed.item()) if keep_prob < 1.0 else 0,
     )
+    dq, dk, dv = (_from_bnsd(t, layout) for t in (dq, dk, dv))
     return dq, dk, dv, torch.empty([0], dtype=query.dtype, device=query.device)
 
 
@@ -276,7 +325,8 @@ _registered = False
 def register_fx_pass() -> None:
     """Register the replacement with Inductor's joint-graph pattern pass
     (reference inductor_x/npu_fusion_attention_graph.py:134-230), for inference and for
-    training graphs; patterns with dropout are not rewritten (the kernels have none)."""
+    training graphs.  Patterns with dropout are not rewritten: the op would serve them over library
+    GEMMs with O(S^2) traffic, slower than the attention Inductor picks for them itself."""
     global _registered
     if _registered:
         return

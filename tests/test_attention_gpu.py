@@ -349,3 +349,116 @@ def test_attention_op_outside_the_fused_kernels(dtype, B, N, S, D, causal):
     for g, r in zip(got, (qf.grad, kf.grad, vf.grad)):
         assert g.dtype == dtype
         assert (g.float() - r).abs().max().item() <= (1e-4 if dtype == torch.float32 else 3e-2) * max(r.abs().max().item(), 1.0)
+
+
+def _unfused_fp32(q, k, v, inv, causal, keep=None, keep_prob=1.0):
+    """fp32 autograd-able definition on [B, N, S, D] tensors; `keep` is a [B, N, S, S] dropout mask."""
+    S = q.size(2)
+    s = (q @ k.transpose(-1, -2)) / inv
+    if causal:
+        s = s.masked_fill(torch.ones(S, S, device=q.device, dtype=torch.bool).triu(1), float("-inf"))
+    p = torch.softmax(s, -1)
+    if keep is not None:
+        p = p * keep / keep_prob
+    return p @ v
+
+
+@pytest.mark.parametrize("layout", ["BSH", "SBH"])
+@pytest.mark.parametrize("dtype,B,N,S,D,causal", [
+    (torch.bfloat16, 2, 3, 256, 128, True),   # the fused kernels
+    (torch.float16, 1, 4, 72, 64, False),     # the GEMM path
+])
+def test_attention_op_layouts(layout, dtype, B, N, S, D, causal):
+    """Layouts BSH and SBH (reference inductor_x/npu_fusion_attention_graph.py:53-61): outputs and
+    gradients come back in the caller's layout and equal the BNSD call on the same numbers bit for bit;
+    the BNSD call itself is checked against fp32 autograd."""
+    announce(f"attention op layout {layout} {dtype} B={B} N={N} S={S} D={D} causal={causal}")
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
+    torch.manual_seed(21)
+    base = [torch.randn(B, N, S, D, device=DEV).to(dtype) for _ in range(4)]
+
+    def to_layout(t):
+        if layout == "BSH":
+            return t.permute(0, 2, 1, 3).reshape(B, S, N * D).contiguous()
+        return t.permute(2, 0, 1, 3).reshape(S, B, N * D).contiguous()
+
+    def from_layout(t):
+        if layout == "BSH":
+            return t.view(B, S, N, D).permute(0, 2, 1, 3)
+        return t.view(S, B, N, D).permute(1, 2, 0, 3)
+
+    inv = D ** 0.5
+    mode = 3 if causal else 0
+    q, k, v = (t.clone().requires_grad_() for t in base[:3])
+    ref = npu_fusion_attention_graph(q, k, v, N, "BNSD", scale=inv, sparse_mode=mode)
+    ref[0].backward(base[3])
+    ql, kl, vl = (to_layout(t).requires_grad_() for t in base[:3])
+    got = npu_fusion_attention_graph(ql, kl, vl, N, layout, scale=inv, sparse_mode=mode)
+    assert got[0].shape == ql.shape and got[0].is_contiguous()
+    assert got[1].shape == (B, N, S, 8) and torch.equal(got[1], ref[1]) and torch.equal(got[2], ref[2])
+    got[0].backward(to_layout(base[3]))
+    assert torch.equal(from_layout(got[0]), ref[0])
+    for g, r in zip((ql.grad, kl.grad, vl.grad), (q.grad, k.grad, v.grad)):
+        assert g.shape == ql.shape and torch.equal(from_layout(g), r)
+    qf, kf, vf = (t.float().requires_grad_() for t in base[:3])
+    want = _unfused_fp32(qf, kf, vf, inv, causal)
+    want.backward(base[3].float())
+    assert (ref[0].float() - want).abs().max().item() <= 2e-2 * max(want.abs().max().item(), 1.0)
+    for g, r in zip((q.grad, k.grad, v.grad), (qf.grad, kf.grad, vf.grad)):
+        assert (g.float() - r).abs().max().item() <= 3e-2 * max(r.abs().max().item(), 1.0)
+    with pytest.raises(NotImplementedError):
+        npu_fusion_attention_graph(ql, kl, vl, N, "TND", scale=inv)
+    with pytest.raises(ValueError):
+        npu_fusion_attention_graph(ql, kl, vl, 7, layout, scale=inv)  # 7 divides neither hidden size
+
+
+@pytest.mark.parametrize("dtype,B,N,S,D,causal,keep_prob", [
+    (torch.bfloat16, 2, 2, 256, 128, True, 0.8), (torch.float32, 1, 3, 100, 32, False, 0.5),
+])
+def test_attention_op_dropout(dtype, B, N, S, D, causal, keep_prob):
+    """keep_prob < 1 (reference inductor_x/npu_fusion_attention_graph.py:150-164 passes
+    keep_prob = 1 - dropout_p): output and gradients against fp32 autograd of the unfused graph under
+    the mask that the op's seed output regenerates; the kept fraction; repeatability under
+    torch.manual_seed; keep_prob 0 gives zeros, as torch's dropout with p = 1 does."""
+    announce(f"attention op dropout {dtype} B={B} N={N} S={S} D={D} causal={causal} keep={keep_prob}")
+    from inductor_x_amd.attention_backward import _heads_per_round, dropout_keep_mask
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
+    torch.manual_seed(33)
+    q, k, v = (torch.randn(B, N, S, D, device=DEV).to(dtype).requires_grad_() for _ in range(3))
+    do = torch.randn(B, N, S, D, device=DEV).to(dtype)
+    inv = D ** 0.5
+    mode = 3 if causal else 0
+    torch.manual_seed(5)
+    res = npu_fusion_attention_graph(q, k, v, N, "BNSD", scale=inv, keep_prob=keep_prob, sparse_mode=mode)
+    out, seed, numels = res[0], res[4], res[6]
+    assert seed.dtype == torch.int64 and seed.device.type == "cpu" and int(numels) == B * N * S * S
+    out.backward(do)
+    heads, step = B * N, _heads_per_round(B * N, S)
+    keep = torch.cat([dropout_keep_mask(int(seed), h0, min(step, heads - h0), S, keep_prob, DEV)
+                      for h0 in range(0, heads, step)]).view(B, N, S, S)
+    assert abs(keep.float().mean().item() - keep_prob) < 0.01
+    qf, kf, vf = (t.detach().float().requires_grad_() for t in (q, k, v))
+    want = _unfused_fp32(qf, kf, vf, inv, causal, keep, keep_prob)
+    want.backward(do.float())
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert (out.float() - want).abs().max().item() <= tol * max(want.abs().max().item(), 1.0)
+    for g, r in zip((q.grad, k.grad, v.grad), (qf.grad, kf.grad, vf.grad)):
+        assert (g.float() - r).abs().max().item() <= (1e-4 if dtype == torch.float32 else 3e-2) * max(r.abs().max().item(), 1.0)
+    # the row statistics are those of the undropped softmax
+    plain = npu_fusion_attention_graph(q.detach(), k.detach(), v.detach(), N, "BNSD", scale=inv, sparse_mode=mode)
+    torch.testing.assert_close(res[1], plain[1], rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(res[2], plain[2], rtol=2e-2, atol=1e-2)
+    torch.manual_seed(5)
+    again = npu_fusion_attention_graph(q.detach(), k.detach(), v.detach(), N, "BNSD", scale=inv,
+                                       keep_prob=keep_prob, sparse_mode=mode)
+    assert int(again[4]) == int(seed) and torch.equal(again[0], out.detach())
+    other = npu_fusion_attention_graph(q.detach(), k.detach(), v.detach(), N, "BNSD", scale=inv,
+                                       keep_prob=keep_prob, sparse_mode=mode)
+    assert int(other[4]) != int(seed) and not torch.equal(other[0], out.detach())
+    zero = npu_fusion_attention_graph(q.detach(), k.detach(), v.detach(), N, "BNSD", scale=inv, keep_prob=0.0,
+                                      sparse_mode=mode)
+    assert zero[0].abs().max().item() == 0.0
+    with pytest.raises(ValueError):
+        npu_fusion_attention_graph(q, k, v, N, "BNSD", scale=inv, keep_prob=1.5)
