@@ -16,6 +16,7 @@ import os
 import shutil
 import subprocess
 import tempfile
+import threading
 from typing import Iterable, Optional
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -53,8 +54,23 @@ def hipcc_path() -> str:
     return cand
 
 
+def toolchain_version() -> str:
+    """ROCm release the code objects are built with (part of every cache key: an object built by
+    another compiler release is never reused).  Read from the installation's version file; running
+    the compiler for its banner would cost more than most cache hits save."""
+    root = os.path.dirname(os.path.dirname(os.path.realpath(hipcc_path())))
+    for rel in (".info/version", ".info/version-dev"):
+        try:
+            with open(os.path.join(root, rel)) as f:
+                return f.read().strip()
+        except OSError:
+            continue
+    return "unknown"
+
+
 def _headers_digest() -> str:
     h = hashlib.sha256()
+    h.update(toolchain_version().encode())
     for name in sorted(os.listdir(HEADER_DIR)):
         if name.endswith(".h"):
             with open(os.path.join(HEADER_DIR, name), "rb") as f:
@@ -101,7 +117,8 @@ def _writable_store(prefer_intree: bool) -> str:
     for d in order:
         try:
             os.makedirs(d, exist_ok=True)
-            probe = os.path.join(d, f".w{os.getpid()}")
+            # one probe name per thread: the compile pool's threads run this concurrently
+            probe = os.path.join(d, f".w{os.getpid()}.{threading.get_ident()}")
             with open(probe, "w"):
                 pass
             os.unlink(probe)
@@ -155,6 +172,23 @@ def compile_source(
             return out
         finally:
             fcntl.flock(lock, fcntl.LOCK_UN)
+
+
+def harvest(source_dir: Optional[str] = None) -> int:
+    """Copy the code objects of `source_dir` (default: the per-user store) into the package's
+    store of generated kernels, so that a tree shipped to a machine without a warm per-user store
+    starts with them.  Returns the number of objects copied."""
+    source_dir = source_dir or user_store()
+    os.makedirs(GENERATED_STORE, exist_ok=True)
+    copied = 0
+    for name in sorted(os.listdir(source_dir)) if os.path.isdir(source_dir) else ():
+        dst = os.path.join(GENERATED_STORE, name)
+        if name.endswith(".hsaco") and not os.path.exists(dst) and not os.path.exists(os.path.join(INTREE_STORE, name)):
+            tmp = dst + f".tmp{os.getpid()}"
+            shutil.copyfile(os.path.join(source_dir, name), tmp)
+            os.replace(tmp, dst)
+            copied += 1
+    return copied
 
 
 def aot_source(name: str) -> str:

@@ -239,6 +239,51 @@ class CachingLauncher:
         self._save_best(best, timings)
         return best
 
+    def pick(self, shape_key: str, default_idx: int, eligible: Sequence[int], args, grid_arg, stream: int) -> int:
+        """Configuration for one problem shape of a kernel family whose best variant depends on the
+        extents: the heuristic's `default_idx` unless config.autotune is on; then the fastest of
+        `eligible`, timed once per shape (outputs are overwritten with the same values by every
+        variant) and remembered in `<code object>.<shape_key>.best_config` for later processes."""
+        if not config.autotune or len(eligible) < 2:
+            return default_idx
+        tuned = self.__dict__.setdefault("_tuned", {})
+        idx = tuned.get(shape_key)
+        if idx is not None:
+            return idx
+        import torch
+
+        if torch.cuda.is_current_stream_capturing():
+            return default_idx
+        path = (self._hsaco_path[: -len(".hsaco")] + f".{shape_key}.best_config") if self._hsaco_path else None
+        symbols = {cfg.symbol: i for i, (cfg, _) in enumerate(self.launchers)}
+        if path and os.path.exists(path):
+            try:
+                with open(path) as f:
+                    rec = json.load(f)
+                if rec.get("symbol") in symbols and symbols[rec["symbol"]] in eligible:
+                    tuned[shape_key] = symbols[rec["symbol"]]
+                    return tuned[shape_key]
+            except (OSError, ValueError):
+                pass
+        timings, best, best_ms = {}, default_idx, float("inf")
+        for i in eligible:
+            try:
+                ms = self.bench(i, args, grid_arg, stream, warmup=5, rep=20)
+            except launcher.LauncherError as e:
+                log.debug("config %s of %s failed to launch: %s", self.launchers[i][0].symbol, self.name, e)
+                continue
+            timings[self.launchers[i][0].symbol] = ms
+            if ms < best_ms:
+                best, best_ms = i, ms
+        tuned[shape_key] = best
+        if path:
+            try:
+                with open(path, "w") as f:
+                    json.dump({"symbol": self.launchers[best][0].symbol, "shape": shape_key, "timings_ms": timings}, f)
+            except OSError:
+                pass
+        return best
+
     def run(self, *args, grid, stream: int) -> None:
         if not self.launchers:
             self.precompile()

@@ -23,6 +23,7 @@ from .hip_heuristics import (
     LaunchConfig,
     cdiv,
     col_fold_lds_bytes,
+    grid as row_grid,
     next_power_of_2,
     row_reduction_plan,
     split_reduction_plan,
@@ -250,12 +251,18 @@ def fused_relu_sigmoid_rowsum(x: torch.Tensor, variant: Optional[tuple] = None) 
     _require(rnumel % 4 == 0 and _aligned(x), "row length must be a multiple of 4 and x 16-byte aligned")
     _require(x.numel() < 2**31, "numel must fit int32 indexing")
     l = _rowsum_launcher()
+    args = (x.data_ptr(), out.data_ptr(), xnumel, rnumel)
     if variant is None:
         plan = row_reduction_plan(xnumel, rnumel, 4, persistent=False)
-        variant = (plan.block, max(plan.tpr, 64))  # instantiated shapes start at one wavefront per row
-    b, t = variant
-    idx = _find(l, f"fused_relu_sigmoid_rowsum_f32_b{b}_t{t}")
-    l._launch(idx, (x.data_ptr(), out.data_ptr(), xnumel, rnumel), (cdiv(xnumel, b // t), 1, 1), _stream())
+        b, t = plan.block, max(plan.tpr, 64)  # instantiated shapes start at one wavefront per row
+        idx = _find(l, f"fused_relu_sigmoid_rowsum_f32_b{b}_t{t}")
+        # every instantiated shape loops over any row length: all are candidates when tuning
+        if config.autotune:
+            idx = l.pick(f"{xnumel}x{rnumel}", idx, range(len(l.launchers)), args, row_grid(xnumel), _stream())
+    else:
+        b, t = variant
+        idx = _find(l, f"fused_relu_sigmoid_rowsum_f32_b{b}_t{t}")
+    l._launch(idx, args, (cdiv(xnumel, l.launchers[idx][0].meta["PER_WG0"]), 1, 1), _stream())
     return out
 
 
@@ -289,15 +296,18 @@ def add_rmsnorm(
         while variant not in have and variant[2] < 8:
             variant = (variant[0], variant[1], variant[2] * 2)
         _require(variant in have, f"row length {cols} exceeds the persistent kernel's reach")
+        tuned = True
+    else:
+        tuned = False
     b, t, i = variant
     _require(cols <= t * 8 * i, "variant too small for the row length")
     idx = _find(l, f"add_rmsnorm_bf16_b{b}_t{t}_i{i}")
-    l._launch(
-        idx,
-        (h.data_ptr(), r.data_ptr(), w.data_ptr(), out.data_ptr(), s.data_ptr(), rows, cols, float(eps)),
-        (cdiv(rows, b // t), 1, 1),
-        _stream(),
-    )
+    args = (h.data_ptr(), r.data_ptr(), w.data_ptr(), out.data_ptr(), s.data_ptr(), rows, cols, float(eps))
+    if tuned and config.autotune:
+        # candidates when tuning: the register-resident shapes that hold a whole row
+        fits = [k for k, (cfg, _) in enumerate(l.launchers) if cols <= cfg.meta["TPR"] * 8 * cfg.meta["ITERS"]]
+        idx = l.pick(f"{rows}x{cols}", idx, fits, args, row_grid(rows), _stream())
+    l._launch(idx, args, (cdiv(rows, l.launchers[idx][0].meta["PER_WG0"]), 1, 1), _stream())
     return out, s
 
 

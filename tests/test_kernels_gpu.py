@@ -5,6 +5,8 @@ Tolerances: bit-exact for integer / index / byte-moving outputs; <= 1e-5
 relative for fp32 outputs; <= 2e-2 absolute for bf16 outputs.  Shapes follow
 the reference's own test shapes where it has them (cited per test).
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -392,3 +394,55 @@ def test_bandwidth_print(K, tmp_path, monkeypatch, capsys):
     line = [l for l in capsys.readouterr().out.splitlines() if l.startswith("gather_rows:")]
     assert len(line) == 1 and line[0].endswith("GB/s") and " ms " in line[0]
     assert torch.equal(out, table)
+
+
+def test_autotune_reaches_the_product_entry_points(K, O, tmp_path, monkeypatch):
+    """With config.autotune on, kernels.fused_relu_sigmoid_rowsum and kernels.add_rmsnorm time the
+    instantiated shapes that fit the problem once per extents, write a per-shape record beside the
+    code object, launch the winner, and return the same numbers as without tuning."""
+    import glob
+    import json
+    import shutil
+
+    from inductor_x_amd import config, kernels
+    from inductor_x_amd.hip_heuristics import CachingLauncher
+
+    announce("autotune through kernels.*")
+    torch.manual_seed(8)
+    x = torch.randn(300, 2048, device=DEV)
+    h, r = (torch.randn(129, 1024, device=DEV).bfloat16() for _ in range(2))
+    w = torch.ones(1024, device=DEV).bfloat16()
+    plain_sum = K.fused_relu_sigmoid_rowsum(x)
+    plain_norm = K.add_rmsnorm(h, r, w, 1e-6)
+    # a private copy of each family's code object, so the records land in tmp_path
+    for getter in (kernels._rowsum_launcher, kernels._rmsnorm_launcher):
+        fam = getter()
+        fam.precompile()
+        private = str(tmp_path / os.path.basename(fam._hsaco_path))
+        shutil.copyfile(fam._hsaco_path, private)
+        monkeypatch.setattr(fam, "_hsaco_path", private)
+        monkeypatch.setattr(fam, "_tuned", {}, raising=False)
+    monkeypatch.setattr(config, "autotune", True)
+    launched = []
+    real = CachingLauncher._launch
+    monkeypatch.setattr(CachingLauncher, "_launch",
+                        lambda self, idx, *a, **k: (launched.append(self.launchers[idx][0].symbol), real(self, idx, *a, **k))[1])
+    tuned_sum = K.fused_relu_sigmoid_rowsum(x)
+    last_of_sum = launched[-1]  # the timing launches come first, the launch that counts last
+    tuned_norm = K.add_rmsnorm(h, r, w, 1e-6)
+    last_of_norm = launched[-1]
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(tuned_sum.cpu().numpy(), plain_sum.cpu().numpy(), rtol=1e-6)
+    assert torch.equal(tuned_norm[1], plain_norm[1])
+    assert (tuned_norm[0].float() - plain_norm[0].float()).abs().max().item() <= 2e-2
+    records = {os.path.basename(p).split(".", 1)[1]: json.loads(open(p).read()) for p in glob.glob(str(tmp_path / "*.best_config"))}
+    assert set(records) == {"300x2048.best_config", "129x1024.best_config"}
+    rs, rn = records["300x2048.best_config"], records["129x1024.best_config"]
+    assert len(rs["timings_ms"]) == len(kernels._ROWSUM_VARIANTS) and rs["timings_ms"][rs["symbol"]] == min(rs["timings_ms"].values())
+    # rows of 1024 bf16 = 128 vectors: only shapes with TPR * ITERS >= 128 are candidates
+    assert all(int(s.split("_t")[1].split("_i")[0]) * int(s.rsplit("_i", 1)[1]) >= 128 for s in rn["timings_ms"])
+    assert (last_of_sum, last_of_norm) == (rs["symbol"], rn["symbol"])
+    # the second call of a shape times nothing
+    monkeypatch.setattr(CachingLauncher, "bench", lambda *a, **k: pytest.fail("timed a second time"))
+    again = K.fused_relu_sigmoid_rowsum(x)
+    assert torch.equal(again, tuned_sum) and launched[-1] == rs["symbol"]
