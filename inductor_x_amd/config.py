@@ -132,3 +132,14 @@ def apply_inductor_settings() -> None:
     # reduction and the column reduction stay two kernels
     if hasattr(inductor_config.triton, "mix_order_reduction"):
         inductor_config.triton.mix_order_reduction = False
+
+
+def streaming_read_bytes() -> int:
+    """A generated kernel whose read set exceeds this many bytes loads with the non-temporal hint
+    (it reads each element once, and a set of more than half the memory-side cache is not found
+    there again by the next kernel).  INDUCTOR_X_AMD_STREAM_READS overrides the limit in bytes;
+    0 switches the hint off."""
+    forced = os.environ.get("INDUCTOR_X_AMD_STREAM_READS")
+    if forced is not None:
+        return int(forced)
+    return hardware().mall_bytes // 2

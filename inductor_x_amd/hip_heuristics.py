@@ -624,7 +624,9 @@ class GeneratedKernel:
         m = self.meta
         if self.mode == "pointwise":
             # a tiled kernel (static shapes) carries its own workgroup count
-            grid = (m["grid"] if "grid" in m else cdiv(xnumel, m["block"] * m["vec"] * m.get("unroll", 1)), 1, 1)
+            g = m["grid"] if "grid" in m else cdiv(xnumel, m["block"] * m["vec"] * m.get("unroll", 1))
+            mult = int(m.get("grid_multiple", 1))  # the kernel deals workgroups out to the dies itself
+            grid = (cdiv(g, mult) * mult, 1, 1)
             return LaunchPlan([("main", grid, (m["block"],), 0, (xnumel,), False)], 0, cand)
         if self.mode == "row":
             rounds = cdiv(xnumel, m["block"] // m["tpr"])

@@ -149,7 +149,7 @@ def test_graph4_gather_and_permute(O):
     assert torch.equal(emb, out)
     t = torch.randn(4, 2048, 32, 128).bfloat16()
     out, code = compile_and_code(lambda t: t.permute(0, 2, 1, 3).contiguous(), t.to(DEV))
-    assert "mi::vload<VEC>" in code and "mi::vstore<VEC" in code  # 16-byte accesses on both sides
+    assert "mi::vload_x<VEC, STREAM_READS>" in code and "mi::vstore<VEC" in code  # 16-byte accesses on both sides
     assert np.array_equal(bits(out), O.permute4(bits(t), (0, 2, 1, 3)))
 
 
