@@ -36,27 +36,27 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
 # copy kernel of known size in the same run.  Keyed by (configuration, path); an entry
 # applies only while the call still launches exactly the symbols that were profiled.
 MEASURED_TRAFFIC: dict = {
-    ('1', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_817_884, "write_bytes": 32_742,
+    ('1', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_817_904, "write_bytes": 32_740,
         "profile": "profiles/rowsum_f32_1024x4096_warm_pmc.txt"},
-    ('1', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 16_805_597, "write_bytes": 32_742,
+    ('1', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 16_805_617, "write_bytes": 32_740,
         "profile": "profiles/rowsum_f32_1024x4096_warm_pmc.txt"},
-    ('1cold', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_819_024, "write_bytes": 32_740,
+    ('1cold', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_817_850, "write_bytes": 32_741,
         "profile": "profiles/rowsum_f32_1024x4096_cold_pmc.txt"},
-    ('2', 'kernel'): {"symbols": ["add_rmsnorm_bf16_b512_t512_i1"], "fetch_bytes": 134_289_498, "write_bytes": 134_240_626,
+    ('2', 'kernel'): {"symbols": ["add_rmsnorm_bf16_b512_t512_i1"], "fetch_bytes": 134_290_266, "write_bytes": 134_228_892,
         "profile": "profiles/add_rmsnorm_bf16_8192x4096_pmc.txt"},
-    ('2', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 134_297_689, "write_bytes": 134_277_240,
+    ('2', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 134_298_458, "write_bytes": 134_324_096,
         "profile": "profiles/add_rmsnorm_bf16_8192x4096_pmc.txt"},
-    ('3', 'kernel'): {"symbols": ["col_mean_var_argmax_partial_f32_c32_r8_u8", "col_mean_var_argmax_final_f32_c4_s16"], "fetch_bytes": 138_611_172, "write_bytes": 536_141,
+    ('3', 'kernel'): {"symbols": ["col_mean_var_argmax_partial_f32_c32_r8_u8", "col_mean_var_argmax_final_f32_c4_s16"], "fetch_bytes": 138_611_205, "write_bytes": 536_106,
         "profile": "profiles/col_mean_var_argmax_f32_65536x512_pmc.txt"},
-    ('3', 'torch.compile'): {"symbols": ["hip_col_0_partial", "hip_col_0_final"], "fetch_bytes": 147_016_534, "write_bytes": 1_583_867,
+    ('3', 'torch.compile'): {"symbols": ["hip_col_0_partial", "hip_col_0_final"], "fetch_bytes": 147_016_569, "write_bytes": 1_583_762,
         "profile": "profiles/col_mean_var_argmax_f32_65536x512_pmc.txt"},
-    ('4a', 'kernel'): {"symbols": ["gather_rows_b16_b256_t128_r2"], "fetch_bytes": 66_447_574, "write_bytes": 67_213_165,
+    ('4a', 'kernel'): {"symbols": ["gather_rows_b16_b256_t128_r2"], "fetch_bytes": 66_444_435, "write_bytes": 67_185_799,
         "profile": "profiles/gather_rows_bf16_50304x1024_32768_pmc.txt"},
-    ('4a', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 67_434_256, "write_bytes": 67_096_785,
+    ('4a', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 65_558_445, "write_bytes": 67_105_289,
         "profile": "profiles/gather_rows_bf16_50304x1024_32768_pmc.txt"},
-    ('4b', 'kernel'): {"symbols": ["permute_copy_b16_b256_p16_t32x4"], "fetch_bytes": 268_466_890, "write_bytes": 268_421_811,
+    ('4b', 'kernel'): {"symbols": ["permute_copy_b16_b256_p16_t32x4"], "fetch_bytes": 268_466_801, "write_bytes": 268_438_653,
         "profile": "profiles/permute_0213_bf16_16x2048x32x128_pmc.txt"},
-    ('4b', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 268_441_292, "write_bytes": 268_519_390,
+    ('4b', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 268_441_203, "write_bytes": 268_544_924,
         "profile": "profiles/permute_0213_bf16_16x2048x32x128_pmc.txt"},
 }
 
