@@ -62,6 +62,7 @@ from torch.utils._sympy.printers import ExprPrinter
 from torch.utils._sympy.value_ranges import ValueRanges
 
 from .. import config as backend_config
+from ..hip_heuristics import col_fold_all_planes
 
 DTYPE_TO_HIP = {
     torch.float32: "float",
@@ -2050,6 +2051,21 @@ class HipKernel(SIMDKernel):
         if not self.col_reductions:
             raise UnsupportedHipCodegen("column kernel without a reduction")
         ct, rl, vec = self.col_ct, self.col_rl, self.vec
+        # A plain fp32 sum of a value whose moments the kernel accumulates anyway (mean beside
+        # variance) is read off the moments (mean * count) instead of being summed once more.
+        alias: dict[str, ColReduction] = {}
+        for c in self.col_reductions:
+            if c.cxx == "mi::RedSum":
+                twin = next((w for w in self.col_reductions if w.kind == "welford_reduce" and w.value == c.value), None)
+                if twin is not None:
+                    alias[c.acc] = twin
+        all_reductions = list(self.col_reductions)
+        self.col_reductions = [c for c in all_reductions if c.acc not in alias]
+        self.ws_words = 0
+        for c in self.col_reductions:
+            c.ws_offset_words = self.ws_words
+            self.ws_words += c.words
+        aliased = [c for c in all_reductions if c.acc in alias]
         max_words = max(c.words for c in self.col_reductions)
         extra = [f"float* __restrict__ ws", f"const {idx_t} xnumel", f"const {idx_t} rnumel", "const int nsplit"]
         # rows handed to a thread between two looks at the loop counter
@@ -2079,6 +2095,8 @@ class HipKernel(SIMDKernel):
                     kind = c.cxx
                     src.writeline(f"mi::ColAcc<{kind}, VEC> {c.acc};")
                     src.writeline(f"{c.acc}.init();")
+                for c in aliased:
+                    src.writeline(f"mi::ColAccNone {c.acc};  // read off {alias[c.acc].acc}")
                 src.writeline("if (xmask) {")
                 with src.indent():
                     src.splice(self._entry_code(self.x_entries))
@@ -2141,14 +2159,17 @@ class HipKernel(SIMDKernel):
                     src.writeline("}")
                 src.writeline("}")
                 for c in self.col_reductions:
-                    kind = c.cxx
-                    src.writeline(f"typename {kind}::M {c.acc}_m[VEC];")
+                    src.writeline(f"typename {c.cxx}::M {c.acc}_m[VEC];")
                     src.writeline("#pragma unroll")
                     src.writeline(f"for (int i = 0; i < VEC; ++i) {c.acc}_m[i] = {c.acc}.finish(i);")
-                    src.writeline(f"mi::col_fold<{kind}, VEC, CT, RL>({c.acc}_m, ct, rl, lds_dyn);")
-                    if not direct:
+                # one fold for all reductions: lane exchanges inside a wavefront, one or two LDS rounds
+                kinds_ = ", ".join(c.cxx for c in self.col_reductions)
+                states_ = ", ".join(f"{c.acc}_m" for c in self.col_reductions)
+                src.writeline(f"mi::col_fold_all<VEC, CT, RL, {kinds_}>(lds_dyn, ct, rl, {states_});")
+                if not direct:
+                    for c in self.col_reductions:
                         src.writeline(
-                            f"if (rl == 0) mi::col_store_partial<{kind}, VEC>(ws + {c.ws_offset_words} * "
+                            f"if (rl == 0) mi::col_store_partial<{c.cxx}, VEC>(ws + {c.ws_offset_words} * "
                             f"static_cast<mi::i64>(nsplit) * xnumel, {c.acc}_m, xindex, xnumel, split, nsplit);"
                         )
                 if direct:
@@ -2168,6 +2189,9 @@ class HipKernel(SIMDKernel):
                                 src.writeline("const int sl = 0;")
                                 for c in self.col_reductions:
                                     src.writeline(f"const auto {c.result} = {c.acc}_m[col_];")
+                                for c in aliased:
+                                    w = alias[c.acc]
+                                    src.writeline(f"const auto {c.result} = {w.acc}_m[col_].mean * {w.acc}_m[col_].n;")
                                 for line in self._result_defs_col:
                                     src.writeline(line)
                                 src.splice(self._final_indexing_code())
@@ -2206,13 +2230,16 @@ class HipKernel(SIMDKernel):
             kinds = ", ".join(c.cxx for c in self.col_reductions)
             states = ", ".join(c.result for c in self.col_reductions)
             src.writeline(f"mi::col_final_fold_all<CPW, SL, {kinds}>(lds_fin, slot, sl, {states});")
+            for c in aliased:
+                src.writeline(f"const auto {c.result} = {alias[c.acc].result}.mean * {alias[c.acc].result}.n;")
             for line in self._result_defs_col:
                 src.writeline(line)
             src.splice(self._final_indexing_code())
             src.splice(self.final_body)
         src.writeline("}")
         meta.update({"ct": ct, "rl": rl, "cpw": cpw, "sl": sl, "ws_words": self.ws_words, "col_unroll": unroll,
-                     "lds_partial": (rl // 2) * ct * vec * max_words * 4})
+                     "lds_partial": max((rl // 2) * ct * vec * max_words * 4,
+                                        col_fold_all_planes(ct, rl) * ct * vec * sum(c.words for c in self.col_reductions) * 4)})
         return codes + "P" + idx_code + idx_code + "i"
 
     def _final_indexing_code(self) -> IndentedBuffer:

@@ -1195,6 +1195,12 @@ struct ColAcc {
   }
 };
 
+// Stands in for the accumulator of a reduction whose result is derived from another one's state.
+struct ColAccNone {
+  template <class VT>
+  __device__ __forceinline__ void step(const VT&, int, bool) {}
+};
+
 // Per-thread: N independent columns whose inputs are moments already.
 template <int N>
 struct ColMomentsAcc {
@@ -1245,6 +1251,98 @@ __device__ __forceinline__ void col_fold(typename R::M (&m)[N], int ct, int rl, 
 #pragma unroll
           for (int k = 0; k < R::W; ++k) w[k] = lds[k * PLANE + slot + i];
           m[i] = R::merge(m[i], R::dec(w));
+        }
+      }
+    }
+  }
+}
+
+// The fold of col_fold for every reduction of a kernel at once, with as few barriers as the
+// shape allows: row lanes that share a wavefront (CT < 64) meet through lane exchanges, the
+// remaining groups are halved through LDS while more than four are left and then collected in
+// one round.  Every state travels as its float words (enc / dec), so a state of any width folds
+// the same way.  lds holds col_fold_all_planes(CT, RL) * CT * N * (sum of R::W) floats.
+// Afterwards threads with rl == 0 own the results.  Merges are commutative up to rounding
+// (arg-reductions break ties by index, moments by Chan's symmetric formula).
+__host__ __device__ constexpr int col_fold_all_in_wave(int ct, int rl) {
+  return ct >= kWave ? 1 : (kWave / ct < rl ? kWave / ct : rl);
+}
+__host__ __device__ constexpr int col_fold_all_planes(int ct, int rl) {
+  const int groups = rl / col_fold_all_in_wave(ct, rl);
+  if (groups <= 1) return 0;
+  const int tree = groups > 4 ? groups / 2 : 0;
+  const int last = (groups < 4 ? groups : 4) - 1;
+  return tree > last ? tree : last;
+}
+template <class R, int N>
+__device__ __forceinline__ void col_state_exchange(typename R::M (&m)[N], int off) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    float w[R::W];
+    R::enc(m[i], w);
+#pragma unroll
+    for (int k = 0; k < R::W; ++k) w[k] = __shfl_xor(w[k], off, kWave);
+    m[i] = R::merge(m[i], R::dec(w));
+  }
+}
+template <class R, int N>
+__device__ __forceinline__ void col_state_put(float* lds, int plane, int slot, int& word, const typename R::M (&m)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    float w[R::W];
+    R::enc(m[i], w);
+#pragma unroll
+    for (int k = 0; k < R::W; ++k) lds[(word + k) * plane + slot + i] = w[k];
+  }
+  word += R::W;
+}
+template <class R, int N>
+__device__ __forceinline__ void col_state_take(const float* lds, int plane, int slot, int& word, typename R::M (&m)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    float w[R::W];
+#pragma unroll
+    for (int k = 0; k < R::W; ++k) w[k] = lds[(word + k) * plane + slot + i];
+    m[i] = R::merge(m[i], R::dec(w));
+  }
+  word += R::W;
+}
+template <int N, int CT, int RL, class... R>
+__device__ __forceinline__ void col_fold_all(float* lds, int ct, int rl, typename R::M (&... m)[N]) {
+  if constexpr (RL > 1) {
+    constexpr int IN_WAVE = col_fold_all_in_wave(CT, RL);
+    constexpr int GROUPS = RL / IN_WAVE;
+    constexpr int PLANE = col_fold_all_planes(CT, RL) * CT * N;
+#pragma unroll
+    for (int off = CT; off < CT * IN_WAVE; off <<= 1) (col_state_exchange<R, N>(m, off), ...);
+    if constexpr (GROUPS > 1) {
+      const int grp = rl / IN_WAVE;
+      const bool lead = rl % IN_WAVE == 0;
+      int left = GROUPS;
+#pragma unroll
+      for (int half = GROUPS / 2; half >= 4; half >>= 1) {
+        if (lead && grp >= half && grp < 2 * half) {
+          int word = 0;
+          (col_state_put<R, N>(lds, PLANE, ((grp - half) * CT + ct) * N, word, m), ...);
+        }
+        __syncthreads();
+        if (lead && grp < half) {
+          int word = 0;
+          (col_state_take<R, N>(lds, PLANE, (grp * CT + ct) * N, word, m), ...);
+        }
+        __syncthreads();
+        left = half;
+      }
+      // at most four groups are left: one round
+      if (lead && grp >= 1 && grp < left) {
+        int word = 0;
+        (col_state_put<R, N>(lds, PLANE, ((grp - 1) * CT + ct) * N, word, m), ...);
+      }
+      __syncthreads();
+      if (rl == 0) {
+        for (int g2 = 1; g2 < left; ++g2) {
+          int word = 0;
+          (col_state_take<R, N>(lds, PLANE, ((g2 - 1) * CT + ct) * N, word, m), ...);
         }
       }
     }
@@ -1404,41 +1502,55 @@ template <class R>
 struct RedTag {
   typedef R type;
 };
+template <class R>
+__device__ __forceinline__ void col_final_exchange(typename R::M& m, int off) {
+  float w[R::W];
+  R::enc(m, w);
+#pragma unroll
+  for (int k = 0; k < R::W; ++k) w[k] = __shfl_xor(w[k], off, kWave);
+  m = R::merge(m, R::dec(w));
+}
+// Thread (slot, sl) = sl * CPW + slot.  The split lanes of a column that share a wavefront meet
+// through lane exchanges (CPW * SL <= 64: no LDS and no barrier at all); with several wavefronts
+// the first lane of every further wavefront hands its state over through LDS in one round
+// (lds: (waves - 1) * CPW * (sum of R::W) floats at least).  Valid afterwards where sl == 0.
 template <int CPW, int SL, class... R>
 __device__ __forceinline__ void col_final_fold_all(float* lds, int slot, int sl, typename R::M&... m) {
-  constexpr int PLANE = CPW * SL;
-  const int me = sl * CPW + slot;
-  auto put = [&](auto tag, auto& mm, int& off) {
-    typedef typename decltype(tag)::type RR;
-    float w[RR::W];
-    RR::enc(mm, w);
+  static_assert(CPW <= kWave && (CPW & (CPW - 1)) == 0 && (SL & (SL - 1)) == 0, "CPW, SL: powers of two, CPW <= 64");
+  constexpr int SLW = (kWave / CPW) < SL ? (kWave / CPW) : SL;  // split lanes of a column per wavefront
+  constexpr int WAVES = SL / SLW;
 #pragma unroll
-    for (int k = 0; k < RR::W; ++k) lds[(off + k) * PLANE + me] = w[k];
-    off += RR::W;
-  };
-  auto take = [&](auto tag, auto& mm, int& off, int half) {
-    typedef typename decltype(tag)::type RR;
-    float w[RR::W];
+  for (int off = CPW; off < CPW * SLW; off <<= 1) (col_final_exchange<R>(m, off), ...);
+  if constexpr (WAVES > 1) {
+    constexpr int PLANE = (WAVES - 1) * CPW;
+    const int wave = sl / SLW;
+    auto put = [&](auto tag, auto& mm, int& off) {
+      typedef typename decltype(tag)::type RR;
+      float w[RR::W];
+      RR::enc(mm, w);
 #pragma unroll
-    for (int k = 0; k < RR::W; ++k) w[k] = lds[(off + k) * PLANE + (sl + half) * CPW + slot];
-    mm = RR::merge(mm, RR::dec(w));
-    off += RR::W;
-  };
-  __syncthreads();
-  {
-    int off = 0;
-    (put(RedTag<R>{}, m, off), ...);
-  }
-  __syncthreads();
+      for (int k = 0; k < RR::W; ++k) lds[(off + k) * PLANE + (wave - 1) * CPW + slot] = w[k];
+      off += RR::W;
+    };
+    auto take = [&](auto tag, auto& mm, int& off, int from) {
+      typedef typename decltype(tag)::type RR;
+      float w[RR::W];
 #pragma unroll
-  for (int half = SL / 2; half >= 1; half >>= 1) {
-    if (sl < half) {
+      for (int k = 0; k < RR::W; ++k) w[k] = lds[(off + k) * PLANE + (from - 1) * CPW + slot];
+      mm = RR::merge(mm, RR::dec(w));
+      off += RR::W;
+    };
+    if (wave >= 1 && sl % SLW == 0) {
       int off = 0;
-      (take(RedTag<R>{}, m, off, half), ...);
-      off = 0;
       (put(RedTag<R>{}, m, off), ...);
     }
     __syncthreads();
+    if (sl == 0) {
+      for (int from = 1; from < WAVES; ++from) {
+        int off = 0;
+        (take(RedTag<R>{}, m, off, from), ...);
+      }
+    }
   }
 }
 

@@ -371,6 +371,20 @@ def row_reduction_plan(xnumel: int, rnumel: int, elem_bytes: int, persistent: bo
     return RowPlan(block=block, tpr=tpr, vec=vec, iters=iters, rows_per_wg=block // tpr)
 
 
+def col_fold_all_planes(ct: int, rl: int, wave: int = 64) -> int:
+    """LDS planes of the generated column sweep's fold over row lanes (mi::col_fold_all computes
+    the same number on the device): row lanes that share a wavefront meet through lane exchanges,
+    the remaining groups are halved through LDS while more than four are left, then collected in
+    one round.  One plane is CT * VEC * (words of all reduction states) floats."""
+    in_wave = min(wave // ct, rl) if ct < wave else 1
+    groups = rl // max(in_wave, 1)
+    if groups <= 1:
+        return 0
+    tree = groups // 2 if groups > 4 else 0
+    last = min(groups, 4) - 1
+    return max(tree, last)
+
+
 def col_fold_lds_bytes(ct: int, rl: int, wave: int = 64) -> int:
     """Dynamic LDS of the hand-written column sweep's fold over row lanes: row lanes that share a
     wavefront meet through lane exchanges, the remaining groups are halved through LDS while more than
