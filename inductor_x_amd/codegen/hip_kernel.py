@@ -1953,7 +1953,8 @@ class HipKernel(SIMDKernel):
                     # 61 -> 46 us, a plain bf16 add of 96 MiB tensors 42.1 -> 41.0 us.
                     src.writeline(f"const {idx_t} per_die_ = static_cast<{idx_t}>(gridDim.x) >> 3;")
                     src.writeline(
-                        f"const {idx_t} wg_ = static_cast<{idx_t}>(blockIdx.x & 7) * per_die_ + static_cast<{idx_t}>(blockIdx.x >> 3);"
+                        f"const {idx_t} wg_ = (gridDim.x & 7) == 0 ? static_cast<{idx_t}>(blockIdx.x & 7) * per_die_ + "
+                        f"static_cast<{idx_t}>(blockIdx.x >> 3) : static_cast<{idx_t}>(blockIdx.x);"
                     )
                     src.writeline(f"const {idx_t} xbase = (wg_ * UNROLL * {self.block} + threadIdx.x) * VEC;")
                     meta["grid_multiple"] = 8

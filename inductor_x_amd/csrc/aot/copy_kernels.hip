@@ -51,6 +51,11 @@ PERMUTE_VARIANT(256, 8, 1, 32)
 PERMUTE_VARIANT(256, 4, 1, 64)
 PERMUTE_VARIANT(256, 64, 1, 4)
 PERMUTE_VARIANT(256, 64, 4, 4)
+PERMUTE_VARIANT(256, 16, 8, 4)
+PERMUTE_VARIANT(256, 16, 16, 4)
+PERMUTE_VARIANT(256, 16, 4, 8)
+PERMUTE_VARIANT(256, 16, 8, 2)
+PERMUTE_VARIANT(256, 16, 4, 4)
 
 extern "C" __global__ __launch_bounds__(256) void permute_copy_b32_b256_p16_t8x8(
     const uint32_t* in, uint32_t* out, int n0, int n1, int n2, int inner, long long s0,
