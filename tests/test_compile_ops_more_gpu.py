@@ -75,6 +75,12 @@ CASES = {
 }
 
 
+# Accumulation into a 16-bit tensor through atomics rounds after every addition, in whatever order
+# the additions arrive (eager's result depends on that order as well): the bar for these is two
+# units in the last place of bf16 at the magnitudes involved instead of one.
+ORDER_DEPENDENT_16BIT = {"index_put_inplace_accumulate_bf16"}
+
+
 def _compare(got, ref, name):
     got = got if isinstance(got, (tuple, list)) else (got,)
     ref = ref if isinstance(ref, (tuple, list)) else (ref,)
@@ -83,6 +89,8 @@ def _compare(got, ref, name):
         assert g.shape == r.shape and g.dtype == r.dtype, (name, g.shape, r.shape, g.dtype, r.dtype)
         if r.dtype.is_floating_point:
             tol = dict(rtol=2e-2, atol=2e-2) if r.dtype in (torch.bfloat16, torch.float16) else dict(rtol=2e-4, atol=2e-4)
+            if name in ORDER_DEPENDENT_16BIT:
+                tol = dict(rtol=4e-2, atol=4e-2)
             torch.testing.assert_close(g, r, equal_nan=True, **tol)
         else:
             assert torch.equal(g, r), name
