@@ -46,17 +46,17 @@ MEASURED_TRAFFIC: dict = {
         "profile": "profiles/add_rmsnorm_bf16_8192x4096_pmc.txt"},
     ('2', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 134_298_458, "write_bytes": 134_324_096,
         "profile": "profiles/add_rmsnorm_bf16_8192x4096_pmc.txt"},
-    ('3', 'kernel'): {"symbols": ["col_mean_var_argmax_partial_f32_c32_r8_u8", "col_mean_var_argmax_final_f32_c4_s16"], "fetch_bytes": 138_611_205, "write_bytes": 536_106,
+    ('3', 'kernel'): {"symbols": ["col_mean_var_argmax_partial_f32_c32_r8_u8", "col_mean_var_argmax_final_f32_c4_s16"], "fetch_bytes": 138_610_524, "write_bytes": 536_139,
         "profile": "profiles/col_mean_var_argmax_f32_65536x512_pmc.txt"},
-    ('3', 'torch.compile'): {"symbols": ["hip_col_0_partial", "hip_col_0_final"], "fetch_bytes": 147_016_569, "write_bytes": 1_583_762,
+    ('3', 'torch.compile'): {"symbols": ["hip_col_0_partial", "hip_col_0_final"], "fetch_bytes": 144_902_485, "write_bytes": 1_321_930,
         "profile": "profiles/col_mean_var_argmax_f32_65536x512_pmc.txt"},
-    ('4a', 'kernel'): {"symbols": ["gather_rows_b16_b256_t128_r2"], "fetch_bytes": 66_444_435, "write_bytes": 67_185_799,
+    ('4a', 'kernel'): {"symbols": ["gather_rows_b16_b256_t128_r2"], "fetch_bytes": 66_427_429, "write_bytes": 67_191_160,
         "profile": "profiles/gather_rows_bf16_50304x1024_32768_pmc.txt"},
-    ('4a', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 65_558_445, "write_bytes": 67_105_289,
+    ('4a', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 65_552_757, "write_bytes": 67_063_580,
         "profile": "profiles/gather_rows_bf16_50304x1024_32768_pmc.txt"},
-    ('4b', 'kernel'): {"symbols": ["permute_copy_b16_b256_p16_t32x4"], "fetch_bytes": 268_466_801, "write_bytes": 268_438_653,
+    ('4b', 'kernel'): {"symbols": ["permute_copy_b16_b256_p16_t8x2"], "fetch_bytes": 268_431_975, "write_bytes": 268_559_077,
         "profile": "profiles/permute_0213_bf16_16x2048x32x128_pmc.txt"},
-    ('4b', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 268_441_203, "write_bytes": 268_544_924,
+    ('4b', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 268_441_190, "write_bytes": 268_543_678,
         "profile": "profiles/permute_0213_bf16_16x2048x32x128_pmc.txt"},
 }
 
