@@ -165,12 +165,12 @@ extern "C" __global__ __launch_bounds__(512, 1) void fused_attention_fwd_bf16_d1
 
 // v5: the v4 schedule with K and V tiles loaded straight into LDS and V read back transposed
 // (attention_v5.h).  Same workgroup shape and grid as v4; 64 KiB of LDS.
-template <bool CAUSAL>
+template <bool CAUSAL, int WAVES = kAttnV5Waves>
 __device__ __forceinline__ void attention_entry_v5(const bf16_t* q, const bf16_t* k, const bf16_t* v,
                                                    bf16_t* o, float* smax, float* ssum, int n_heads,
                                                    int S, float scale_log2e) {
   constexpr int XCDS = 8;
-  const int n_qb = S / kAttnV5BM;
+  const int n_qb = S / (32 * WAVES);
   const int id = blockIdx.x;
   const int xcd = id % XCDS;
   const int slot = id / XCDS;
@@ -183,12 +183,12 @@ __device__ __forceinline__ void attention_entry_v5(const bf16_t* q, const bf16_t
     const int n_pass = lo != hi ? 2 : 1;
 #pragma nounroll
     for (int pass = 0; pass < n_pass; ++pass)
-      attention_fwd_d128_v5<true>(q, k, v, o, smax, ssum, S, pass == 0 ? hi : lo, head, scale_log2e);
+      attention_fwd_d128_v5<true, WAVES>(q, k, v, o, smax, ssum, S, pass == 0 ? hi : lo, head, scale_log2e);
   } else {
     const int head = (slot / n_qb) * XCDS + xcd;
     const int qb = slot % n_qb;
     if (head >= n_heads) return;
-    attention_fwd_d128_v5<false>(q, k, v, o, smax, ssum, S, qb, head, scale_log2e);
+    attention_fwd_d128_v5<false, WAVES>(q, k, v, o, smax, ssum, S, qb, head, scale_log2e);
   }
 }
 
@@ -201,4 +201,16 @@ extern "C" __global__ __launch_bounds__(512, 1) void fused_attention_fwd_bf16_d1
     const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
     int n_heads, int S, float scale_log2e) {
   attention_entry_v5<false>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
+}
+
+// v5h: the v5 kernel with four wavefronts (128 queries) per workgroup and two workgroups per CU.
+extern "C" __global__ __launch_bounds__(256, 2) void fused_attention_fwd_bf16_d128_causal_v5h(
+    const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
+    int n_heads, int S, float scale_log2e) {
+  attention_entry_v5<true, 4>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
+}
+extern "C" __global__ __launch_bounds__(256, 2) void fused_attention_fwd_bf16_d128_full_v5h(
+    const bf16_t* q, const bf16_t* k, const bf16_t* v, bf16_t* o, float* smax, float* ssum,
+    int n_heads, int S, float scale_log2e) {
+  attention_entry_v5<false, 4>(q, k, v, o, smax, ssum, n_heads, S, scale_log2e);
 }

@@ -27,7 +27,10 @@ namespace mi {
 constexpr int kAttnV5Waves = 8;
 constexpr int kAttnV5BM = kAttnV5Waves * 32;
 
-template <bool CAUSAL>
+// WAVES = 8: one workgroup of 256 queries per CU.  WAVES = 4: 128 queries per workgroup and two
+// workgroups per CU (64 KiB of LDS each), so the two wavefronts of a SIMD belong to different
+// workgroups, share no barrier and drift apart in phase.
+template <bool CAUSAL, int WAVES = kAttnV5Waves>
 __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__ Q,
                                                       const bf16_t* __restrict__ K,
                                                       const bf16_t* __restrict__ V,
@@ -54,7 +57,9 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
   const bf16_t* __restrict__ Kh = K + head_off;
   const bf16_t* __restrict__ Vh = V + head_off;
 
-  const int q0 = q_block * kAttnV5BM;
+  static_assert(WAVES == 8 || WAVES == 4, "8 or 4 wavefronts");
+  constexpr int BM = WAVES * 32;
+  const int q0 = q_block * BM;
   // Wavefronts 4..7 take the 32-query sub-blocks in reverse order: with a causal mask a sub-block
   // needs 1 + sub / 2 of the four diagonal tiles, and the two wavefronts that share a SIMD
   // (w and w + 4) then have five tiles of diagonal work between them on every SIMD instead of
@@ -62,7 +67,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
 #ifndef MI_ATTN_V5_BALANCE
 #define MI_ATTN_V5_BALANCE 1
 #endif
-  const int sub = (CAUSAL && MI_ATTN_V5_BALANCE && wave >= 4) ? 11 - wave : wave;
+  const int sub = (CAUSAL && MI_ATTN_V5_BALANCE && WAVES == 8 && wave >= 4) ? 11 - wave : wave;
   const int qi = q0 + sub * 32 + li;
 
   bf16x8_t qf[8];
@@ -77,8 +82,8 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
     for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
   float m_run = -__builtin_inff(), m_true = -__builtin_inff(), l_run = 0.f, alpha = 1.f;
 
-  const int n_tiles = CAUSAL ? (q0 + kAttnV5BM) / kAttnBN : S / kAttnBN;
-  const int first_masked = CAUSAL ? n_tiles - kAttnV5BM / kAttnBN : n_tiles;
+  const int n_tiles = CAUSAL ? (q0 + BM) / kAttnBN : S / kAttnBN;
+  const int first_masked = CAUSAL ? n_tiles - BM / kAttnBN : n_tiles;
 
   // direct global -> LDS copies: block b of a tile (rows 4 b .. 4 b + 3) is written by one wavefront
   // instruction, lane l filling LDS chunk l of the block (row 4 b + l / 16, chunk position l % 16)
@@ -87,8 +92,8 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
   const int blk_pos = lane & 15;
   auto issue_tile = [&](const bf16_t* __restrict__ src, bf16_t* dst, int tile, auto swz) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int b = 2 * wave + u;
+    for (int u = 0; u < 16 / WAVES; ++u) {
+      const int b = (16 / WAVES) * wave + u;
       const int row = 4 * b + blk_row;
       const int gchunk = blk_pos ^ swz(row);
       const bf16_t* gp = src + (static_cast<size_t>(tile) * kAttnBN + row) * kAttnD + 8 * gchunk;

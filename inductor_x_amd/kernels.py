@@ -530,6 +530,14 @@ def _attention_launcher() -> CachingLauncher:
             lds_bytes=4 * 64 * 128 * 2,  # two K and two V tiles of [64, 128] bf16
         )
         for c in (1, 0)
+    ] + [
+        LaunchConfig(
+            f"fused_attention_fwd_bf16_d128_{'causal' if c else 'full'}_v5h",
+            256,
+            meta={"CAUSAL": c, "WAVES": 4, "INTERLEAVED": 1, "DIRECT_LDS": 1, "WORKGROUPS_PER_CU": 2},
+            lds_bytes=4 * 64 * 128 * 2,
+        )
+        for c in (1, 0)
     ]
     return CachingLauncher(
         "fused_attention_fwd_bf16_d128",
@@ -566,13 +574,15 @@ def fused_attention(
         return out, smax, ssum
     if variant is None and waves is None and pingpong is None:
         variant = _ATTN_DEFAULT_VARIANT if S % 256 == 0 else None
-    if variant in ("v2", "v4", "v5"):
-        # 256 queries per workgroup (4 wavefronts of 64 or 8 of 32), causal query blocks paired
+    if variant in ("v2", "v4", "v5", "v5h"):
+        # 256 queries per workgroup (4 wavefronts of 64 or 8 of 32; v5h: 128 queries, 4 wavefronts of 32),
+        # causal query blocks paired
+        bm = 128 if variant == "v5h" else 256
         _require(S % 256 == 0, "the interleaved kernels need S to be a multiple of 256")
         l = _attention_launcher()
         i = _find(l, f"fused_attention_fwd_bf16_d128_{'causal' if causal else 'full'}_{variant}")
         heads = B * N
-        n_qb = S // 256
+        n_qb = S // bm
         per_head = (n_qb + 1) // 2 if causal else n_qb
         l._launch(
             i,
@@ -582,7 +592,7 @@ def fused_attention(
             _stream(),
         )
         return out, smax, ssum
-    _require(variant is None, "variant must be None, 'v2', 'v4' or 'v5'")
+    _require(variant is None, "variant must be None, 'v2', 'v4', 'v5' or 'v5h'")
     if waves is None:
         waves = _ATTN_DEFAULT_WAVES if S % 256 == 0 else 4
     _require(waves in (4, 8) and S % (32 * waves) == 0, "waves must be 4 or 8 and 32*waves must divide S")

@@ -52,7 +52,7 @@ def test_attention_vs_oracle(K, O, B, N, S, causal, waves):
     np.testing.assert_allclose(ssum.cpu().numpy(), l_ref, rtol=2e-3)
 
 
-@pytest.mark.parametrize("variant", ["v5", "v4", "v2"])
+@pytest.mark.parametrize("variant", ["v5", "v5h", "v4", "v2"])
 @pytest.mark.parametrize(
     "B,N,S,causal,qmul",
     [
@@ -151,6 +151,9 @@ def test_attention_causality_and_sdpa_full_size_slice(K):
     # the direct-to-LDS kernel computes what the register-staged one does, bit for bit
     out4, smax4, ssum4 = K.fused_attention(q, k, v, scale, True, variant="v4")
     assert torch.equal(outd, out4) and torch.equal(smaxd, smax4) and torch.equal(ssumd, ssum4)
+    # and so does the four-wavefront form of it that runs two workgroups per CU
+    outh, smaxh, ssumh = K.fused_attention(q, k, v, scale, True, variant="v5h")
+    assert torch.equal(outd, outh) and torch.equal(smaxd, smaxh) and torch.equal(ssumd, ssumh)
     out, smax, ssum = outd, smaxd, ssumd
     for causal in (False,):
         a = K.fused_attention(q, k, v, scale, causal, waves=4)
