@@ -36,27 +36,27 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
 # copy kernel of known size in the same run.  Keyed by (configuration, path); an entry
 # applies only while the call still launches exactly the symbols that were profiled.
 MEASURED_TRAFFIC: dict = {
-    ('1', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_817_904, "write_bytes": 32_740,
+    ('1', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_817_904, "write_bytes": 32_739,
         "profile": "profiles/rowsum_f32_1024x4096_warm_pmc.txt"},
-    ('1', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 16_805_617, "write_bytes": 32_740,
+    ('1', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 16_805_617, "write_bytes": 32_739,
         "profile": "profiles/rowsum_f32_1024x4096_warm_pmc.txt"},
-    ('1cold', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_817_850, "write_bytes": 32_741,
+    ('1cold', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_817_842, "write_bytes": 32_741,
         "profile": "profiles/rowsum_f32_1024x4096_cold_pmc.txt"},
-    ('2', 'kernel'): {"symbols": ["add_rmsnorm_bf16_b512_t512_i1"], "fetch_bytes": 134_290_266, "write_bytes": 134_228_892,
+    ('2', 'kernel'): {"symbols": ["add_rmsnorm_bf16_b512_t512_i1"], "fetch_bytes": 134_289_921, "write_bytes": 134_238_139,
         "profile": "profiles/add_rmsnorm_bf16_8192x4096_pmc.txt"},
-    ('2', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 134_298_458, "write_bytes": 134_324_096,
+    ('2', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 134_298_112, "write_bytes": 134_342_635,
         "profile": "profiles/add_rmsnorm_bf16_8192x4096_pmc.txt"},
-    ('3', 'kernel'): {"symbols": ["col_mean_var_argmax_partial_f32_c32_r8_u8", "col_mean_var_argmax_final_f32_c4_s16"], "fetch_bytes": 138_610_524, "write_bytes": 536_139,
+    ('3', 'kernel'): {"symbols": ["col_mean_var_argmax_partial_f32_c32_r8_u8", "col_mean_var_argmax_final_f32_c4_s16"], "fetch_bytes": 138_610_822, "write_bytes": 536_096,
         "profile": "profiles/col_mean_var_argmax_f32_65536x512_pmc.txt"},
-    ('3', 'torch.compile'): {"symbols": ["hip_col_0_partial", "hip_col_0_final"], "fetch_bytes": 144_902_485, "write_bytes": 1_321_930,
+    ('3', 'torch.compile'): {"symbols": ["hip_col_0_partial", "hip_col_0_final"], "fetch_bytes": 144_902_796, "write_bytes": 1_321_824,
         "profile": "profiles/col_mean_var_argmax_f32_65536x512_pmc.txt"},
-    ('4a', 'kernel'): {"symbols": ["gather_rows_b16_b256_t128_r2"], "fetch_bytes": 66_427_429, "write_bytes": 67_191_160,
+    ('4a', 'kernel'): {"symbols": ["gather_rows_b16_b256_t128_r2"], "fetch_bytes": 66_448_240, "write_bytes": 67_196_420,
         "profile": "profiles/gather_rows_bf16_50304x1024_32768_pmc.txt"},
-    ('4a', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 65_552_757, "write_bytes": 67_063_580,
+    ('4a', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 65_560_705, "write_bytes": 67_087_919,
         "profile": "profiles/gather_rows_bf16_50304x1024_32768_pmc.txt"},
-    ('4b', 'kernel'): {"symbols": ["permute_copy_b16_b256_p16_t8x2"], "fetch_bytes": 268_431_975, "write_bytes": 268_559_077,
+    ('4b', 'kernel'): {"symbols": ["permute_copy_b16_b256_p16_t8x2"], "fetch_bytes": 268_432_000, "write_bytes": 268_550_121,
         "profile": "profiles/permute_0213_bf16_16x2048x32x128_pmc.txt"},
-    ('4b', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 268_441_190, "write_bytes": 268_543_678,
+    ('4b', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 268_441_216, "write_bytes": 268_551_202,
         "profile": "profiles/permute_0213_bf16_16x2048x32x128_pmc.txt"},
 }
 
