@@ -288,6 +288,26 @@ for name, (fn, args) in cases.items():
 '''
 
 
+DRY_SHAPES = DRY_HEAD + r'''
+import re
+def code_of(fn, *args):
+    torch._dynamo.reset()
+    _, codes = run_and_get_code(torch.compile(fn), *args)
+    return "\n".join(codes)
+# read set above / below half of the 256 MiB memory-side cache; a weight vector does not count
+big = code_of(lambda a, b: a + b, torch.zeros(36 << 20, dtype=torch.bfloat16), torch.zeros(36 << 20, dtype=torch.bfloat16))
+small = code_of(lambda a, b, w: (a + b) * w, torch.zeros(8192, 4096, dtype=torch.bfloat16), torch.zeros(8192, 4096, dtype=torch.bfloat16),
+                torch.zeros(4096, dtype=torch.bfloat16))
+flag = lambda c: re.findall(r"constexpr bool STREAM_READS = (\w+);", c)
+print("STREAM", flag(big), flag(small))
+print("ORDER", "blockIdx.x & 7" in big and "gridDim.x & 7" in big, re.search(r"'grid_multiple': (\d+)", big).group(1))
+col = code_of(lambda x: (x.mean(0), x.var(0, unbiased=False), x.argmax(0)), torch.randn(65536, 512))
+print("COL", "mi::ColAccNone acc0" in col, re.search(r"'ws_words': (\d+)", col).group(1),
+      len(re.findall(r"mi::col_fold_all<VEC, CT, RL, mi::RedWelford, mi::RedArgMax>", col)),
+      "red2.mean * red2.n" in col, re.search(r"'lds_partial': (\d+)", col).group(1))
+'''
+
+
 def _run_dry(tmp_path, text):
     script = tmp_path / "dry_case.py"
     script.write_text(text)
@@ -317,6 +337,22 @@ def test_indirect_accesses_stay_inside_their_buffer(tmp_path, built):
     assert got["embedding"][0] == "100" and got["scatter"][0] == "64"
     for name, (size, found, uses_raw, guarded) in got.items():
         assert found == "True" and uses_raw == "False" and guarded == "True", (name, got[name])
+
+
+def test_generated_kernel_shapes_follow_read_set_and_reduction_set(tmp_path, built):
+    """Emitted source of three graphs (nothing launched): a pointwise kernel reads with the
+    non-temporal hint only when its large operands exceed half the memory-side cache, it deals
+    workgroups to the dies in eighths with a grid that is a multiple of 8, and the column pair of the
+    third benchmark graph folds its two states in one call, takes the mean's sum from the moments
+    (five partial words) and sizes its LDS for three planes of 32 x 4 columns x 5 words."""
+    from inductor_x_amd.hip_heuristics import col_fold_all_planes
+
+    out = _run_dry(tmp_path, DRY_SHAPES)
+    line = {l.split()[0]: l.split(None, 1)[1] for l in out.splitlines() if l.split() and l.split()[0] in ("STREAM", "ORDER", "COL")}
+    assert line["STREAM"] == "['true'] ['false']"
+    assert line["ORDER"] == "True 8"
+    assert line["COL"].split() == ["True", "5", "2", "True", str(col_fold_all_planes(32, 8) * 32 * 4 * 5 * 4)]
+    assert [col_fold_all_planes(ct, rl) for ct, rl in ((32, 8), (64, 8), (16, 16), (64, 1), (128, 2), (32, 2))] == [3, 4, 3, 0, 1, 0]
 
 
 def test_import_hook_keeps_cpu_inductor_working():
