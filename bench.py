@@ -572,6 +572,26 @@ def _cpu_baseline() -> dict:
     }
 
 
+def _launch_floor(K, torch) -> dict:
+    """Per-launch time of a kernel that moves next to nothing (a 4 KiB copy by one workgroup) and
+    of the cfg 1 row sum, both as 20 dependent launches per HIP graph: the first is what this
+    machine charges for a launch in a chain, whatever the kernel does."""
+    dev = "cuda:0"
+    torch.manual_seed(0)
+    a = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    b = torch.empty_like(a)
+    x = torch.randn(1024, 4096, device=dev)
+    for _ in range(30):
+        K.copy_bytes(b, a)
+        K.fused_relu_sigmoid_rowsum(x)
+    tiny = min(_graph_time_ms(lambda: K.copy_bytes(b, a)) for _ in range(3))
+    rows = min(_graph_time_ms(lambda: K.fused_relu_sigmoid_rowsum(x)) for _ in range(3))
+    return {"launch_floor_us": round(tiny * 1e3, 3), "kernel": "copy_b128 (4 KiB, one workgroup)",
+            "cfg1_us": round(rows * 1e3, 3), "cfg1_kernel": _launched_symbols(lambda: K.fused_relu_sigmoid_rowsum(x)),
+            "cfg1_at_peak_us": round(ALGO_BYTES["rowsum"] / HBM_PEAK_GBS / 1e3, 3),
+            "timing": "hip-graph replay, 20 dependent launches per graph, best of 3 x 5 replays"}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=int(os.environ.get("WORLD_SIZE", "1")))
@@ -584,6 +604,9 @@ def main() -> None:
     ap.add_argument("--pmc-config", default=None,
                     help="run only plain launches of one configuration (1, 1cold, 2, 3, 4a, 4b, 5), both paths, and the "
                          "copy probe: the program for a rocprofv3 --pmc counter run")
+    ap.add_argument("--launch-floor", action="store_true",
+                    help="time a 4 KiB copy (one workgroup) and the cfg 1 row sum the same way, 20 dependent launches per "
+                         "HIP graph: what a launch costs on this machine before any data moves")
     ap.add_argument("--cpu-baseline-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
 
@@ -604,6 +627,9 @@ def main() -> None:
 
     if args.pmc_config is not None:
         print(json.dumps(_pmc_run(K, torch, args.pmc_config, args.steps, args.warmup)))
+        return
+    if args.launch_floor:
+        print(json.dumps(_launch_floor(K, torch)))
         return
     dev = "cuda:0"
     torch.manual_seed(0)
