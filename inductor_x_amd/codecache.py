@@ -13,6 +13,7 @@ from __future__ import annotations
 import fcntl
 import hashlib
 import os
+import re
 import shutil
 import subprocess
 import tempfile
@@ -68,26 +69,50 @@ def toolchain_version() -> str:
     return "unknown"
 
 
-def _headers_digest() -> str:
+_INCLUDE = re.compile(r'^\s*#\s*include\s+"(?:\.\./)?(?:mi/)?([A-Za-z0-9_.]+\.h)"', re.M)
+_header_text_cache: dict[str, str] = {}
+
+
+def _header_text(name: str) -> Optional[str]:
+    if name not in _header_text_cache:
+        try:
+            with open(os.path.join(HEADER_DIR, name)) as f:
+                _header_text_cache[name] = f.read()
+        except OSError:
+            _header_text_cache[name] = ""
+    return _header_text_cache[name] or None
+
+
+def reachable_headers(source: str) -> list[str]:
+    """Names of the device headers (csrc/mi/*.h) a translation unit includes, directly or through
+    other headers, sorted.  Only these enter its cache key: editing the attention kernels does not
+    invalidate the code objects of generated row or column kernels."""
+    seen: set[str] = set()
+    todo = list(_INCLUDE.findall(source))
+    while todo:
+        name = todo.pop()
+        if name in seen:
+            continue
+        text = _header_text(name)
+        if text is None:
+            continue
+        seen.add(name)
+        todo.extend(_INCLUDE.findall(text))
+    return sorted(seen)
+
+
+def _headers_digest(source: str) -> str:
     h = hashlib.sha256()
     h.update(toolchain_version().encode())
-    for name in sorted(os.listdir(HEADER_DIR)):
-        if name.endswith(".h"):
-            with open(os.path.join(HEADER_DIR, name), "rb") as f:
-                h.update(name.encode())
-                h.update(f.read())
+    for name in reachable_headers(source):
+        h.update(name.encode())
+        h.update(_header_text(name).encode())
     return h.hexdigest()
 
 
-_headers_digest_cache: Optional[str] = None
-
-
 def source_key(source: str, extra_flags: Iterable[str] = ()) -> str:
-    global _headers_digest_cache
-    if _headers_digest_cache is None:
-        _headers_digest_cache = _headers_digest()
     h = hashlib.sha256()
-    h.update(_headers_digest_cache.encode())
+    h.update(_headers_digest(source).encode())
     h.update("\0".join(HIPCC_FLAGS + tuple(extra_flags)).encode())
     h.update(source.encode())
     return h.hexdigest()[:32]

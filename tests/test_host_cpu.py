@@ -355,6 +355,23 @@ def test_generated_kernel_shapes_follow_read_set_and_reduction_set(tmp_path, bui
     assert [col_fold_all_planes(ct, rl) for ct, rl in ((32, 8), (64, 8), (16, 16), (64, 1), (128, 2), (32, 2))] == [3, 4, 3, 0, 1, 0]
 
 
+def test_code_object_key_follows_only_the_headers_a_source_includes(monkeypatch):
+    """A generated kernel includes mi/codegen.h (and through it common.h): its key moves with those
+    and not with the attention headers; the compiler flags and the source text move it as well."""
+    from inductor_x_amd import codecache
+
+    gen = '#include "mi/codegen.h"\nextern "C" __global__ void k() {}\n'
+    assert codecache.reachable_headers(gen) == ["codegen.h", "common.h"]
+    assert "attention_v5.h" in codecache.reachable_headers(codecache.aot_source("attention_kernels.hip"))
+    key = codecache.source_key(gen)
+    assert key == codecache.source_key(gen) and key != codecache.source_key(gen, ("-DX=1",)) and key != codecache.source_key(gen + " ")
+    real = codecache._header_text
+    monkeypatch.setattr(codecache, "_header_text", lambda n: real(n) + "// edited" if n == "attention_v5.h" else real(n))
+    assert codecache.source_key(gen) == key
+    monkeypatch.setattr(codecache, "_header_text", lambda n: real(n) + "// edited" if n == "common.h" else real(n))
+    assert codecache.source_key(gen) != key
+
+
 def test_import_hook_keeps_cpu_inductor_working():
     """The table patches only act on GPU tensors: CPU compilation in the same
     process still goes through Inductor's C++ backend and matches eager."""
