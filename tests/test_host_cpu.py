@@ -235,6 +235,7 @@ DRY_HEAD = r'''
 import os, sys
 os.environ["INDUCTOR_X_AMD_DRYRUN"] = "1"
 os.environ["INDUCTOR_X_AMD_CACHE"] = sys.argv[1]
+os.environ["TORCHINDUCTOR_FORCE_DISABLE_CACHES"] = "1"  # every graph is lowered here, never served from disk
 sys.path.insert(0, sys.argv[2])
 import torch
 import inductor_x_amd
