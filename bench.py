@@ -592,6 +592,51 @@ def _launch_floor(K, torch) -> dict:
             "timing": "hip-graph replay, 20 dependent launches per graph, best of 3 x 5 replays"}
 
 
+def _attention_ceiling(torch) -> dict:
+    """Rates of the probe kernels (one workgroup of eight wavefronts per CU, 256 workgroups): nanoseconds per
+    step -- one MFMA 32x32x16 bf16 and / or one 1 KiB LDS fragment -- and what follows from them."""
+    from inductor_x_amd import codecache, launcher
+
+    path = codecache.compile_source(codecache.aot_source("probe_kernels.hip"), label="probe_kernels", prefer_intree=True)
+    with open(path, "rb") as f:
+        mod = launcher.Module(f.read(), label="probe_kernels")
+    out = torch.zeros(512, device="cuda:0")
+    stream = torch._C._cuda_getCurrentRawStream(0)
+    iters = 20000
+    names = ["mfma_only", "ds_read_b128_only", "ds_read_b64_x2_only", "ds_read_b64_tr_b16_x2_only",
+             "fragment_per_mfma", "mfma_with_vector_work", "fragment_per_mfma_with_vector_work"]
+    ns = {}
+    for mode, name in enumerate(names):
+        fn = mod.function(f"attention_resource_probe_m{mode}")
+        launch = lambda: fn.launch("Pi", (out.data_ptr(), iters), (256, 1, 1), (512,), stream, 65536)  # noqa: E731
+        for _ in range(3):
+            launch()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0.record()
+            launch()
+            t1.record()
+            t1.synchronize()
+            best = min(best, t0.elapsed_time(t1))
+        ns[name] = best * 1e6 / (iters * 16) / 2  # per step per SIMD (two wavefronts share one)
+    mfma = ns["mfma_only"]  # 32 cycles
+    clock_ghz = 32 / mfma
+    lds = lambda n: round(4 * 1024 / (ns[n] / mfma * 32), 1)  # noqa: E731  bytes per clock per CU
+    frac = lambda n: round(mfma / ns[n], 3)  # noqa: E731
+    return {
+        "ns_per_step_per_simd": {k: round(v, 2) for k, v in ns.items()},
+        "clock_ghz_under_mfma_load": round(clock_ghz, 3),
+        "lds_bytes_per_clock_per_cu": {n: lds(n) for n in names[1:4]},
+        "lds_bytes_per_clock_needed_at_full_mfma_rate": 128.0,
+        "mfma_rate_vs_alone": {n: frac(n) for n in names[4:]},
+        "ceiling_of_datasheet_peak": round(frac(names[6]) * clock_ghz / 2.4, 3),
+        "note": "fragment_per_mfma_with_vector_work is the instruction mix of the attention loop (one fragment, four "
+                "fma, one exp2, one add per MFMA, two wavefronts per SIMD) with no dependence between the three streams",
+    }
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=int(os.environ.get("WORLD_SIZE", "1")))
@@ -607,6 +652,9 @@ def main() -> None:
     ap.add_argument("--launch-floor", action="store_true",
                     help="time a 4 KiB copy (one workgroup) and the cfg 1 row sum the same way, 20 dependent launches per "
                          "HIP graph: what a launch costs on this machine before any data moves")
+    ap.add_argument("--attention-ceiling", action="store_true",
+                    help="run the resource probes of csrc/aot/probe_kernels.hip: what one CU sustains of MFMA, LDS operand "
+                         "reads and softmax-like vector work, alone and together (the ceiling of the attention design)")
     ap.add_argument("--cpu-baseline-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
 
@@ -630,6 +678,9 @@ def main() -> None:
         return
     if args.launch_floor:
         print(json.dumps(_launch_floor(K, torch)))
+        return
+    if args.attention_ceiling:
+        print(json.dumps(_attention_ceiling(torch)))
         return
     dev = "cuda:0"
     torch.manual_seed(0)

@@ -1,0 +1,122 @@
+// Measurement kernels, not part of any graph: what one CU sustains of the three resources the fused
+// attention forward needs per MFMA -- the matrix pipe, one 1 KiB operand fragment from LDS, and the
+// softmax's share of vector work -- alone and together, free of any data dependence between them.
+// Launched as one workgroup of eight wavefronts per CU (two per SIMD), the shape of the attention
+// kernels.  bench.py --attention-ceiling runs them and prints the rates.
+#include "../mi/attention.h"
+
+using namespace mi;
+
+namespace {
+
+typedef __bf16 probe_bf16x4_t __attribute__((__vector_size__(4 * sizeof(__bf16))));
+
+// MODE 0  MFMA only (four independent accumulators)
+//      1  ds_read_b128 only, the K fragment addresses of the attention kernel (XOR-swizzled rows)
+//      2  the same bytes as two ds_read_b64
+//      3  two transposing ds_read_b64_tr_b16 per fragment
+//      4  one ds_read_b128 fragment per MFMA, requested two steps ahead
+//      5  MFMA beside four fused multiply-adds, one exponential and one add per step on other registers
+//      6  4 and 5 together: the instruction mix of the attention loop without its dependences
+template <int MODE>
+__device__ __forceinline__ void attention_resource_probe(float* out, int iters) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char probe_lds[];  // 64 KiB
+  const int lane = threadIdx.x & 63;
+  const int li = lane & 31, g = lane >> 5;
+  for (int i = threadIdx.x; i < 16384; i += blockDim.x) reinterpret_cast<float*>(probe_lds)[i] = 1.0f + i * 1e-6f;
+  __syncthreads();
+  const bf16_t* base = reinterpret_cast<const bf16_t*>(probe_lds);
+  int off[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) off[ks] = li * 128 + 8 * ((2 * ks + g) ^ (li & 15));
+  f32x16_t acc[4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[a][r] = 0.f;
+  bf16x8_t q;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) q[e] = static_cast<bf16_t>(0.5f + lane);
+  float w[8], psum = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) w[e] = 0.001f * (lane + e);
+  for (int it = 0; it < iters; ++it) {
+    const bf16_t* tile = base + (it & 1) * 16384;  // two 16 KiB tiles 32 KiB apart; every read stays below 56 KiB
+    if constexpr (MODE == 0) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(q, q, acc[i & 3], 0, 0, 0);
+    } else if constexpr (MODE == 1) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(tile + 32 * (i >> 3) * 128 + off[i & 7]);
+        asm volatile("" ::"v"(v));
+      }
+    } else if constexpr (MODE == 2) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const u32x2_t a = *reinterpret_cast<const u32x2_t*>(tile + 32 * (i >> 3) * 128 + off[i & 7]);
+        const u32x2_t b = *reinterpret_cast<const u32x2_t*>(tile + 32 * (i >> 3) * 128 + off[i & 7] + 4);
+        asm volatile("" ::"v"(a), "v"(b));
+      }
+    } else if constexpr (MODE == 3) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const bf16_t* p0 = tile + 16 * (i >> 2) * 128 + off[i & 3];
+        const probe_bf16x4_t lo =
+            __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) probe_bf16x4_t*)(p0));
+        const probe_bf16x4_t hi =
+            __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) probe_bf16x4_t*)(p0 + 8 * 128));
+        asm volatile("" ::"v"(lo), "v"(hi));
+      }
+    } else {
+      bf16x8_t f[16];
+      if constexpr (MODE == 4 || MODE == 6) {
+        f[0] = *reinterpret_cast<const bf16x8_t*>(tile + off[0]);
+        f[1] = *reinterpret_cast<const bf16x8_t*>(tile + off[1]);
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        if constexpr (MODE == 4 || MODE == 6) {
+          if (i + 2 < 16) f[i + 2] = *reinterpret_cast<const bf16x8_t*>(tile + 32 * ((i + 2) >> 3) * 128 + off[(i + 2) & 7]);
+          acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], q, acc[i & 3], 0, 0, 0);
+        } else {
+          acc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(q, q, acc[i & 3], 0, 0, 0);
+        }
+        if constexpr (MODE == 5 || MODE == 6) {
+          float a = w[i & 7], b = w[(i + 3) & 7];
+          a = fmaf(a, 1.0001f, -0.5f);
+          b = fmaf(b, 0.9999f, 0.25f);
+          a = __builtin_amdgcn_exp2f(a);
+          b = fmaf(b, a, 0.125f);
+          psum += a;
+          w[i & 7] = fmaf(a, 0.5f, b);
+          asm volatile("" : "+v"(w[i & 7]), "+v"(psum));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  float s = psum;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) s += w[e];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += acc[a][r];
+  if (s == 12345.678f) out[threadIdx.x] = s;  // keeps the work alive; never true for these inputs
+}
+
+}  // namespace
+
+#define PROBE(MODE)                                                                                   \
+  extern "C" __global__ __launch_bounds__(512, 1) void attention_resource_probe_m##MODE(float* out,   \
+                                                                                         int iters) { \
+    attention_resource_probe<MODE>(out, iters);                                                       \
+  }
+PROBE(0)
+PROBE(1)
+PROBE(2)
+PROBE(3)
+PROBE(4)
+PROBE(5)
+PROBE(6)
