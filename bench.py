@@ -621,6 +621,20 @@ def _attention_ceiling(torch) -> dict:
             t1.synchronize()
             best = min(best, t0.elapsed_time(t1))
         ns[name] = best * 1e6 / (iters * 16) / 2  # per step per SIMD (two wavefronts share one)
+    # the 64-queries-per-wavefront design: four wavefronts (one per SIMD), two MFMAs per step
+    fn = mod.function("attention_resource_probe_m7")
+    for _ in range(3):
+        fn.launch("Pi", (out.data_ptr(), iters), (256, 1, 1), (256,), stream, 65536)
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(3):
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        fn.launch("Pi", (out.data_ptr(), iters), (256, 1, 1), (256,), stream, 65536)
+        t1.record()
+        t1.synchronize()
+        best = min(best, t0.elapsed_time(t1))
+    ns_wide = best * 1e6 / (iters * 16) / 2  # per MFMA per SIMD
     mfma = ns["mfma_only"]  # 32 cycles
     clock_ghz = 32 / mfma
     lds = lambda n: round(4 * 1024 / (ns[n] / mfma * 32), 1)  # noqa: E731  bytes per clock per CU
@@ -632,6 +646,8 @@ def _attention_ceiling(torch) -> dict:
         "lds_bytes_per_clock_needed_at_full_mfma_rate": 128.0,
         "mfma_rate_vs_alone": {n: frac(n) for n in names[4:]},
         "ceiling_of_datasheet_peak": round(frac(names[6]) * clock_ghz / 2.4, 3),
+        "one_wavefront_per_simd_64_queries": {"ns_per_mfma_per_simd": round(ns_wide, 2), "mfma_rate_vs_alone": round(mfma / ns_wide, 3),
+                                              "ceiling_of_datasheet_peak": round(mfma / ns_wide * clock_ghz / 2.4, 3)},
         "note": "fragment_per_mfma_with_vector_work is the instruction mix of the attention loop (one fragment, four "
                 "fma, one exp2, one add per MFMA, two wavefronts per SIMD) with no dependence between the three streams",
     }

@@ -18,6 +18,8 @@ typedef __bf16 probe_bf16x4_t __attribute__((__vector_size__(4 * sizeof(__bf16))
 //      4  one ds_read_b128 fragment per MFMA, requested two steps ahead
 //      5  MFMA beside four fused multiply-adds, one exponential and one add per step on other registers
 //      6  4 and 5 together: the instruction mix of the attention loop without its dependences
+//      7  the mix of the 64-queries-per-wavefront design, launched with four wavefronts (one per SIMD):
+//         every fragment feeds two MFMAs, twice the vector work per step
 template <int MODE>
 __device__ __forceinline__ void attention_resource_probe(float* out, int iters) {
   extern __shared__ __attribute__((aligned(16))) unsigned char probe_lds[];  // 64 KiB
@@ -67,6 +69,28 @@ __device__ __forceinline__ void attention_resource_probe(float* out, int iters) 
         const probe_bf16x4_t hi =
             __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) probe_bf16x4_t*)(p0 + 8 * 128));
         asm volatile("" ::"v"(lo), "v"(hi));
+      }
+    } else if constexpr (MODE == 7) {
+      bf16x8_t f[16];
+      f[0] = *reinterpret_cast<const bf16x8_t*>(tile + off[0]);
+      f[1] = *reinterpret_cast<const bf16x8_t*>(tile + off[1]);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        if (i + 2 < 16) f[i + 2] = *reinterpret_cast<const bf16x8_t*>(tile + 32 * ((i + 2) >> 3) * 128 + off[(i + 2) & 7]);
+        acc[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], q, acc[i & 1], 0, 0, 0);
+        acc[2 + (i & 1)] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], q, acc[2 + (i & 1)], 0, 0, 0);
+#pragma unroll
+        for (int rep = 0; rep < 2; ++rep) {
+          float a = w[(i + 4 * rep) & 7], b = w[(i + 3 + 4 * rep) & 7];
+          a = fmaf(a, 1.0001f, -0.5f);
+          b = fmaf(b, 0.9999f, 0.25f);
+          a = __builtin_amdgcn_exp2f(a);
+          b = fmaf(b, a, 0.125f);
+          psum += a;
+          w[(i + 4 * rep) & 7] = fmaf(a, 0.5f, b);
+          asm volatile("" : "+v"(w[(i + 4 * rep) & 7]), "+v"(psum));
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     } else {
       bf16x8_t f[16];
@@ -120,3 +144,6 @@ PROBE(3)
 PROBE(4)
 PROBE(5)
 PROBE(6)
+extern "C" __global__ __launch_bounds__(256, 1) void attention_resource_probe_m7(float* out, int iters) {
+  attention_resource_probe<7>(out, iters);
+}
