@@ -373,6 +373,10 @@ def _ring_merge_configs(torch, add) -> None:
     st = lambda off: (torch.rand(B, N, DS, device=dev) + off).unsqueeze(3).repeat(1, 1, 1, 8).contiguous()  # noqa: E731
     args = (torch.randn(DS, B, H, device=dev).bfloat16(), st(0.0), st(0.5), torch.randn(DS, B, H, device=dev).bfloat16(),
             st(0.0), st(0.5))
+    from inductor_x_amd import kernels as K
+
+    add("f1a ring forward_update bf16 [8192,1,6144] N=48", "kernel", lambda: K.ring_forward_update(*args),
+        3 * DS * B * H * 2 + 6 * B * N * DS * 8 * 4, "hbm")
     one("f1a ring forward_update bf16 [8192,1,6144] N=48", forward_update, args, 3 * DS * B * H * 2 + 6 * B * N * DS * 8 * 4)
     del args
     B, N, DS, D = 1, 48, 8192, 128
@@ -597,7 +601,7 @@ def _attention_ceiling(torch) -> dict:
     step -- one MFMA 32x32x16 bf16 and / or one 1 KiB LDS fragment -- and what follows from them."""
     from inductor_x_amd import codecache, launcher
 
-    path = codecache.compile_source(codecache.aot_source("probe_kernels.hip"), label="probe_kernels", prefer_intree=True)
+    path = codecache.compile_source(codecache.probe_source("probe_kernels.hip"), label="probe_kernels", prefer_intree=True)
     with open(path, "rb") as f:
         mod = launcher.Module(f.read(), label="probe_kernels")
     out = torch.zeros(512, device="cuda:0")
@@ -669,7 +673,7 @@ def main() -> None:
                     help="time a 4 KiB copy (one workgroup) and the cfg 1 row sum the same way, 20 dependent launches per "
                          "HIP graph: what a launch costs on this machine before any data moves")
     ap.add_argument("--attention-ceiling", action="store_true",
-                    help="run the resource probes of csrc/aot/probe_kernels.hip: what one CU sustains of MFMA, LDS operand "
+                    help="run the resource probes of csrc/probes/probe_kernels.hip: what one CU sustains of MFMA, LDS operand "
                          "reads and softmax-like vector work, alone and together (the ceiling of the attention design)")
     ap.add_argument("--cpu-baseline-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()

@@ -143,12 +143,19 @@ def install_unsupported_retry() -> None:
 
         if not config.retry_unsupported_with_eager:
             return original(self, gm, example_inputs, inputs_to_check, graph_kwargs)
-        pristine = copy.deepcopy(gm)  # the post-grad passes rewrite gm in place
+        try:
+            pristine = copy.deepcopy(gm)  # the post-grad passes rewrite gm in place
+        except Exception as e:  # a graph that cannot be copied compiles without the retry
+            log.debug("graph module cannot be copied (%s): no eager retry for this compile", e)
+            return original(self, gm, example_inputs, inputs_to_check, graph_kwargs)
         for _ in range(4):
             try:
                 return original(self, gm, example_inputs, inputs_to_check, graph_kwargs)
             except Exception as e:
                 unsupported = _find_unsupported(e)
+                # The fallbacks registered here stay for the rest of the process (lowering tables are
+                # process-wide): later graphs run these ops as eager kernels too.
+                # lowering.RUNTIME_FALLBACKS lists them, lowering.clear_runtime_fallbacks() undoes them.
                 changed = [op for op in getattr(unsupported, "ops", ()) if add_runtime_fallback(op)]
                 if unsupported is None or not changed:
                     raise

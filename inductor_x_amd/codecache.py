@@ -24,6 +24,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC_DIR = os.path.join(_HERE, "csrc")
 HEADER_DIR = os.path.join(CSRC_DIR, "mi")
 AOT_DIR = os.path.join(CSRC_DIR, "aot")
+PROBE_DIR = os.path.join(CSRC_DIR, "probes")
 INTREE_STORE = os.path.join(_HERE, "_hsaco")
 # Code objects of generated (torch.compile) kernels that ship with the tree, so a
 # machine that has seen a graph before does not invoke hipcc for it again.
@@ -221,6 +222,21 @@ def aot_source(name: str) -> str:
     with its relative includes rewritten to the include root."""
     with open(os.path.join(AOT_DIR, name)) as f:
         return f.read().replace('#include "../mi/', '#include "mi/')
+
+
+def probe_source(name: str) -> str:
+    """Text of a measurement kernel file under csrc/probes (resource probes that no graph launches;
+    they are compiled for the benchmark program only and are not part of the ahead-of-time set)."""
+    with open(os.path.join(PROBE_DIR, name)) as f:
+        return f.read().replace('#include "../mi/', '#include "mi/')
+
+
+def build_probes(force: bool = True) -> dict[str, str]:
+    """Compile the measurement kernels of csrc/probes into the in-tree store."""
+    out = {}
+    for name in sorted(n for n in os.listdir(PROBE_DIR) if n.endswith(".hip")):
+        out[name] = compile_source(probe_source(name), label=name[:-4], prefer_intree=True, force=force)
+    return out
 
 
 def aot_files() -> list[str]:

@@ -1380,6 +1380,7 @@ class HipKernel(SIMDKernel):
             # (every one of the thread's VEC elements contributes, also when they share an address)
             idx = self.index_to_str(index) if kind == "uniform" else self.index_to_vec_str(index)
             line = f"mi::scatter_add_m<VEC>({var}, {idx}, {value}, {mask or 'true'});"
+            self.__dict__.setdefault("accumulated_args", set()).add(str(var))
             self.stores.writeline(DeferredLine(name, line))
             return
         if kind == "contiguous":
@@ -1805,6 +1806,17 @@ class HipKernel(SIMDKernel):
         _, call_args, signature, _ = self.args.python_argdefs()
         call_args = [str(a) for a in call_args]
         params, codes = [], []
+        # buffers a launch both reads and writes (in-place operands, targets of accumulating stores):
+        # launching twice is not the same as launching once, so whoever times the kernel must do it on copies
+        accumulated = self.__dict__.get("accumulated_args", set())
+        self.mutated_arg_positions = [
+            pos for pos, arg in enumerate(signature)
+            if isinstance(arg, TensorArg) and (arg.name.startswith("in_out_ptr") or arg.name in accumulated)
+        ]
+        self.written_arg_positions = [
+            pos for pos, arg in enumerate(signature)
+            if isinstance(arg, TensorArg) and (arg.name.startswith("out_ptr") or arg.name.startswith("in_out_ptr"))
+        ]
         for pos, arg in enumerate(signature):
             if isinstance(arg, TensorArg) and should_unwrap_unspec_arg(arg.buffer):
                 # a zero-dimensional CPU tensor among GPU operands (a Python number dynamo chose not
@@ -1958,6 +1970,7 @@ class HipKernel(SIMDKernel):
                     )
                     src.writeline(f"const {idx_t} xbase = (wg_ * UNROLL * {self.block} + threadIdx.x) * VEC;")
                     meta["grid_multiple"] = 8
+                    meta["index_bits"] = 32 if idx_t == "int" else 64
                 # each thread handles UNROLL vectors one workgroup-width apart, so a
                 # wavefront still touches 1 KiB runs and has UNROLL loads in flight
                 src.writeline("#pragma unroll")
@@ -2045,6 +2058,8 @@ class HipKernel(SIMDKernel):
             sig = self._codegen_col(src, kname, params, codes, idx_t, idx_code, meta)
         meta["signature"] = sig
         meta["n_buffer_args"] = len(codes)
+        meta["mutated_args"] = list(getattr(self, "mutated_arg_positions", []))
+        meta["written_args"] = list(getattr(self, "written_arg_positions", []))
         self.meta = meta
         return src.getvalue()
 

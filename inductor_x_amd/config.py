@@ -35,7 +35,11 @@ retry_unsupported_with_eager = os.environ.get("INDUCTOR_X_AMD_RETRY_UNSUPPORTED"
 
 # sum of a 16-bit floating-point tensor: accumulate in fp32 and round the result back to the input
 # type, which is the type eager PyTorch returns (False), or return the fp32 sum itself as the
-# reference's lowering does (True; reference inductor_x/lowering.py:204-215).
+# reference's lowering does (True; reference inductor_x/lowering.py:204-215).  True is for inference
+# graphs that compare against the reference's outputs only: the buffer's type then differs from the
+# type dynamo and AOTAutograd traced for the node, so a graph output, a guard or a backward pass that
+# relies on the traced type can see a mismatch; the lowering applies it to inference graphs only
+# (no backward graph is compiled for the function).
 sum_returns_fp32 = os.environ.get("INDUCTOR_X_AMD_SUM_FP32", "0") == "1"
 
 # Generated indirect accesses (embedding, index, gather, index_put, scatter): "clamp" keeps every

@@ -13,6 +13,23 @@ using namespace mi;
     col_stats_partial<CT, RL, UNROLL>(x, part, rows, cols, nsplit);                           \
   }
 
+// the same with PF batches of loads held per thread instead of two
+#define COL_PARTIAL_VARIANT_PF(CT, RL, UNROLL, PF)                                            \
+  extern "C" __global__ __launch_bounds__(CT* RL) void                                        \
+      col_mean_var_argmax_partial_f32_c##CT##_r##RL##_u##UNROLL##_p##PF(                      \
+          const float* x, float* part, int rows, int cols, int nsplit) {                      \
+    col_stats_partial<CT, RL, UNROLL, PF>(x, part, rows, cols, nsplit);                       \
+  }
+
+COL_PARTIAL_VARIANT_PF(32, 8, 8, 3)
+COL_PARTIAL_VARIANT_PF(32, 8, 8, 4)
+COL_PARTIAL_VARIANT_PF(32, 8, 4, 3)
+COL_PARTIAL_VARIANT_PF(32, 8, 4, 4)
+COL_PARTIAL_VARIANT_PF(32, 16, 4, 3)
+COL_PARTIAL_VARIANT_PF(32, 16, 8, 3)
+COL_PARTIAL_VARIANT_PF(32, 8, 16, 3)
+COL_PARTIAL_VARIANT_PF(64, 8, 8, 3)
+
 COL_PARTIAL_VARIANT(128, 2, 4)
 COL_PARTIAL_VARIANT(128, 2, 8)
 COL_PARTIAL_VARIANT(128, 4, 4)

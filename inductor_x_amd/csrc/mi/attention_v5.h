@@ -355,16 +355,33 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
   const float l_tot = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
   const float inv_l = 1.0f / l_tot;
   const float l_true = l_tot * __builtin_amdgcn_exp2f(m_run - m_true);
-  bf16_t* __restrict__ orow = O + head_off + static_cast<size_t>(qi) * kAttnD;
+  // The accumulators hold O^T: a lane owns one query and, per register quad, four consecutive d.
+  // Stored from there a wavefront instruction would write 32 separate 16-byte pieces, one per row;
+  // measured on MI355X those partial-line writes kept a workgroup's CU busy for about 5 us per query
+  // block (7 % of the causal launch).  So the tile goes through LDS once: every wavefront writes its
+  // 32 x 128 block into its own 8 KiB of the (now idle) K/V buffers, 16-byte chunks XOR-swizzled by the
+  // row, and reads it back row-wise, so that one instruction stores four whole 256-byte rows.
+  __syncthreads();  // every wavefront is done with the K and V tiles
+  {
+    bf16_t* stage = reinterpret_cast<bf16_t*>(attn_lds) + wave * (32 * kAttnD);
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+    for (int db = 0; db < 4; ++db)
 #pragma unroll
-    for (int rq = 0; rq < 4; ++rq) {
-      bf16x4_t o4;
+      for (int rq = 0; rq < 4; ++rq) {
+        bf16x4_t o4;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o4[e] = static_cast<bf16_t>(oacc[db][4 * rq + e] * inv_l);
-      *reinterpret_cast<bf16x4_t*>(orow + 32 * db + 8 * rq + 4 * g) = o4;
+        for (int e = 0; e < 4; ++e) o4[e] = static_cast<bf16_t>(oacc[db][4 * rq + e] * inv_l);
+        *reinterpret_cast<bf16x4_t*>(stage + li * kAttnD + 8 * ((4 * db + rq) ^ (li & 15)) + 4 * g) = o4;
+      }
+    bf16_t* __restrict__ oblk = O + head_off + static_cast<size_t>(q0 + sub * 32) * kAttnD;
+    const int c16 = lane & 15;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int row = 4 * j + (lane >> 4);
+      const u32x4_t v16 = *reinterpret_cast<const u32x4_t*>(stage + row * kAttnD + 8 * (c16 ^ (row & 15)));
+      *reinterpret_cast<u32x4_t*>(oblk + row * kAttnD + 8 * c16) = v16;
     }
+  }
   if (g == 0) {
     const size_t so = (static_cast<size_t>(head) * S + qi) * 8;
     const float m_nat = m_true * 0.69314718055994530942f;
@@ -379,6 +396,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
     store_vec<float, 4>(softmax_sum + so, lv);
     store_vec<float, 4>(softmax_sum + so + 4, lv);
   }
+  __syncthreads();  // the staging reads are done before a following query block refills the K buffers
 }
 
 }  // namespace mi

@@ -476,7 +476,7 @@ __device__ __forceinline__ auto clamp_index(const A& a, S size) {
   return apply(
       [size](auto x) {
         typedef decltype(x) T;
-        const T hi = static_cast<T>(size) - 1;
+        const T hi = size > 0 ? static_cast<T>(size) - 1 : static_cast<T>(0);  // an empty axis clamps to 0, not -1
         return x < 0 ? static_cast<T>(0) : (x > hi ? hi : x);
       },
       a);

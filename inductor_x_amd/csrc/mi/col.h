@@ -160,7 +160,7 @@ __device__ __forceinline__ void col_fold_row_lanes(ColState (&st)[4], int ct, in
 // contiguous slice of rows per workgroup: 27.2 us against 28.6 us for both passes,
 // and half as many workgroups (each with twice the loads in flight) do as well,
 // which halves the partials the second pass reads.
-template <int CT, int RL, int UNROLL>
+template <int CT, int RL, int UNROLL, int PF = 2>
 __device__ __forceinline__ void col_stats_sweep(const float* __restrict__ x, int rows, int cols,
                                                 int nsplit, ColState (&st)[4], float* lds_dyn) {
   constexpr int BATCH = RL * UNROLL;
@@ -194,36 +194,45 @@ __device__ __forceinline__ void col_stats_sweep(const float* __restrict__ x, int
     }
     int cnt = 0;
     int b = split;
-    Vec<float, 4> v[UNROLL];
-    if (b < full) {
+    // PF batches of UNROLL rows each are held per thread: while one is folded, the loads of the
+    // other PF - 1 are in flight (buffer j is refilled with the batch PF turns ahead as soon as
+    // its values have been used, so the order of rows a thread sees stays increasing).
+    Vec<float, 4> v[PF][UNROLL];
 #pragma unroll
-      for (int u = 0; u < UNROLL; ++u) v[u] = load_vec_readonly<float, 4>(base + b * batch_step + u * row_step);
+    for (int j = 0; j < PF; ++j) {
+      if (b + j * nsplit < full) {
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+          v[j][u] = load_vec_readonly<float, 4>(base + (b + j * nsplit) * batch_step + u * row_step);
+      }
     }
     while (b < full) {
-      const int bn = b + nsplit;
-      Vec<float, 4> vn[UNROLL];
-      if (bn < full) {
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) vn[u] = load_vec_readonly<float, 4>(base + bn * batch_step + u * row_step);
-      }
-      const int r = b * BATCH + rl;
+      for (int j = 0; j < PF; ++j) {
+        if (b < full) {
+          const int r = b * BATCH + rl;
 #pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
+          for (int u = 0; u < UNROLL; ++u) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const float xv = v[u][k];
-          const float d = xv - c[k];
-          s1[k] += d;
-          s2[k] = fmaf(d, d, s2[k]);
-          const bool upd = xv > best[k];
-          best[k] = upd ? xv : best[k];
-          bi[k] = upd ? (r + u * RL) : bi[k];
+            for (int k = 0; k < 4; ++k) {
+              const float xv = v[j][u][k];
+              const float d = xv - c[k];
+              s1[k] += d;
+              s2[k] = fmaf(d, d, s2[k]);
+              const bool upd = xv > best[k];
+              best[k] = upd ? xv : best[k];
+              bi[k] = upd ? (r + u * RL) : bi[k];
+            }
+          }
+          cnt += UNROLL;
+          const int bn = b + PF * nsplit;
+          if (bn < full) {
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) v[j][u] = load_vec_readonly<float, 4>(base + bn * batch_step + u * row_step);
+          }
+          b += nsplit;
         }
       }
-      cnt += UNROLL;
-      b = bn;
-#pragma unroll
-      for (int u = 0; u < UNROLL; ++u) v[u] = vn[u];
     }
     // the last, partly filled batch belongs to workgroup full % nsplit
     if (b == full) {
@@ -279,13 +288,13 @@ __device__ __forceinline__ void col_stats_sweep(const float* __restrict__ x, int
 }
 
 // Pass 1 of the two-launch form: sweep, then one plain partial per (split, column).
-template <int CT, int RL, int UNROLL>
+template <int CT, int RL, int UNROLL, int PF = 2>
 __device__ __forceinline__ void col_stats_partial(const float* __restrict__ x,
                                                          float* __restrict__ part, int rows,
                                                          int cols, int nsplit) {
   extern __shared__ float lds_dyn[];
   ColState st[4];
-  col_stats_sweep<CT, RL, UNROLL>(x, rows, cols, nsplit, st, lds_dyn);
+  col_stats_sweep<CT, RL, UNROLL, PF>(x, rows, cols, nsplit, st, lds_dyn);
   const int ct = threadIdx.x % CT;
   const int rl = threadIdx.x / CT;
   const int col = (blockIdx.x * CT + ct) * 4;

@@ -77,6 +77,25 @@ __device__ __forceinline__ Vec<T, N> load_vec(const T* __restrict__ p) {
   return out;
 }
 
+// Load whose non-temporal hint is a template argument of the kernel itself (not a build-time
+// switch): for kernel families that are instantiated both ways and picked per launch from the size
+// of what the launch reads.
+template <typename T, int N, bool NONTEMPORAL>
+__device__ __forceinline__ Vec<T, N> load_vec_hint(const T* __restrict__ p) {
+  constexpr int B = sizeof(T) * N;
+  static_assert(B == 16 || B == 8 || B == 4 || B == 2 || B == 1, "vector must be 1..16 bytes");
+  typedef typename RawBits<B>::type raw_t;
+  raw_t r;
+  if constexpr (NONTEMPORAL) {
+    r = __builtin_nontemporal_load(reinterpret_cast<const raw_t*>(p));
+  } else {
+    r = *reinterpret_cast<const raw_t*>(p);
+  }
+  Vec<T, N> out;
+  __builtin_memcpy(&out, &r, B);
+  return out;
+}
+
 // Load for kernels that only read (a reduction's sweep over its input), with a hint switch of
 // its own.  Measured on MI355X with a plain summing kernel: 1 GiB streams at 7.2-7.3 TB/s with
 // the non-temporal hint against 6.5-6.7 TB/s without, 128 MiB takes 17.9 us against 19.0 us.

@@ -181,7 +181,9 @@ int mi_launch_packed_scratch(void* function, uint32_t grid_x, uint32_t grid_y, u
   if (function == nullptr || arg_segment == nullptr) return rc(hipErrorInvalidValue);
   if (scratch_bytes_needed > MI355_SCRATCH_BYTES) return MI_ERROR_SCRATCH_TOO_LARGE;
   if (arg_segment_bytes > kMaxArgSegment) return rc(hipErrorInvalidValue);
-  if (scratch_arg_offset % sizeof(void*) != 0 || scratch_arg_offset + sizeof(void*) > arg_segment_bytes)
+  // written so that an offset near SIZE_MAX cannot wrap past the check
+  if (scratch_arg_offset % sizeof(void*) != 0 || arg_segment_bytes < sizeof(void*) ||
+      scratch_arg_offset > arg_segment_bytes - sizeof(void*))
     return rc(hipErrorInvalidValue);
   if (grid_x == 0 || grid_y == 0 || grid_z == 0 || block_x == 0 || block_y == 0 || block_z == 0)
     return rc(hipErrorInvalidConfiguration);

@@ -407,6 +407,7 @@ class SplitPlan:
     nsplit: int  # workgroups along the reduced axis
     rows_per_split: int
     col_tiles: int
+    prefetch: int = 2  # batches of `unroll` loads a thread holds (one being folded, the others in flight)
 
     @property
     def block(self) -> int:
@@ -640,7 +641,13 @@ class GeneratedKernel:
             # a tiled kernel (static shapes) carries its own workgroup count
             g = m["grid"] if "grid" in m else cdiv(xnumel, m["block"] * m["vec"] * m.get("unroll", 1))
             mult = int(m.get("grid_multiple", 1))  # the kernel deals workgroups out to the dies itself
-            grid = (cdiv(g, mult) * mult, 1, 1)
+            padded = cdiv(g, mult) * mult
+            # up to mult - 1 extra workgroups compute a start index before their bounds check: keep the
+            # exact count (the kernel then takes the plain workgroup order) when that index would
+            # leave the kernel's index type
+            if padded * m["block"] * m["vec"] * m.get("unroll", 1) >= 2 ** (int(m.get("index_bits", 64)) - 1):
+                padded = g
+            grid = (padded, 1, 1)
             return LaunchPlan([("main", grid, (m["block"],), 0, (xnumel,), False)], 0, cand)
         if self.mode == "row":
             rounds = cdiv(xnumel, m["block"] // m["tpr"])
@@ -725,6 +732,18 @@ class GeneratedKernel:
         wrapper's raw stream is)."""
         import torch
 
+        private = self._args_to_copy(args)
+        if private:
+            # in-place operands, targets of accumulating stores and outputs that share memory with an
+            # input (a mutated graph input arrives as both): time on copies, the caller's buffers see
+            # exactly one launch (reference inductor_x/npu_triton_heuristics.py:395-429 hands its
+            # tuner the mutated argument names for the same reason)
+            args = list(args)
+            for i in private:
+                t = args[i]  # same sizes and strides as the original: the kernel's index arithmetic is baked in
+                args[i] = torch.empty_strided(t.size(), t.stride(), dtype=t.dtype, device=t.device).copy_(t)
+            args = tuple(args)
+            raw = tuple(self._raw(a) for a in args)
         for _ in range(warmup):
             self._launch_plan(plan, args, raw, stream)
         start = torch.cuda.Event(enable_timing=True)
@@ -735,6 +754,22 @@ class GeneratedKernel:
         end.record()
         end.synchronize()
         return start.elapsed_time(end) / rep
+
+    def _args_to_copy(self, args) -> list:
+        """Positions of the tensor arguments a repeated launch would change the result of: buffers
+        the kernel reads and writes (in-place operands, accumulation targets), and written buffers
+        whose memory overlaps another argument's."""
+        is_t = lambda a: hasattr(a, "data_ptr") and hasattr(a, "untyped_storage")  # noqa: E731
+        out = {i for i in self.meta.get("mutated_args", ()) if i < len(args) and is_t(args[i])}
+        span = {}
+        for i, a in enumerate(args):
+            if is_t(a) and a.numel() > 0:
+                st = a.untyped_storage()
+                span[i] = (st.data_ptr(), st.data_ptr() + st.nbytes())
+        for i in self.meta.get("written_args", ()):
+            if i in span and any(j != i and span[j][0] < span[i][1] and span[i][0] < span[j][1] for j in span):
+                out.add(i)
+        return sorted(out)
 
     def num_bytes(self, args) -> int:
         """Bytes of every tensor argument, read or written once: the figure the reference's

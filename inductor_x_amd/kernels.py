@@ -99,6 +99,9 @@ _COL_PARTIAL_VARIANTS = [
     (128, 2, 16),
     (16, 16, 8),
 ]
+# (ct, rl, unroll, batches held per thread) beyond the default two
+_COL_PARTIAL_PF_VARIANTS = [(32, 8, 8, 3), (32, 8, 8, 4), (32, 8, 4, 3), (32, 8, 4, 4), (32, 16, 4, 3), (32, 16, 8, 3),
+                            (32, 8, 16, 3), (64, 8, 8, 3)]
 _COL_FINAL_VARIANTS = [(16, 16), (16, 32), (8, 64), (8, 32), (4, 64), (64, 4), (4, 16), (4, 32), (2, 64), (2, 32),
                        (8, 16), (8, 8), (16, 4), (16, 8)]
 _GATHER_VARIANTS = [(256, 128, 1), (256, 128, 2), (256, 128, 4), (256, 64, 1), (256, 64, 2), (256, 64, 4), (256, 16, 1), (256, 16, 4)]
@@ -159,6 +162,14 @@ def _col_partial_launcher() -> CachingLauncher:
             lds_bytes=col_fold_lds_bytes(ct, rl),
         )
         for ct, rl, u in _COL_PARTIAL_VARIANTS
+    ] + [
+        LaunchConfig(
+            f"col_mean_var_argmax_partial_f32_c{ct}_r{rl}_u{u}_p{pf}",
+            ct * rl,
+            meta={"CT": ct, "RL": rl, "UNROLL": u, "PF": pf},
+            lds_bytes=col_fold_lds_bytes(ct, rl),
+        )
+        for ct, rl, u, pf in _COL_PARTIAL_PF_VARIANTS
     ]
     return CachingLauncher(
         "col_mean_var_argmax_partial_f32", codecache.aot_source("col_kernels.hip"), "PPiii", cfgs, prefer_intree=True
@@ -373,7 +384,8 @@ def col_mean_var_argmax(
     _require(plan.col_tiles * plan.ct * 4 >= cols, "split plan does not cover all columns")
     need = plan.workspace_floats(cols)
     lp, lf = _col_partial_launcher(), _col_final_launcher()
-    ip = _find(lp, f"col_mean_var_argmax_partial_f32_c{plan.ct}_r{plan.rl}_u{plan.unroll}")
+    pf = "" if plan.prefetch == 2 else f"_p{plan.prefetch}"
+    ip = _find(lp, f"col_mean_var_argmax_partial_f32_c{plan.ct}_r{plan.rl}_u{plan.unroll}{pf}")
     if final_variant is None:
         # few columns per workgroup so that the second pass has hundreds of workgroups, and as many
         # split lanes as there are splits up to 16 (measured at 512 columns x 64 splits: (4, 16) 25.3 us
@@ -479,6 +491,89 @@ def permute_0213_contiguous(t: torch.Tensor, variant: Optional[tuple] = None) ->
     tiles = n0 * cdiv(n1, t1) * cdiv(n2, t2)
     l._launch(i, (t.data_ptr(), out.data_ptr(), n0, n1, n2, inner, s0, s1, s2), (tiles, 1, 1), _stream())
     return out
+
+
+# ---------------------------------------------------------------------------
+# ring-attention merge step: (prev_out, prev_max, prev_sum) + (cur_out, cur_max, cur_sum)
+# ---------------------------------------------------------------------------
+_RING_DTYPES = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}
+_RING_VARIANTS = [("bf16", 128, 16), ("bf16", 128, 32), ("bf16", 128, 8), ("f16", 128, 16), ("f32", 128, 16),
+                  ("bf16", 64, 16), ("f32", 64, 16)]
+
+
+@functools.lru_cache(maxsize=None)
+def _ring_launcher() -> CachingLauncher:
+    cfgs = [
+        LaunchConfig(f"ring_forward_update_{t}_d{d}_s{st}{'_nt' if nt else ''}", 256,
+                     meta={"DTYPE": t, "D": d, "ST": st, "STREAM": nt})
+        for t, d, st in _RING_VARIANTS for nt in (0, 1)
+    ]
+    return CachingLauncher(
+        "ring_forward_update", codecache.aot_source("ring_kernels.hip"), "PPPPPPPPPiiiqq", cfgs, prefer_intree=True
+    )
+
+
+def ring_forward_update(
+    prev_attn_out: torch.Tensor, prev_softmax_max: torch.Tensor, prev_softmax_sum: torch.Tensor,
+    cur_attn_out: torch.Tensor, cur_softmax_max: torch.Tensor, cur_softmax_sum: torch.Tensor,
+    variant: Optional[tuple] = None,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """One merge step of ring attention in a single kernel: returns (attn_out, softmax_max,
+    softmax_sum) of the union of the two key sets.  Attention outputs are [S, B, H] (bf16, fp16 or
+    fp32, H = N * D with D 64 or 128), statistics fp32 [B, N, S, 8] whose head stride may differ
+    between the two steps (a slice of a larger buffer); the returned statistics take the current
+    step's strides.  Argument order, layouts and result as the reference's hand-written
+    forward_update_triton (reference test/npu_indexing/written/attn_cp_triton_kernel_3d.py:88-139).
+    variant = (ST, streaming loads) overrides the launch choice."""
+    stats = (prev_softmax_max, prev_softmax_sum, cur_softmax_max, cur_softmax_sum)
+    _check_cuda(prev_attn_out, cur_attn_out, *stats)
+    _require(prev_attn_out.dtype == cur_attn_out.dtype and prev_attn_out.dtype in _RING_DTYPES,
+             "attention outputs must share one of bf16, fp16, fp32")
+    _require(prev_attn_out.dim() == 3 and prev_attn_out.shape == cur_attn_out.shape, "attention outputs must share an [S, B, H] shape")
+    _require(prev_attn_out.is_contiguous() and cur_attn_out.is_contiguous(), "attention outputs must be contiguous")
+    S, B, H = cur_attn_out.shape
+    for t in stats:
+        _require(t.dtype == torch.float32 and t.dim() == 4 and t.shape == cur_softmax_max.shape, "statistics must share a fp32 [B, N, S, 8] shape")
+    _require(cur_softmax_max.shape[0] == B and cur_softmax_max.shape[2] == S and cur_softmax_max.shape[3] == 8,
+             "statistics must be [B, N, S, 8] for [S, B, H] outputs")
+    N = cur_softmax_max.shape[1]
+    _require(N > 0 and H % N == 0, "H must be a multiple of the head count")
+    D = H // N
+    _require(prev_softmax_max.stride() == prev_softmax_sum.stride() and cur_softmax_max.stride() == cur_softmax_sum.stride(),
+             "maximum and sum of one step must share their strides")
+    for t in (prev_softmax_max, cur_softmax_max):
+        _require(t.stride(3) == 1 and t.stride(2) == 8, "statistics must be contiguous along their last two axes")
+        _require(B == 1 or t.stride(0) == N * t.stride(1), "the batch stride must be N head strides (no slice along N)")
+        _require(t.stride(1) % 4 == 0, "the head stride must be a multiple of 16 bytes")
+    out = torch.empty_like(cur_attn_out)
+    smax = torch.empty_strided(cur_softmax_max.shape, cur_softmax_max.stride(), dtype=torch.float32, device=cur_attn_out.device)
+    ssum = torch.empty_strided(cur_softmax_sum.shape, cur_softmax_sum.stride(), dtype=torch.float32, device=cur_attn_out.device)
+    if S * B * H == 0:
+        return out, smax, ssum
+    _require(all(_aligned(t) for t in (prev_attn_out, cur_attn_out, out, smax, ssum) + stats), "operands must be 16-byte aligned")
+    _require(out.numel() < 2**31 and B * N < 2**31 // max(S, 1), "extents must fit int32 indexing")
+    name = _RING_DTYPES[cur_attn_out.dtype]
+    shapes = [(d, st) for t, d, st in _RING_VARIANTS if t == name]
+    _require(any(d == D for d, _ in shapes), f"no forward_update kernel for head dimension {D} in {name}")
+    if variant is None:
+        # the operands are read once: loads carry the non-temporal hint when they exceed what the
+        # memory-side cache would keep for a later kernel anyway
+        read_bytes = 2 * out.numel() * out.element_size()
+        variant = (16, read_bytes > config.streaming_read_bytes() > 0)
+    st, stream = variant
+    _require((D, st) in shapes, f"no forward_update kernel with {st} sequence positions per workgroup")
+    l = _ring_launcher()
+    i = _find(l, f"ring_forward_update_{name}_d{D}_s{st}{'_nt' if stream else ''}")
+    nt = 256 // (D * out.element_size() // 16)  # heads per workgroup
+    l._launch(
+        i,
+        (prev_attn_out.data_ptr(), prev_softmax_max.data_ptr(), prev_softmax_sum.data_ptr(), cur_attn_out.data_ptr(),
+         cur_softmax_max.data_ptr(), cur_softmax_sum.data_ptr(), out.data_ptr(), smax.data_ptr(), ssum.data_ptr(),
+         S, B, N, prev_softmax_max.stride(1), cur_softmax_max.stride(1)),
+        (cdiv(S, st), cdiv(N, nt), B),
+        _stream(),
+    )
+    return out, smax, ssum
 
 
 # ---------------------------------------------------------------------------

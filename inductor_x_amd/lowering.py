@@ -41,6 +41,7 @@ from torch._inductor.lowering import (
     to_dtype,
 )
 from torch._inductor.utils import sympy_product
+from torch._inductor.virtualized import V
 from torch._prims_common import is_boolean_dtype, is_integer_dtype
 
 from . import config as backend_config
@@ -133,7 +134,8 @@ FALLBACK_OPS = [
 FALLBACK_LIST: list = []
 # Ops sent to eager kernels after the code generator refused a fused node that came from them
 # (filled at compile time by add_runtime_fallback; process-wide, so later graphs skip the retry).
-RUNTIME_FALLBACKS: list = []
+RUNTIME_FALLBACKS: list = []  # ops sent to eager kernels after a refused fused node (process-wide)
+_RUNTIME_FALLBACK_ORIGINALS: dict = {}
 _registered = False
 
 
@@ -166,7 +168,20 @@ def add_runtime_fallback(op) -> bool:
         return False
     lowerings[op] = _device_aware(op, original, handler)
     RUNTIME_FALLBACKS.append(op)
+    _RUNTIME_FALLBACK_ORIGINALS[op] = original
     return True
+
+
+def clear_runtime_fallbacks() -> list:
+    """Give every op in RUNTIME_FALLBACKS its generated lowering back; returns the ops restored.
+    The lowering tables are per process, so a fallback registered while one graph compiled also
+    applies to every graph compiled later; a caller that wants the generated lowering tried again
+    (after a fix, or for an unrelated model) calls this between compiles."""
+    restored = list(RUNTIME_FALLBACKS)
+    for op in restored:
+        lowerings[op] = _RUNTIME_FALLBACK_ORIGINALS.pop(op)
+    RUNTIME_FALLBACKS.clear()
+    return restored
 
 
 def _register_inductor_fallbacks() -> None:
@@ -209,7 +224,8 @@ def _register_inductor_fallbacks() -> None:
         if in_dtype in (torch.float16, torch.bfloat16):
             x = to_dtype(x, torch.float32)
         result = tagged_sum(x, axis, keepdims, dtype=torch.float32 if out_dtype != torch.float64 else None)
-        if backend_config.sum_returns_fp32 and dtype is None and in_dtype in (torch.float16, torch.bfloat16):
+        if (backend_config.sum_returns_fp32 and dtype is None and in_dtype in (torch.float16, torch.bfloat16)
+                and getattr(V.graph, "is_inference", False)):
             return result  # the reference's result type: the fp32 sum, not rounded back
         return to_dtype(result, out_dtype)
 

@@ -649,3 +649,76 @@ def test_generated_kernel_autotune_record_and_bandwidth_print(tmp_path, monkeypa
     torch.cuda.synchronize()
     assert again._plans[(256, 40000)].candidate == rec["best"]
     torch.testing.assert_close(out2, out)
+
+
+def test_timing_switches_leave_mutated_buffers_alone(tmp_path, monkeypatch, capsys):
+    """With the bandwidth print (and autotuning) on, a generated kernel is launched several extra
+    times for its timing.  A kernel that updates an operand in place (x.add_(y)) or accumulates
+    through atomic stores (index_put with accumulate=True) must do that on copies: the caller's
+    buffers see exactly one update (reference inductor_x/npu_triton_heuristics.py:395-429 passes the
+    mutated argument names to its tuner for the same reason)."""
+    from inductor_x_amd import config, hip_heuristics
+
+    announce("timing switches on in-place and accumulating kernels")
+    monkeypatch.setenv("INDUCTOR_X_AMD_CACHE", str(tmp_path))
+    monkeypatch.setattr(config, "autotune", True)
+    monkeypatch.setattr(config, "profile_bandwidth", True)
+    made = []
+    original = hip_heuristics.generated_kernel
+    monkeypatch.setattr(hip_heuristics, "generated_kernel", lambda *a, **k: made.append(original(*a, **k)) or made[-1])
+    torch.manual_seed(0)
+
+    def inplace(x, y):
+        x.add_(y * 3.0)
+        return x
+
+    x = torch.randn(3001, 517, device=DEV)
+    y = torch.randn(3001, 517, device=DEV)
+    want = x + y * 3.0
+    torch._dynamo.reset()
+    got = torch.compile(inplace)(x, y)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(x, want, rtol=1e-6, atol=1e-6)
+
+    def accumulate(base, idx, vals):
+        return torch.index_put(base * 1.0, (idx,), vals, accumulate=True)
+
+    base = torch.zeros(257, 64, device=DEV)
+    idx = torch.randint(0, 257, (5000,), device=DEV)
+    vals = torch.ones(5000, 64, device=DEV)  # integers-valued sums: exact whatever the order
+    want = torch.index_put(base * 1.0, (idx,), vals, accumulate=True)
+    torch._dynamo.reset()
+    got = torch.compile(accumulate)(base, idx, vals)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert any(k.meta.get("mutated_args") for k in made), [k.meta.get("mutated_args") for k in made]
+    assert "GB/s" in capsys.readouterr().out
+
+
+def test_sum_fp32_switch_applies_to_inference_graphs_only(monkeypatch):
+    """config.sum_returns_fp32 (the reference's `sum` returns the fp32 accumulator for 16-bit inputs,
+    reference inductor_x/lowering.py:204-215): in an inference graph the fp32 sum is what a consumer
+    reads and what the graph returns; a graph with a backward keeps the traced 16-bit type."""
+    from inductor_x_amd import config
+
+    announce("sum of bf16 returning fp32: inference graph, consumer, training graph")
+    monkeypatch.setattr(config, "sum_returns_fp32", True)
+    torch.manual_seed(0)
+    x = torch.randn(64, 4096, device=DEV).bfloat16()
+    f = lambda x: (x.sum(-1) * 2.0, x.sum(-1))  # noqa: E731
+    exact = x.double().sum(-1)
+    torch._dynamo.reset()
+    with torch.no_grad():
+        doubled, plain = torch.compile(f)(x)
+    assert plain.dtype == torch.float32 and doubled.dtype == torch.float32
+    # fp32 accumulation of 4096 terms of size ~1: far inside bf16's rounding step of 0.25 - 0.5 at |sum| ~ 64
+    assert (plain.double() - exact).abs().max().item() < 1e-2
+    assert (doubled.double() - 2 * exact).abs().max().item() < 2e-2
+    xg = x.clone().requires_grad_(True)
+    torch._dynamo.reset()
+    out = torch.compile(lambda x: x.sum(-1))(xg)
+    assert out.dtype == torch.bfloat16
+    out.float().sum().backward()
+    assert xg.grad is not None and xg.grad.dtype == torch.bfloat16 and torch.equal(xg.grad, torch.ones_like(xg))
+    torch._dynamo.reset()

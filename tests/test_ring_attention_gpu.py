@@ -89,6 +89,67 @@ def test_forward_update_reference_shapes(O, S, B, H, N, dtype):
         np.testing.assert_allclose(got, ref_out, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize(
+    "S,B,H,N,dtype",
+    [(4096, 1, 6144, 48, torch.bfloat16), (4096, 1, 1536, 12, torch.float32), (37, 2, 5 * 128, 5, torch.bfloat16),
+     (100, 1, 3 * 64, 3, torch.float32), (33, 2, 17 * 128, 17, torch.float16)],
+)
+def test_forward_update_single_kernel(O, S, B, H, N, dtype):
+    """The hand-written one-launch form (kernels.ring_forward_update; reference
+    written/attn_cp_triton_kernel_3d.py:15-139) at the reference's two shapes and at extents that
+    leave partly filled tiles along the sequence and the head axis, against the fp64 oracle; the
+    previous step's statistics are a slice of a longer buffer (their head stride differs)."""
+    from inductor_x_amd import kernels, launcher
+
+    DS = 2 * S
+    announce(f"ring forward_update, one kernel (2S,B,H,N)=({DS},{B},{H},{N}) {dtype}")
+    torch.manual_seed(0)
+    mk_out = lambda: torch.randn(DS, B, H).to(dtype)  # noqa: E731
+    mk_st = lambda off, s=DS: (torch.rand(B, N, s) + off).unsqueeze(3).repeat(1, 1, 1, F32_BLK).contiguous()  # noqa: E731
+    prev_out, cur_out = mk_out(), mk_out()
+    cur_max, cur_sum = mk_st(0.0), mk_st(0.5)
+    prev_max_buf, prev_sum_buf = mk_st(0.0, DS + 24), mk_st(0.5, DS + 24)
+    prev_max, prev_sum = prev_max_buf[:, :, :DS], prev_sum_buf[:, :, :DS]
+    dev = lambda t: t.to(DEV)  # noqa: E731
+    pm_d, ps_d = dev(prev_max_buf)[:, :, :DS], dev(prev_sum_buf)[:, :, :DS]
+    launcher.launch_log = []
+    try:
+        out, smax, ssum = kernels.ring_forward_update(dev(prev_out), pm_d, ps_d, dev(cur_out), dev(cur_max), dev(cur_sum))
+        torch.cuda.synchronize()
+    finally:
+        log, launcher.launch_log = launcher.launch_log, None
+    assert len(log) == 1 and log[0].startswith("ring_forward_update_"), log
+    ref_out, ref_max, ref_sum = O.forward_update(prev_out.float().numpy(), prev_max.contiguous().numpy(), prev_sum.contiguous().numpy(),
+                                                 cur_out.float().numpy(), cur_max.numpy(), cur_sum.numpy())
+    assert out.dtype == dtype and out.shape == (DS, B, H) and smax.shape == cur_max.shape
+    np.testing.assert_allclose(smax.cpu().numpy(), ref_max, rtol=1e-6)
+    np.testing.assert_allclose(ssum.cpu().numpy(), ref_sum, rtol=1e-5)
+    got = out.float().cpu().numpy()
+    if dtype == torch.float32:
+        np.testing.assert_allclose(got, ref_out, rtol=1e-5, atol=1e-5)
+    else:
+        assert np.abs(got - ref_out).max() <= 2e-2
+    # both load forms give the same bits
+    for variant in ((16, False), (16, True)):
+        o2, m2, l2 = kernels.ring_forward_update(dev(prev_out), pm_d, ps_d, dev(cur_out), dev(cur_max), dev(cur_sum), variant=variant)
+        assert torch.equal(o2, out) and torch.equal(m2, smax) and torch.equal(l2, ssum)
+
+
+def test_forward_update_single_kernel_rejects_what_it_was_not_written_for():
+    from inductor_x_amd import kernels
+
+    announce("ring forward_update, one kernel: argument checks")
+    o = torch.zeros(8, 1, 256, device=DEV, dtype=torch.bfloat16)
+    st = torch.zeros(1, 2, 8, 8, device=DEV)
+    with pytest.raises(ValueError):
+        kernels.ring_forward_update(o, st, st, o.float(), st, st)  # mixed element types
+    with pytest.raises(ValueError):
+        kernels.ring_forward_update(o, st, st, o, st[..., :4].repeat(1, 1, 1, 2)[:, :, ::2], st)  # wrong sequence extent
+    with pytest.raises(ValueError):
+        kernels.ring_forward_update(o[:, :, :96].contiguous(), st, st, o[:, :, :96].contiguous(), st, st)  # head dimension 48
+    assert kernels.ring_forward_update(o[:0], st[:, :, :0], st[:, :, :0], o[:0], st[:, :, :0], st[:, :, :0])[0].shape == (0, 1, 256)
+
+
 def forward_update_la(prev_out, prev_lse, cur_out, cur_lse):
     lse = torch.log(torch.exp(cur_lse) + torch.exp(prev_lse))
     out = torch.exp(prev_lse - lse) * prev_out + torch.exp(cur_lse - lse) * cur_out
