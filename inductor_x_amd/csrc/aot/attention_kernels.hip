@@ -164,31 +164,37 @@ extern "C" __global__ __launch_bounds__(512, 1) void fused_attention_fwd_bf16_d1
 }
 
 // v5: the v4 schedule with K and V tiles loaded straight into LDS and V read back transposed
-// (attention_v5.h).  Same workgroup shape and grid as v4; 64 KiB of LDS.
+// (attention_v5.h).  64 KiB of LDS.  The launch is persistent: the grid is at most one workgroup
+// per CU and every workgroup walks the work items id = blockIdx.x, blockIdx.x + gridDim.x, ...
+// (gridDim.x is a multiple of 8, so a workgroup stays on the heads of its own die).  Between two
+// items nothing waits: the output stores of one item drain while the next one loads its queries
+// and first key tiles, and no workgroup has to be dispatched in between.  Measured on MI355X at
+// [4,32,4096,128]: one workgroup per item spent about 3.4 us per query block on the drain and the
+// next dispatch.
 template <bool CAUSAL, int WAVES = kAttnV5Waves>
 __device__ __forceinline__ void attention_entry_v5(const bf16_t* q, const bf16_t* k, const bf16_t* v,
                                                    bf16_t* o, float* smax, float* ssum, int n_heads,
                                                    int S, float scale_log2e) {
   constexpr int XCDS = 8;
   const int n_qb = S / (32 * WAVES);
-  const int id = blockIdx.x;
-  const int xcd = id % XCDS;
-  const int slot = id / XCDS;
-  if (CAUSAL) {
-    const int n_pair = (n_qb + 1) / 2;
-    const int head = (slot / n_pair) * XCDS + xcd;
-    const int lo = slot % n_pair;
-    const int hi = n_qb - 1 - lo;
-    if (head >= n_heads) return;
-    const int n_pass = lo != hi ? 2 : 1;
+  const int per_head = CAUSAL ? (n_qb + 1) / 2 : n_qb;
+  const int total = XCDS * ((n_heads + XCDS - 1) / XCDS) * per_head;
 #pragma nounroll
-    for (int pass = 0; pass < n_pass; ++pass)
-      attention_fwd_d128_v5<true, WAVES>(q, k, v, o, smax, ssum, S, pass == 0 ? hi : lo, head, scale_log2e);
-  } else {
-    const int head = (slot / n_qb) * XCDS + xcd;
-    const int qb = slot % n_qb;
-    if (head >= n_heads) return;
-    attention_fwd_d128_v5<false, WAVES>(q, k, v, o, smax, ssum, S, qb, head, scale_log2e);
+  for (int id = blockIdx.x; id < total; id += gridDim.x) {
+    const int xcd = id % XCDS;
+    const int slot = id / XCDS;
+    const int head = (slot / per_head) * XCDS + xcd;
+    if (head >= n_heads) continue;
+    if (CAUSAL) {
+      const int lo = slot % per_head;
+      const int hi = n_qb - 1 - lo;
+      const int n_pass = lo != hi ? 2 : 1;
+#pragma nounroll
+      for (int pass = 0; pass < n_pass; ++pass)
+        attention_fwd_d128_v5<true, WAVES>(q, k, v, o, smax, ssum, S, pass == 0 ? hi : lo, head, scale_log2e);
+    } else {
+      attention_fwd_d128_v5<false, WAVES>(q, k, v, o, smax, ssum, S, slot % per_head, head, scale_log2e);
+    }
   }
 }
 

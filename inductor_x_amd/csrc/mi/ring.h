@@ -31,7 +31,7 @@ __device__ __forceinline__ float ring_max_nan(float a, float b) {
 // by TPR = D / VEC lanes of 16 bytes, so a workgroup spans NT = 256 / TPR heads.
 // STREAM: loads and stores of the attention outputs carry the non-temporal hint (the caller
 // sets it when the operands are larger than the memory-side cache can hold anyway).
-template <typename T, int D, int ST, bool STREAM>
+template <typename T, int D, int ST, bool STREAM, int BATCH_ = 4, bool EARLY = true>
 __device__ __forceinline__ void ring_forward_update(
     const T* __restrict__ prev_out, const float* __restrict__ prev_max, const float* __restrict__ prev_sum,
     const T* __restrict__ cur_out, const float* __restrict__ cur_max, const float* __restrict__ cur_sum,
@@ -55,7 +55,7 @@ __device__ __forceinline__ void ring_forward_update(
   const int n = n0 + n_l;
   const size_t H = static_cast<size_t>(N) * D;
   const size_t col = static_cast<size_t>(n) * D + static_cast<size_t>(tid % TPR) * VEC;
-  constexpr int BATCH = ST % 8 == 0 ? 8 : (ST % 4 == 0 ? 4 : 1);
+  constexpr int BATCH = ST % BATCH_ == 0 ? BATCH_ : 1;
   Vec<T, VEC> pv[BATCH], cv[BATCH];
   auto load_rows = [&](int r0) {
 #pragma unroll
@@ -69,7 +69,7 @@ __device__ __forceinline__ void ring_forward_update(
     }
   };
   // the first rows are requested before the statistics are touched: they do not depend on them
-  load_rows(0);
+  if constexpr (EARLY) load_rows(0);
 
   // ---- statistics: one thread per (head, s), s fastest, eight fp32 per array ----
   for (int p = tid; p < PAIRS; p += 256) {
@@ -111,7 +111,7 @@ __device__ __forceinline__ void ring_forward_update(
   if (n >= N) return;
 #pragma unroll
   for (int r0 = 0; r0 < ST; r0 += BATCH) {
-    if (r0 > 0) load_rows(r0);
+    if (!EARLY || r0 > 0) load_rows(r0);
 #pragma unroll
     for (int j = 0; j < BATCH; ++j) {
       const int s = s0 + r0 + j;

@@ -679,11 +679,19 @@ def fused_attention(
         heads = B * N
         n_qb = S // bm
         per_head = (n_qb + 1) // 2 if causal else n_qb
+        items = 8 * cdiv(heads, 8) * per_head
+        if variant in ("v5", "v5h"):
+            # persistent launch: at most one workgroup per CU slot, a multiple of 8 (one per die in turn);
+            # every workgroup walks items blockIdx.x, blockIdx.x + gridDim.x, ...
+            slots = config.hardware().cu_count * (2 if variant == "v5h" else 1)
+            grid = min(items, max(slots // 8, 1) * 8)
+        else:
+            grid = items
         l._launch(
             i,
             (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), smax.data_ptr(), ssum.data_ptr(), heads, S,
              float(scale) * 1.4426950408889634),
-            (8 * cdiv(heads, 8) * per_head, 1, 1),
+            (grid, 1, 1),
             _stream(),
         )
         return out, smax, ssum
