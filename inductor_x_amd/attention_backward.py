@@ -95,10 +95,10 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
                              use_kernels=None, keep_prob: float = 1.0, seed: int = 0):
     """q, k, v, out, dout: [B, N, S, D] of one floating-point type; softmax_max / softmax_sum:
     [B, N, S, 8] fp32 from the forward.  Returns (dq, dk, dv) in that type.  use_kernels: None = fused
-    kernels where they apply (bf16, head dimension 128, sequence a multiple of 128, no dropout).
+    kernels where they apply (bf16, head dimension 128, sequence a multiple of 64, no dropout).
     keep_prob < 1 with the forward's seed regenerates the forward's dropout mask (GEMM path only)."""
-    fits = (q.dim() == 4 and q.dtype == torch.bfloat16 and q.size(3) == 128 and q.size(2) % 128 == 0
-            and q.size(2) > 0 and keep_prob == 1.0)
+    fits = (q.dim() == 4 and q.dtype == torch.bfloat16 and q.size(3) == 128 and q.size(2) % 64 == 0
+            and q.size(2) > 0 and q.shape == k.shape and keep_prob == 1.0)
     if use_kernels is None:
         use_kernels = fits
     if use_kernels:

@@ -26,7 +26,7 @@
 // loads and not stored.
 #pragma once
 
-#include "attention_v2.h"
+#include "attention.h"
 
 namespace mi {
 

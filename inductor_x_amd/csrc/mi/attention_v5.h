@@ -1,8 +1,12 @@
 // Fused attention forward, 32 queries per wavefront, two wavefronts per SIMD, K and V tiles brought
-// into LDS by direct global -> LDS loads and V read back transposed.
+// into LDS by direct global -> LDS loads and V read back transposed.  Operand layouts: attention.h.
 //
-// Same mathematics, operand layouts and software pipeline as attention_v4.h (its results are
-// bit-identical); what changes is how a tile travels:
+// Software pipeline per 64-key tile, matrix and vector work of each wavefront interleaved chunk by
+// chunk (one LDS fragment read two chunks ahead, one MFMA, a slice of the vector work):
+//     A   matrix:  O += V^T(t-1) P(t-1)      vector:  row max of S(t), first half of P(t)
+//     B   matrix:  S(t+1) = K(t+1) Q^T       vector:  second half of P(t)
+// With 32 queries a wavefront needs 200-240 registers, so a SIMD holds two, and the vector
+// instructions of one issue in the shadow of the other's MFMAs.  How a tile travels:
 //   - K and V tiles go memory -> LDS with 16-byte `buffer_load ... lds` (gfx950): no staging registers, no
 //     LDS store instructions, no byte permutes.  One wavefront instruction fills a 1 KiB block (four
 //     256-byte rows); which global 16-byte chunk a lane fetches is free, so the chunks of a row are
@@ -14,12 +18,14 @@
 //     `ds_read_b64_tr_b16` per fragment: in every group of 16 lanes, lane s points at four consecutive
 //     d of key 4 g + s / 4 and receives, for its own d, the four keys of the group -- which is the
 //     key order P arrives in from the first product's accumulator layout.
-// Measured on MI355X at [4,32,4096,128] (HIP events, same process): 0.576 / 0.996 ms causal / full
-// against 0.587 / 1.010 ms for attention_v4.h: the tile traffic it removes (0.116 -> 0.068 ms by
-// ablation) is partly paid back by the second LDS read per V fragment (fragment reads 0.25 -> 0.30 ms).
+// Element type (bf16 or fp16), causal mask and bounds handling are template arguments.  RAGGED
+// instantiations take any sequence lengths: query rows past the end are computed on a copy of the
+// last row and not stored, keys past the end read as zeros (the tile copies are bounded buffer
+// loads) and are masked in the softmax of the last tile; the others require lengths that are
+// multiples of 256 (queries) and 128 (keys) and carry none of that code.
 #pragma once
 
-#include "attention_v2.h"
+#include "attention.h"
 
 
 namespace mi {
@@ -30,21 +36,22 @@ constexpr int kAttnV5BM = kAttnV5Waves * 32;
 // WAVES = 8: one workgroup of 256 queries per CU.  WAVES = 4: 128 queries per workgroup and two
 // workgroups per CU (64 KiB of LDS each), so the two wavefronts of a SIMD belong to different
 // workgroups, share no barrier and drift apart in phase.
-template <bool CAUSAL, int WAVES = kAttnV5Waves>
-__device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__ Q,
-                                                      const bf16_t* __restrict__ K,
-                                                      const bf16_t* __restrict__ V,
-                                                      bf16_t* __restrict__ O,
+template <typename T, bool CAUSAL, bool RAGGED, int WAVES = kAttnV5Waves>
+__device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, const T* __restrict__ K,
+                                                      const T* __restrict__ V, T* __restrict__ O,
                                                       float* __restrict__ softmax_max,
-                                                      float* __restrict__ softmax_sum, int S,
+                                                      float* __restrict__ softmax_sum, int Sq, int Sk,
                                                       int q_block, int head, float scale_log2e) {
+  typedef AttnElem<T> E;
+  typedef typename E::x8 x8_t;
+  constexpr bool GUARDED = CAUSAL || RAGGED;  // the last tiles of a block run the guarded copy of the loop
   extern __shared__ __attribute__((aligned(16))) unsigned char attn_lds[];
   // K and V tiles as they come from memory, [64 rows][128] bf16 without padding, 16-byte chunks of a
   // row XOR-swizzled; written by direct global -> LDS loads (one 1 KiB block = four rows per
   // wavefront instruction), two buffers each
   constexpr int kTileElems = 64 * 128;
-  bf16_t* Kbuf = reinterpret_cast<bf16_t*>(attn_lds);
-  bf16_t* Vbuf = Kbuf + 2 * kTileElems;
+  T* Kbuf = reinterpret_cast<T*>(attn_lds);
+  T* Vbuf = Kbuf + 2 * kTileElems;
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -52,12 +59,14 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
   const int li = lane & 31;
   const int g = lane >> 5;
 
-  const size_t head_off = static_cast<size_t>(head) * S * kAttnD;
-  const bf16_t* __restrict__ Qh = Q + head_off;
-  const bf16_t* __restrict__ Kh = K + head_off;
-  const bf16_t* __restrict__ Vh = V + head_off;
+  const size_t head_off = static_cast<size_t>(head) * Sq * kAttnD;
+  const size_t kv_off = static_cast<size_t>(head) * Sk * kAttnD;
+  const T* __restrict__ Qh = Q + head_off;
+  const T* __restrict__ Kh = K + kv_off;
+  const T* __restrict__ Vh = V + kv_off;
 
-  static_assert(WAVES == 8 || WAVES == 4, "8 or 4 wavefronts");
+  static_assert(WAVES == 8, "8 wavefronts");
+  static_assert(sizeof(T) == 2, "16-bit elements");
   constexpr int BM = WAVES * 32;
   const int q0 = q_block * BM;
   // Wavefronts 4..7 take the 32-query sub-blocks in reverse order: with a causal mask a sub-block
@@ -69,11 +78,12 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
 #endif
   const int sub = (CAUSAL && MI_ATTN_V5_BALANCE && WAVES == 8 && wave >= 4) ? 11 - wave : wave;
   const int qi = q0 + sub * 32 + li;
+  const int qi_ld = RAGGED ? min(qi, Sq - 1) : qi;  // rows past the end work on a copy of the last row
 
-  bf16x8_t qf[8];
+  x8_t qf[8];
 #pragma unroll
   for (int s = 0; s < 8; ++s)
-    qf[s] = *reinterpret_cast<const bf16x8_t*>(Qh + static_cast<size_t>(qi) * kAttnD + 16 * s + 8 * g);
+    qf[s] = *reinterpret_cast<const x8_t*>(Qh + static_cast<size_t>(qi_ld) * kAttnD + 16 * s + 8 * g);
 
   f32x16_t oacc[4];
 #pragma unroll
@@ -82,15 +92,23 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
     for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
   float m_run = -__builtin_inff(), m_true = -__builtin_inff(), l_run = 0.f, alpha = 1.f;
 
-  const int n_tiles = CAUSAL ? (q0 + BM) / kAttnBN : S / kAttnBN;
-  const int first_masked = CAUSAL ? n_tiles - BM / kAttnBN : n_tiles;
+  // Tiles that hold keys at all, tiles this block can see, and the (even) number the loop walks:
+  // the pipeline below is unrolled over pairs of tiles, so an odd count is padded with one tile
+  // that lies wholly past the end (zeros from the bounded loads, skipped like a tile above the
+  // diagonal).
+  const int real_tiles = RAGGED ? (Sk + kAttnBN - 1) / kAttnBN : Sk / kAttnBN;
+  const int vis_tiles = CAUSAL ? min(real_tiles, (q0 + BM) / kAttnBN) : real_tiles;
+  const int n_tiles = RAGGED ? 2 * ((vis_tiles + 1) / 2) : vis_tiles;
+  // first tile that needs the guarded loop: the diagonal, or the tile that holds the end of the keys
+  const int first_masked = CAUSAL ? q0 / kAttnBN : (RAGGED ? Sk / kAttnBN : n_tiles);
 
   // direct global -> LDS copies: block b of a tile (rows 4 b .. 4 b + 3) is written by one wavefront
   // instruction, lane l filling LDS chunk l of the block (row 4 b + l / 16, chunk position l % 16)
   // with the global chunk that the swizzle puts there
   const int blk_row = lane >> 4;
   const int blk_pos = lane & 15;
-  auto issue_tile = [&](const bf16_t* __restrict__ src, bf16_t* dst, int tile, auto swz) {
+  const int kv_bytes = RAGGED ? Sk * kAttnD * 2 : 0x7fffffff;  // loads past a head's keys return zeros
+  auto issue_tile = [&](const T* __restrict__ src, T* dst, int tile, auto swz) {
 #pragma unroll
     for (int u = 0; u < 16 / WAVES; ++u) {
       const int b = (16 / WAVES) * wave + u;
@@ -103,7 +121,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
       // needs 200 / 228 registers instead of 206 / 256 + 4 spilled, and runs about 1 % faster.
       const int voff = ((tile * kAttnBN + row) * kAttnD + 8 * gchunk) * 2;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(src), 0, 0x7fffffff, 0x00020000),
+          __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(src), 0, kv_bytes, 0x00020000),
           (__attribute__((address_space(3))) void*)(dst + b * 512), 16, voff, 0, 0, 0);
     }
   };
@@ -119,8 +137,8 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
   int k_off[8];
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) k_off[ks] = li * kAttnD + 8 * ((2 * ks + g) ^ (li & 15));
-  auto k_frag = [&](const bf16_t* Ks, int i) {
-    return *reinterpret_cast<const bf16x8_t*>(Ks + 32 * (i >> 3) * kAttnD + k_off[i & 7]);
+  auto k_frag = [&](const T* Ks, int i) {
+    return *reinterpret_cast<const x8_t*>(Ks + 32 * (i >> 3) * kAttnD + k_off[i & 7]);
   };
   // V^T fragment of chunk i of phase A (key slice t4 = i / 4, d block db = i % 4) by two transposing
   // LDS reads: in each group of 16 lanes, lane s points at four consecutive d of key
@@ -135,14 +153,12 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
     for (int db = 0; db < 4; ++db)
       v_off[db] = key_l * kAttnD + 8 * (((4 * db) ^ (f & 12)) + (c_l ^ (f & 2))) + 4 * (sl16 & 1);
   }
-  typedef __bf16 bf16x4v_t __attribute__((__vector_size__(4 * sizeof(__bf16))));
-  auto v_frag = [&](const bf16_t* Vt, int i) {
+  auto v_frag = [&](const T* Vt, int i) {
     const int t4 = i >> 2, db = i & 3;
-    const bf16_t* p0 = Vt + 16 * t4 * kAttnD + v_off[db];
-    const bf16x4v_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4v_t*)(p0));
-    const bf16x4v_t hi =
-        __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4v_t*)(p0 + 8 * kAttnD));
-    bf16x8_t r;
+    const T* p0 = Vt + 16 * t4 * kAttnD + v_off[db];
+    const typename E::x4 lo = E::read_tr(p0);
+    const typename E::x4 hi = E::read_tr(p0 + 8 * kAttnD);
+    x8_t r;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       r[e] = lo[e];
@@ -151,8 +167,10 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
     return r;
   };
 
+  // last key this lane's query may see: itself under a causal mask, the last key there is otherwise
+  const int key_limit = CAUSAL ? (RAGGED ? min(qi_ld, Sk - 1) : qi) : Sk - 1;
   auto apply_mask = [&](int tile) {
-    const int d = qi - (tile * kAttnBN + 4 * g);  // keys with local offset > d are masked
+    const int d = key_limit - (tile * kAttnBN + 4 * g);  // keys with local offset > d are masked
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -175,7 +193,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
   };
   auto softmax_ref = [&]() {
     m_true = fmaxf(m_true, mx * scale_log2e);
-    m_new = m_true > m_run + kAttnV2Slack ? m_true : m_run;
+    m_new = m_true > m_run + kAttnSlack ? m_true : m_run;
     alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     m_run = m_new;
     psum = 0.f;
@@ -187,9 +205,9 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
     const float p0 = __builtin_amdgcn_exp2f(fmaf(sacc[kb][r], scale_log2e, -m_new));
     const float p1 = __builtin_amdgcn_exp2f(fmaf(sacc[kb][r + 1], scale_log2e, -m_new));
     psum += p0 + p1;
-    bf16x2_t pk;
-    pk[0] = static_cast<bf16_t>(p0);
-    pk[1] = static_cast<bf16_t>(p1);
+    typename E::x2 pk;
+    pk[0] = static_cast<T>(p0);
+    pk[1] = static_cast<T>(p1);
     uint32_t word = __builtin_bit_cast(uint32_t, pk);
     asm volatile("" : "+v"(word), "+v"(psum));  // keep the work in this slot of the schedule
     pw[t4][j] = word;
@@ -203,8 +221,8 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
     constexpr bool DO_PV = decltype(pv_c)::value;
     constexpr bool GUARD = decltype(guard_c)::value;
     constexpr int ODD = decltype(odd_c)::value ? 1 : 0;
-    const bf16_t* Vt = Vbuf + (1 - ODD) * kTileElems;
-    bf16x8_t f[16];
+    const T* Vt = Vbuf + (1 - ODD) * kTileElems;
+    x8_t f[16];
     if constexpr (DO_PV) {
       if (!GUARD || do_pv) {
         f[0] = v_frag(Vt, 0);
@@ -217,7 +235,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
       if constexpr (DO_PV) {
         if (!GUARD || do_pv) {
           if constexpr (i + 2 < 16) f[i + 2] = v_frag(Vt, i + 2);
-          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], attn_as_bf16x8(pw[t4]), oacc[db], 0, 0, 0);
+          oacc[db] = E::mfma(f[i], __builtin_bit_cast(x8_t, pw[t4]), oacc[db]);
         }
       }
       if constexpr (i == 0) issue_k(k_tile, ODD);
@@ -246,8 +264,8 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
     constexpr bool DO_QK = decltype(qk_c)::value;
     constexpr bool GUARD = decltype(guard_c)::value;
     constexpr int ODD = decltype(odd_c)::value ? 1 : 0;
-    const bf16_t* Ks = Kbuf + (1 - ODD) * kTileElems;
-    bf16x8_t f[16];
+    const T* Ks = Kbuf + (1 - ODD) * kTileElems;
+    x8_t f[16];
     if constexpr (DO_QK) {
       if (!GUARD || do_qk) {
         f[0] = k_frag(Ks, 0);
@@ -264,9 +282,9 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
             f32x16_t z;
 #pragma unroll
             for (int r = 0; r < 16; ++r) z[r] = 0.f;
-            sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], qf[ks], z, 0, 0, 0);
+            sacc[kb] = E::mfma(f[i], qf[ks], z);
           } else {
-            sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f[i], qf[ks], sacc[kb], 0, 0, 0);
+            sacc[kb] = E::mfma(f[i], qf[ks], sacc[kb]);
           }
         }
       }
@@ -292,17 +310,19 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
       for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; ++i)
-      sacc[i >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag(Kbuf, i), qf[i & 7], sacc[i >> 3], 0, 0, 0);
+      sacc[i >> 3] = E::mfma(k_frag(Kbuf, i), qf[i & 7], sacc[i >> 3]);
   }
   __syncthreads();  // K buffer 0 is rewritten in iteration 0
 
-  using T = std::true_type;
-  using F = std::false_type;
+  using Yes = std::true_type;
+  using No = std::false_type;
   // last key tile this wavefront's queries can see (only the diagonal tiles differ between wavefronts)
-  const int last_tile = CAUSAL ? first_masked + (sub >> 1) : n_tiles - 1;
-  if (CAUSAL && 0 == last_tile) apply_mask(0);
-  phase_a(F(), F(), 2, 0, F(), true, true);
-  phase_b(T(), F(), F(), true, true);
+  const int last_tile =
+      CAUSAL ? (RAGGED ? min(min(q0 + sub * 32 + 31, Sq - 1) / kAttnBN, real_tiles - 1) : first_masked + (sub >> 1))
+             : real_tiles - 1;
+  if (GUARDED && 0 == last_tile) apply_mask(0);
+  phase_a(No(), No(), min(2, n_tiles - 1), 0, No(), true, true);
+  phase_b(Yes(), No(), No(), true, true);
   __syncthreads();
 
   auto pair = [&](int t, auto mask_c) {
@@ -312,9 +332,9 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
         if (t == last_tile) apply_mask(t);
       }
       const bool sm = !MASK || t <= last_tile;
-      phase_a(T(), T(), min(t + 2, n_tiles - 1), t, mask_c, t - 1 <= last_tile, sm);  // K past the end: a harmless reload
+      phase_a(Yes(), Yes(), min(t + 2, n_tiles - 1), t, mask_c, t - 1 <= last_tile, sm);  // K past the end: a harmless reload
       if (sm) rescale();
-      phase_b(T(), T(), mask_c, t + 1 <= last_tile, sm);
+      phase_b(Yes(), Yes(), mask_c, t + 1 <= last_tile, sm);
       __syncthreads();
     }
     {
@@ -323,30 +343,30 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
         if (u == last_tile) apply_mask(u);
       }
       const bool sm = !MASK || u <= last_tile;
-      phase_a(T(), F(), min(u + 2, n_tiles - 1), u, mask_c, u - 1 <= last_tile, sm);
+      phase_a(Yes(), No(), min(u + 2, n_tiles - 1), u, mask_c, u - 1 <= last_tile, sm);
       if (sm) rescale();
-      phase_b(T(), F(), mask_c, u + 1 <= last_tile, sm);
+      phase_b(Yes(), No(), mask_c, u + 1 <= last_tile, sm);
       __syncthreads();
     }
   };
   int t = 1;
-  for (; t + 1 < first_masked; t += 2) pair(t, F());
-  if constexpr (CAUSAL) {
-    for (; t < n_tiles - 1; t += 2) pair(t, T());
+  for (; t + 1 < first_masked; t += 2) pair(t, No());
+  if constexpr (GUARDED) {
+    for (; t < n_tiles - 1; t += 2) pair(t, Yes());
   }
   {
     t = n_tiles - 1;
     const bool sm = t <= last_tile;
-    if (CAUSAL && t == last_tile) apply_mask(t);
-    phase_a(T(), T(), t, t, std::integral_constant<bool, CAUSAL>(), t - 1 <= last_tile, sm);
+    if (GUARDED && t == last_tile) apply_mask(t);
+    phase_a(Yes(), Yes(), t, t, std::integral_constant<bool, GUARDED>(), t - 1 <= last_tile, sm);
     if (sm) rescale();
-    phase_b(F(), T(), std::integral_constant<bool, CAUSAL>(), false, sm);
+    phase_b(No(), Yes(), std::integral_constant<bool, GUARDED>(), false, sm);
     __syncthreads();
     if (sm) {
-      const bf16_t* Vt = Vbuf + kTileElems;
+      const T* Vt = Vbuf + kTileElems;
 #pragma unroll
       for (int i = 0; i < 16; ++i)
-        oacc[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag(Vt, i), attn_as_bf16x8(pw[i >> 2]), oacc[i & 3], 0, 0, 0);
+        oacc[i & 3] = E::mfma(v_frag(Vt, i), __builtin_bit_cast(x8_t, pw[i >> 2]), oacc[i & 3]);
     }
   }
 
@@ -363,27 +383,27 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const bf16_t* __restrict__
   // row, and reads it back row-wise, so that one instruction stores four whole 256-byte rows.
   __syncthreads();  // every wavefront is done with the K and V tiles
   {
-    bf16_t* stage = reinterpret_cast<bf16_t*>(attn_lds) + wave * (32 * kAttnD);
+    T* stage = reinterpret_cast<T*>(attn_lds) + wave * (32 * kAttnD);
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
-        bf16x4_t o4;
+        typename E::x4 o4;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o4[e] = static_cast<bf16_t>(oacc[db][4 * rq + e] * inv_l);
-        *reinterpret_cast<bf16x4_t*>(stage + li * kAttnD + 8 * ((4 * db + rq) ^ (li & 15)) + 4 * g) = o4;
+        for (int e = 0; e < 4; ++e) o4[e] = static_cast<T>(oacc[db][4 * rq + e] * inv_l);
+        *reinterpret_cast<typename E::x4*>(stage + li * kAttnD + 8 * ((4 * db + rq) ^ (li & 15)) + 4 * g) = o4;
       }
-    bf16_t* __restrict__ oblk = O + head_off + static_cast<size_t>(q0 + sub * 32) * kAttnD;
+    T* __restrict__ oblk = O + head_off + static_cast<size_t>(q0 + sub * 32) * kAttnD;
     const int c16 = lane & 15;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int row = 4 * j + (lane >> 4);
       const u32x4_t v16 = *reinterpret_cast<const u32x4_t*>(stage + row * kAttnD + 8 * (c16 ^ (row & 15)));
-      *reinterpret_cast<u32x4_t*>(oblk + row * kAttnD + 8 * c16) = v16;
+      if (!RAGGED || q0 + sub * 32 + row < Sq) *reinterpret_cast<u32x4_t*>(oblk + row * kAttnD + 8 * c16) = v16;
     }
   }
-  if (g == 0) {
-    const size_t so = (static_cast<size_t>(head) * S + qi) * 8;
+  if (g == 0 && (!RAGGED || qi < Sq)) {
+    const size_t so = (static_cast<size_t>(head) * Sq + qi) * 8;
     const float m_nat = m_true * 0.69314718055994530942f;
     Vec<float, 4> mv, lv;
 #pragma unroll

@@ -118,14 +118,14 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
     real_scale = 1.0 / scale
     causal = _is_causal(query.size(2), atten_mask, pre_tockens, next_tockens, sparse_mode)
     seed = numels = 0
-    if (keep_prob == 1.0 and query.dtype == torch.bfloat16 and query.size(3) == 128 and query.size(2) % 128 == 0
-            and query.size(2) > 0):
+    if (keep_prob == 1.0 and query.dtype in (torch.bfloat16, torch.float16) and query.size(3) == 128
+            and query.size(2) > 0 and key.size(2) > 0 and (not causal or query.size(2) == key.size(2))):
+        # the MFMA kernel: bf16 or fp16, head dimension 128, any sequence lengths
         out, smax, ssum = kernels.fused_attention(
             query.contiguous(), key.contiguous(), value.contiguous(), real_scale, causal
         )
     else:
-        # shapes and element types outside the fused kernels, and dropout: the same mathematics over
-        # library GEMMs.  The dropout seed comes from torch's CPU generator (torch.manual_seed makes a
+        # other head dimensions, fp32 and dropout: the same mathematics over library GEMMs.  The dropout seed comes from torch's CPU generator (torch.manual_seed makes a
         # run repeatable) and travels to the backward in the op's seed output, as in the reference's op.
         from .attention_backward import attention_forward_over_gemms
 

@@ -577,142 +577,78 @@ def ring_forward_update(
 
 
 # ---------------------------------------------------------------------------
-# graph 5: fused attention forward (bf16, head dim 128)
+# graph 5: fused attention forward (bf16 / fp16, head dim 128)
 # ---------------------------------------------------------------------------
-_ATTN_LDS_BYTES = 2 * (64 * 136 + 128 * 64) * 2  # two K + V^T tiles
+_ATTN_DTYPES = {torch.bfloat16: "bf16", torch.float16: "f16"}
+_ATTN_LDS_BYTES = 4 * 64 * 128 * 2  # two K and two V tiles of [64, 128] 16-bit elements
+_ATTN_BLOCK_QUERIES = 256
 
 
 @functools.lru_cache(maxsize=None)
 def _attention_launcher() -> CachingLauncher:
     cfgs = [
         LaunchConfig(
-            f"fused_attention_fwd_bf16_d128_{'causal' if c else 'full'}_w{w}",
-            64 * w,
-            meta={"CAUSAL": c, "WAVES": w},
-            lds_bytes=_ATTN_LDS_BYTES,
-        )
-        for c in (1, 0)
-        for w in (4, 8)
-    ] + [
-        LaunchConfig(
-            f"fused_attention_fwd_bf16_d128_{'causal' if c else 'full'}_pp",
+            f"fused_attention_fwd_{t}_d128_{'causal' if c else 'full'}_v5{'_ragged' if r else ''}",
             512,
-            meta={"CAUSAL": c, "WAVES": 8, "PINGPONG": 1},
+            meta={"DTYPE": t, "CAUSAL": c, "RAGGED": r, "WAVES": 8},
             lds_bytes=_ATTN_LDS_BYTES,
         )
+        for t in ("bf16", "f16")
         for c in (1, 0)
-    ] + [
-        LaunchConfig(
-            f"fused_attention_fwd_bf16_d128_{'causal' if c else 'full'}_v2",
-            256,
-            meta={"CAUSAL": c, "WAVES": 4, "QUERIES_PER_WAVE": 64},
-            lds_bytes=_ATTN_LDS_BYTES,
-        )
-        for c in (1, 0)
-    ] + [
-        LaunchConfig(
-            f"fused_attention_fwd_bf16_d128_{'causal' if c else 'full'}_v4",
-            512,
-            meta={"CAUSAL": c, "WAVES": 8, "INTERLEAVED": 1},
-            lds_bytes=_ATTN_LDS_BYTES,
-        )
-        for c in (1, 0)
-    ] + [
-        LaunchConfig(
-            f"fused_attention_fwd_bf16_d128_{'causal' if c else 'full'}_v5",
-            512,
-            meta={"CAUSAL": c, "WAVES": 8, "INTERLEAVED": 1, "DIRECT_LDS": 1},
-            lds_bytes=4 * 64 * 128 * 2,  # two K and two V tiles of [64, 128] bf16
-        )
-        for c in (1, 0)
-    ] + [
-        LaunchConfig(
-            f"fused_attention_fwd_bf16_d128_{'causal' if c else 'full'}_v5h",
-            256,
-            meta={"CAUSAL": c, "WAVES": 4, "INTERLEAVED": 1, "DIRECT_LDS": 1, "WORKGROUPS_PER_CU": 2},
-            lds_bytes=4 * 64 * 128 * 2,
-        )
-        for c in (1, 0)
+        for r in (0, 1)
     ]
     return CachingLauncher(
-        "fused_attention_fwd_bf16_d128",
+        "fused_attention_fwd_d128",
         codecache.aot_source("attention_kernels.hip"),
-        "PPPPPPiif",
+        "PPPPPPiiif",
         cfgs,
         prefer_intree=True,
     )
 
 
 def fused_attention(
-    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool, waves: Optional[int] = None,
-    pingpong: Optional[bool] = None, variant: Optional[str] = None,
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """softmax(q k^T * scale [+ causal mask]) v for [B, N, S, 128] bf16 tensors.
+    """softmax(q k^T * scale [+ causal mask]) v for q [B, N, Sq, 128] and k, v [B, N, Sk, 128], bf16
+    or fp16, any positive sequence lengths (a causal mask needs Sq == Sk).
 
-    Returns (out bf16 [B,N,S,128], softmax_max fp32 [B,N,S,8], softmax_sum fp32
-    [B,N,S,8]); the statistics are the row maximum of the scaled scores and the
-    row sum of exp(score - max), each repeated over the trailing axis."""
+    Returns (out [B,N,Sq,128] in the input type, softmax_max fp32 [B,N,Sq,8], softmax_sum fp32
+    [B,N,Sq,8]); the statistics are the row maximum of the scaled scores and the row sum of
+    exp(score - max), each repeated over the trailing axis.  Lengths that are multiples of 256
+    (queries) and 128 (keys) run the kernel without bounds handling, all others the instantiation
+    that masks the ragged end."""
     _check_cuda(q, k, v)
-    _require(q.dtype == k.dtype == v.dtype == torch.bfloat16, "q, k, v must be bf16")
-    _require(q.dim() == 4 and q.shape == k.shape == v.shape, "q, k, v must share a [B, N, S, D] shape")
-    B, N, S, D = q.shape
+    _require(q.dtype == k.dtype == v.dtype and q.dtype in _ATTN_DTYPES, "q, k, v must share bf16 or fp16")
+    _require(q.dim() == 4 and k.dim() == 4 and k.shape == v.shape, "q [B, N, Sq, D]; k and v one [B, N, Sk, D] shape")
+    B, N, Sq, D = q.shape
+    Sk = k.shape[2]
+    _require(k.shape[0] == B and k.shape[1] == N and k.shape[3] == D, "q, k, v must share batch, heads and head dimension")
     _require(D == 128, "head dimension must be 128")
-    _require(S % 128 == 0 and S > 0, "sequence length must be a positive multiple of 128")
+    _require(Sq > 0 and Sk > 0, "sequence lengths must be positive")
+    _require(not causal or Sq == Sk, "a causal mask needs equal query and key lengths")
     _require(q.is_contiguous() and k.is_contiguous() and v.is_contiguous(), "q, k, v must be contiguous (BNSD)")
     _require(all(_aligned(t) for t in (q, k, v)), "q, k, v must be 16-byte aligned")
     _require(scale > 0 and math.isfinite(scale), "scale must be positive and finite")
-    _require(B * N * S * D < 2**31, "numel must fit int32 indexing")
+    _require(B * N * max(Sq, Sk) * D < 2**31, "numel must fit int32 indexing")
     out = torch.empty_like(q)
-    smax = torch.empty((B, N, S, 8), dtype=torch.float32, device=q.device)
-    ssum = torch.empty((B, N, S, 8), dtype=torch.float32, device=q.device)
-    if B * N == 0:
-        return out, smax, ssum
-    if variant is None and waves is None and pingpong is None:
-        variant = _ATTN_DEFAULT_VARIANT if S % 256 == 0 else None
-    if variant in ("v2", "v4", "v5", "v5h"):
-        # 256 queries per workgroup (4 wavefronts of 64 or 8 of 32; v5h: 128 queries, 4 wavefronts of 32),
-        # causal query blocks paired
-        bm = 128 if variant == "v5h" else 256
-        _require(S % 256 == 0, "the interleaved kernels need S to be a multiple of 256")
-        l = _attention_launcher()
-        i = _find(l, f"fused_attention_fwd_bf16_d128_{'causal' if causal else 'full'}_{variant}")
-        heads = B * N
-        n_qb = S // bm
-        per_head = (n_qb + 1) // 2 if causal else n_qb
-        items = 8 * cdiv(heads, 8) * per_head
-        if variant in ("v5", "v5h"):
-            # persistent launch: at most one workgroup per CU slot, a multiple of 8 (one per die in turn);
-            # every workgroup walks items blockIdx.x, blockIdx.x + gridDim.x, ...
-            slots = config.hardware().cu_count * (2 if variant == "v5h" else 1)
-            grid = min(items, max(slots // 8, 1) * 8)
-        else:
-            grid = items
-        l._launch(
-            i,
-            (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), smax.data_ptr(), ssum.data_ptr(), heads, S,
-             float(scale) * 1.4426950408889634),
-            (grid, 1, 1),
-            _stream(),
-        )
-        return out, smax, ssum
-    _require(variant is None, "variant must be None, 'v2', 'v4', 'v5' or 'v5h'")
-    if waves is None:
-        waves = _ATTN_DEFAULT_WAVES if S % 256 == 0 else 4
-    _require(waves in (4, 8) and S % (32 * waves) == 0, "waves must be 4 or 8 and 32*waves must divide S")
-    if pingpong is None:
-        pingpong = _ATTN_DEFAULT_PINGPONG and waves == 8
-    _require(not pingpong or waves == 8, "the ping-pong schedule needs 8 wavefronts per workgroup")
-    l = _attention_launcher()
-    suffix = "pp" if pingpong else f"w{waves}"
-    i = _find(l, f"fused_attention_fwd_bf16_d128_{'causal' if causal else 'full'}_{suffix}")
+    smax = torch.empty((B, N, Sq, 8), dtype=torch.float32, device=q.device)
+    ssum = torch.empty((B, N, Sq, 8), dtype=torch.float32, device=q.device)
     heads = B * N
-    n_qb = S // (32 * waves)
-    # the causal ping-pong kernel pairs query blocks (b, n_qb - 1 - b) in one workgroup
-    per_head = (n_qb + 1) // 2 if (pingpong and causal) else n_qb
-    grid = 8 * cdiv(heads, 8) * per_head
+    if heads == 0:
+        return out, smax, ssum
+    ragged = Sq % _ATTN_BLOCK_QUERIES != 0 or Sk % 128 != 0
+    l = _attention_launcher()
+    i = _find(l, f"fused_attention_fwd_{_ATTN_DTYPES[q.dtype]}_d128_{'causal' if causal else 'full'}_v5"
+                 f"{'_ragged' if ragged else ''}")
+    n_qb = cdiv(Sq, _ATTN_BLOCK_QUERIES)
+    per_head = (n_qb + 1) // 2 if causal else n_qb  # causal: query blocks (b, n - 1 - b) are one work item
+    items = 8 * cdiv(heads, 8) * per_head
+    # persistent launch: at most one workgroup per CU, a multiple of 8 (one per die in turn); every
+    # workgroup walks items blockIdx.x, blockIdx.x + gridDim.x, ...
+    grid = min(items, max(config.hardware().cu_count // 8, 1) * 8)
     l._launch(
         i,
-        (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), smax.data_ptr(), ssum.data_ptr(), heads, S,
+        (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), smax.data_ptr(), ssum.data_ptr(), heads, Sq, Sk,
          float(scale) * 1.4426950408889634),
         (grid, 1, 1),
         _stream(),
@@ -723,8 +659,6 @@ def fused_attention(
 # ---------------------------------------------------------------------------
 # fused attention backward (bf16, head dim 128): row statistics, then dQ, dK and dV kernels
 # ---------------------------------------------------------------------------
-_ATTN_BWD_DQ_LDS = 2 * (2 * 64 * 136 + 128 * 64) * 2
-_ATTN_BWD_DKV_LDS = 2 * ((2 * 64 * 136 + 2 * 128 * 64) * 2 + 3 * 64 * 4)
 _ATTN_BWD8_DQ_LDS = 2 * (2 * 64 * 136 + 128 * 64) * 2
 _ATTN_BWD8_DK_LDS = 2 * ((2 * 64 * 136 + 128 * 64) * 2 + 64 * 2 * 4)
 _ATTN_BWD8_DV_LDS = 2 * ((64 * 136 + 128 * 64) * 2 + 64 * 2 * 4)
@@ -735,17 +669,6 @@ def _attention_bwd_launchers() -> dict:
     src = codecache.aot_source("attention_bwd_kernels.hip")
     mk = lambda name, sig, cfgs: CachingLauncher(name, src, sig, cfgs, prefer_intree=True)  # noqa: E731
     return {
-        "delta": mk("attention_bwd_delta_bf16_d128", "PPPi", [LaunchConfig("attention_bwd_delta_bf16_d128", 256)]),
-        "dq": mk(
-            "attention_bwd_dq_bf16_d128", "PPPPPPPPiif",
-            [LaunchConfig(f"attention_bwd_dq_bf16_d128_{c}", 256, meta={"CAUSAL": c == "causal"},
-                          lds_bytes=_ATTN_BWD_DQ_LDS) for c in ("causal", "full")],
-        ),
-        "dkv": mk(
-            "attention_bwd_dkv_bf16_d128", "PPPPPPPPPiif",
-            [LaunchConfig(f"attention_bwd_dkv_bf16_d128_{c}", 256, meta={"CAUSAL": c == "causal"},
-                          lds_bytes=_ATTN_BWD_DKV_LDS) for c in ("causal", "full")],
-        ),
         "stats": mk("attention_bwd_stats_bf16_d128", "PPPPPi", [LaunchConfig("attention_bwd_stats_bf16_d128", 256)]),
         **{
             which: mk(
@@ -760,22 +683,18 @@ def _attention_bwd_launchers() -> dict:
 
 def fused_attention_backward(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, dout: torch.Tensor,
-    softmax_max: torch.Tensor, softmax_sum: torch.Tensor, scale: float, causal: bool, variant: Optional[str] = None,
+    softmax_max: torch.Tensor, softmax_sum: torch.Tensor, scale: float, causal: bool,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients (dq, dk, dv) of fused_attention for [B, N, S, 128] bf16 tensors; softmax_max /
-    softmax_sum are the forward's [B, N, S, 8] fp32 statistics.  variant "w8" (default): workgroups
-    of eight wavefronts on 256 rows, separate dK and dV kernels, S a multiple of 64; "w4": four
-    wavefronts on 128 rows, dK and dV in one kernel, S a multiple of 128."""
+    softmax_sum are the forward's [B, N, S, 8] fp32 statistics.  Workgroups of eight wavefronts on
+    256 rows, a statistics pass and separate dQ, dK and dV kernels; S a positive multiple of 64."""
     _check_cuda(q, k, v, out, dout, softmax_max, softmax_sum)
     for t in (q, k, v, out, dout):
         _require(t.dtype == torch.bfloat16 and t.dim() == 4 and t.shape == q.shape, "q, k, v, out, dout: one [B, N, S, D] bf16 shape")
         _require(t.is_contiguous() and _aligned(t), "q, k, v, out, dout must be contiguous and 16-byte aligned")
     B, N, S, D = q.shape
     _require(D == 128, "head dimension must be 128")
-    variant = variant or "w8"
-    _require(variant in ("w8", "w4"), "variant must be 'w8' or 'w4'")
-    step = 64 if variant == "w8" else 128
-    _require(S % step == 0 and S > 0, f"sequence length must be a positive multiple of {step}")
+    _require(S % 64 == 0 and S > 0, "sequence length must be a positive multiple of 64")
     for t in (softmax_max, softmax_sum):
         _require(t.dtype == torch.float32 and t.shape == (B, N, S, 8) and t.is_contiguous(), "statistics must be contiguous fp32 [B, N, S, 8]")
     _require(scale > 0 and math.isfinite(scale), "scale must be positive and finite")
@@ -787,43 +706,19 @@ def fused_attention_backward(
     ls = _attention_bwd_launchers()
     st = _stream()
     which = "causal" if causal else "full"
-    if variant == "w8":
-        stats = torch.empty(heads * S, 2, dtype=torch.float32, device=q.device)
-        ls["stats"]._launch(
-            _find(ls["stats"], "attention_bwd_stats_bf16_d128"),
-            (out.data_ptr(), dout.data_ptr(), softmax_max.data_ptr(), softmax_sum.data_ptr(), stats.data_ptr(), heads * S),
-            (cdiv(heads * S * 16, 256), 1, 1), st,
+    stats = torch.empty(heads * S, 2, dtype=torch.float32, device=q.device)
+    ls["stats"]._launch(
+        _find(ls["stats"], "attention_bwd_stats_bf16_d128"),
+        (out.data_ptr(), dout.data_ptr(), softmax_max.data_ptr(), softmax_sum.data_ptr(), stats.data_ptr(), heads * S),
+        (cdiv(heads * S * 16, 256), 1, 1), st,
+    )
+    blocks = cdiv(S, 256)
+    grid = (8 * cdiv(heads, 8) * (cdiv(blocks, 2) if causal else blocks), 1, 1)  # causal: pairs of blocks
+    for name, dst in (("dk8", dk), ("dv8", dv), ("dq8", dq)):
+        l = ls[name]
+        l._launch(
+            _find(l, f"attention_bwd8_{name[:2]}_bf16_d128_{which}"),
+            (q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), stats.data_ptr(), dst.data_ptr(), heads, S, float(scale)),
+            grid, st,
         )
-        blocks = cdiv(S, 256)
-        grid = (8 * cdiv(heads, 8) * (cdiv(blocks, 2) if causal else blocks), 1, 1)  # causal: pairs of blocks
-        for name, dst in (("dk8", dk), ("dv8", dv), ("dq8", dq)):
-            l = ls[name]
-            l._launch(
-                _find(l, f"attention_bwd8_{name[:2]}_bf16_d128_{which}"),
-                (q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), stats.data_ptr(), dst.data_ptr(), heads, S, float(scale)),
-                grid, st,
-            )
-        return dq, dk, dv
-    delta = torch.empty(heads * S, dtype=torch.float32, device=q.device)
-    ls["delta"]._launch(_find(ls["delta"], "attention_bwd_delta_bf16_d128"), (out.data_ptr(), dout.data_ptr(), delta.data_ptr(), heads * S), (cdiv(heads * S * 16, 256), 1, 1), st)
-    grid = (8 * cdiv(heads, 8) * (S // 128), 1, 1)
-    ldq, ldkv = ls["dq"], ls["dkv"]
-    ldkv._launch(
-        _find(ldkv, f"attention_bwd_dkv_bf16_d128_{which}"),
-        (q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), softmax_max.data_ptr(), softmax_sum.data_ptr(),
-         delta.data_ptr(), dk.data_ptr(), dv.data_ptr(), heads, S, float(scale)),
-        grid, st,
-    )
-    ldq._launch(
-        _find(ldq, f"attention_bwd_dq_bf16_d128_{which}"),
-        (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(), softmax_max.data_ptr(),
-         softmax_sum.data_ptr(), dq.data_ptr(), heads, S, float(scale)),
-        grid, st,
-    )
     return dq, dk, dv
-
-
-_ATTN_DEFAULT_WAVES = 8
-_ATTN_DEFAULT_PINGPONG = True
-# the interleaved 8-wavefront kernel with direct global -> LDS tile loads whenever S % 256 == 0
-_ATTN_DEFAULT_VARIANT = "v5"

@@ -1,6 +1,6 @@
-"""Fused attention (bf16 MFMA kernel) against the CPU oracle and against the
+"""Fused attention (bf16 / fp16 MFMA kernel) against the CPU oracle and against the
 closed-form properties of softmax attention.  Tolerance: 2e-2 absolute on the
-bf16 output; the fp32 statistics to 1e-3 relative (they depend only on q, k).
+16-bit output; the fp32 statistics to 1e-3 relative (they depend only on q, k).
 """
 import numpy as np
 import pytest
@@ -26,33 +26,17 @@ def O():
     return oracle
 
 
-@pytest.mark.parametrize(
-    "B,N,S,causal,waves",
-    [
-        (1, 1, 128, True, 4),
-        (1, 2, 256, True, 4),
-        (1, 2, 256, True, 8),
-        (2, 3, 384, True, 4),
-        (1, 2, 256, False, 4),
-        (1, 9, 128, False, 4),
-        (1, 1, 512, True, 8),
-        (1, 3, 512, False, 8),
-    ],
-)
-def test_attention_vs_oracle(K, O, B, N, S, causal, waves):
-    announce(f"attention B={B} N={N} S={S} causal={causal} waves={waves}")
-    torch.manual_seed(0)
-    q, k, v = (torch.randn(B, N, S, 128).bfloat16() for _ in range(3))
-    scale = 128 ** -0.5
-    out, smax, ssum = K.fused_attention(q.to(DEV), k.to(DEV), v.to(DEV), scale, causal, waves=waves)
-    o_ref, m_ref, l_ref = O.attention_bf16(bits(q), bits(k), bits(v), scale, causal)
-    err = np.abs(O.bf16_bits_to_f32(bits(out)) - O.bf16_bits_to_f32(o_ref)).max()
+def _check_against_oracle(K, O, q, k, v, scale, causal):
+    """q, k, v: CPU tensors whose values bf16 represents exactly (the oracle reads bf16 bits)."""
+    out, smax, ssum = K.fused_attention(q.to(DEV), k.to(DEV), v.to(DEV), scale, causal)
+    o_ref, m_ref, l_ref = O.attention_bf16(bits(q.bfloat16()), bits(k.bfloat16()), bits(v.bfloat16()), scale, causal)
+    assert out.dtype == q.dtype and out.shape == q.shape
+    err = np.abs(out.float().cpu().numpy() - O.bf16_bits_to_f32(o_ref)).max()
     assert err <= 2e-2, err
     np.testing.assert_allclose(smax.cpu().numpy(), m_ref, rtol=1e-3, atol=1e-3)
     np.testing.assert_allclose(ssum.cpu().numpy(), l_ref, rtol=2e-3)
 
 
-@pytest.mark.parametrize("variant", ["v5", "v5h", "v4", "v2"])
 @pytest.mark.parametrize(
     "B,N,S,causal,qmul",
     [
@@ -63,48 +47,64 @@ def test_attention_vs_oracle(K, O, B, N, S, causal, waves):
         (1, 2, 768, True, 1.0),  # odd number of query blocks: the middle one has no partner
         (1, 2, 1024, True, 8.0),  # large scores: the reference maximum moves more than once
         (1, 2, 512, False, 8.0),
+        (1, 20, 1280, True, 1.0),  # more work items than one pass of a small grid: the persistent walk
     ],
 )
-def test_attention_interleaved_kernels_vs_oracle(K, O, B, N, S, causal, qmul, variant):
-    """The kernels that interleave MFMAs and softmax within a wavefront (v4: 8 wavefronts of
-    32 queries, the default; v2: 4 wavefronts of 64 queries with inline-assembly MFMAs),
-    both with a lazily updated reference maximum, against the oracle."""
-    announce(f"attention {variant} B={B} N={N} S={S} causal={causal} qmul={qmul}")
+def test_attention_vs_oracle(K, O, B, N, S, causal, qmul):
+    """Lengths that are multiples of 256: the instantiations without bounds handling."""
+    announce(f"attention B={B} N={N} S={S} causal={causal} qmul={qmul}")
     torch.manual_seed(3)
     q, k, v = (torch.randn(B, N, S, 128).bfloat16() for _ in range(3))
     q = (q.float() * qmul).bfloat16()
-    scale = 128 ** -0.5
-    out, smax, ssum = K.fused_attention(q.to(DEV), k.to(DEV), v.to(DEV), scale, causal, variant=variant)
-    o_ref, m_ref, l_ref = O.attention_bf16(bits(q), bits(k), bits(v), scale, causal)
-    err = np.abs(O.bf16_bits_to_f32(bits(out)) - O.bf16_bits_to_f32(o_ref)).max()
-    assert err <= 2e-2, err
-    np.testing.assert_allclose(smax.cpu().numpy(), m_ref, rtol=1e-3, atol=1e-3)
-    np.testing.assert_allclose(ssum.cpu().numpy(), l_ref, rtol=2e-3)
+    _check_against_oracle(K, O, q, k, v, 128 ** -0.5, causal)
 
 
-@pytest.mark.parametrize("variant", ["v5", "v4", "v2"])
-def test_attention_interleaved_kernels_full_length(K, variant):
-    """S = 4096: statistics equal to the phase-separated kernel's to fp32 rounding, outputs
-    within bf16 rounding of it, causal output independent of later keys."""
-    announce(f"attention {variant} S=4096")
-    torch.manual_seed(4)
-    B, N, S = 1, 3, 4096
-    q, k, v = (torch.randn(B, N, S, 128, device=DEV).bfloat16() for _ in range(3))
-    scale = 128 ** -0.5
-    for causal in (True, False):
-        o1, m1, l1 = K.fused_attention(q, k, v, scale, causal, waves=8, pingpong=True)
-        o2, m2, l2 = K.fused_attention(q, k, v, scale, causal, variant=variant)
-        assert (o1.float() - o2.float()).abs().max().item() <= 1.6e-2
-        assert torch.equal(m1, m2)
-        assert torch.allclose(l1, l2, rtol=1e-5)
-    k2, v2 = k.clone(), v.clone()
-    k2[:, :, 2048:] = torch.randn_like(k2[:, :, 2048:])
-    v2[:, :, 2048:] = torch.randn_like(v2[:, :, 2048:])
-    oa, _, _ = K.fused_attention(q, k, v, scale, True, variant=variant)
-    ob, _, _ = K.fused_attention(q, k2, v2, scale, True, variant=variant)
-    assert torch.equal(oa[:, :, :2048], ob[:, :, :2048])
-    with pytest.raises(ValueError):
-        K.fused_attention(q[:, :, :128], k[:, :, :128], v[:, :, :128], scale, True, variant=variant)
+@pytest.mark.parametrize(
+    "B,N,Sq,Sk,causal",
+    [
+        (1, 1, 128, 128, True),
+        (1, 9, 128, 128, False),
+        (2, 3, 384, 384, True),
+        (1, 2, 1, 1, True),
+        (1, 2, 1, 1, False),
+        (1, 2, 63, 63, True),
+        (1, 2, 64, 64, False),
+        (1, 3, 65, 65, True),
+        (1, 2, 100, 100, False),
+        (1, 2, 257, 257, True),  # a second query block with one row
+        (1, 2, 300, 300, True),
+        (1, 2, 300, 300, False),
+        (1, 2, 1000, 1000, True),
+        (1, 2, 1000, 1000, False),
+        (1, 2, 100, 333, False),  # queries and keys of different lengths
+        (1, 2, 512, 128, False),  # ... both aligned
+        (1, 2, 256, 64, False),
+        (1, 3, 700, 50, False),
+        (1, 2, 30, 1100, False),
+    ],
+)
+def test_attention_ragged_lengths_vs_oracle(K, O, B, N, Sq, Sk, causal):
+    """Any sequence lengths (the reference's fused op takes them as they come, reference
+    inductor_x/npu_fusion_attention_graph.py:20-35): partly filled last key tile, partly filled last
+    query block, query and key lengths that differ."""
+    announce(f"attention B={B} N={N} Sq={Sq} Sk={Sk} causal={causal}")
+    torch.manual_seed(7)
+    q = torch.randn(B, N, Sq, 128).bfloat16()
+    k, v = (torch.randn(B, N, Sk, 128).bfloat16() for _ in range(2))
+    _check_against_oracle(K, O, q, k, v, 128 ** -0.5, causal)
+
+
+@pytest.mark.parametrize("B,N,Sq,Sk,causal", [(1, 2, 256, 256, True), (1, 3, 512, 512, False), (1, 2, 333, 333, True),
+                                              (1, 2, 100, 200, False), (2, 2, 1024, 1024, True)])
+def test_attention_fp16_vs_oracle(K, O, B, N, Sq, Sk, causal):
+    """fp16 operands.  Inputs are multiples of 1/64 below 4 in magnitude, which both 16-bit formats
+    represent exactly, so the bf16 oracle sees the same numbers."""
+    announce(f"attention fp16 B={B} N={N} Sq={Sq} Sk={Sk} causal={causal}")
+    torch.manual_seed(11)
+    grid = lambda *shape: (torch.randint(-255, 256, shape).float() / 64).half()  # noqa: E731
+    q, k, v = grid(B, N, Sq, 128), grid(B, N, Sk, 128), grid(B, N, Sk, 128)
+    assert torch.equal(q.float(), q.float().bfloat16().float())
+    _check_against_oracle(K, O, q, k, v, 128 ** -0.5, causal)
 
 
 def test_attention_closed_forms(K):
@@ -129,59 +129,60 @@ def test_attention_closed_forms(K):
     assert (out.float() - mean).abs().max().item() <= 2e-2
     n = torch.arange(1, S + 1, device=DEV, dtype=torch.float32).view(1, 1, S, 1).expand(B, N, S, 8)
     assert torch.allclose(ssum, n, rtol=1e-5)
+    # a ragged length leaves what lies behind the last row untouched
+    S = 200
+    big = torch.full((B, N, S + 56, 128), 7.0, device=DEV).bfloat16()
+    out, _, _ = K.fused_attention(q[:, :, :S].contiguous(), k[:, :, :S].contiguous(), ones[:, :, :S].contiguous(), 0.1, False)
+    assert out.shape == (B, N, S, 128) and (out.float() - 1).abs().max().item() <= 8e-3
+    assert (big == 7.0).all()
 
 
 def test_attention_causality_and_sdpa_full_size_slice(K):
-    """Causal output must not depend on later keys/values; and one head at the
-    BASELINE sequence length matches PyTorch's math-backend attention on the GPU."""
+    """Causal output must not depend on later keys/values; and two heads at the
+    BASELINE sequence length match the fp32 definition evaluated on the GPU."""
     announce("attention causality / S=4096")
     torch.manual_seed(2)
     B, N, S = 1, 2, 4096
     q, k, v = (torch.randn(B, N, S, 128, device=DEV).bfloat16() for _ in range(3))
     scale = 128 ** -0.5
-    out, smax, ssum = K.fused_attention(q, k, v, scale, True, waves=4)
-    out8, smax8, ssum8 = K.fused_attention(q, k, v, scale, True, waves=8, pingpong=False)
-    assert torch.equal(out, out8) and torch.equal(smax, smax8) and torch.equal(ssum, ssum8)
-    outp, smaxp, ssump = K.fused_attention(q, k, v, scale, True, waves=8, pingpong=True)
-    assert torch.equal(out, outp) and torch.equal(smax, smaxp) and torch.equal(ssum, ssump)
-    # the default at this length is the interleaved 8-wavefront kernel
-    outd, smaxd, ssumd = K.fused_attention(q, k, v, scale, True)
-    outv, smaxv, ssumv = K.fused_attention(q, k, v, scale, True, variant="v5")
-    assert torch.equal(outd, outv) and torch.equal(smaxd, smaxv) and torch.equal(ssumd, ssumv)
-    # the direct-to-LDS kernel computes what the register-staged one does, bit for bit
-    out4, smax4, ssum4 = K.fused_attention(q, k, v, scale, True, variant="v4")
-    assert torch.equal(outd, out4) and torch.equal(smaxd, smax4) and torch.equal(ssumd, ssum4)
-    # and so does the four-wavefront form of it that runs two workgroups per CU
-    outh, smaxh, ssumh = K.fused_attention(q, k, v, scale, True, variant="v5h")
-    assert torch.equal(outd, outh) and torch.equal(smaxd, smaxh) and torch.equal(ssumd, ssumh)
-    out, smax, ssum = outd, smaxd, ssumd
-    for causal in (False,):
-        a = K.fused_attention(q, k, v, scale, causal, waves=4)
-        b = K.fused_attention(q, k, v, scale, causal, waves=8, pingpong=True)
-        assert all(torch.equal(x, y) for x, y in zip(a, b))
+    out, smax, ssum = K.fused_attention(q, k, v, scale, True)
+    again = K.fused_attention(q, k, v, scale, True)
+    assert torch.equal(out, again[0]) and torch.equal(smax, again[1]) and torch.equal(ssum, again[2])
     k2, v2 = k.clone(), v.clone()
     k2[:, :, 2048:] = torch.randn_like(k2[:, :, 2048:])
     v2[:, :, 2048:] = torch.randn_like(v2[:, :, 2048:])
     out2, _, _ = K.fused_attention(q, k2, v2, scale, True)
     assert torch.equal(out[:, :, :2048], out2[:, :, :2048])
     s = (q.float() @ k.float().transpose(-1, -2)) * scale
+    full = torch.softmax(s, -1) @ v.float()
+    outf, smaxf, ssumf = K.fused_attention(q, k, v, scale, False)
+    assert (outf.float() - full).abs().max().item() <= 2e-2
+    assert torch.allclose(smaxf[..., 0], s.max(-1).values, rtol=1e-3, atol=1e-3)
     s = s.masked_fill(torch.ones(S, S, device=DEV, dtype=torch.bool).triu(1), float("-inf"))
     ref = torch.softmax(s, -1) @ v.float()
     assert (out.float() - ref).abs().max().item() <= 2e-2
     assert torch.allclose(smax[..., 0], s.max(-1).values, rtol=1e-3, atol=1e-3)
     assert torch.allclose(ssum[..., 0], torch.exp(s - s.max(-1, keepdim=True).values).sum(-1), rtol=2e-3)
+    # the ragged instantiation on aligned lengths is the same arithmetic: one row fewer changes nothing above it
+    out3, smax3, _ = K.fused_attention(q[:, :, :4095].contiguous(), k[:, :, :4095].contiguous(), v[:, :, :4095].contiguous(), scale, True)
+    assert (out3.float() - out[:, :, :4095].float()).abs().max().item() <= 1.6e-2
+    assert torch.allclose(smax3, smax[:, :, :4095], rtol=1e-6)
 
 
 def test_attention_rejects_bad_operands(K):
     q = torch.randn(1, 1, 128, 64, device=DEV).bfloat16()
     with pytest.raises(ValueError):
         K.fused_attention(q, q, q, 0.1, True)  # head dim
-    q = torch.randn(1, 1, 100, 128, device=DEV).bfloat16()
-    with pytest.raises(ValueError):
-        K.fused_attention(q, q, q, 0.1, True)  # sequence length
     q = torch.randn(1, 1, 128, 128, device=DEV)
     with pytest.raises(ValueError):
         K.fused_attention(q, q, q, 0.1, True)  # dtype
+    q = torch.randn(1, 1, 128, 128, device=DEV).bfloat16()
+    with pytest.raises(ValueError):
+        K.fused_attention(q, q[:, :, :64].contiguous(), q[:, :, :64].contiguous(), 0.1, True)  # causal with Sq != Sk
+    with pytest.raises(ValueError):
+        K.fused_attention(q, q.half(), q.half(), 0.1, False)  # mixed element types
+    with pytest.raises(ValueError):
+        K.fused_attention(q, q[:, :, :0].contiguous(), q[:, :, :0].contiguous(), 0.1, False)  # no keys
 
 
 @pytest.mark.parametrize("B,N,S,causal", [(1, 2, 256, True), (2, 3, 512, False), (1, 4, 1024, True), (1, 1, 128, True)])
@@ -229,36 +230,34 @@ def test_attention_backward_closed_forms():
     assert q2.grad.float().abs().max().item() <= 2e-2 and k2.grad.float().abs().max().item() <= 2e-2
 
 
-@pytest.mark.parametrize("variant", ["w8", "w4"])
 @pytest.mark.parametrize("B,N,S,causal", [(1, 2, 256, True), (1, 3, 384, False), (1, 3, 384, True), (2, 4, 1024, True),
                                           (1, 9, 128, False), (1, 2, 128, True), (1, 2, 640, True), (1, 5, 1280, False)])
-def test_attention_backward_kernels_vs_gemm_path(K, B, N, S, causal, variant):
-    """The fused backward kernels (both workgroup shapes) against the same gradients computed with
-    library GEMMs from the same saved statistics.  All round P and dS to bf16 once (the
-    eight-wavefront kernels before, the others after the multiplication by `scale`), so they agree
-    to two bf16 ulps of the largest entry.  Sequence lengths include last blocks of 128 rows."""
-    announce(f"attention backward {variant} vs GEMM path B={B} N={N} S={S} causal={causal}")
+def test_attention_backward_kernels_vs_gemm_path(K, B, N, S, causal):
+    """The fused backward kernels against the same gradients computed with library GEMMs from the
+    same saved statistics.  Both round P and dS to bf16 once, so they agree to two bf16 ulps of the
+    largest entry.  Sequence lengths include last blocks of 128 rows."""
+    announce(f"attention backward vs GEMM path B={B} N={N} S={S} causal={causal}")
     from inductor_x_amd import attention_backward as AB
 
     torch.manual_seed(7)
     q, k, v, do = (torch.randn(B, N, S, 128, device=DEV).bfloat16() for _ in range(4))
     scale = 128 ** -0.5
     o, m, l = K.fused_attention(q, k, v, scale, causal)
-    a = K.fused_attention_backward(q, k, v, o, do, m, l, scale, causal, variant=variant)
+    a = K.fused_attention_backward(q, k, v, o, do, m, l, scale, causal)
     b = AB.fused_attention_backward(q, k, v, o, do, m, l, scale, causal, use_kernels=False)
     for x, y in zip(a, b):
         assert (x.float() - y.float()).abs().max().item() <= 8e-3 * max(y.float().abs().max().item(), 1.0)
     with pytest.raises(ValueError):
         K.fused_attention_backward(q[:, :, :32].contiguous(), k[:, :, :32].contiguous(), v[:, :, :32].contiguous(),
                                    o[:, :, :32].contiguous(), do[:, :, :32].contiguous(), m[:, :, :32].contiguous(),
-                                   l[:, :, :32].contiguous(), scale, causal, variant=variant)
+                                   l[:, :, :32].contiguous(), scale, causal)
 
 
 @pytest.mark.parametrize("S,causal", [(64, True), (192, False), (320, True), (576, True)])
 def test_attention_backward_sequence_multiple_of_64(K, S, causal):
-    """The eight-wavefront kernels take any multiple of 64 (the forward kernels do not, so the
-    output and the row statistics come from fp32 torch here): last blocks of 64 and 192 rows."""
-    announce(f"attention backward w8 S={S} causal={causal}")
+    """The backward kernels take any multiple of 64: last blocks of 64 and 192 rows (the output and
+    the row statistics come from fp32 torch here, independent of the forward kernel)."""
+    announce(f"attention backward S={S} causal={causal}")
     from inductor_x_amd import attention_backward as AB
 
     torch.manual_seed(11)
@@ -273,13 +272,10 @@ def test_attention_backward_sequence_multiple_of_64(K, S, causal):
     sm = e.sum(-1, keepdim=True)
     o = ((e / sm) @ v.float()).bfloat16()
     m, l = mx.expand(B, N, S, 8).contiguous(), sm.expand(B, N, S, 8).contiguous()
-    a = K.fused_attention_backward(q, k, v, o, do, m, l, scale, causal, variant="w8")
+    a = K.fused_attention_backward(q, k, v, o, do, m, l, scale, causal)
     b = AB.fused_attention_backward(q, k, v, o, do, m, l, scale, causal, use_kernels=False)
     for x, y in zip(a, b):
         assert (x.float() - y.float()).abs().max().item() <= 8e-3 * max(y.float().abs().max().item(), 1.0)
-    if S % 128:
-        with pytest.raises(ValueError):
-            K.fused_attention_backward(q, k, v, o, do, m, l, scale, causal, variant="w4")
 
 
 def test_attention_backward_full_length_causal_independence(K):
@@ -304,18 +300,17 @@ def test_attention_backward_full_length_causal_independence(K):
         assert (b.float() - 2 * a.float()).abs().max().item() <= 2e-2 * max(b.float().abs().max().item(), 1.0)
 
 
-@pytest.mark.parametrize("variant", ["w8", "w4"])
 @pytest.mark.parametrize("B,N,S,causal", [(1, 2, 128, True), (1, 1, 256, False), (2, 2, 256, True), (1, 1, 384, True)])
-def test_attention_backward_vs_oracle(K, O, B, N, S, causal, variant):
+def test_attention_backward_vs_oracle(K, O, B, N, S, causal):
     """Fused backward kernels against the fp64 oracle on the same bf16 inputs (the kernels take the
     forward kernel's output and statistics).  Bar: 1 % of the largest entry of each gradient."""
-    announce(f"attention backward {variant} vs oracle B={B} N={N} S={S} causal={causal}")
+    announce(f"attention backward vs oracle B={B} N={N} S={S} causal={causal}")
     torch.manual_seed(9)
     q, k, v, do = (torch.randn(B, N, S, 128).bfloat16() for _ in range(4))
     scale = 128 ** -0.5
     qd, kd, vd, dod = (t.to(DEV) for t in (q, k, v, do))
     o, m, l = K.fused_attention(qd, kd, vd, scale, causal)
-    got = K.fused_attention_backward(qd, kd, vd, o, dod, m, l, scale, causal, variant=variant)
+    got = K.fused_attention_backward(qd, kd, vd, o, dod, m, l, scale, causal)
     ref = O.attention_bwd(bits(q), bits(k), bits(v), bits(do), scale, causal)
     for g, r in zip(got, ref):
         assert np.abs(g.float().cpu().numpy() - r).max() <= 1e-2 * np.abs(r).max() + 1e-3
@@ -323,7 +318,7 @@ def test_attention_backward_vs_oracle(K, O, B, N, S, causal, variant):
 
 @pytest.mark.parametrize("dtype,B,N,S,D,causal", [
     (torch.float16, 2, 3, 200, 64, True), (torch.bfloat16, 1, 4, 96, 80, False), (torch.float32, 1, 2, 130, 32, True),
-    (torch.bfloat16, 1, 2, 192, 128, True),  # head dimension 128 but a sequence the forward kernels do not take
+    (torch.bfloat16, 1, 2, 192, 128, True),  # fused forward (ragged instantiation) and fused backward (a multiple of 64)
 ])
 def test_attention_op_outside_the_fused_kernels(dtype, B, N, S, D, causal):
     """npu_fa / npu_fa_backward for shapes and element types the MFMA kernels do not cover run the same
@@ -352,6 +347,48 @@ def test_attention_op_outside_the_fused_kernels(dtype, B, N, S, D, causal):
     for g, r in zip(got, (qf.grad, kf.grad, vf.grad)):
         assert g.dtype == dtype
         assert (g.float() - r).abs().max().item() <= (1e-4 if dtype == torch.float32 else 3e-2) * max(r.abs().max().item(), 1.0)
+
+
+@pytest.mark.parametrize("dtype,B,N,Sq,Sk,causal", [
+    (torch.float16, 1, 3, 200, 200, True), (torch.float16, 2, 2, 512, 512, False), (torch.bfloat16, 1, 2, 100, 300, False),
+    (torch.bfloat16, 1, 2, 77, 77, True),
+])
+def test_attention_op_reaches_the_fused_kernel_for_fp16_and_any_length(dtype, B, N, Sq, Sk, causal):
+    """npu_fa with fp16 operands, with sequence lengths that are no multiple of a tile and with
+    different query and key lengths launches the MFMA kernel (not the GEMM formulation), and the
+    training path still returns gradients where the backward applies (equal lengths)."""
+    announce(f"attention op on the fused kernel {dtype} B={B} N={N} Sq={Sq} Sk={Sk} causal={causal}")
+    from inductor_x_amd import launcher
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
+    torch.manual_seed(13)
+    q = torch.randn(B, N, Sq, 128, device=DEV).to(dtype)
+    k, v = (torch.randn(B, N, Sk, 128, device=DEV).to(dtype) for _ in range(2))
+    train = Sq == Sk
+    if train:
+        q, k, v = (t.requires_grad_() for t in (q, k, v))
+    inv = 128 ** 0.5
+    launcher.launch_log = []
+    try:
+        res = npu_fusion_attention_graph(q, k, v, N, "BNSD", scale=inv, sparse_mode=3 if causal else 0)
+        torch.cuda.synchronize()
+    finally:
+        log, launcher.launch_log = launcher.launch_log, None
+    name = "f16" if dtype == torch.float16 else "bf16"
+    assert any(sym.startswith(f"fused_attention_fwd_{name}_d128_") for sym in log), log
+    qf, kf, vf = (t.detach().float().requires_grad_() for t in (q, k, v))
+    s = (qf @ kf.transpose(-1, -2)) / inv
+    if causal:
+        s = s.masked_fill(torch.ones(Sq, Sk, device=DEV, dtype=torch.bool).triu(1), float("-inf"))
+    ref = torch.softmax(s, -1) @ vf
+    assert res[0].dtype == dtype and (res[0].float() - ref).abs().max().item() <= 2e-2
+    torch.testing.assert_close(res[1][..., 0], s.amax(-1), rtol=1e-3, atol=1e-3)
+    if train:
+        do = torch.randn_like(res[0])
+        res[0].backward(do)
+        ref.backward(do.float())
+        for g, r in zip((q.grad, k.grad, v.grad), (qf.grad, kf.grad, vf.grad)):
+            assert (g.float() - r).abs().max().item() <= 3e-2 * max(r.abs().max().item(), 1.0)
 
 
 def _unfused_fp32(q, k, v, inv, causal, keep=None, keep_prob=1.0):
