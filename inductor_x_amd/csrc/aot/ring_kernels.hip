@@ -1,6 +1,6 @@
 // Ring-attention merge step (forward_update) instantiations: one kernel per element type of the
-// attention outputs, head dimension 128, 16 sequence positions per workgroup; each with plain and
-// with non-temporal loads of the outputs (`_nt`).
+// attention outputs, head dimensions 128 and 64, 8 (or 16) sequence positions per workgroup; each
+// with plain and with non-temporal loads of the outputs (`_nt`).
 #include "../mi/ring.h"
 
 using namespace mi;
@@ -17,35 +17,14 @@ using namespace mi;
 
 RING_FWD_VARIANT(ring_forward_update_bf16_d128_s16, bf16_t, 128, 16, false)
 RING_FWD_VARIANT(ring_forward_update_bf16_d128_s16_nt, bf16_t, 128, 16, true)
-RING_FWD_VARIANT(ring_forward_update_bf16_d128_s32, bf16_t, 128, 32, false)
-RING_FWD_VARIANT(ring_forward_update_bf16_d128_s32_nt, bf16_t, 128, 32, true)
 RING_FWD_VARIANT(ring_forward_update_bf16_d128_s8, bf16_t, 128, 8, false)
 RING_FWD_VARIANT(ring_forward_update_bf16_d128_s8_nt, bf16_t, 128, 8, true)
-RING_FWD_VARIANT(ring_forward_update_f16_d128_s16, f16_t, 128, 16, false)
-RING_FWD_VARIANT(ring_forward_update_f16_d128_s16_nt, f16_t, 128, 16, true)
-RING_FWD_VARIANT(ring_forward_update_f32_d128_s16, float, 128, 16, false)
-RING_FWD_VARIANT(ring_forward_update_f32_d128_s16_nt, float, 128, 16, true)
-RING_FWD_VARIANT(ring_forward_update_bf16_d64_s16, bf16_t, 64, 16, false)
-RING_FWD_VARIANT(ring_forward_update_bf16_d64_s16_nt, bf16_t, 64, 16, true)
-RING_FWD_VARIANT(ring_forward_update_f32_d64_s16, float, 64, 16, false)
-RING_FWD_VARIANT(ring_forward_update_f32_d64_s16_nt, float, 64, 16, true)
+RING_FWD_VARIANT(ring_forward_update_f16_d128_s8, f16_t, 128, 8, false)
+RING_FWD_VARIANT(ring_forward_update_f16_d128_s8_nt, f16_t, 128, 8, true)
+RING_FWD_VARIANT(ring_forward_update_f32_d128_s8, float, 128, 8, false)
+RING_FWD_VARIANT(ring_forward_update_f32_d128_s8_nt, float, 128, 8, true)
+RING_FWD_VARIANT(ring_forward_update_bf16_d64_s8, bf16_t, 64, 8, false)
+RING_FWD_VARIANT(ring_forward_update_bf16_d64_s8_nt, bf16_t, 64, 8, true)
+RING_FWD_VARIANT(ring_forward_update_f32_d64_s8, float, 64, 8, false)
+RING_FWD_VARIANT(ring_forward_update_f32_d64_s8_nt, float, 64, 8, true)
 
-// experiment shapes: rows per batch and whether the first batch is requested before the statistics
-#define RING_FWD_EXP(NAME, ST, BATCH, EARLY)                                                       \
-  extern "C" __global__ __launch_bounds__(256) void NAME(                                          \
-      const bf16_t* prev_out, const float* prev_max, const float* prev_sum, const bf16_t* cur_out, \
-      const float* cur_max, const float* cur_sum, bf16_t* out, float* out_max, float* out_sum,     \
-      int S, int B, int N, long long prev_n_stride, long long cur_n_stride) {                      \
-    ring_forward_update<bf16_t, 128, ST, false, BATCH, EARLY>(prev_out, prev_max, prev_sum,        \
-        cur_out, cur_max, cur_sum, out, out_max, out_sum, S, B, N, prev_n_stride, cur_n_stride);   \
-  }
-RING_FWD_EXP(ring_exp_s8_b4_e0, 8, 4, false)
-RING_FWD_EXP(ring_exp_s8_b4_e1, 8, 4, true)
-RING_FWD_EXP(ring_exp_s8_b8_e0, 8, 8, false)
-RING_FWD_EXP(ring_exp_s8_b8_e1, 8, 8, true)
-RING_FWD_EXP(ring_exp_s16_b4_e0, 16, 4, false)
-RING_FWD_EXP(ring_exp_s16_b4_e1, 16, 4, true)
-RING_FWD_EXP(ring_exp_s16_b8_e0, 16, 8, false)
-RING_FWD_EXP(ring_exp_s16_b8_e1, 16, 8, true)
-RING_FWD_EXP(ring_exp_s4_b4_e0, 4, 4, false)
-RING_FWD_EXP(ring_exp_s4_b4_e1, 4, 4, true)

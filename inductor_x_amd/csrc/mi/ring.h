@@ -28,10 +28,13 @@ __device__ __forceinline__ float ring_max_nan(float a, float b) {
 
 // T: element type of the attention outputs (bf16_t, f16_t or float); D: head dimension;
 // ST: consecutive sequence positions per workgroup.  256 threads; a head's D columns are covered
-// by TPR = D / VEC lanes of 16 bytes, so a workgroup spans NT = 256 / TPR heads.
+// by TPR = D / VEC lanes of 16 bytes, so a workgroup spans NT = 256 / TPR heads.  Measured on MI355X
+// at bf16 [8192, 1, 6144] with 48 heads (377 MB per call, replayed): ST = 8 with all eight rows of a
+// thread in flight 58.3 us, ST = 4 60.0, ST = 16 62.6 (four rows in flight) / 70.1 (eight), ST = 32 74;
+// requesting the first rows before the statistics are read costs 1 - 9 us in every shape.
 // STREAM: loads and stores of the attention outputs carry the non-temporal hint (the caller
 // sets it when the operands are larger than the memory-side cache can hold anyway).
-template <typename T, int D, int ST, bool STREAM, int BATCH_ = 4, bool EARLY = true>
+template <typename T, int D, int ST, bool STREAM>
 __device__ __forceinline__ void ring_forward_update(
     const T* __restrict__ prev_out, const float* __restrict__ prev_max, const float* __restrict__ prev_sum,
     const T* __restrict__ cur_out, const float* __restrict__ cur_max, const float* __restrict__ cur_sum,
@@ -55,7 +58,7 @@ __device__ __forceinline__ void ring_forward_update(
   const int n = n0 + n_l;
   const size_t H = static_cast<size_t>(N) * D;
   const size_t col = static_cast<size_t>(n) * D + static_cast<size_t>(tid % TPR) * VEC;
-  constexpr int BATCH = ST % BATCH_ == 0 ? BATCH_ : 1;
+  constexpr int BATCH = ST % 8 == 0 ? 8 : (ST % 4 == 0 ? 4 : 1);  // rows whose loads are in flight together
   Vec<T, VEC> pv[BATCH], cv[BATCH];
   auto load_rows = [&](int r0) {
 #pragma unroll
@@ -68,8 +71,6 @@ __device__ __forceinline__ void ring_forward_update(
       }
     }
   };
-  // the first rows are requested before the statistics are touched: they do not depend on them
-  if constexpr (EARLY) load_rows(0);
 
   // ---- statistics: one thread per (head, s), s fastest, eight fp32 per array ----
   for (int p = tid; p < PAIRS; p += 256) {
@@ -111,7 +112,7 @@ __device__ __forceinline__ void ring_forward_update(
   if (n >= N) return;
 #pragma unroll
   for (int r0 = 0; r0 < ST; r0 += BATCH) {
-    if (!EARLY || r0 > 0) load_rows(r0);
+    load_rows(r0);
 #pragma unroll
     for (int j = 0; j < BATCH; ++j) {
       const int s = s0 + r0 + j;

@@ -130,7 +130,7 @@ def test_forward_update_single_kernel(O, S, B, H, N, dtype):
     else:
         assert np.abs(got - ref_out).max() <= 2e-2
     # both load forms give the same bits
-    for variant in ((16, False), (16, True)):
+    for variant in ((8, False), (8, True)):
         o2, m2, l2 = kernels.ring_forward_update(dev(prev_out), pm_d, ps_d, dev(cur_out), dev(cur_max), dev(cur_sum), variant=variant)
         assert torch.equal(o2, out) and torch.equal(m2, smax) and torch.equal(l2, ssum)
 
