@@ -60,6 +60,12 @@ MEASURED_TRAFFIC: dict = {
         "profile": "profiles/permute_0213_bf16_16x2048x32x128_pmc.txt"},
 }
 
+# Kernel durations (microseconds, average over the dispatches of a warm run) from the committed
+# rocprofv3 kernel traces of `bench.py --pmc-config <n>`: the benchmark definition's "GPU time" of a
+# graph is the sum over its kernels.  Keyed like MEASURED_TRAFFIC and used under the same rule.
+KERNEL_TRACE_US: dict = {
+}
+
 ALGO_BYTES = {
     "rowsum": 16_781_312,
     "add_rmsnorm": 268_443_648,
@@ -86,6 +92,14 @@ def _event_time_ms(fn, reps: int) -> float:
 
 # input sets visited in turn by the cold rows of all_configs (reads of about 1 GiB per pass)
 COLD_COPIES = {"2": 8, "3": 8, "4a": 8, "4b": 4}
+
+
+def _cold_sets(torch, args, copies: int) -> list:
+    """`copies` input sets for one configuration: the given one plus fresh random copies of its
+    large floating-point operands (small operands and index tensors are shared)."""
+    dev = "cuda:0"
+    return [args] + [tuple(torch.randn(a.shape, device=dev).to(a.dtype) if a.is_floating_point() and a.numel() > (1 << 20)
+                           else a for a in args) for _ in range(copies - 1)]
 
 
 def _graph_time_ms(fn, launches_per_graph: int = 20, replays: int = 5) -> float:
@@ -177,6 +191,7 @@ def _config_table(K, torch, only=None):
         "4b permute(0,2,1,3) bf16 [16,2048,32,128]": c4b,
         "5 causal attention bf16 [4,32,4096,128]": c5,
     }
+    table.update(_ring_merge_table(K, torch))
     if only is not None:
         table = {k: v for k, v in table.items() if k.split()[0] == only}
     return table
@@ -203,6 +218,32 @@ def _traffic_for(config: str, path: str, symbols: list, work):
     total = rec["fetch_bytes"] + rec["write_bytes"]
     return {"bytes": total, "fetch_bytes": rec["fetch_bytes"], "write_bytes": rec["write_bytes"],
             "over_algorithmic": round(total / work, 4), "profile": rec["profile"]}
+
+
+def _kernel_us_for(config: str, path: str, symbols: list):
+    """Sum of the committed kernel-trace durations of a call's kernels, or None when the call no
+    longer launches the symbols that were traced."""
+    rec = KERNEL_TRACE_US.get((config.split()[0], path))
+    if rec is None or list(rec["symbols"]) != list(symbols):
+        return None
+    return round(sum(rec["us"]), 2)
+
+
+def _per_config_summary(rows: list) -> dict:
+    """Compact table of all_configs for the roofline object: configuration -> fraction of the roofline
+    per path (and the traced kernel time where the committed trace covers the launched symbols)."""
+    per: dict = {}
+    for rec in rows:
+        if "frac" not in rec:
+            continue
+        key = rec["config"].split()[0]
+        path = "kernel" if rec["path"] == "kernel" else "compile"
+        e = per.setdefault(key, {})
+        e[path] = rec["frac"]
+        kus = _kernel_us_for(rec["config"], rec["path"], rec.get("kernels", []))
+        if kus is not None:
+            e[path + "_kernel_us"] = kus
+    return per
 
 
 def _all_configs(K, torch) -> list:
@@ -246,7 +287,8 @@ def _all_configs(K, torch) -> list:
         out.append(rec)
 
     def both(name, direct, graph_fn, args, work, bound):
-        add(name, "kernel", lambda: direct(*args), work, bound)
+        if direct is not None:
+            add(name, "kernel", lambda: direct(*args), work, bound)
         try:
             torch._dynamo.reset()
             cf = torch.compile(graph_fn)
@@ -287,8 +329,7 @@ def _all_configs(K, torch) -> list:
             # visited in turn, one pass over all of them per graph replay.  The rows above replay
             # one input set, whose reads the 256 MiB cache can partly serve again.
             copies = COLD_COPIES[name.split()[0]]
-            sets = [args] + [tuple(torch.randn(a.shape, device=dev).to(a.dtype) if a.is_floating_point() and a.numel() > (1 << 20)
-                                   else a for a in args) for _ in range(copies - 1)]
+            sets = _cold_sets(torch, args, copies)
             cname = name.split()[0] + "cold " + name.split(" ", 1)[1] + f" (cold: {copies} input sets in turn)"
             for path, call in (("kernel", direct), ("torch.compile", None)):
                 turn = [0]
@@ -325,14 +366,14 @@ def _all_configs(K, torch) -> list:
                 lambda: K.fused_attention_backward(q, k, v, o, do, m, l, 128 ** -0.5, True), 2.5 * ATTN_FLOPS_CAUSAL, "mfma")
             del o, m, l, do
         del direct, graph_fn, args
-    _ring_merge_configs(torch, add)
     return out
 
 
-def _ring_merge_configs(torch, add) -> None:
+def _ring_merge_table(K, torch) -> dict:
     """The merge steps of ring attention at the reference's shapes (the callers next to the fused
-    attention op on a sequence-parallel path), compiled through the backend; HBM-bound.  Algorithmic
-    bytes: every operand read once, every result written once.  `add` records one measurement."""
+    attention op on a sequence-parallel path); HBM-bound.  Algorithmic bytes: every operand read
+    once, every result written once.  name -> builder of (direct call or None, graph function,
+    arguments, algorithmic bytes, bound), as _config_table."""
     dev = "cuda:0"
 
     def trans(x):
@@ -358,38 +399,33 @@ def _ring_merge_configs(torch, add) -> None:
         dk.add_(cdk.view(dk.shape))
         dv.add_(cdv.view(dv.shape))
 
-    def one(name, fn, args, work):
-        try:
-            torch._dynamo.reset()
-            cf = torch.compile(fn)
-            cf(*args)
-        except Exception as e:
-            add(name, "torch.compile", None, work, "hbm", error=f"{type(e).__name__}: {e}"[:200])
-            return
-        add(name, "torch.compile", lambda: cf(*args), work, "hbm")
+    def f1a():
+        torch.manual_seed(0)
+        DS, B, H, N = 8192, 1, 6144, 48
+        st = lambda off: (torch.rand(B, N, DS, device=dev) + off).unsqueeze(3).repeat(1, 1, 1, 8).contiguous()  # noqa: E731
+        args = (torch.randn(DS, B, H, device=dev).bfloat16(), st(0.0), st(0.5), torch.randn(DS, B, H, device=dev).bfloat16(),
+                st(0.0), st(0.5))
+        return K.ring_forward_update, forward_update, args, 3 * DS * B * H * 2 + 6 * B * N * DS * 8 * 4, "hbm"
 
-    torch.manual_seed(0)
-    DS, B, H, N = 8192, 1, 6144, 48
-    st = lambda off: (torch.rand(B, N, DS, device=dev) + off).unsqueeze(3).repeat(1, 1, 1, 8).contiguous()  # noqa: E731
-    args = (torch.randn(DS, B, H, device=dev).bfloat16(), st(0.0), st(0.5), torch.randn(DS, B, H, device=dev).bfloat16(),
-            st(0.0), st(0.5))
-    from inductor_x_amd import kernels as K
+    def f1b():
+        torch.manual_seed(0)
+        B, N, DS, D = 1, 48, 8192, 128
+        args = (torch.randn(B, N, DS, D, device=dev), torch.rand(B, N, DS, 1, device=dev), torch.randn(B, N, DS, D, device=dev),
+                torch.rand(B, N, DS, 1, device=dev))
+        return None, forward_update_la, args, 3 * B * N * DS * D * 4 + 3 * B * N * DS * 4, "hbm"
 
-    add("f1a ring forward_update bf16 [8192,1,6144] N=48", "kernel", lambda: K.ring_forward_update(*args),
-        3 * DS * B * H * 2 + 6 * B * N * DS * 8 * 4, "hbm")
-    one("f1a ring forward_update bf16 [8192,1,6144] N=48", forward_update, args, 3 * DS * B * H * 2 + 6 * B * N * DS * 8 * 4)
-    del args
-    B, N, DS, D = 1, 48, 8192, 128
-    args = (torch.randn(B, N, DS, D, device=dev), torch.rand(B, N, DS, 1, device=dev), torch.randn(B, N, DS, D, device=dev),
-            torch.rand(B, N, DS, 1, device=dev))
-    one("f1b ring forward_update (log-sum-exp) fp32 [1,48,8192,128]", forward_update_la, args,
-        3 * B * N * DS * D * 4 + 3 * B * N * DS * 4)
-    del args
-    S, B, H = 16384, 1, 1536
-    args = tuple(torch.randn(2, S, B, H, device=dev).bfloat16() for _ in range(3)) + tuple(
-        torch.randn(2 * S, B, H, device=dev).bfloat16() for _ in range(3))
-    one("f1c ring backward_update bf16 3 x [2,16384,1,1536]", backward_update, args, 3 * 3 * 2 * S * B * H * 2)
-    del args
+    def f1c():
+        torch.manual_seed(0)
+        S, B, H = 16384, 1, 1536
+        args = tuple(torch.randn(2, S, B, H, device=dev).bfloat16() for _ in range(3)) + tuple(
+            torch.randn(2 * S, B, H, device=dev).bfloat16() for _ in range(3))
+        return None, backward_update, args, 3 * 3 * 2 * S * B * H * 2, "hbm"
+
+    return {
+        "f1a ring forward_update bf16 [8192,1,6144] N=48": f1a,
+        "f1b ring forward_update (log-sum-exp) fp32 [1,48,8192,128]": f1b,
+        "f1c ring backward_update bf16 3 x [2,16384,1,1536]": f1c,
+    }
 
 
 def _pmc_run(K, torch, which: str, steps: int, warmup: int) -> dict:
@@ -400,25 +436,28 @@ def _pmc_run(K, torch, which: str, steps: int, warmup: int) -> dict:
 
     dev = "cuda:0"
     res = {"pmc_config": which, "steps": steps}
-    cold = which == "1cold"
-    table = _config_table(K, torch, only="1" if cold else which)
-    if not table:
-        raise SystemExit(f"bench.py: no configuration {which!r} (1, 1cold, 2, 3, 4a, 4b, 5)")
+    cold = which.endswith("cold")
+    base = which[:-4] if cold else which
+    table = _config_table(K, torch, only=base)
+    if not table or (cold and base != "1" and base not in COLD_COPIES):
+        raise SystemExit(f"bench.py: no configuration {which!r} (1, 1cold, 2, 2cold, 3, 3cold, 4a, 4acold, 4b, 4bcold, 5, f1a, f1b, f1c)")
     (name, build), = table.items()
     direct, graph_fn, args, work, bound = build()
-    if cold:
-        xs = [args[0]] + [torch.randn(1024, 4096, device=dev) for _ in range(71)]
-        for i in range(warmup + steps):
-            K.fused_relu_sigmoid_rowsum(xs[i % len(xs)])
-        res["kernels"] = _launched_symbols(lambda: K.fused_relu_sigmoid_rowsum(xs[0]))
+    if cold and base == "1":
+        sets = [args] + [(torch.randn(1024, 4096, device=dev),) for _ in range(71)]
+    elif cold:
+        sets = _cold_sets(torch, args, COLD_COPIES[base])
     else:
-        for _ in range(warmup + steps):
-            direct(*args)
+        sets = [args]
+    if direct is not None:
+        for i in range(warmup + steps):
+            direct(*sets[i % len(sets)])
         res["kernels"] = _launched_symbols(lambda: direct(*args))
+    if not (cold and base == "1"):
         torch._dynamo.reset()
         cf = torch.compile(graph_fn)
-        for _ in range(warmup + steps):
-            cf(*args)
+        for i in range(warmup + steps):
+            cf(*sets[i % len(sets)])
         res["compiled_kernels"] = _launched_symbols(lambda: cf(*args))
     torch.cuda.synchronize()
     src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -667,7 +706,8 @@ def main() -> None:
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB copy kernel 10 times (calibrates HBM byte counters under rocprofv3 --pmc)")
     ap.add_argument("--pmc-config", default=None,
-                    help="run only plain launches of one configuration (1, 1cold, 2, 3, 4a, 4b, 5), both paths, and the "
+                    help="run only plain launches of one configuration (1, 2, 3, 4a, 4b, 5, f1a, f1b, f1c; 1cold, 2cold, 3cold, "
+                         "4acold, 4bcold visit several input sets in turn), both paths, and the "
                          "copy probe: the program for a rocprofv3 --pmc counter run")
     ap.add_argument("--launch-floor", action="store_true",
                     help="time a 4 KiB copy (one workgroup) and the cfg 1 row sum the same way, 20 dependent launches per "
@@ -771,6 +811,15 @@ def main() -> None:
         del src, dst
     if not args.no_all_configs:
         line["all_configs"] = _all_configs(K, torch)
+        per = _per_config_summary(line["all_configs"])
+        # `frac` replays one input set, whose reads the 256 MiB memory-side cache partly serves again;
+        # `frac_cold` visits eight input sets in turn (1 GiB of reads per pass): the figure for HBM itself
+        line["roofline"]["frac_cold"] = per.get("2cold", {}).get("kernel")
+        line["roofline"]["per_config"] = per
+        line["roofline"]["per_config_note"] = ("fraction of 8 TB/s (configs 1-4, f1*) or of 2.5 PFLOP/s bf16 (5, 5b); 'kernel' = "
+                                               "hand-written family, 'compile' = through torch.compile; '*cold' rows visit several "
+                                               "input sets in turn so nothing is cache-resident; '*_kernel_us' = committed rocprofv3 "
+                                               "kernel-trace duration of the launched symbols")
     line["cpu_baseline"] = (
         {"value": None, "unit": "GB/s", "cores": None, "kind": "port", "sample": "skipped (--no-cpu-baseline)"}
         if args.no_cpu_baseline else _cpu_baseline()

@@ -415,9 +415,28 @@ class HipOverrides(OpOverrides):
     def identity(x) -> str:
         return f"{x}"
 
+    # -- random numbers (reference inductor_x/npu_fusion_attention_graph.py:150-164 carries dropout in its
+    #    training pattern; Inductor lowers rand / randn / randint / dropout to these three ops and a seed
+    #    load when config.fallback_random is off) ------------------------------------------------------
     @staticmethod
-    def load_seed(name: str, offset) -> str:
-        raise UnsupportedHipCodegen("random number generation is not generated; the op falls back to eager")
+    def load_seed(name: str, offset):
+        kernel: HipKernel = V.kernel
+        var = kernel.args.input(name)
+        out = kernel.cse.generate(kernel.compute, f"{var}[{offset}]", dtype=torch.int64)
+        out.is_vec = False  # one seed per kernel
+        return out
+
+    @staticmethod
+    def rand(seed, offset) -> str:
+        return f"mi::rand({seed}, {offset})"
+
+    @staticmethod
+    def randn(seed, offset) -> str:
+        return f"mi::randn({seed}, {offset})"
+
+    @staticmethod
+    def randint64(seed, offset, low, high) -> str:
+        return f"mi::randint64({seed}, {offset}, {low}, {high})"
 
 
 def _add_unary(name: str) -> None:

@@ -120,5 +120,90 @@ class HipScheduling(SIMDScheduling):
     def codegen_sync(self) -> None:
         V.graph.wrapper_code.writeline(V.graph.device_ops.synchronize())
 
-    def benchmark_fused_nodes(self, nodes):
-        raise NotImplementedError("fusion benchmarking is not used by this backend")
+    # -- fusion benchmarking ----------------------------------------------------
+    def generate_kernel_code_from_nodes(self, nodes, benchmark_kernel=False, hint_override=None):
+        """Python source of a module that holds the kernel for `nodes` (under the attribute name
+        Inductor's scheduler looks up, `triton_`), random operands of the graph's hinted sizes
+        (`get_args`) and one launch (`call`): what Inductor's scheduler compiles and times when
+        `benchmark_fusion` asks whether fusing two nodes pays (the reference inherits Triton's
+        form of it, reference inductor_x/codegen/triton.py:525-526,550-553,613-614)."""
+        from torch._inductor import config as inductor_config
+        from torch._inductor.codegen.common import SizeArg, TensorArg, WorkspaceArg
+        from torch._inductor.utils import IndentedBuffer
+
+        if any(n.is_template() for n in nodes):
+            raise NotImplementedError("this backend has no template kernels")
+        _, (numel, rnumel) = max(nodes, key=lambda x: int(x.is_reduction())).group
+        node_schedule = self.generate_node_schedule(nodes, numel, rnumel)
+        tiling = self.select_tiling(node_schedule, numel, rnumel)
+        kernel = self.kernel_type(tiling, features=SIMDKernelFeatures(node_schedule, numel, rnumel))
+        self.codegen_node_schedule_with_kernel(node_schedule, kernel)
+        with V.set_kernel_handler(kernel):
+            src_code = kernel.codegen_kernel()
+        name = "hip_bench"
+        device = V.graph.get_current_device_or_throw()
+        hint = lambda e: V.graph.sizevars.size_hint(e, fallback=inductor_config.unbacked_symint_fallback)  # noqa: E731
+        hints = lambda es: [hint(e) for e in es]  # noqa: E731
+        out = IndentedBuffer()
+        out.splice(
+            "import torch\nfrom torch._dynamo.testing import rand_strided\n"
+            "from inductor_x_amd.hip_heuristics import generated_kernel\n\n"
+        )
+        out.writeline(f"triton_ = generated_kernel(\n    name={name!r},\n    meta={kernel.meta!r},\n    source='''")
+        out.splice(src_code.replace(KERNEL_PLACEHOLDER, name))
+        out.writeline("''',\n)")
+        out.writelines(["", "", "def get_args():"])
+        _argdefs, call_args, signature, _ = kernel.args.python_argdefs()
+        with out.indent():
+            names = []
+            for i, (arg_name, sig) in enumerate(zip(call_args, signature)):
+                arg_name, var = str(arg_name), f"arg_{i}"
+                buf = V.graph.try_get_buffer(arg_name) if isinstance(sig, TensorArg) else None
+                if buf is not None:
+                    line = (f"{var} = rand_strided({hints(buf.get_size())}, {hints(buf.get_stride())}, "
+                            f"device='{buf.get_device()}', dtype={buf.get_dtype()})")
+                    # a zero-dimensional CPU tensor among GPU operands is a scalar kernel argument
+                    if buf.get_device().type == "cpu" and len(buf.get_size()) == 0:
+                        line += ".item()"
+                    out.writeline(line)
+                elif arg_name in V.graph.constants:
+                    c = V.graph.constants[arg_name]
+                    out.writeline(f"{var} = rand_strided({hints(c.size())}, {hints(c.stride())}, device='{device}', dtype={c.dtype})")
+                elif isinstance(sig, SizeArg):
+                    out.writeline(f"{var} = {0 if 'seed_offset' in sig.name else hint(sig.expr)}")
+                elif isinstance(sig, WorkspaceArg):
+                    out.writeline(f"{var} = torch.zeros({hint(sig.count)}, device='{device}', dtype={sig.dtype})")
+                else:
+                    raise KeyError(f"no buffer or constant behind kernel argument {arg_name}")
+                names.append(var)
+            extents = {f"{tree.prefix}numel": hint(tree.numel) for tree in kernel.range_trees}
+            out.writeline(f"return ({', '.join(names)}{',' if names else ''}), {extents!r}")
+        out.writelines(["", "", "def call(args):"])
+        with out.indent():
+            out.writeline("operands, extents = args")
+            out.writeline(f"with torch.cuda.device({device.index or 0}):")
+            with out.indent():
+                out.writeline(f"triton_.run(*operands, **extents, stream=torch._C._cuda_getCurrentRawStream({device.index or 0}))")
+        return out.getvalue()
+
+    def benchmark_codegened_module(self, mod, n_spills_threshold=8, node_names=None) -> tuple[float, str]:
+        """Milliseconds per launch of a module made by generate_kernel_code_from_nodes, and its path."""
+        args = mod.get_args()
+        for _ in range(3):
+            mod.call(args)
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(10):
+            mod.call(args)
+        end.record()
+        end.synchronize()
+        ms = start.elapsed_time(end) / 10
+        log.debug("kernel for %s: %.4f ms (%s)", node_names, ms, mod.__file__)
+        return ms, mod.__file__
+
+    def benchmark_fused_nodes(self, nodes, n_spills_threshold=8) -> tuple[float, str]:
+        """Milliseconds one launch of the kernel for `nodes` takes on random operands."""
+        from torch._inductor.codecache import PyCodeCache
+
+        mod = PyCodeCache.load(self.generate_kernel_code_from_nodes(nodes, benchmark_kernel=True))
+        return self.benchmark_codegened_module(mod, n_spills_threshold, OrderedSet(n.get_name() for n in nodes))

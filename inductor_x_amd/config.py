@@ -42,6 +42,13 @@ retry_unsupported_with_eager = os.environ.get("INDUCTOR_X_AMD_RETRY_UNSUPPORTED"
 # (no backward graph is compiled for the function).
 sum_returns_fp32 = os.environ.get("INDUCTOR_X_AMD_SUM_FP32", "0") == "1"
 
+# Random numbers in compiled graphs (rand, randn, randint, dropout): True generates them inside the
+# fused kernels with a counter-based Philox generator keyed by the graph's seed (what Inductor does
+# on its own GPU backends and what the reference's Triton path does; the values then differ from
+# eager's for one torch.manual_seed, and a backward pass regenerates the forward's dropout mask from
+# the same seed), False calls the ATen generators as separate kernels (eager's stream, bit for bit).
+generate_random = os.environ.get("INDUCTOR_X_AMD_GENERATE_RANDOM", "1") == "1"
+
 # Generated indirect accesses (embedding, index, gather, index_put, scatter): "clamp" keeps every
 # index inside its buffer (loads read the nearest valid element, stores and atomics outside the
 # range are dropped), "none" uses the index as it comes, as the reference's generated code does

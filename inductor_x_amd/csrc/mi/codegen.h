@@ -466,6 +466,68 @@ __device__ __forceinline__ V<T, N> tile_col(const Tile<T, N>& t, int u) {
   return r;
 }
 
+// ---------------------------------------------------------------------------
+// Random numbers: counter-based Philox-4x32 with ten rounds, keyed by the graph's 64-bit seed and
+// counted by the element's offset -- the generator and the integer -> float maps that Inductor's
+// own GPU code generation uses (triton.language.random: philox, uint_to_uniform_float,
+// pair_uniform_to_normal; torch/_inductor/runtime/triton_helpers.py: randint64), so a graph sees the
+// same stream whichever backend compiled it.  Stateless: the value of an element depends on
+// (seed, offset) only.
+// ---------------------------------------------------------------------------
+struct Philox4 {
+  uint32_t r[4];
+};
+__device__ __forceinline__ Philox4 philox4x32_10(i64 seed, uint32_t offset) {
+  constexpr uint32_t KEY_A = 0x9E3779B9u, KEY_B = 0xBB67AE85u, ROUND_A = 0xD2511F53u, ROUND_B = 0xCD9E8D57u;
+  uint32_t k0 = static_cast<uint32_t>(static_cast<unsigned long long>(seed));
+  uint32_t k1 = static_cast<uint32_t>(static_cast<unsigned long long>(seed) >> 32);
+  uint32_t c0 = offset, c1 = 0, c2 = 0, c3 = 0;
+#pragma unroll
+  for (int round = 0; round < 10; ++round) {
+    const uint32_t p0 = c0, p2 = c2;
+    c0 = __umulhi(ROUND_B, p2) ^ c1 ^ k0;
+    c2 = __umulhi(ROUND_A, p0) ^ c3 ^ k1;
+    c1 = ROUND_B * p2;
+    c3 = ROUND_A * p0;
+    k0 += KEY_A;
+    k1 += KEY_B;
+  }
+  return {{c0, c1, c2, c3}};
+}
+// uniform in [0, 1): the 31 low bits of |x| as a signed integer, scaled by 2^-31 (rounded down a little)
+__device__ __forceinline__ float philox_uniform(uint32_t bits) {
+  int x = static_cast<int>(bits);
+  x = x < 0 ? -x - 1 : x;
+  return static_cast<float>(x) * 4.6566127342e-10f;
+}
+template <class S, class O>
+__device__ __forceinline__ auto rand(const S& seed, const O& offset) {
+  return apply([](auto s, auto o) { return philox_uniform(philox4x32_10(static_cast<i64>(s), static_cast<uint32_t>(o)).r[0]); },
+               seed, offset);
+}
+template <class S, class O>
+__device__ __forceinline__ auto randn(const S& seed, const O& offset) {
+  return apply(
+      [](auto s, auto o) {
+        const Philox4 p = philox4x32_10(static_cast<i64>(s), static_cast<uint32_t>(o));
+        const float u1 = ::fmaxf(1.0e-7f, philox_uniform(p.r[0]));
+        const float th = 6.283185307179586f * philox_uniform(p.r[1]);
+        return ::sqrtf(-2.0f * ::logf(u1)) * ::cosf(th);
+      },
+      seed, offset);
+}
+template <class S, class O, class L, class H>
+__device__ __forceinline__ auto randint64(const S& seed, const O& offset, const L& low, const H& high) {
+  return apply(
+      [](auto s, auto o, auto lo, auto hi) {
+        const Philox4 p = philox4x32_10(static_cast<i64>(s), static_cast<uint32_t>(o));
+        const unsigned long long word = static_cast<unsigned long long>(p.r[0]) | (static_cast<unsigned long long>(p.r[1]) << 32);
+        const unsigned long long size = static_cast<unsigned long long>(static_cast<i64>(hi) - static_cast<i64>(lo));
+        return static_cast<i64>(word % size) + static_cast<i64>(lo);
+      },
+      seed, offset, low, high);
+}
+
 // Element-wise indexed load: idx scalar -> scalar, idx vector -> vector.
 // Indirect indices: the index a generated indirect load reads with when the one it was given lies
 // outside [0, size) (the nearest valid one), and whether an index is inside (stores and atomics

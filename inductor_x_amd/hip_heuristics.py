@@ -590,11 +590,35 @@ class GeneratedKernel:
         # calls from its worker pool)
         self._pending = _compile_pool().submit(codecache.compile_source, source, label=name)
 
-    def precompile(self) -> None:
+    # -- what Inductor's AsyncCompile asks of a kernel object (its worker pool compiles the kernels of
+    #    a benchmark module and sends the objects back pickled; reference
+    #    inductor_x/npu_triton_heuristics.py:53-109 is the same protocol on the reference's side) ------
+    autotune_cache_info = None
+
+    def set_compile_info(self, compile_id=None, is_backward: bool = False) -> None:
+        self.compile_id, self.is_backward = compile_id, is_backward
+
+    def prepare_for_pickle(self):
+        return None
+
+    def restore_after_unpickle(self, old_values=None) -> None:
+        return None
+
+    def __getstate__(self):
+        # the code object is on disk by now; module handles and the pending compile stay behind
+        self._pending.result()
+        return {"name": self.name, "meta": self.meta, "source": self.source}
+
+    def __setstate__(self, state):
+        self.__init__(state["name"], state["meta"], state["source"])
+
+    def precompile(self, warm_cache_only: bool = False, **_unused) -> None:
         if self._fns is not None:
             return
         path = self._pending.result()
         self.hsaco_path = path
+        if warm_cache_only:  # a compile worker: the code object is in the store, nothing to load
+            return
         if _DRYRUN:
             self._fns = {}
             return

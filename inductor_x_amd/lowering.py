@@ -194,8 +194,8 @@ def _register_inductor_fallbacks() -> None:
         return
     _registered = True
 
-    # device-side random numbers are not generated: let Inductor call ATen for them
-    inductor_config.fallback_random = True
+    # random numbers: generated inside the fused kernels, or ATen's generators as separate kernels
+    inductor_config.fallback_random = not backend_config.generate_random
 
     fb_set: set = set()
     _init_set(FALLBACK_OPS, fb_set)

@@ -722,3 +722,42 @@ def test_sum_fp32_switch_applies_to_inference_graphs_only(monkeypatch):
     out.float().sum().backward()
     assert xg.grad is not None and xg.grad.dtype == torch.bfloat16 and torch.equal(xg.grad, torch.ones_like(xg))
     torch._dynamo.reset()
+
+
+def test_fusion_benchmarking_times_generated_kernels(monkeypatch):
+    """With Inductor's `benchmark_fusion` on, the scheduler asks the backend for the run time of
+    candidate kernels (fused against separate) before it fuses: the backend compiles each
+    candidate, runs it on random operands and returns milliseconds.  The compiled graph is the
+    same function either way (the reference inherits this from Triton's scheduling, reference
+    inductor_x/codegen/triton.py:525-526,550-553,613-614)."""
+    import torch._inductor.config as inductor_config
+
+    from inductor_x_amd.codegen.scheduling import HipScheduling
+
+    announce("fusion benchmarking")
+    timed = []
+    original = HipScheduling.benchmark_codegened_module
+
+    def counting(self, mod, *a, **k):
+        ms, path = original(self, mod, *a, **k)
+        timed.append((path, ms))
+        return ms, path
+
+    monkeypatch.setattr(HipScheduling, "benchmark_codegened_module", counting)
+    torch.manual_seed(0)
+    x = torch.randn(4096, 2048, device=DEV)
+    w = torch.randn(2048, device=DEV)
+
+    def f(x, w):
+        y = torch.relu(x * w + 1.0)
+        return y.sum(-1), (y * 2.0).amax(-1), y.mean(0)
+
+    want = f(x, w)
+    torch._dynamo.reset()
+    with inductor_config.patch(benchmark_fusion=True):
+        got = torch.compile(f)(x, w)
+    torch.cuda.synchronize()
+    for g, r in zip(got, want):
+        torch.testing.assert_close(g, r, rtol=1e-4, atol=1e-3)
+    assert timed and all(ms > 0 for _, ms in timed), timed
+    torch._dynamo.reset()

@@ -149,13 +149,110 @@ def test_embedding_gradient_accumulates_with_atomics():
     torch.testing.assert_close(got, ref, rtol=1e-5, atol=1e-5)
 
 
-def test_dropout_in_training_keeps_its_rate():
-    """Random numbers come from the library generator (no device-side generator is emitted);
-    the mask is applied by generated code."""
-    announce("compile dropout, training")
+def _philox4x32_10(seed: int, offset: int):
+    """Philox-4x32-10 in plain Python (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3";
+    key = the 64-bit seed, counter = (offset, 0, 0, 0)), the reference the device code is held to."""
+    M = 0xFFFFFFFF
+    k0, k1 = seed & M, (seed >> 32) & M
+    c = [offset & M, 0, 0, 0]
+    for _ in range(10):
+        p0, p2 = c[0], c[2]
+        c = [((0xCD9E8D57 * p2) >> 32) ^ c[1] ^ k0, (0xCD9E8D57 * p2) & M, ((0xD2511F53 * p0) >> 32) ^ c[3] ^ k1, (0xD2511F53 * p0) & M]
+        k0, k1 = (k0 + 0x9E3779B9) & M, (k1 + 0xBB67AE85) & M
+    return c
+
+
+def test_philox_reference_matches_the_published_vectors():
+    """The plain-Python generator above reproduces the known-answer vectors of the Random123
+    distribution (kat_vectors: philox4x32-10) -- counter and key all zeros, all ones, and the digits
+    of pi -- so the device code below is compared with the published algorithm, not with a copy of itself."""
+    def full(counter, key):
+        M = 0xFFFFFFFF
+        c, (k0, k1) = list(counter), key
+        for _ in range(10):
+            p0, p2 = c[0], c[2]
+            c = [((0xCD9E8D57 * p2) >> 32) ^ c[1] ^ k0, (0xCD9E8D57 * p2) & M, ((0xD2511F53 * p0) >> 32) ^ c[3] ^ k1, (0xD2511F53 * p0) & M]
+            k0, k1 = (k0 + 0x9E3779B9) & M, (k1 + 0xBB67AE85) & M
+        return c
+
+    assert full((0, 0, 0, 0), (0, 0)) == [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]
+    assert full((0xFFFFFFFF,) * 4, (0xFFFFFFFF, 0xFFFFFFFF)) == [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]
+    assert full((0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344), (0xA4093822, 0x299F31D0)) == [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]
+    assert _philox4x32_10(0, 0) == full((0, 0, 0, 0), (0, 0))
+
+
+def test_generated_random_numbers():
+    """rand / randn / randint / dropout inside generated kernels (reference
+    inductor_x/npu_fusion_attention_graph.py:150-164 carries dropout through its training pattern):
+    the uniform stream equals Philox-4x32-10 keyed by the graph's seed element by element, a fixed
+    torch.manual_seed repeats it, moments and ranges are right, and the backward of dropout reuses
+    the forward's mask."""
+    from torch._inductor.utils import run_and_get_code
+
+    from inductor_x_amd import config
+
+    announce("generated random numbers")
+    assert config.generate_random
     torch._dynamo.reset()
-    kept = torch.compile(lambda a: (F.dropout(a, 0.5, training=True) != 0).float().mean(), dynamic=False)(t(512, 512))
-    assert abs(kept.item() - 0.5) < 0.02
+    f = torch.compile(lambda a: torch.rand_like(a) + a * 0, dynamic=False)
+    x = t(300, 77)
+    torch.manual_seed(123)
+    u1, codes = run_and_get_code(f, x)
+    code = "\n".join(codes)
+    assert "mi::rand(" in code and "aten.rand_like" not in code and "aten.rand.default" not in code
+    torch.manual_seed(123)
+    u2 = f(x)
+    assert torch.equal(u1, u2)
+    torch.manual_seed(124)
+    assert not torch.equal(u1, f(x))
+    assert 0.0 <= u1.min().item() and u1.max().item() < 1.0 and abs(u1.mean().item() - 0.5) < 0.01
+    # the stream is philox(seed, element index): recover the seed Inductor drew and check 64 elements
+    torch.manual_seed(123)
+    # (the wrapper draws it with aten.randint over the whole int64 range as its first random call)
+    seed = int(torch.randint(-2 ** 63, 2 ** 63 - 1, (1,), device=DEV).item())
+    flat = u1.flatten().cpu()
+    for i in (0, 1, 2, 63, 64, 1000, 23099):
+        bits = _philox4x32_10(seed, i)[0]
+        v = bits - (1 << 32) if bits >= (1 << 31) else bits
+        v = -v - 1 if v < 0 else v
+        assert abs(flat[i].item() - v * 4.6566127342e-10) <= 1e-7, i
+    torch._dynamo.reset()
+    n = torch.compile(lambda a: torch.randn_like(a) + a * 0, dynamic=False)(t(1024, 512))
+    assert abs(n.mean().item()) < 0.01 and abs(n.std().item() - 1.0) < 0.01
+    torch._dynamo.reset()
+    r = torch.compile(lambda a: torch.randint(-3, 9, a.shape, device=a.device) + (a * 0).long(), dynamic=False)(t(256, 256))
+    assert r.min().item() == -3 and r.max().item() == 8 and abs(r.float().mean().item() - 2.5) < 0.1
+    # dropout: rate, scaling, and the same mask in the backward
+    torch._dynamo.reset()
+    a = t(512, 512).requires_grad_()
+    g = torch.compile(lambda a: F.dropout(a * 2.0, 0.25, training=True), dynamic=False)
+    torch.manual_seed(5)
+    y = g(a)
+    y.sum().backward()
+    kept = y != 0
+    assert abs(kept.float().mean().item() - 0.75) < 0.01
+    torch.testing.assert_close(y[kept], (a.detach() * 2.0 / 0.75)[kept])
+    torch.testing.assert_close(a.grad, kept.float() * (2.0 / 0.75))
+    torch._dynamo.reset()
+
+
+def test_random_numbers_from_the_library_generator(monkeypatch):
+    """With the generator switched off the random ops run as ATen kernels (eager's stream for one
+    seed, bit for bit) and generated code applies the mask."""
+    import torch._inductor.config as inductor_config
+
+    announce("compile dropout, library generator")
+    torch._dynamo.reset()
+    with inductor_config.patch(fallback_random=True):
+        f = torch.compile(lambda a: F.dropout(a, 0.5, training=True), dynamic=False)
+        x = t(512, 512)
+        torch.manual_seed(9)
+        got = f(x)
+        torch.manual_seed(9)
+        want = F.dropout(x, 0.5, training=True)
+    assert torch.equal(got, want)
+    assert abs((got != 0).float().mean().item() - 0.5) < 0.02
+    torch._dynamo.reset()
 
 
 def _setitem(a, p, v):

@@ -1,7 +1,8 @@
-"""Parity at the exact shapes the benchmark times, for the three graphs whose other tests run at
-reduced extents: the row gather at 32,768 indices, add + RMSNorm through torch.compile at 8,192
-rows, and fused causal attention on the 4 x 32 head grid (128 heads over 8 dies, paired query
-blocks).  Bars: bit-exact for gather and h + r; 2e-2 absolute for bf16 outputs.
+"""Parity at the exact shapes the benchmark times, for the graphs whose other tests run at
+reduced extents: the row gather at 32,768 indices, add + RMSNorm and the permuted copy through
+torch.compile at their full extents, and fused causal attention, forward and backward, on the
+4 x 32 head grid (128 heads over 8 dies, paired query blocks).  Bars: bit-exact for gather,
+permute and h + r; 2e-2 absolute for bf16 outputs; 1 % of the largest entry for gradients.
 """
 import numpy as np
 import pytest
@@ -129,3 +130,73 @@ def test_attention_full_grid_through_the_graph_pattern(K):
     a = npu_fusion_attention_graph(q, k, v, 32, "BNSD", scale=128 ** 0.5, sparse_mode=3)[0]
     b = K.fused_attention(q, k, v, 128 ** -0.5, True)[0]
     assert torch.equal(a, b)
+
+
+def test_permute_compiled_full_shape(K, O):
+    """t [16, 2048, 32, 128] bf16 through torch.compile: permute(0, 2, 1, 3).contiguous() as one
+    generated kernel, bit-exact against the oracle's copy and against the hand-written kernel."""
+    announce("full-shape compiled permute 16x2048x32x128")
+    torch.manual_seed(0)
+    t = torch.randn(16, 2048, 32, 128).bfloat16()
+    tg = t.to(DEV)
+    out, code = _compile(lambda t: t.permute(0, 2, 1, 3).contiguous(), tg)
+    assert code.count("generated_kernel(") == 1
+    assert out.shape == (16, 32, 2048, 128) and out.is_contiguous()
+    hand = K.permute_0213_contiguous(tg)
+    assert torch.equal(out, hand)
+    ref = O.permute4(bits(t), (0, 2, 1, 3))
+    assert np.array_equal(bits(out), ref)
+
+
+# heads of the 128-head grid whose gradients are checked against the fp64 oracle (one on the first die,
+# one across the batch boundary, the last), on the first 512 positions of each: the causal gradients of
+# a prefix depend on nothing behind it when only the prefix carries upstream gradient
+_BWD_ORACLE_HEADS = (0, 64, 127)
+
+
+def test_attention_backward_full_grid(K, O):
+    """Backward at [4, 32, 4096, 128] bf16, causal, the launch the benchmark times.  Oracle-sampled:
+    with upstream gradient only on the first 512 queries of three heads, dq / dk / dv of those
+    heads' first 512 positions equal the oracle's gradients of the 512-long problem (everything
+    behind is masked for those queries), and every other entry of all 128 heads is exactly zero.
+    On the whole tensor with a dense upstream gradient: linear in dO and equal to the gradients
+    computed with library GEMMs on 8 sampled heads."""
+    announce("full-shape attention backward 4x32x4096x128 causal")
+    from inductor_x_amd import attention_backward as AB
+
+    torch.manual_seed(3)
+    B, N, S, D, P = 4, 32, 4096, 128, 512
+    q, k, v = (torch.randn(B, N, S, D).bfloat16() for _ in range(3))
+    scale = D ** -0.5
+    qg, kg, vg = q.to(DEV), k.to(DEV), v.to(DEV)
+    o, m, l = K.fused_attention(qg, kg, vg, scale, True)
+    do = torch.zeros(B * N, S, D).bfloat16()
+    for hd in _BWD_ORACLE_HEADS:
+        do[hd, :P] = torch.randn(P, D).bfloat16()
+    dog = do.view(B, N, S, D).to(DEV)
+    dq, dk, dv = K.fused_attention_backward(qg, kg, vg, o, dog, m, l, scale, True)
+    torch.cuda.synchronize()
+    flat = lambda t: t.view(B * N, S, t.shape[-1])  # noqa: E731
+    for name, g in (("dq", dq), ("dk", dk), ("dv", dv)):
+        gf = flat(g)
+        mask = torch.ones(B * N, S, dtype=torch.bool, device=DEV)
+        for hd in _BWD_ORACLE_HEADS:
+            mask[hd, :P] = False
+        assert gf[mask].float().abs().max().item() == 0.0, name
+    for hd in _BWD_ORACLE_HEADS:
+        sl = lambda t: bits(flat(t)[hd:hd + 1, :P].reshape(1, 1, P, D).contiguous())  # noqa: E731
+        ref = O.attention_bwd(sl(q), sl(k), sl(v), bits(do[hd:hd + 1, :P].reshape(1, 1, P, D).contiguous()), scale, True)
+        for name, g, r in zip(("dq", "dk", "dv"), (dq, dk, dv), ref):
+            got = flat(g)[hd, :P].float().cpu().numpy()
+            assert np.abs(got - r[0, 0]).max() <= 1e-2 * np.abs(r).max() + 1e-3, (hd, name)
+    # dense upstream gradient: GEMM formulation on 8 heads (one per die), and linearity
+    dense = torch.randn(B, N, S, D, device=DEV).bfloat16()
+    dq, dk, dv = K.fused_attention_backward(qg, kg, vg, o, dense, m, l, scale, True)
+    pick = [0, 17, 34, 51, 68, 85, 102, 119]
+    sub = lambda t: flat(t)[pick].reshape(1, len(pick), S, t.shape[-1]).contiguous()  # noqa: E731
+    ref = AB.fused_attention_backward(sub(qg), sub(kg), sub(vg), sub(o), sub(dense), sub(m), sub(l), scale, True, use_kernels=False)
+    for g, r in zip((dq, dk, dv), ref):
+        assert (sub(g).float() - r.float()).abs().max().item() <= 8e-3 * max(r.float().abs().max().item(), 1.0)
+    dq2, dk2, dv2 = K.fused_attention_backward(qg, kg, vg, o, (dense.float() * 2).bfloat16(), m, l, scale, True)
+    for a, b in ((dq, dq2), (dk, dk2), (dv, dv2)):
+        assert (b.float() - 2 * a.float()).abs().max().item() <= 2e-2 * max(b.float().abs().max().item(), 1.0)
