@@ -1,6 +1,7 @@
 """Backward of the fused attention forward (npu_graph::npu_fa_backward).
 
-Two paths.  bf16 with head dimension 128 and a sequence length that is a multiple of 128 runs the fused MFMA
+Two paths.  bf16 with a head dimension up to 128 (a multiple of 8; smaller ones are padded with zero columns)
+and a sequence length that is a multiple of 64 runs the fused MFMA
 kernels (kernels.fused_attention_backward, csrc/mi/attention_bwd_w8.h).  Other shapes run the matrix
 products as library GEMMs (torch.bmm, hipBLASLt underneath) on a bounded number of heads at a time
 and move O(S^2) intermediates through HBM.  Both recompute the probabilities from the forward's
@@ -95,10 +96,10 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
                              use_kernels=None, keep_prob: float = 1.0, seed: int = 0):
     """q, k, v, out, dout: [B, N, S, D] of one floating-point type; softmax_max / softmax_sum:
     [B, N, S, 8] fp32 from the forward.  Returns (dq, dk, dv) in that type.  use_kernels: None = fused
-    kernels where they apply (bf16, head dimension 128, sequence a multiple of 64, no dropout).
+    kernels where they apply (bf16, head dimension up to 128, sequence a multiple of 64, no dropout).
     keep_prob < 1 with the forward's seed regenerates the forward's dropout mask (GEMM path only)."""
-    fits = (q.dim() == 4 and q.dtype == torch.bfloat16 and q.size(3) == 128 and q.size(2) % 64 == 0
-            and q.size(2) > 0 and q.shape == k.shape and keep_prob == 1.0)
+    fits = (q.dim() == 4 and q.dtype == torch.bfloat16 and 0 < q.size(3) <= 128 and q.size(3) % 8 == 0
+            and q.size(2) % 64 == 0 and q.size(2) > 0 and q.shape == k.shape and keep_prob == 1.0)
     if use_kernels is None:
         use_kernels = fits
     if use_kernels:
@@ -106,10 +107,15 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
             raise NotImplementedError("attention backward: the fused kernels have no dropout")
         from . import kernels
 
-        return kernels.fused_attention_backward(
-            q.contiguous(), k.contiguous(), v.contiguous(), out.contiguous(), dout.contiguous(),
+        # a head dimension below 128 is padded with zero columns: scores, probabilities and
+        # rowsum(dO * O) do not change, the extra gradient columns are zero and dropped
+        d = q.size(3)
+        widen = (lambda t: torch.nn.functional.pad(t, (0, 128 - d))) if d < 128 else (lambda t: t.contiguous())  # noqa: E731
+        grads = kernels.fused_attention_backward(
+            widen(q), widen(k), widen(v), widen(out), widen(dout),
             softmax_max.contiguous(), softmax_sum.contiguous(), scale, causal,
         )
+        return tuple(g[..., :d].contiguous() for g in grads) if d < 128 else grads
     return _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale, causal, keep_prob, seed)
 
 

@@ -118,14 +118,19 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
     real_scale = 1.0 / scale
     causal = _is_causal(query.size(2), atten_mask, pre_tockens, next_tockens, sparse_mode)
     seed = numels = 0
-    if (keep_prob == 1.0 and query.dtype in (torch.bfloat16, torch.float16) and query.size(3) == 128
-            and query.size(2) > 0 and key.size(2) > 0 and (not causal or query.size(2) == key.size(2))):
-        # the MFMA kernel: bf16 or fp16, head dimension 128, any sequence lengths
-        out, smax, ssum = kernels.fused_attention(
-            query.contiguous(), key.contiguous(), value.contiguous(), real_scale, causal
-        )
+    head_dim = query.size(3)
+    if (keep_prob == 1.0 and query.dtype in (torch.bfloat16, torch.float16) and head_dim <= 128 and head_dim % 8 == 0
+            and head_dim > 0 and query.size(2) > 0 and key.size(2) > 0 and (not causal or query.size(2) == key.size(2))):
+        # the MFMA kernel: bf16 or fp16, head dimension 128, any sequence lengths.  A smaller head
+        # dimension is padded with zero columns (scores and statistics do not change, the extra output
+        # columns are zero and dropped): twice the matrix work at 64, but no S x S tensor in memory
+        pad = 128 - head_dim
+        widen = (lambda t: torch.nn.functional.pad(t, (0, pad))) if pad else (lambda t: t.contiguous())  # noqa: E731
+        out, smax, ssum = kernels.fused_attention(widen(query), widen(key), widen(value), real_scale, causal)
+        if pad:
+            out = out[..., :head_dim].contiguous()
     else:
-        # other head dimensions, fp32 and dropout: the same mathematics over library GEMMs.  The dropout seed comes from torch's CPU generator (torch.manual_seed makes a
+        # head dimensions above 128 or not a multiple of 8, fp32 and dropout: the same mathematics over library GEMMs.  The dropout seed comes from torch's CPU generator (torch.manual_seed makes a
         # run repeatable) and travels to the backward in the op's seed output, as in the reference's op.
         from .attention_backward import attention_forward_over_gemms
 

@@ -317,8 +317,11 @@ def test_attention_backward_vs_oracle(K, O, B, N, S, causal):
 
 
 @pytest.mark.parametrize("dtype,B,N,S,D,causal", [
-    (torch.float16, 2, 3, 200, 64, True), (torch.bfloat16, 1, 4, 96, 80, False), (torch.float32, 1, 2, 130, 32, True),
+    (torch.float16, 2, 3, 200, 64, True),    # fused forward on a padded head dimension, GEMM backward (fp16)
+    (torch.bfloat16, 1, 4, 96, 80, False),   # fused forward (padded), GEMM backward (96 is no multiple of 64)
+    (torch.float32, 1, 2, 130, 32, True),    # fp32: GEMMs both ways
     (torch.bfloat16, 1, 2, 192, 128, True),  # fused forward (ragged instantiation) and fused backward (a multiple of 64)
+    (torch.bfloat16, 1, 2, 100, 160, False), (torch.float16, 1, 2, 64, 36, True),  # head dimensions the kernel does not take
 ])
 def test_attention_op_outside_the_fused_kernels(dtype, B, N, S, D, causal):
     """npu_fa / npu_fa_backward for shapes and element types the MFMA kernels do not cover run the same
@@ -349,25 +352,27 @@ def test_attention_op_outside_the_fused_kernels(dtype, B, N, S, D, causal):
         assert (g.float() - r).abs().max().item() <= (1e-4 if dtype == torch.float32 else 3e-2) * max(r.abs().max().item(), 1.0)
 
 
-@pytest.mark.parametrize("dtype,B,N,Sq,Sk,causal", [
-    (torch.float16, 1, 3, 200, 200, True), (torch.float16, 2, 2, 512, 512, False), (torch.bfloat16, 1, 2, 100, 300, False),
-    (torch.bfloat16, 1, 2, 77, 77, True),
+@pytest.mark.parametrize("dtype,B,N,Sq,Sk,causal,D", [
+    (torch.float16, 1, 3, 200, 200, True, 128), (torch.float16, 2, 2, 512, 512, False, 128),
+    (torch.bfloat16, 1, 2, 100, 300, False, 128), (torch.bfloat16, 1, 2, 77, 77, True, 128),
+    (torch.bfloat16, 2, 3, 256, 256, True, 64), (torch.float16, 1, 2, 130, 130, False, 64), (torch.bfloat16, 1, 2, 192, 192, True, 80),
 ])
-def test_attention_op_reaches_the_fused_kernel_for_fp16_and_any_length(dtype, B, N, Sq, Sk, causal):
-    """npu_fa with fp16 operands, with sequence lengths that are no multiple of a tile and with
-    different query and key lengths launches the MFMA kernel (not the GEMM formulation), and the
-    training path still returns gradients where the backward applies (equal lengths)."""
-    announce(f"attention op on the fused kernel {dtype} B={B} N={N} Sq={Sq} Sk={Sk} causal={causal}")
+def test_attention_op_reaches_the_fused_kernel_for_fp16_and_any_length(dtype, B, N, Sq, Sk, causal, D):
+    """npu_fa with fp16 operands, with sequence lengths that are no multiple of a tile, with
+    different query and key lengths and with head dimensions below 128 (zero-padded) launches the
+    MFMA kernel (not the GEMM formulation), and the training path still returns gradients where the
+    backward applies (equal lengths)."""
+    announce(f"attention op on the fused kernel {dtype} B={B} N={N} Sq={Sq} Sk={Sk} D={D} causal={causal}")
     from inductor_x_amd import launcher
     from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
 
     torch.manual_seed(13)
-    q = torch.randn(B, N, Sq, 128, device=DEV).to(dtype)
-    k, v = (torch.randn(B, N, Sk, 128, device=DEV).to(dtype) for _ in range(2))
+    q = torch.randn(B, N, Sq, D, device=DEV).to(dtype)
+    k, v = (torch.randn(B, N, Sk, D, device=DEV).to(dtype) for _ in range(2))
     train = Sq == Sk
     if train:
         q, k, v = (t.requires_grad_() for t in (q, k, v))
-    inv = 128 ** 0.5
+    inv = D ** 0.5
     launcher.launch_log = []
     try:
         res = npu_fusion_attention_graph(q, k, v, N, "BNSD", scale=inv, sparse_mode=3 if causal else 0)
@@ -381,11 +386,18 @@ def test_attention_op_reaches_the_fused_kernel_for_fp16_and_any_length(dtype, B,
     if causal:
         s = s.masked_fill(torch.ones(Sq, Sk, device=DEV, dtype=torch.bool).triu(1), float("-inf"))
     ref = torch.softmax(s, -1) @ vf
-    assert res[0].dtype == dtype and (res[0].float() - ref).abs().max().item() <= 2e-2
+    assert res[0].dtype == dtype and res[0].shape == q.shape and (res[0].float() - ref).abs().max().item() <= 2e-2
     torch.testing.assert_close(res[1][..., 0], s.amax(-1), rtol=1e-3, atol=1e-3)
     if train:
         do = torch.randn_like(res[0])
-        res[0].backward(do)
+        launcher.launch_log = []
+        try:
+            res[0].backward(do)
+            torch.cuda.synchronize()
+        finally:
+            log, launcher.launch_log = launcher.launch_log, None
+        if dtype == torch.bfloat16 and Sq % 64 == 0:
+            assert any(sym.startswith("attention_bwd8_") for sym in log), log
         ref.backward(do.float())
         for g, r in zip((q.grad, k.grad, v.grad), (qf.grad, kf.grad, vf.grad)):
             assert (g.float() - r).abs().max().item() <= 3e-2 * max(r.abs().max().item(), 1.0)
