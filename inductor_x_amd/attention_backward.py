@@ -53,14 +53,32 @@ def _check_keep_prob(keep_prob: float) -> float:
     return 0.0 if keep_prob == 0.0 else 1.0 / keep_prob
 
 
-def attention_forward_over_gemms(q, k, v, scale: float, causal: bool, keep_prob: float = 1.0, seed: int = 0):
+def _per_head(t, B: int, N: int, Sq: int, Sk: int, what: str):
+    """A bias or mask given as [Sq, Sk] or broadcastable to [B, N, Sq, Sk], as a [B * N or 1, Sq, Sk] view
+    (no copy when it broadcasts over batch and heads)."""
+    if t.dim() == 2:
+        t = t.view(1, 1, *t.shape)
+    if t.dim() != 4 or t.shape[2:] != (Sq, Sk) or t.shape[0] not in (1, B) or t.shape[1] not in (1, N):
+        raise ValueError(f"attention: {what} of shape {tuple(t.shape)} does not broadcast to [{B}, {N}, {Sq}, {Sk}]")
+    if t.shape[0] == 1 and t.shape[1] == 1:
+        return t.view(1, Sq, Sk)
+    return t.expand(B, N, Sq, Sk).reshape(B * N, Sq, Sk)
+
+
+def attention_forward_over_gemms(q, k, v, scale: float, causal: bool, keep_prob: float = 1.0, seed: int = 0,
+                                 pse=None, atten_mask=None):
     """softmax(q k^T * scale [+ causal mask]) v with library GEMMs for shapes and element types the
     fused forward kernels do not cover (any head dimension and sequence length; bf16, fp16, fp32).
     Returns (out, softmax_max, softmax_sum) like kernels.fused_attention: the row statistics are
     fp32 [B, N, S, 8], the probabilities are rounded to the operand type before the second product
     and O(S^2) intermediates move through HBM, a bounded number of heads at a time.
     keep_prob < 1 drops probabilities after the softmax (dropout_keep_mask) and scales the kept ones
-    by 1 / keep_prob; the row statistics are those of the undropped softmax."""
+    by 1 / keep_prob; the row statistics are those of the undropped softmax.
+    pse (a positional bias, [Sq, Sk] or broadcastable to [B, N, Sq, Sk]) is added to q k^T before the
+    scaling and atten_mask (boolean or integer, non-zero = the key is hidden from the query) is
+    applied after it -- softmax(mask(scale * (pse + q k^T))) as the fused op of the reference's
+    device library documents it (call site: reference inductor_x/npu_fusion_attention_graph.py:31);
+    a row with every key hidden gives zeros."""
     inv_keep = _check_keep_prob(keep_prob)
     for t in (q, k, v):
         if not (t.is_cuda and t.dtype in _GEMM_DTYPES and t.dtype == q.dtype and t.dim() == 4):
@@ -76,14 +94,25 @@ def attention_forward_over_gemms(q, k, v, scale: float, causal: bool, keep_prob:
     if heads and S:
         chunk = _heads_per_round(heads, S)
         mask = torch.ones(S, S, dtype=torch.bool, device=q.device).triu_(1) if causal else None
+        bias = _per_head(pse, B, N, S, S, "pse") if pse is not None else None
+        hide = _per_head(atten_mask != 0, B, N, S, S, "atten_mask") if atten_mask is not None else None
         for h0 in range(0, heads, chunk):
             sl = slice(h0, min(h0 + chunk, heads))
-            s = _bmm_f32(qh[sl], kh[sl].transpose(1, 2)).mul_(scale)
+            s = _bmm_f32(qh[sl], kh[sl].transpose(1, 2))
+            if bias is not None:
+                s.add_(bias if bias.shape[0] == 1 else bias[sl])
+            s.mul_(scale)
             if mask is not None:
                 s.masked_fill_(mask, float("-inf"))
+            if hide is not None:
+                s.masked_fill_(hide if hide.shape[0] == 1 else hide[sl], float("-inf"))
             m = s.amax(-1)
+            if hide is not None:
+                m = torch.where(torch.isinf(m), torch.zeros_like(m), m)  # rows with every key hidden
             p = s.sub_(m.unsqueeze(-1)).exp_()
             l = p.sum(-1)
+            if hide is not None:
+                l = torch.where(l == 0, torch.ones_like(l), l)
             smax[sl], ssum[sl] = m, l
             if keep_prob < 1.0:
                 p.mul_(dropout_keep_mask(seed, h0, sl.stop - h0, S, keep_prob, q.device)).mul_(inv_keep)
@@ -93,11 +122,18 @@ def attention_forward_over_gemms(q, k, v, scale: float, causal: bool, keep_prob:
 
 
 def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale: float, causal: bool,
-                             use_kernels=None, keep_prob: float = 1.0, seed: int = 0):
+                             use_kernels=None, keep_prob: float = 1.0, seed: int = 0, pse=None, atten_mask=None):
     """q, k, v, out, dout: [B, N, S, D] of one floating-point type; softmax_max / softmax_sum:
     [B, N, S, 8] fp32 from the forward.  Returns (dq, dk, dv) in that type.  use_kernels: None = fused
     kernels where they apply (bf16, head dimension up to 128, sequence a multiple of 64, no dropout).
-    keep_prob < 1 with the forward's seed regenerates the forward's dropout mask (GEMM path only)."""
+    keep_prob < 1 with the forward's seed regenerates the forward's dropout mask (GEMM path only).
+    With pse or atten_mask (GEMM path only) the result has a fourth member, the gradient of pse in
+    pse's own shape (None without pse)."""
+    if pse is not None or atten_mask is not None:
+        if use_kernels:
+            raise NotImplementedError("attention backward: the fused kernels take no bias or mask")
+        return _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale, causal, keep_prob, seed,
+                                    pse=pse, atten_mask=atten_mask)
     fits = (q.dim() == 4 and q.dtype == torch.bfloat16 and 0 < q.size(3) <= 128 and q.size(3) % 8 == 0
             and q.size(2) % 64 == 0 and q.size(2) > 0 and q.shape == k.shape and keep_prob == 1.0)
     if use_kernels is None:
@@ -120,7 +156,7 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
 
 
 def _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale: float, causal: bool,
-                         keep_prob: float = 1.0, seed: int = 0):
+                         keep_prob: float = 1.0, seed: int = 0, pse=None, atten_mask=None):
     # With dropout, Pd = P * keep / keep_prob takes P's place in dV = Pd^T dO, and dP = (dO V^T) * keep /
     # keep_prob; D = rowsum(dO * O) = rowsum(P * dP) still holds because O = Pd V.
     inv_keep = _check_keep_prob(keep_prob)
@@ -145,14 +181,22 @@ def _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale: fl
     mask = None
     if causal:
         mask = torch.ones(S, S, dtype=torch.bool, device=q.device).triu_(1)
+    extras = pse is not None or atten_mask is not None
+    bias = _per_head(pse, B, N, S, S, "pse") if pse is not None else None
+    hide = _per_head(atten_mask != 0, B, N, S, S, "atten_mask") if atten_mask is not None else None
+    dpse = torch.zeros(heads, S, S, dtype=torch.float32, device=q.device) if pse is not None else None
     for h0 in range(0, heads, chunk):
         sl = slice(h0, min(h0 + chunk, heads))
         qc, kc, vc, oc, doc = qh[sl], kh[sl], vh[sl], oh[sl], doh[sl]
         s = _bmm_f32(qc, kc.transpose(1, 2))
+        if bias is not None:
+            s.add_(bias if bias.shape[0] == 1 else bias[sl])
         # P = exp(S * scale - m) / l, masked entries exactly zero
         s.mul_(scale).sub_(m[sl].unsqueeze(-1))
         if mask is not None:
             s.masked_fill_(mask, float("-inf"))
+        if hide is not None:
+            s.masked_fill_(hide if hide.shape[0] == 1 else hide[sl], float("-inf"))
         p = s.exp_().div_(l[sl].unsqueeze(-1))
         dp = _bmm_f32(doc, vc.transpose(1, 2))
         if keep_prob < 1.0:
@@ -163,7 +207,21 @@ def _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale: fl
         else:
             dv[sl] = torch.bmm(p.to(q.dtype).transpose(1, 2), doc)
         delta = (doc.float() * oc.float()).sum(-1, keepdim=True)
-        ds16 = p.mul_(dp.sub_(delta)).mul_(scale).to(q.dtype)
+        ds = p.mul_(dp.sub_(delta)).mul_(scale)
+        if dpse is not None:
+            dpse[sl] = ds  # d loss / d (q k^T) is also d loss / d pse: the bias sits beside the product
+        ds16 = ds.to(q.dtype)
         dq[sl] = torch.bmm(ds16, kc)
         dk[sl] = torch.bmm(ds16.transpose(1, 2), qc)
-    return dq.view(B, N, S, D), dk.view(B, N, S, D), dv.view(B, N, S, D)
+    grads = (dq.view(B, N, S, D), dk.view(B, N, S, D), dv.view(B, N, S, D))
+    if not extras:
+        return grads
+    if dpse is not None:
+        # fold the [B, N, S, S] gradient onto the axes pse broadcast over
+        g = dpse.view(B, N, S, S)
+        shape = pse.shape if pse.dim() == 4 else (1, 1) + tuple(pse.shape)
+        for axis in (0, 1):
+            if shape[axis] == 1 and g.shape[axis] != 1:
+                g = g.sum(axis, keepdim=True)
+        dpse = g.reshape(pse.shape).to(pse.dtype)
+    return grads + (dpse,)

@@ -86,14 +86,17 @@ def _check_layout(op: str, layout: str):
 
 
 def _is_causal(seq_len: int, atten_mask, pre_tockens: int, next_tockens: int, sparse_mode: int) -> bool:
+    """True when the arguments describe the plain causal mask (which the kernels apply themselves and
+    for which a mask tensor, if given, is the compressed triangle of the reference's device library and is
+    not read).  Otherwise a given atten_mask is applied as it stands."""
     if sparse_mode in (2, 3):
         return True
     if sparse_mode == 0 and next_tockens == 0 and pre_tockens >= seq_len:
         return True
-    if atten_mask is not None:
+    if sparse_mode != 0 or (atten_mask is None and (next_tockens < seq_len or pre_tockens < seq_len)):
         raise NotImplementedError(
-            "npu_fa: an attention mask is only supported as the causal mask "
-            "(sparse_mode 2/3, or next_tockens=0 with pre_tockens >= sequence length)"
+            "npu_fa: band masks (pre_tockens / next_tockens short of the sequence length) and sparse modes other "
+            "than 0, 2 and 3 are not supported"
         )
     return False
 
@@ -106,8 +109,8 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
     _check_layout("npu_fa", input_layout)
     layout = input_layout
     query, key, value = (_to_bnsd(t, head_num, layout) for t in (query, key, value))
-    if pse is not None or padding_mask is not None or prefix or actual_seq_qlen or actual_seq_kvlen:
-        raise NotImplementedError("npu_fa: pse / padding_mask / prefix / variable sequence lengths")
+    if padding_mask is not None or prefix or actual_seq_qlen or actual_seq_kvlen:
+        raise NotImplementedError("npu_fa: padding_mask / prefix / variable sequence lengths")
     if not (0.0 <= keep_prob <= 1.0):
         raise ValueError(f"npu_fa: keep_prob {keep_prob} outside [0, 1]")
     if query.size(1) != head_num:
@@ -117,9 +120,10 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
     # the graph pattern passes the divisor of the scores; the kernel multiplies
     real_scale = 1.0 / scale
     causal = _is_causal(query.size(2), atten_mask, pre_tockens, next_tockens, sparse_mode)
+    mask = None if causal else atten_mask  # under the causal modes the mask tensor is the library's compressed triangle
     seed = numels = 0
     head_dim = query.size(3)
-    if (keep_prob == 1.0 and query.dtype in (torch.bfloat16, torch.float16) and head_dim <= 128 and head_dim % 8 == 0
+    if (pse is None and mask is None and keep_prob == 1.0 and query.dtype in (torch.bfloat16, torch.float16) and head_dim <= 128 and head_dim % 8 == 0
             and head_dim > 0 and query.size(2) > 0 and key.size(2) > 0 and (not causal or query.size(2) == key.size(2))):
         # the MFMA kernel: bf16 or fp16, head dimension 128, any sequence lengths.  A smaller head
         # dimension is padded with zero columns (scores and statistics do not change, the extra output
@@ -130,14 +134,16 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
         if pad:
             out = out[..., :head_dim].contiguous()
     else:
-        # head dimensions above 128 or not a multiple of 8, fp32 and dropout: the same mathematics over library GEMMs.  The dropout seed comes from torch's CPU generator (torch.manual_seed makes a
+        # head dimensions above 128 or not a multiple of 8, fp32, dropout, a positional bias or a general mask: the
+        # same mathematics over library GEMMs.  The dropout seed comes from torch's CPU generator (torch.manual_seed makes a
         # run repeatable) and travels to the backward in the op's seed output, as in the reference's op.
         from .attention_backward import attention_forward_over_gemms
 
         if keep_prob < 1.0:
             seed = int(torch.randint(0, 1 << 62, (1,), dtype=torch.int64).item())
             numels = query.size(0) * query.size(1) * query.size(2) * key.size(2)
-        out, smax, ssum = attention_forward_over_gemms(query, key, value, real_scale, causal, keep_prob, seed)
+        out, smax, ssum = attention_forward_over_gemms(query, key, value, real_scale, causal, keep_prob, seed,
+                                                       pse=pse, atten_mask=mask)
     softmax_out = torch.empty([0], dtype=query.dtype, device=query.device)
     word = lambda v: torch.tensor([v], dtype=torch.int64)  # noqa: E731  seed / offset / numels live on the host
     return _from_bnsd(out, layout), smax, ssum, softmax_out, word(seed), word(0), word(numels)
@@ -157,8 +163,8 @@ def npu_fa_backward_gpu(query, key, value, dy, head_num, input_layout, *, pse=No
 
     _check_layout("npu_fa_backward", input_layout)
     layout = input_layout
-    if pse is not None or padding_mask is not None or prefix or actual_seq_qlen or actual_seq_kvlen:
-        raise NotImplementedError("npu_fa_backward: pse / padding_mask / prefix / variable sequence lengths")
+    if padding_mask is not None or prefix or actual_seq_qlen or actual_seq_kvlen:
+        raise NotImplementedError("npu_fa_backward: padding_mask / prefix / variable sequence lengths")
     if not (0.0 <= keep_prob <= 1.0):
         raise ValueError(f"npu_fa_backward: keep_prob {keep_prob} outside [0, 1]")
     if keep_prob < 1.0 and seed is None:
@@ -171,12 +177,14 @@ def npu_fa_backward_gpu(query, key, value, dy, head_num, input_layout, *, pse=No
         _to_bnsd(t, head_num, layout).contiguous() for t in (query, key, value, attention_in, dy)
     )
     causal = _is_causal(query.size(2), atten_mask, pre_tockens, next_tockens, sparse_mode)
-    dq, dk, dv = fused_attention_backward(
+    mask = None if causal else atten_mask
+    grads = fused_attention_backward(
         query, key, value, attention_in, dy, softmax_max, softmax_sum, 1.0 / scale_value, causal,
-        keep_prob=keep_prob, seed=int(seed.item()) if keep_prob < 1.0 else 0,
+        keep_prob=keep_prob, seed=int(seed.item()) if keep_prob < 1.0 else 0, pse=pse, atten_mask=mask,
     )
-    dq, dk, dv = (_from_bnsd(t, layout) for t in (dq, dk, dv))
-    return dq, dk, dv, torch.empty([0], dtype=query.dtype, device=query.device)
+    dq, dk, dv = (_from_bnsd(t, layout) for t in grads[:3])
+    dpse = grads[3] if len(grads) > 3 and grads[3] is not None else torch.empty([0], dtype=query.dtype, device=query.device)
+    return dq, dk, dv, dpse
 
 
 gpu_lib.impl("npu_fa_backward", npu_fa_backward_gpu)
@@ -214,7 +222,7 @@ def npu_fa_backward_meta(query, key, value, dy, head_num, input_layout, *, pse=N
         torch.empty_like(query).contiguous(),
         torch.empty_like(key).contiguous(),
         torch.empty_like(value).contiguous(),
-        torch.empty([0], dtype=query.dtype, device=query.device),
+        torch.empty_like(pse).contiguous() if pse is not None else torch.empty([0], dtype=query.dtype, device=query.device),
     )
 
 

@@ -403,6 +403,59 @@ def test_attention_op_reaches_the_fused_kernel_for_fp16_and_any_length(dtype, B,
             assert (g.float() - r).abs().max().item() <= 3e-2 * max(r.abs().max().item(), 1.0)
 
 
+@pytest.mark.parametrize("dtype,B,N,S,D,pse_shape,mask_shape", [
+    (torch.bfloat16, 2, 3, 128, 128, (1, 3, 128, 128), (2, 1, 128, 128)),
+    (torch.float32, 1, 2, 100, 64, (100, 100), None),
+    (torch.float16, 2, 2, 96, 128, None, (96, 96)),
+    (torch.float32, 2, 2, 64, 32, (2, 2, 64, 64), (1, 1, 64, 64)),
+])
+def test_attention_op_positional_bias_and_mask(dtype, B, N, S, D, pse_shape, mask_shape):
+    """pse (added to q k^T before the scaling) and a general atten_mask (non-zero = hidden) through
+    npu_fa / npu_fa_backward: softmax(mask(scale * (pse + q k^T))) v, as the fused op of the
+    reference's device library documents it (call site reference
+    inductor_x/npu_fusion_attention_graph.py:31; PARITY UNPINNED against that library, pinned here by
+    fp32 autograd of the written-out formula), outputs and gradients including the gradient of pse
+    in pse's own (broadcast) shape.  One query row has every key hidden: it returns zeros."""
+    announce(f"attention op pse {pse_shape} mask {mask_shape} {dtype} B={B} N={N} S={S} D={D}")
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
+    torch.manual_seed(31)
+    q, k, v = (torch.randn(B, N, S, D, device=DEV).to(dtype).requires_grad_() for _ in range(3))
+    pse = torch.randn(*pse_shape, device=DEV).to(dtype).requires_grad_() if pse_shape else None
+    mask = None
+    if mask_shape:
+        mask = torch.rand(*mask_shape, device=DEV) < 0.3
+        mask[..., 5, :] = True   # query 5 sees nothing
+        mask[..., 6, :] = False  # query 6 sees everything
+    inv = D ** 0.5
+    res = npu_fusion_attention_graph(q, k, v, N, "BNSD", pse, None, mask, scale=inv)
+    do = torch.randn_like(res[0])
+    res[0].backward(do)
+    qf, kf, vf = (t.detach().float().requires_grad_() for t in (q, k, v))
+    pf = pse.detach().float().requires_grad_() if pse is not None else None
+    s = qf @ kf.transpose(-1, -2)
+    if pf is not None:
+        s = s + pf
+    s = s / inv
+    if mask is not None:
+        s = s.masked_fill(mask, float("-inf"))
+    p = torch.softmax(s, -1)
+    p = torch.nan_to_num(p, nan=0.0)  # the row with every key hidden
+    ref = p @ vf
+    ref.backward(do.float())
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert (res[0].float() - ref).abs().max().item() <= tol * max(ref.abs().max().item(), 1.0)
+    if mask is not None:
+        assert res[0][..., 5, :].abs().max().item() == 0.0
+    gtol = 1e-4 if dtype == torch.float32 else 3e-2
+    pairs = [(q.grad, qf.grad), (k.grad, kf.grad), (v.grad, vf.grad)]
+    if pse is not None:
+        assert pse.grad is not None and pse.grad.shape == pse.shape
+        pairs.append((pse.grad, pf.grad))
+    for g, r in pairs:
+        assert (g.float() - r).abs().max().item() <= gtol * max(r.abs().max().item(), 1.0)
+
+
 def _unfused_fp32(q, k, v, inv, causal, keep=None, keep_prob=1.0):
     """fp32 autograd-able definition on [B, N, S, D] tensors; `keep` is a [B, N, S, S] dropout mask."""
     S = q.size(2)
