@@ -36,34 +36,68 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
 # copy kernel of known size in the same run.  Keyed by (configuration, path); an entry
 # applies only while the call still launches exactly the symbols that were profiled.
 MEASURED_TRAFFIC: dict = {
-    ('1', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_817_904, "write_bytes": 32_739,
+    ('1', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_817_825, "write_bytes": 32_732,
         "profile": "profiles/rowsum_f32_1024x4096_warm_pmc.txt"},
-    ('1', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 16_805_617, "write_bytes": 32_739,
+    ('1', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 16_805_538, "write_bytes": 32_732,
         "profile": "profiles/rowsum_f32_1024x4096_warm_pmc.txt"},
-    ('1cold', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_817_842, "write_bytes": 32_741,
+    ('1cold', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "fetch_bytes": 16_819_020, "write_bytes": 32_741,
         "profile": "profiles/rowsum_f32_1024x4096_cold_pmc.txt"},
-    ('2', 'kernel'): {"symbols": ["add_rmsnorm_bf16_b512_t512_i1"], "fetch_bytes": 134_289_921, "write_bytes": 134_238_139,
+    ('2', 'kernel'): {"symbols": ["add_rmsnorm_bf16_b512_t512_i1"], "fetch_bytes": 134_289_613, "write_bytes": 134_203_759,
         "profile": "profiles/add_rmsnorm_bf16_8192x4096_pmc.txt"},
-    ('2', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 134_298_112, "write_bytes": 134_342_635,
+    ('2', 'torch.compile'): {"symbols": ["hip_row_0"], "fetch_bytes": 134_297_805, "write_bytes": 134_282_709,
         "profile": "profiles/add_rmsnorm_bf16_8192x4096_pmc.txt"},
-    ('3', 'kernel'): {"symbols": ["col_mean_var_argmax_partial_f32_c32_r8_u8", "col_mean_var_argmax_final_f32_c4_s16"], "fetch_bytes": 138_610_822, "write_bytes": 536_096,
+    ('3', 'kernel'): {"symbols": ["col_mean_var_argmax_partial_f32_c32_r8_u8", "col_mean_var_argmax_final_f32_c4_s16"], "fetch_bytes": 138_623_472, "write_bytes": 536_020,
         "profile": "profiles/col_mean_var_argmax_f32_65536x512_pmc.txt"},
-    ('3', 'torch.compile'): {"symbols": ["hip_col_0_partial", "hip_col_0_final"], "fetch_bytes": 144_902_796, "write_bytes": 1_321_824,
+    ('3', 'torch.compile'): {"symbols": ["hip_col_0_partial", "hip_col_0_final"], "fetch_bytes": 144_903_176, "write_bytes": 1_321_636,
         "profile": "profiles/col_mean_var_argmax_f32_65536x512_pmc.txt"},
-    ('4a', 'kernel'): {"symbols": ["gather_rows_b16_b256_t128_r2"], "fetch_bytes": 66_448_240, "write_bytes": 67_196_420,
+    ('4a', 'kernel'): {"symbols": ["gather_rows_b16_b256_t128_r2"], "fetch_bytes": 66_422_229, "write_bytes": 67_173_304,
         "profile": "profiles/gather_rows_bf16_50304x1024_32768_pmc.txt"},
-    ('4a', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 65_560_705, "write_bytes": 67_087_919,
+    ('4a', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 65_564_107, "write_bytes": 67_078_688,
         "profile": "profiles/gather_rows_bf16_50304x1024_32768_pmc.txt"},
-    ('4b', 'kernel'): {"symbols": ["permute_copy_b16_b256_p16_t8x2"], "fetch_bytes": 268_432_000, "write_bytes": 268_550_121,
+    ('4b', 'kernel'): {"symbols": ["permute_copy_b16_b256_p16_t8x2"], "fetch_bytes": 268_432_000, "write_bytes": 268_533_552,
         "profile": "profiles/permute_0213_bf16_16x2048x32x128_pmc.txt"},
-    ('4b', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 268_441_216, "write_bytes": 268_551_202,
+    ('4b', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "fetch_bytes": 268_441_216, "write_bytes": 268_522_739,
         "profile": "profiles/permute_0213_bf16_16x2048x32x128_pmc.txt"},
+    ('f1a', 'kernel'): {"symbols": ["ring_forward_update_bf16_d128_s8"], "fetch_bytes": 251_735_288, "write_bytes": 126_523_105,
+        "profile": "profiles/ring_forward_update_bf16_8192x1x6144_n48_pmc.txt"},
+    ('f1a', 'torch.compile'): {"symbols": ["hip_pointwise_0", "hip_pointwise_1"], "fetch_bytes": 327_170_359, "write_bytes": 125_696_749,
+        "profile": "profiles/ring_forward_update_bf16_8192x1x6144_n48_pmc.txt"},
+    ('f1b', 'torch.compile'): {"symbols": ["hip_pointwise_0", "hip_pointwise_1"], "fetch_bytes": 410_535_752, "write_bytes": 202_736_322,
+        "profile": "profiles/ring_forward_update_lse_f32_1x48x8192x128_pmc.txt"},
+    ('f1c', 'torch.compile'): {"symbols": ["hip_pointwise_0", "hip_pointwise_0", "hip_pointwise_0"], "fetch_bytes": 604_001_787, "write_bytes": 301_749_079,
+        "profile": "profiles/ring_backward_update_bf16_3x2x16384x1x1536_pmc.txt"},
 }
 
 # Kernel durations (microseconds, average over the dispatches of a warm run) from the committed
 # rocprofv3 kernel traces of `bench.py --pmc-config <n>`: the benchmark definition's "GPU time" of a
 # graph is the sum over its kernels.  Keyed like MEASURED_TRAFFIC and used under the same rule.
 KERNEL_TRACE_US: dict = {
+    ('1', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "us": [4.1], "profile": "profiles/rowsum_f32_1024x4096_warm_pmc.txt"},
+    ('1', 'torch.compile'): {"symbols": ["hip_row_0"], "us": [4.04], "profile": "profiles/rowsum_f32_1024x4096_warm_pmc.txt"},
+    ('1cold', 'kernel'): {"symbols": ["fused_relu_sigmoid_rowsum_f32_b256_t256"], "us": [6.17], "profile": "profiles/rowsum_f32_1024x4096_cold_pmc.txt"},
+    ('2', 'kernel'): {"symbols": ["add_rmsnorm_bf16_b512_t512_i1"], "us": [37.99], "profile": "profiles/add_rmsnorm_bf16_8192x4096_pmc.txt"},
+    ('2', 'torch.compile'): {"symbols": ["hip_row_0"], "us": [37.56], "profile": "profiles/add_rmsnorm_bf16_8192x4096_pmc.txt"},
+    ('3', 'kernel'): {"symbols": ["col_mean_var_argmax_partial_f32_c32_r8_u8", "col_mean_var_argmax_final_f32_c4_s16"], "us": [23.65, 4.12], "profile": "profiles/col_mean_var_argmax_f32_65536x512_pmc.txt"},
+    ('3', 'torch.compile'): {"symbols": ["hip_col_0_partial", "hip_col_0_final"], "us": [24.02, 4.78], "profile": "profiles/col_mean_var_argmax_f32_65536x512_pmc.txt"},
+    ('4a', 'kernel'): {"symbols": ["gather_rows_b16_b256_t128_r2"], "us": [20.61], "profile": "profiles/gather_rows_bf16_50304x1024_32768_pmc.txt"},
+    ('4a', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "us": [20.31], "profile": "profiles/gather_rows_bf16_50304x1024_32768_pmc.txt"},
+    ('4b', 'kernel'): {"symbols": ["permute_copy_b16_b256_p16_t8x2"], "us": [76.29], "profile": "profiles/permute_0213_bf16_16x2048x32x128_pmc.txt"},
+    ('4b', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "us": [76.01], "profile": "profiles/permute_0213_bf16_16x2048x32x128_pmc.txt"},
+    ('f1a', 'kernel'): {"symbols": ["ring_forward_update_bf16_d128_s8"], "us": [59.16], "profile": "profiles/ring_forward_update_bf16_8192x1x6144_n48_pmc.txt"},
+    ('f1a', 'torch.compile'): {"symbols": ["hip_pointwise_0", "hip_pointwise_1"], "us": [11.9, 58.43], "profile": "profiles/ring_forward_update_bf16_8192x1x6144_n48_pmc.txt"},
+    ('f1b', 'torch.compile'): {"symbols": ["hip_pointwise_0", "hip_pointwise_1"], "us": [5.0, 92.55], "profile": "profiles/ring_forward_update_lse_f32_1x48x8192x128_pmc.txt"},
+    ('f1c', 'torch.compile'): {"symbols": ["hip_pointwise_0", "hip_pointwise_0", "hip_pointwise_0"], "us": [47.96, 47.96, 47.96], "profile": "profiles/ring_backward_update_bf16_3x2x16384x1x1536_pmc.txt"},
+    ('2cold', 'kernel'): {"symbols": ["add_rmsnorm_bf16_b512_t512_i1"], "us": [45.47], "profile": "profiles/kernel_traces_per_config.txt"},
+    ('2cold', 'torch.compile'): {"symbols": ["hip_row_0"], "us": [45.06], "profile": "profiles/kernel_traces_per_config.txt"},
+    ('3cold', 'kernel'): {"symbols": ["col_mean_var_argmax_partial_f32_c32_r8_u8", "col_mean_var_argmax_final_f32_c4_s16"], "us": [26.39, 4.01], "profile": "profiles/kernel_traces_per_config.txt"},
+    ('3cold', 'torch.compile'): {"symbols": ["hip_col_0_partial", "hip_col_0_final"], "us": [25.89, 4.74], "profile": "profiles/kernel_traces_per_config.txt"},
+    ('4acold', 'kernel'): {"symbols": ["gather_rows_b16_b256_t128_r2"], "us": [23.89], "profile": "profiles/kernel_traces_per_config.txt"},
+    ('4acold', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "us": [24.02], "profile": "profiles/kernel_traces_per_config.txt"},
+    ('4bcold', 'kernel'): {"symbols": ["permute_copy_b16_b256_p16_t8x2"], "us": [84.4], "profile": "profiles/kernel_traces_per_config.txt"},
+    ('4bcold', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "us": [86.53], "profile": "profiles/kernel_traces_per_config.txt"},
+    ('5', 'kernel'): {"symbols": ["fused_attention_fwd_bf16_d128_causal_v5"], "us": [595.45], "profile": "profiles/kernel_traces_per_config.txt"},
+    ('5', 'torch.compile'): {"symbols": ["fused_attention_fwd_bf16_d128_causal_v5"], "us": [595.45], "profile": "profiles/kernel_traces_per_config.txt"},
+    ('5b', 'kernel'): {"symbols": ["attention_bwd_stats_bf16_d128", "attention_bwd8_dk_bf16_d128_causal", "attention_bwd8_dv_bf16_d128_causal", "attention_bwd8_dq_bf16_d128_causal"], "us": [53.01, 994.78, 684.17, 851.43], "profile": "profiles/kernel_traces_per_config.txt"},
 }
 
 ALGO_BYTES = {
