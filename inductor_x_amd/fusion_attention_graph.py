@@ -12,14 +12,18 @@ The device implementation runs the MFMA kernel of this package.  As in the
 reference the op receives the *inverse* scale from the pattern and inverts it
 (:20-35, :162).  The reference's pattern carries no mask; a causal mask enters
 through the op's own arguments: sparse_mode 2 or 3, or next_tockens == 0 with
-pre_tockens covering the sequence.  Supported: layouts "BNSD", "BSH", "SBH"; the fused kernels take bf16, head
-dimension 128, no pse / padding mask; dropout (keep_prob < 1) runs the GEMM path; anything else raises.  Layouts
-"BSH" and "SBH" are viewed as [B, N, S, D], copied once into that order for the
-kernels and copied back.
-The backward op recomputes the probabilities from the saved row statistics inside fused
-gradient kernels (head dimension 128; kernels.fused_attention_backward) and falls back to the
-same mathematics over library GEMMs for other head dimensions (attention_backward.py); the
-training variant of the pattern is registered beside the inference one.
+pre_tockens covering the sequence.  Supported: layouts "BNSD", "BSH", "SBH" ("BSH" and "SBH" are
+viewed as [B, N, S, D], copied once into that order for the kernels and copied back).  The fused
+kernel takes bf16 and fp16 operands with a head dimension that is a multiple of 8 up to 128
+(smaller heads are zero-padded to 128) at any query and key lengths; a positional bias (pse), a
+general boolean mask, fp32 operands, other head dimensions and dropout (keep_prob < 1) run the same
+mathematics over library GEMMs; padding masks, prefixes, variable sequence lengths and band masks
+raise.
+The backward op recomputes the probabilities from the saved row statistics inside fused gradient
+kernels (bf16, head dimension up to 128, equal lengths that are multiples of 64;
+kernels.fused_attention_backward) and falls back to the GEMM formulation otherwise
+(attention_backward.py), which also returns the gradient of pse; the training variant of the
+pattern is registered beside the inference one.
 """
 from __future__ import annotations
 
