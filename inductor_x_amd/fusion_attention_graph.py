@@ -306,23 +306,32 @@ def _attention_replacement_1(query, key, value, inv_scale_factor, dropout_p):
     )[0]
 
 
-def _extra_check(match) -> bool:
-    """Only rewrite what the op can run: bf16 GPU tensors with head dim 128, query, key and value of
-    one shape and type (no cross attention: the kernels take one sequence length), and a positive
-    divisor of the scores when it is a constant.  Anything else stays on Inductor's own path."""
+def _extra_check(match, training: bool = False) -> bool:
+    """Only rewrite what the fused kernels run; anything else stays on Inductor's own path.
+    Inference graphs: bf16 or fp16 GPU tensors [B, S, N, 128], any sequence lengths, key and value of
+    one shape that may differ from the query's in its length (cross attention).  Training graphs,
+    whose backward runs the fused gradient kernels: bf16, query, key and value of one shape, a
+    sequence length that is a multiple of 64.  Either way the divisor of the scores, when it is a
+    constant, must be positive and finite."""
     try:
         q = match.kwargs["query"].meta["val"]
         k = match.kwargs["key"].meta["val"]
         v = match.kwargs["value"].meta["val"]
     except Exception:
         return False
-    if not (
-        q.device.type == "cuda" and q.dtype == torch.bfloat16 and q.dim() == 4 and q.size(3) == 128
-        and q.size(1) % 128 == 0
-    ):
+    if not (q.device.type == "cuda" and q.dim() == 4 and q.size(3) == 128 and q.size(1) > 0):
+        return False
+    if training:
+        if q.dtype != torch.bfloat16 or q.size(1) % 64 != 0 or tuple(k.shape) != tuple(q.shape):
+            return False
+    elif q.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    if k.dim() != 4 or k.size(1) <= 0 or (k.size(0), k.size(2), k.size(3)) != (q.size(0), q.size(2), q.size(3)):
+        return False
+    if tuple(v.shape) != tuple(k.shape):
         return False
     for t in (k, v):
-        if tuple(t.shape) != tuple(q.shape) or t.dtype != q.dtype or t.device != q.device:
+        if t.dtype != q.dtype or t.device != q.device:
             return False
     # the divisor of the scores: a keyword of the match when the pattern captured it, otherwise the
     # second operand of the division node that was matched
@@ -360,20 +369,24 @@ def register_fx_pass() -> None:
         replacement = partialize_and_update_signature(_attention_replacement_1, dropout_p=0.0)
         # The search function is traced once per element type: a softmax of 16-bit tensors
         # decomposes with conversions to fp32 and back that the fp32 trace does not contain, and
-        # bf16 is the type the kernels run (the reference traces fp32 only, :218-224).
+        # bf16 is the type the kernels run (the reference traces fp32 only, :218-224); and once more
+        # with a batch of one, for which the batched products trace to different view operations
+        # (Inductor's own attention patterns carry the same second variant).
         for dtype in (torch.float, torch.bfloat16, torch.half):
-            g = functools.partial(torch.empty, (2, 4, 8, 16), device=device, dtype=dtype)
-            register_replacement(
-                pattern, replacement, [g(), g(), g(), c()], fwd_only, joint_graph.patterns,
-                extra_check=_extra_check, scalar_workaround={},
-            )
-            # training: the same search function traced with its backward; the replacement's
-            # autograd.Function supplies npu_fa_backward (reference :196-204, without dropout)
-            gr = functools.partial(torch.empty, (2, 4, 8, 16), device=device, dtype=dtype, requires_grad=True)
-            register_replacement(
-                pattern, replacement, [gr(), gr(), gr(), c()], joint_fwd_bwd, joint_graph.patterns,
-                extra_check=_extra_check, scalar_workaround={},
-            )
+            for batch in (2, 1):
+                g = functools.partial(torch.empty, (batch, 4, 8, 16), device=device, dtype=dtype)
+                register_replacement(
+                    pattern, replacement, [g(), g(), g(), c()], fwd_only, joint_graph.patterns,
+                    extra_check=_extra_check, scalar_workaround={}, skip_duplicates=True,
+                )
+                # training: the same search function traced with its backward; the replacement's
+                # autograd.Function supplies npu_fa_backward (reference :196-204, without dropout)
+                gr = functools.partial(torch.empty, (batch, 4, 8, 16), device=device, dtype=dtype, requires_grad=True)
+                register_replacement(
+                    pattern, replacement, [gr(), gr(), gr(), c()], joint_fwd_bwd, joint_graph.patterns,
+                    extra_check=functools.partial(_extra_check, training=True), scalar_workaround={},
+                    skip_duplicates=True,
+                )
 
     original_lazy_init = joint_graph.lazy_init
 

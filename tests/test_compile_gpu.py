@@ -245,20 +245,20 @@ def test_attention_op_and_pattern():
     assert (out32 - ref).abs().max().item() <= 2e-2
 
 
-def test_attention_pattern_leaves_cross_attention_and_negative_divisors_alone():
-    """Query and key of different sequence lengths, or a negative divisor of the scores, are not
-    what the fused op runs: the pattern must not fire.  For cross attention the compiled result is
-    also compared with eager; with a negative divisor Inductor's own pattern hands the graph to the
-    library's flash attention, whose result for a negative scale is the library's business (it
-    differs from eager by several units on this stack), so only the rewrite is checked there."""
-    announce("compile attention pattern: cross attention / negative divisor")
+def test_attention_pattern_cross_attention_fp16_and_negative_divisors():
+    """Inference graphs: the pattern also fires for query and key of different sequence lengths
+    (cross attention), for fp16 and for lengths that are no multiple of the kernel's tiles, which
+    the fused kernel all runs; a negative divisor of the scores is not what the op runs and the
+    pattern must not fire (Inductor's own pattern then hands the graph to the library's flash
+    attention, whose result for a negative scale is the library's business, so only the rewrite is
+    checked there)."""
+    announce("compile attention pattern: cross attention / fp16 / ragged / negative divisor")
     from torch._inductor.utils import run_and_get_code
 
+    from inductor_x_amd import launcher
+
     torch.manual_seed(1)
-    B, Sq, Sk, N, D = 2, 256, 384, 4, 128
-    q = torch.randn(B, Sq, N, D, device=DEV).bfloat16()
-    k = torch.randn(B, Sk, N, D, device=DEV).bfloat16()
-    v = torch.randn(B, Sk, N, D, device=DEV).bfloat16()
+    N, D = 4, 128
 
     def make(div):
         def g(q, k, v):
@@ -267,15 +267,31 @@ def test_attention_pattern_leaves_cross_attention_and_negative_divisors_alone():
 
         return g
 
-    for args, div in (((q, k, v), D ** 0.5), ((q, q.clone(), q.clone()), -(D ** 0.5))):
+    for dtype, B, Sq, Sk, div, fires in (
+        (torch.bfloat16, 2, 256, 384, D ** 0.5, True),
+        (torch.float16, 2, 333, 333, D ** 0.5, True),
+        (torch.bfloat16, 1, 640, 640, D ** 0.5, True),
+        (torch.float16, 2, 200, 77, 9.0, True),
+        (torch.bfloat16, 2, 256, 256, -(D ** 0.5), False),
+    ):
+        q = torch.randn(B, Sq, N, D, device=DEV).to(dtype)
+        k = torch.randn(B, Sk, N, D, device=DEV).to(dtype)
+        v = torch.randn(B, Sk, N, D, device=DEV).to(dtype)
         g = make(div)
         torch._dynamo.reset()
-        with torch.no_grad():
-            out, codes = run_and_get_code(torch.compile(g), *args)
-            ref = g(*(t.float() for t in args))
-        assert "npu_graph.npu_fa" not in "\n".join(codes)
-        if div > 0:
+        launched = []
+        launcher.launch_log = launched
+        try:
+            with torch.no_grad():
+                out, codes = run_and_get_code(torch.compile(g), q, k, v)
+        finally:
+            launcher.launch_log = None
+        ref = g(q.float(), k.float(), v.float())
+        assert ("npu_graph.npu_fa" in "\n".join(codes)) == fires, (dtype, Sq, Sk, div)
+        if fires:
+            assert any(name.startswith("fused_attention_fwd_") for name in launched), launched
             assert (out.float() - ref).abs().max().item() <= 3e-2
+    torch._dynamo.reset()
 
 
 def test_ring_attention_forward_update():
