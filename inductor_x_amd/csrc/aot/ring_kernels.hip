@@ -25,6 +25,8 @@ RING_FWD_VARIANT(ring_forward_update_f32_d128_s8, float, 128, 8, false)
 RING_FWD_VARIANT(ring_forward_update_f32_d128_s8_nt, float, 128, 8, true)
 RING_FWD_VARIANT(ring_forward_update_bf16_d64_s8, bf16_t, 64, 8, false)
 RING_FWD_VARIANT(ring_forward_update_bf16_d64_s8_nt, bf16_t, 64, 8, true)
+RING_FWD_VARIANT(ring_forward_update_f16_d64_s8, f16_t, 64, 8, false)
+RING_FWD_VARIANT(ring_forward_update_f16_d64_s8_nt, f16_t, 64, 8, true)
 RING_FWD_VARIANT(ring_forward_update_f32_d64_s8, float, 64, 8, false)
 RING_FWD_VARIANT(ring_forward_update_f32_d64_s8_nt, float, 64, 8, true)
 

@@ -497,7 +497,7 @@ def permute_0213_contiguous(t: torch.Tensor, variant: Optional[tuple] = None) ->
 # ring-attention merge step: (prev_out, prev_max, prev_sum) + (cur_out, cur_max, cur_sum)
 # ---------------------------------------------------------------------------
 _RING_DTYPES = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}
-_RING_VARIANTS = [("bf16", 128, 8), ("bf16", 128, 16), ("f16", 128, 8), ("f32", 128, 8), ("bf16", 64, 8), ("f32", 64, 8)]
+_RING_VARIANTS = [("bf16", 128, 8), ("bf16", 128, 16), ("f16", 128, 8), ("f32", 128, 8), ("bf16", 64, 8), ("f16", 64, 8), ("f32", 64, 8)]
 
 
 @functools.lru_cache(maxsize=None)

@@ -92,7 +92,7 @@ def test_forward_update_reference_shapes(O, S, B, H, N, dtype):
 @pytest.mark.parametrize(
     "S,B,H,N,dtype",
     [(4096, 1, 6144, 48, torch.bfloat16), (4096, 1, 1536, 12, torch.float32), (37, 2, 5 * 128, 5, torch.bfloat16),
-     (100, 1, 3 * 64, 3, torch.float32), (33, 2, 17 * 128, 17, torch.float16)],
+     (100, 1, 3 * 64, 3, torch.float32), (33, 2, 17 * 128, 17, torch.float16), (65, 1, 9 * 64, 9, torch.float16)],
 )
 def test_forward_update_single_kernel(O, S, B, H, N, dtype):
     """The hand-written one-launch form (kernels.ring_forward_update; reference
