@@ -33,18 +33,27 @@ def _bmm_f32(a, b):
     return torch.bmm(a, b, out_dtype=torch.float32)
 
 
-def _heads_per_round(heads: int, S: int) -> int:
-    return max(1, min(heads, _SCORE_BYTES_BUDGET // max(2 * S * S * 4, 1)))
+def _heads_per_round(heads: int, Sq: int, Sk: int = None) -> int:
+    Sk = Sq if Sk is None else Sk
+    return max(1, min(heads, _SCORE_BYTES_BUDGET // max(2 * Sq * Sk * 4, 1)))
 
 
-def dropout_keep_mask(seed: int, first_head: int, heads: int, S: int, keep_prob: float, device):
-    """The [heads, S, S] mask of kept probabilities for heads first_head .. first_head + heads - 1 of
+def dropout_keep_mask(seed: int, first_head: int, heads: int, Sq: int, keep_prob: float, device, Sk: int = None):
+    """The [heads, Sq, Sk] mask of kept probabilities for heads first_head .. first_head + heads - 1 of
     a call whose dropout seed is `seed`: a uniform draw per entry from a generator seeded with
     seed + first_head, kept where it is below keep_prob.  Forward and backward walk the heads in the
     same rounds (_heads_per_round) and so regenerate identical masks from the seed alone."""
     gen = torch.Generator(device=device)
     gen.manual_seed((int(seed) + int(first_head)) & ((1 << 63) - 1))
-    return torch.rand(heads, S, S, device=device, generator=gen) < keep_prob
+    return torch.rand(heads, Sq, Sq if Sk is None else Sk, device=device, generator=gen) < keep_prob
+
+
+def _check_shapes(what: str, q, k, v, causal: bool):
+    """q [B, N, Sq, D]; k and v [B, N, Sk, D]; a causal mask needs Sq == Sk."""
+    if not (k.shape == v.shape and q.shape[:2] == k.shape[:2] and q.shape[3] == k.shape[3]):
+        raise ValueError(f"attention {what}: q [B, N, Sq, D] and k, v [B, N, Sk, D] must agree in B, N and D")
+    if causal and q.shape[2] != k.shape[2]:
+        raise ValueError(f"attention {what}: a causal mask needs equal query and key lengths")
 
 
 def _check_keep_prob(keep_prob: float) -> float:
@@ -68,7 +77,8 @@ def _per_head(t, B: int, N: int, Sq: int, Sk: int, what: str):
 def attention_forward_over_gemms(q, k, v, scale: float, causal: bool, keep_prob: float = 1.0, seed: int = 0,
                                  pse=None, atten_mask=None):
     """softmax(q k^T * scale [+ causal mask]) v with library GEMMs for shapes and element types the
-    fused forward kernels do not cover (any head dimension and sequence length; bf16, fp16, fp32).
+    fused forward kernels do not cover (q [B, N, Sq, D], k and v [B, N, Sk, D]: any head dimension
+    and sequence lengths, a causal mask needs Sq == Sk; bf16, fp16, fp32).
     Returns (out, softmax_max, softmax_sum) like kernels.fused_attention: the row statistics are
     fp32 [B, N, S, 8], the probabilities are rounded to the operand type before the second product
     and O(S^2) intermediates move through HBM, a bounded number of heads at a time.
@@ -83,19 +93,22 @@ def attention_forward_over_gemms(q, k, v, scale: float, causal: bool, keep_prob:
     for t in (q, k, v):
         if not (t.is_cuda and t.dtype in _GEMM_DTYPES and t.dtype == q.dtype and t.dim() == 4):
             raise ValueError("attention forward: q, k, v must be 4-D GPU tensors of one floating-point type")
-    if not (q.shape == k.shape == v.shape):
-        raise ValueError("attention forward: q, k, v must share one [B, N, S, D] shape")
+    _check_shapes("forward", q, k, v, causal)
     B, N, S, D = q.shape
+    Sk = k.shape[2]
     heads = B * N
-    qh, kh, vh = (t.contiguous().view(heads, S, D) for t in (q, k, v))
+    qh = q.contiguous().view(heads, S, D)
+    kh, vh = (t.contiguous().view(heads, Sk, D) for t in (k, v))
     out = torch.empty_like(qh)
     smax = torch.empty(heads, S, dtype=torch.float32, device=q.device)
     ssum = torch.empty(heads, S, dtype=torch.float32, device=q.device)
+    if heads and S and Sk == 0:
+        raise ValueError("attention forward: no keys")
     if heads and S:
-        chunk = _heads_per_round(heads, S)
+        chunk = _heads_per_round(heads, S, Sk)
         mask = torch.ones(S, S, dtype=torch.bool, device=q.device).triu_(1) if causal else None
-        bias = _per_head(pse, B, N, S, S, "pse") if pse is not None else None
-        hide = _per_head(atten_mask != 0, B, N, S, S, "atten_mask") if atten_mask is not None else None
+        bias = _per_head(pse, B, N, S, Sk, "pse") if pse is not None else None
+        hide = _per_head(atten_mask != 0, B, N, S, Sk, "atten_mask") if atten_mask is not None else None
         for h0 in range(0, heads, chunk):
             sl = slice(h0, min(h0 + chunk, heads))
             s = _bmm_f32(qh[sl], kh[sl].transpose(1, 2))
@@ -115,7 +128,7 @@ def attention_forward_over_gemms(q, k, v, scale: float, causal: bool, keep_prob:
                 l = torch.where(l == 0, torch.ones_like(l), l)
             smax[sl], ssum[sl] = m, l
             if keep_prob < 1.0:
-                p.mul_(dropout_keep_mask(seed, h0, sl.stop - h0, S, keep_prob, q.device)).mul_(inv_keep)
+                p.mul_(dropout_keep_mask(seed, h0, sl.stop - h0, S, keep_prob, q.device, Sk)).mul_(inv_keep)
             out[sl] = (_bmm_f32(p.to(q.dtype), vh[sl]) / l.unsqueeze(-1)).to(q.dtype)
     stats = lambda t: t.view(B, N, S, 1).expand(B, N, S, 8).contiguous()  # noqa: E731
     return out.view(B, N, S, D), stats(smax), stats(ssum)
@@ -123,8 +136,8 @@ def attention_forward_over_gemms(q, k, v, scale: float, causal: bool, keep_prob:
 
 def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale: float, causal: bool,
                              use_kernels=None, keep_prob: float = 1.0, seed: int = 0, pse=None, atten_mask=None):
-    """q, k, v, out, dout: [B, N, S, D] of one floating-point type; softmax_max / softmax_sum:
-    [B, N, S, 8] fp32 from the forward.  Returns (dq, dk, dv) in that type.  use_kernels: None = fused
+    """q, out, dout: [B, N, Sq, D] and k, v: [B, N, Sk, D] of one floating-point type; softmax_max /
+    softmax_sum: [B, N, Sq, 8] fp32 from the forward.  Returns (dq, dk, dv) in that type.  use_kernels: None = fused
     kernels where they apply (bf16, head dimension up to 128, sequence a multiple of 64, no dropout).
     keep_prob < 1 with the forward's seed regenerates the forward's dropout mask (GEMM path only).
     With pse or atten_mask (GEMM path only) the result has a fourth member, the gradient of pse in
@@ -163,28 +176,31 @@ def _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale: fl
     for t in (q, k, v, out, dout):
         if not (t.is_cuda and t.dtype in _GEMM_DTYPES and t.dtype == q.dtype and t.dim() == 4):
             raise ValueError("attention backward: q, k, v, out, dout must be 4-D GPU tensors of one floating-point type")
-    if not (q.shape == k.shape == v.shape == out.shape == dout.shape):
-        raise ValueError("attention backward: q, k, v, out, dout must share one [B, N, S, D] shape")
+    _check_shapes("backward", q, k, v, causal)
+    if not (q.shape == out.shape == dout.shape):
+        raise ValueError("attention backward: q, out and dout must share one [B, N, Sq, D] shape")
     B, N, S, D = q.shape
+    Sk = k.shape[2]
     if softmax_max.shape != (B, N, S, 8) or softmax_sum.shape != (B, N, S, 8):
         raise ValueError("attention backward: softmax statistics must be [B, N, S, 8]")
     heads = B * N
-    qh, kh, vh, oh, doh = (t.contiguous().view(heads, S, D) for t in (q, k, v, out, dout))
+    qh, oh, doh = (t.contiguous().view(heads, S, D) for t in (q, out, dout))
+    kh, vh = (t.contiguous().view(heads, Sk, D) for t in (k, v))
     m = softmax_max.reshape(heads, S, 8)[..., 0].contiguous()
     l = softmax_sum.reshape(heads, S, 8)[..., 0].contiguous()
     dq = torch.empty_like(qh)
     dk = torch.empty_like(kh)
     dv = torch.empty_like(vh)
-    if heads == 0 or S == 0:
-        return dq.view(B, N, S, D), dk.view(B, N, S, D), dv.view(B, N, S, D)
-    chunk = _heads_per_round(heads, S)
+    if heads == 0 or S == 0 or Sk == 0:
+        return dq.view(B, N, S, D), dk.zero_().view(B, N, Sk, D), dv.zero_().view(B, N, Sk, D)
+    chunk = _heads_per_round(heads, S, Sk)
     mask = None
     if causal:
         mask = torch.ones(S, S, dtype=torch.bool, device=q.device).triu_(1)
     extras = pse is not None or atten_mask is not None
-    bias = _per_head(pse, B, N, S, S, "pse") if pse is not None else None
-    hide = _per_head(atten_mask != 0, B, N, S, S, "atten_mask") if atten_mask is not None else None
-    dpse = torch.zeros(heads, S, S, dtype=torch.float32, device=q.device) if pse is not None else None
+    bias = _per_head(pse, B, N, S, Sk, "pse") if pse is not None else None
+    hide = _per_head(atten_mask != 0, B, N, S, Sk, "atten_mask") if atten_mask is not None else None
+    dpse = torch.zeros(heads, S, Sk, dtype=torch.float32, device=q.device) if pse is not None else None
     for h0 in range(0, heads, chunk):
         sl = slice(h0, min(h0 + chunk, heads))
         qc, kc, vc, oc, doc = qh[sl], kh[sl], vh[sl], oh[sl], doh[sl]
@@ -200,7 +216,7 @@ def _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale: fl
         p = s.exp_().div_(l[sl].unsqueeze(-1))
         dp = _bmm_f32(doc, vc.transpose(1, 2))
         if keep_prob < 1.0:
-            keep = dropout_keep_mask(seed, h0, sl.stop - h0, S, keep_prob, q.device)
+            keep = dropout_keep_mask(seed, h0, sl.stop - h0, S, keep_prob, q.device, Sk)
             dv[sl] = torch.bmm((p * keep).mul_(inv_keep).to(q.dtype).transpose(1, 2), doc)
             dp.mul_(keep).mul_(inv_keep)
             del keep
@@ -213,12 +229,12 @@ def _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale: fl
         ds16 = ds.to(q.dtype)
         dq[sl] = torch.bmm(ds16, kc)
         dk[sl] = torch.bmm(ds16.transpose(1, 2), qc)
-    grads = (dq.view(B, N, S, D), dk.view(B, N, S, D), dv.view(B, N, S, D))
+    grads = (dq.view(B, N, S, D), dk.view(B, N, Sk, D), dv.view(B, N, Sk, D))
     if not extras:
         return grads
     if dpse is not None:
         # fold the [B, N, S, S] gradient onto the axes pse broadcast over
-        g = dpse.view(B, N, S, S)
+        g = dpse.view(B, N, S, Sk)
         shape = pse.shape if pse.dim() == 4 else (1, 1) + tuple(pse.shape)
         for axis in (0, 1):
             if shape[axis] == 1 and g.shape[axis] != 1:

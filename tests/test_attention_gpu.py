@@ -352,6 +352,36 @@ def test_attention_op_outside_the_fused_kernels(dtype, B, N, S, D, causal):
         assert (g.float() - r).abs().max().item() <= (1e-4 if dtype == torch.float32 else 3e-2) * max(r.abs().max().item(), 1.0)
 
 
+@pytest.mark.parametrize("dtype,B,N,Sq,Sk,D", [
+    (torch.bfloat16, 2, 3, 256, 384, 128),   # fused forward, gradients over GEMMs (the gradient kernels take one length)
+    (torch.float16, 1, 2, 100, 333, 64),     # padded head, ragged lengths
+    (torch.float32, 1, 2, 70, 45, 40),       # GEMMs both ways
+])
+def test_attention_op_cross_attention_gradients(dtype, B, N, Sq, Sk, D):
+    """Query and key of different lengths through npu_fa and its backward: output and the three
+    gradients (dk, dv in the key's shape) against fp32 autograd of the unfused graph."""
+    announce(f"attention op cross attention {dtype} B={B} N={N} Sq={Sq} Sk={Sk} D={D}")
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
+    torch.manual_seed(21)
+    q = torch.randn(B, N, Sq, D, device=DEV).to(dtype).requires_grad_()
+    k, v = (torch.randn(B, N, Sk, D, device=DEV).to(dtype).requires_grad_() for _ in range(2))
+    do = torch.randn(B, N, Sq, D, device=DEV).to(dtype)
+    inv = D ** 0.5
+    out = npu_fusion_attention_graph(q, k, v, N, "BNSD", scale=inv)[0]
+    out.backward(do)
+    qf, kf, vf = (t.detach().float().requires_grad_() for t in (q, k, v))
+    ref = torch.softmax((qf @ kf.transpose(-1, -2)) / inv, -1) @ vf
+    ref.backward(do.float())
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert out.shape == q.shape and (out.float() - ref).abs().max().item() <= tol * max(ref.abs().max().item(), 1.0)
+    for g, r, like in zip((q.grad, k.grad, v.grad), (qf.grad, kf.grad, vf.grad), (q, k, v)):
+        assert g.shape == like.shape and g.dtype == dtype
+        assert (g.float() - r).abs().max().item() <= (1e-4 if dtype == torch.float32 else 3e-2) * max(r.abs().max().item(), 1.0)
+    with pytest.raises(ValueError):  # a causal mask is defined for equal lengths only
+        npu_fusion_attention_graph(q.detach().float(), k.detach().float(), v.detach().float(), N, "BNSD", scale=inv, sparse_mode=3)
+
+
 @pytest.mark.parametrize("dtype,B,N,Sq,Sk,causal,D", [
     (torch.float16, 1, 3, 200, 200, True, 128), (torch.float16, 2, 2, 512, 512, False, 128),
     (torch.bfloat16, 1, 2, 100, 300, False, 128), (torch.bfloat16, 1, 2, 77, 77, True, 128),
