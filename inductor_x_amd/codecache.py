@@ -45,8 +45,19 @@ HIPCC_FLAGS = (
 )
 
 
+# second attempt after an internal compiler error (see compile_source)
+BACKEND_ERROR_RETRY_FLAGS = ("-fno-slp-vectorize",)
+
+
 class CompileError(RuntimeError):
     pass
+
+
+def _first_lines(stderr: str, n: int = 3) -> str:
+    """The head of a long compiler message (the tail alone loses the line that names the error)."""
+    if len(stderr) <= 4000:
+        return ""
+    return "\n".join(stderr.splitlines()[:n]) + "\n[...]\n"
 
 
 def hipcc_path() -> str:
@@ -188,8 +199,18 @@ def compile_source(
                 tmp_out = os.path.join(tmp, "out.hsaco")
                 cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, "-I", include_dir or CSRC_DIR, "-o", tmp_out, src]
                 proc = subprocess.run(cmd, capture_output=True, text=True)
+                if proc.returncode != 0 and "error in backend" in proc.stderr:
+                    # The compiler itself gave up, not the source: with packed fp32 instructions switched off,
+                    # this release cannot select some two-element float vectors that its SLP vectorizer forms
+                    # ("Cannot select: v2f32 = bitcast", seen on a generated pointwise kernel with a negated
+                    # select beside an erf).  Without that vectorizer the same source compiles; the code object
+                    # is stored under the key of the request.
+                    first = proc.stderr
+                    proc = subprocess.run(cmd[:-1] + list(BACKEND_ERROR_RETRY_FLAGS) + [src], capture_output=True, text=True)
+                    if proc.returncode != 0:
+                        proc.stderr = _first_lines(first) + proc.stderr
                 if proc.returncode != 0 or not os.path.exists(tmp_out):
-                    raise CompileError(f"hipcc failed for {label} (key {key}):\n{proc.stderr[-4000:]}")
+                    raise CompileError(f"hipcc failed for {label} (key {key}):\n{_first_lines(proc.stderr)}{proc.stderr[-4000:]}")
                 final_tmp = out + f".tmp{os.getpid()}"
                 shutil.copyfile(tmp_out, final_tmp)
                 os.replace(final_tmp, out)

@@ -110,6 +110,45 @@ def test_codecache_compile_hit_and_error(tmp_path, monkeypatch):
     assert "not_a_symbol" in str(e.value)
 
 
+BACKEND_ERROR_KERNEL = r'''
+#include "mi/codegen.h"
+// a generated pointwise kernel (negated select beside an erf, a second output with atan2 / expm1) on which
+// this compiler release stops with "Cannot select: v2f32 = bitcast" when packed fp32 instructions are off
+extern "C" __global__ __launch_bounds__(256) void hip_pointwise_0(const mi::bf16_t* __restrict__ in_ptr0, mi::bf16_t* __restrict__ out_ptr0, mi::bf16_t* __restrict__ out_ptr1, const int xnumel) {
+    constexpr int VEC = 8;
+    const int x0 = (static_cast<int>(blockIdx.x) * 256 + threadIdx.x) * VEC;
+    if (x0 >= xnumel) return;
+    auto tmp0 = mi::cast<float>(mi::vload_u<VEC>(in_ptr0 + (x0)));
+    auto tmp1 = mi::sin(tmp0);
+    auto tmp3 = 0.5f;
+    auto tmp10 = (tmp0 * tmp3) * (mi::erf(tmp0 * 0.7071067811865476f) + 1.0f);
+    auto tmp14 = mi::where(tmp1 > tmp10, tmp1, tmp10 * tmp3);
+    auto tmp15 = (-tmp14);
+    auto tmp16 = mi::abs(tmp0);
+    auto tmp19 = mi::reciprocal(tmp16 + tmp3) * 1.0f;
+    auto tmp21 = tmp19 * tmp19 * tmp19;
+    auto tmp26 = mi::atan2(tmp0, tmp16 + 0.1f) + (tmp0 + tmp0);
+    auto tmp29 = mi::truediv(tmp21, mi::abs(tmp26) + tmp3);
+    auto tmp33 = mi::truediv(tmp0, mi::abs(mi::maximum(tmp0, tmp0)) + tmp3);
+    auto tmp37 = mi::cast<float>(tmp0 > 0.0f) + tmp0;
+    auto tmp44 = mi::expm1(mi::minimum(mi::maximum(tmp37, -5.0f), 5.0f));
+    mi::vstore<VEC>(out_ptr0 + (x0), tmp15);
+    mi::vstore<VEC>(out_ptr1 + (x0), mi::maximum(tmp29, mi::maximum(tmp33, tmp44)));
+}
+'''
+
+
+def test_codecache_retries_an_internal_compiler_error(tmp_path, monkeypatch):
+    """A source on which the compiler's backend gives up is compiled once more without the SLP
+    vectorizer and stored under the key of the request; a source that is wrong still fails."""
+    from inductor_x_amd import codecache
+
+    monkeypatch.setenv("INDUCTOR_X_AMD_CACHE", str(tmp_path))
+    path = codecache.compile_source(BACKEND_ERROR_KERNEL, label="ice")
+    assert os.path.getsize(path) > 0 and os.path.basename(path) == codecache.source_key(BACKEND_ERROR_KERNEL) + ".hsaco"
+    assert codecache.lookup(codecache.source_key(BACKEND_ERROR_KERNEL)) == path
+
+
 def test_aot_code_objects_are_built_for_gfx950(built):
     from inductor_x_amd import codecache
 
