@@ -1,6 +1,6 @@
 """Backward of the fused attention forward (npu_graph::npu_fa_backward).
 
-Two paths.  bf16 with a head dimension up to 128 (a multiple of 8; smaller ones are padded with zero columns)
+Two paths.  bf16 or fp16 with a head dimension up to 128 (a multiple of 8; smaller ones are padded with zero columns)
 and a sequence length that is a multiple of 64 runs the fused MFMA
 kernels (kernels.fused_attention_backward, csrc/mi/attention_bwd_w8.h).  Other shapes run the matrix
 products as library GEMMs (torch.bmm, hipBLASLt underneath) on a bounded number of heads at a time
@@ -138,7 +138,8 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
                              use_kernels=None, keep_prob: float = 1.0, seed: int = 0, pse=None, atten_mask=None):
     """q, out, dout: [B, N, Sq, D] and k, v: [B, N, Sk, D] of one floating-point type; softmax_max /
     softmax_sum: [B, N, Sq, 8] fp32 from the forward.  Returns (dq, dk, dv) in that type.  use_kernels: None = fused
-    kernels where they apply (bf16, head dimension up to 128, sequence a multiple of 64, no dropout).
+    kernels where they apply (bf16 or fp16, head dimension up to 128, one shape for q, k and v, a sequence
+    length that is a multiple of 64, no dropout).
     keep_prob < 1 with the forward's seed regenerates the forward's dropout mask (GEMM path only).
     With pse or atten_mask (GEMM path only) the result has a fourth member, the gradient of pse in
     pse's own shape (None without pse)."""
@@ -147,7 +148,7 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
             raise NotImplementedError("attention backward: the fused kernels take no bias or mask")
         return _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale, causal, keep_prob, seed,
                                     pse=pse, atten_mask=atten_mask)
-    fits = (q.dim() == 4 and q.dtype == torch.bfloat16 and 0 < q.size(3) <= 128 and q.size(3) % 8 == 0
+    fits = (q.dim() == 4 and q.dtype in (torch.bfloat16, torch.float16) and 0 < q.size(3) <= 128 and q.size(3) % 8 == 0
             and q.size(2) % 64 == 0 and q.size(2) > 0 and q.shape == k.shape and keep_prob == 1.0)
     if use_kernels is None:
         use_kernels = fits

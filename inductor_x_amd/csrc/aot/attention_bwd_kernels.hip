@@ -1,4 +1,4 @@
-// Fused attention backward instantiations (bf16, head dimension 128): eight wavefronts per
+// Fused attention backward instantiations (bf16 and fp16, head dimension 128): eight wavefronts per
 // workgroup on 256 rows, a statistics pass and separate dQ, dK and dV kernels (mi/attention_bwd_w8.h).
 // Workgroup -> (head, block): consecutive workgroup ids go to consecutive dies, so the heads of
 // one die share its L2.
@@ -18,10 +18,13 @@ __device__ __forceinline__ bool bwd_block_of(int n_heads, int n_blocks, int& hea
   return head < n_heads;
 }
 
-extern "C" __global__ __launch_bounds__(256) void attention_bwd_stats_bf16_d128(
-    const bf16_t* o, const bf16_t* d_o, const float* smax, const float* ssum, float* stats, int rows) {
-  attention_bwd_stats(o, d_o, smax, ssum, stats, rows);
-}
+#define BWD_STATS(NAME, T)                                                                             \
+  extern "C" __global__ __launch_bounds__(256) void NAME(const T* o, const T* d_o, const float* smax,  \
+                                                         const float* ssum, float* stats, int rows) {  \
+    attention_bwd_stats<T>(o, d_o, smax, ssum, stats, rows);                                           \
+  }
+BWD_STATS(attention_bwd_stats_bf16_d128, bf16_t)
+BWD_STATS(attention_bwd_stats_f16_d128, f16_t)
 
 // Work unit of a workgroup: one block of 256 rows, or under a causal mask the pair of blocks
 // (u, n - 1 - u), whose tile counts add up to the same number for every u, so that all
@@ -44,26 +47,32 @@ __device__ __forceinline__ void bwd8_for_blocks(int n_heads, int S, Body&& body)
   }
 }
 
-#define BWD8_DQ(NAME, CAUSAL)                                                                          \
+#define BWD8_DQ(NAME, T, CAUSAL)                                                                       \
   extern "C" __global__ __launch_bounds__(512, 1) void NAME(                                           \
-      const bf16_t* q, const bf16_t* k, const bf16_t* v, const bf16_t* d_o, const float* stats,         \
-      bf16_t* dq, int n_heads, int S, float scale) {                                                   \
+      const T* q, const T* k, const T* v, const T* d_o, const float* stats, T* dq, int n_heads, int S, \
+      float scale) {                                                                                   \
     bwd8_for_blocks<CAUSAL>(n_heads, S, [&](int head, int block) {                                     \
-      attention_bwd8_dq<CAUSAL>(q, k, v, d_o, stats, dq, S, block, head, scale);                       \
+      attention_bwd8_dq<T, CAUSAL>(q, k, v, d_o, stats, dq, S, block, head, scale);                    \
     });                                                                                                \
   }
-BWD8_DQ(attention_bwd8_dq_bf16_d128_causal, true)
-BWD8_DQ(attention_bwd8_dq_bf16_d128_full, false)
+BWD8_DQ(attention_bwd8_dq_bf16_d128_causal, bf16_t, true)
+BWD8_DQ(attention_bwd8_dq_bf16_d128_full, bf16_t, false)
+BWD8_DQ(attention_bwd8_dq_f16_d128_causal, f16_t, true)
+BWD8_DQ(attention_bwd8_dq_f16_d128_full, f16_t, false)
 
-#define BWD8_DKV(NAME, CAUSAL, WHICH)                                                                  \
+#define BWD8_DKV(NAME, T, CAUSAL, WHICH)                                                               \
   extern "C" __global__ __launch_bounds__(512, 1) void NAME(                                           \
-      const bf16_t* q, const bf16_t* k, const bf16_t* v, const bf16_t* d_o, const float* stats,         \
-      bf16_t* out, int n_heads, int S, float scale) {                                                  \
+      const T* q, const T* k, const T* v, const T* d_o, const float* stats, T* out, int n_heads,       \
+      int S, float scale) {                                                                            \
     bwd8_for_blocks<CAUSAL>(n_heads, S, [&](int head, int block) {                                     \
-      attention_bwd8_dkv<CAUSAL, WHICH>(q, k, v, d_o, stats, out, S, block, head, scale);              \
+      attention_bwd8_dkv<T, CAUSAL, WHICH>(q, k, v, d_o, stats, out, S, block, head, scale);           \
     });                                                                                                \
   }
-BWD8_DKV(attention_bwd8_dk_bf16_d128_causal, true, 0)
-BWD8_DKV(attention_bwd8_dk_bf16_d128_full, false, 0)
-BWD8_DKV(attention_bwd8_dv_bf16_d128_causal, true, 1)
-BWD8_DKV(attention_bwd8_dv_bf16_d128_full, false, 1)
+BWD8_DKV(attention_bwd8_dk_bf16_d128_causal, bf16_t, true, 0)
+BWD8_DKV(attention_bwd8_dk_bf16_d128_full, bf16_t, false, 0)
+BWD8_DKV(attention_bwd8_dv_bf16_d128_causal, bf16_t, true, 1)
+BWD8_DKV(attention_bwd8_dv_bf16_d128_full, bf16_t, false, 1)
+BWD8_DKV(attention_bwd8_dk_f16_d128_causal, f16_t, true, 0)
+BWD8_DKV(attention_bwd8_dk_f16_d128_full, f16_t, false, 0)
+BWD8_DKV(attention_bwd8_dv_f16_d128_causal, f16_t, true, 1)
+BWD8_DKV(attention_bwd8_dv_f16_d128_full, f16_t, false, 1)

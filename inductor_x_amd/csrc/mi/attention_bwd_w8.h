@@ -1,4 +1,4 @@
-// Fused attention backward (bf16, head dimension 128): eight wavefronts per workgroup, two per
+// Fused attention backward (bf16 or fp16, head dimension 128): eight wavefronts per workgroup, two per
 // SIMD, three kernels after a small statistics pass, no atomics.
 //
 // With P = exp(S - m) / l recomputed from the forward's row statistics (S = Q K^T * scale,
@@ -58,7 +58,8 @@ constexpr float kBwd8Log2e = 1.4426950408889634f;
 #endif
 
 // stats[row] = (m log2 e + log2 l, sum_d dO[row, d] * O[row, d]); 16 lanes per row.
-__device__ __forceinline__ void attention_bwd_stats(const bf16_t* __restrict__ O, const bf16_t* __restrict__ dO,
+template <typename T>
+__device__ __forceinline__ void attention_bwd_stats(const T* __restrict__ O, const T* __restrict__ dO,
                                                     const float* __restrict__ softmax_max,
                                                     const float* __restrict__ softmax_sum,
                                                     float* __restrict__ stats, int rows) {
@@ -66,8 +67,9 @@ __device__ __forceinline__ void attention_bwd_stats(const bf16_t* __restrict__ O
   const int part = threadIdx.x & 15;
   float acc = 0.f;
   if (row < rows) {
-    const bf16x8_t o = *reinterpret_cast<const bf16x8_t*>(O + static_cast<size_t>(row) * kAttnD + 8 * part);
-    const bf16x8_t d = *reinterpret_cast<const bf16x8_t*>(dO + static_cast<size_t>(row) * kAttnD + 8 * part);
+    typedef typename AttnElem<T>::x8 x8_t;
+    const x8_t o = *reinterpret_cast<const x8_t*>(O + static_cast<size_t>(row) * kAttnD + 8 * part);
+    const x8_t d = *reinterpret_cast<const x8_t*>(dO + static_cast<size_t>(row) * kAttnD + 8 * part);
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc = fmaf(static_cast<float>(o[e]), static_cast<float>(d[e]), acc);
   }
@@ -83,7 +85,7 @@ __device__ __forceinline__ void attention_bwd_stats(const bf16_t* __restrict__ O
   }
 }
 
-// Staging of a [64][128] bf16 tile by 512 threads.  Row form: 2 x 16 bytes per thread, stored
+// Staging of a [64][128] tile of 16-bit elements by 512 threads.  Row form: 2 x 16 bytes per thread, stored
 // row-major.  Column form: 4 rows x 4 columns per thread (4 x 8 bytes), stored transposed with the
 // row index (the contraction axis of the MFMA that reads the tile) permuted, and optionally
 // row-major as well.
@@ -93,29 +95,34 @@ struct Bwd8RowStage {
 struct Bwd8ColStage {
   u32x2_t r[4];
 };
-__device__ __forceinline__ void bwd8_load(Bwd8RowStage& t, const bf16_t* __restrict__ src, int tid) {
+template <typename T>
+__device__ __forceinline__ void bwd8_load(Bwd8RowStage& t, const T* __restrict__ src, int tid) {
   const int row = tid >> 4, col = (tid & 15) * 8;
 #pragma unroll
   for (int u = 0; u < 2; ++u)
     t.r[u] = *reinterpret_cast<const u32x4_t*>(src + static_cast<size_t>(row + 32 * u) * kAttnD + col);
 }
-__device__ __forceinline__ void bwd8_store_rows(const Bwd8RowStage& t, bf16_t* dst, int tid) {
+template <typename T>
+__device__ __forceinline__ void bwd8_store_rows(const Bwd8RowStage& t, T* dst, int tid) {
   const int row = tid >> 4, col = (tid & 15) * 8;
 #pragma unroll
   for (int u = 0; u < 2; ++u) *reinterpret_cast<u32x4_t*>(dst + (row + 32 * u) * kAttnKStride + col) = t.r[u];
 }
-__device__ __forceinline__ void bwd8_load(Bwd8ColStage& t, const bf16_t* __restrict__ src, int tid) {
+template <typename T>
+__device__ __forceinline__ void bwd8_load(Bwd8ColStage& t, const T* __restrict__ src, int tid) {
   const int rg = tid >> 5, cg = tid & 31;
 #pragma unroll
   for (int u = 0; u < 4; ++u)
     t.r[u] = *reinterpret_cast<const u32x2_t*>(src + static_cast<size_t>(4 * rg + u) * kAttnD + 4 * cg);
 }
-__device__ __forceinline__ void bwd8_store_rows(const Bwd8ColStage& t, bf16_t* dst, int tid) {
+template <typename T>
+__device__ __forceinline__ void bwd8_store_rows(const Bwd8ColStage& t, T* dst, int tid) {
   const int rg = tid >> 5, cg = tid & 31;
 #pragma unroll
   for (int u = 0; u < 4; ++u) *reinterpret_cast<u32x2_t*>(dst + (4 * rg + u) * kAttnKStride + 4 * cg) = t.r[u];
 }
-__device__ __forceinline__ void bwd8_store_cols(const Bwd8ColStage& t, bf16_t* dst, int tid) {
+template <typename T>
+__device__ __forceinline__ void bwd8_store_cols(const Bwd8ColStage& t, T* dst, int tid) {
   const int rg = tid >> 5, cg = tid & 31;
   const int pos = attn_vt_pos(4 * rg);
 #pragma unroll
@@ -131,11 +138,13 @@ __device__ __forceinline__ void bwd8_store_cols(const Bwd8ColStage& t, bf16_t* d
     *reinterpret_cast<u32x2_t*>(dst + attn_vt_offset(4 * cg + 2 * e2 + 1, pos)) = hi;
   }
 }
-__device__ __forceinline__ bf16x8_t bwd8_row_frag(const bf16_t* tile, int row, int s, int g) {
-  return *reinterpret_cast<const bf16x8_t*>(tile + row * kAttnKStride + 16 * s + 8 * g);
+template <typename T>
+__device__ __forceinline__ typename AttnElem<T>::x8 bwd8_row_frag(const T* tile, int row, int s, int g) {
+  return *reinterpret_cast<const typename AttnElem<T>::x8*>(tile + row * kAttnKStride + 16 * s + 8 * g);
 }
-__device__ __forceinline__ bf16x8_t bwd8_col_frag(const bf16_t* tile, int row, int t, int g) {
-  return *reinterpret_cast<const bf16x8_t*>(tile + attn_vt_offset(row, 16 * t + 8 * g));
+template <typename T>
+__device__ __forceinline__ typename AttnElem<T>::x8 bwd8_col_frag(const T* tile, int row, int t, int g) {
+  return *reinterpret_cast<const typename AttnElem<T>::x8*>(tile + attn_vt_offset(row, 16 * t + 8 * g));
 }
 // Accumulators (transposed: lane = row of the output, registers = head dimension) of one wavefront's
 // 32 rows -> memory.  Stored from the registers a wavefront instruction would write 32 separate
@@ -145,9 +154,10 @@ __device__ __forceinline__ bf16x8_t bwd8_col_frag(const bf16_t* tile, int row, i
 // STAGED = false stores from the registers (the causal kernels: they spill registers already and
 // the staging costs them more than it saves -- measured at [4,32,4096,128]: 2.44 against 2.42 ms for
 // the three causal kernels, 4.19 against 4.24 ms for the unmasked ones).
-template <bool STAGED>
-__device__ __forceinline__ void bwd8_store_acc(bf16_t* __restrict__ dst_block, const f32x16_t (&acc)[4], float factor,
-                                               bf16_t* stage, int lane, int rows) {
+template <bool STAGED, typename T>
+__device__ __forceinline__ void bwd8_store_acc(T* __restrict__ dst_block, const f32x16_t (&acc)[4], float factor,
+                                               T* stage, int lane, int rows) {
+  typedef typename AttnElem<T>::x4 x4_t;
   const int li = lane & 31, g = lane >> 5;
   if constexpr (!STAGED) {
   if (li < rows) {
@@ -155,10 +165,10 @@ __device__ __forceinline__ void bwd8_store_acc(bf16_t* __restrict__ dst_block, c
     for (int db = 0; db < 4; ++db)
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
-        bf16x4_t o4;
+        x4_t o4;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o4[e] = static_cast<bf16_t>(acc[db][4 * rq + e] * factor);
-        *reinterpret_cast<bf16x4_t*>(dst_block + li * kAttnD + 32 * db + 8 * rq + 4 * g) = o4;
+        for (int e = 0; e < 4; ++e) o4[e] = static_cast<T>(acc[db][4 * rq + e] * factor);
+        *reinterpret_cast<x4_t*>(dst_block + li * kAttnD + 32 * db + 8 * rq + 4 * g) = o4;
       }
   }
   return;
@@ -167,10 +177,10 @@ __device__ __forceinline__ void bwd8_store_acc(bf16_t* __restrict__ dst_block, c
   for (int db = 0; db < 4; ++db)
 #pragma unroll
     for (int rq = 0; rq < 4; ++rq) {
-      bf16x4_t o4;
+      x4_t o4;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o4[e] = static_cast<bf16_t>(acc[db][4 * rq + e] * factor);
-      *reinterpret_cast<bf16x4_t*>(stage + li * kAttnD + 8 * ((4 * db + rq) ^ (li & 15)) + 4 * g) = o4;
+      for (int e = 0; e < 4; ++e) o4[e] = static_cast<T>(acc[db][4 * rq + e] * factor);
+      *reinterpret_cast<x4_t*>(stage + li * kAttnD + 8 * ((4 * db + rq) ^ (li & 15)) + 4 * g) = o4;
     }
   const int c16 = lane & 15;
 #pragma nounroll
@@ -190,16 +200,18 @@ __device__ __forceinline__ void bwd8_zero(f32x16_t (&acc)[4]) {
 // ---------------------------------------------------------------------------------------------
 // dQ
 // ---------------------------------------------------------------------------------------------
-template <bool CAUSAL>
-__device__ __forceinline__ void attention_bwd8_dq(const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K,
-                                                  const bf16_t* __restrict__ V, const bf16_t* __restrict__ dO,
-                                                  const float* __restrict__ stats, bf16_t* __restrict__ dQ,
+template <typename T, bool CAUSAL>
+__device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const T* __restrict__ K,
+                                                  const T* __restrict__ V, const T* __restrict__ dO,
+                                                  const float* __restrict__ stats, T* __restrict__ dQ,
                                                   int S, int q_block, int head, float scale) {
+  typedef AttnElem<T> E;
+  typedef typename E::x8 x8_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char attn_lds[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
   const size_t head_off = static_cast<size_t>(head) * S * kAttnD;
-  const bf16_t* __restrict__ Kh = K + head_off;
-  const bf16_t* __restrict__ Vh = V + head_off;
+  const T* __restrict__ Kh = K + head_off;
+  const T* __restrict__ Vh = V + head_off;
   const int q0 = q_block * kBwd8BlockRows;
   const int qw = q0 + wave * 32;       // first query of this wavefront
   const int qi = qw + li;
@@ -207,11 +219,11 @@ __device__ __forceinline__ void attention_bwd8_dq(const bf16_t* __restrict__ Q, 
   const int qc = valid ? qi : S - 1;   // rows past the end read the last row and are never stored
   const size_t qrow = head_off + static_cast<size_t>(qc) * kAttnD;
 
-  bf16x8_t qf[8], dof[8];
+  x8_t qf[8], dof[8];
 #pragma unroll
   for (int s = 0; s < 8; ++s) {
-    qf[s] = *reinterpret_cast<const bf16x8_t*>(Q + qrow + 16 * s + 8 * g);
-    dof[s] = *reinterpret_cast<const bf16x8_t*>(dO + qrow + 16 * s + 8 * g);
+    qf[s] = *reinterpret_cast<const x8_t*>(Q + qrow + 16 * s + 8 * g);
+    dof[s] = *reinterpret_cast<const x8_t*>(dO + qrow + 16 * s + 8 * g);
   }
   const Vec<float, 2> st = load_vec<float, 2>(stats + 2 * (static_cast<size_t>(head) * S + qc));
   const float m2 = st[0], delta = st[1];
@@ -224,7 +236,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const bf16_t* __restrict__ Q, 
   const int n_tiles = CAUSAL ? min((q0 + kBwd8BlockRows) / kAttnBN, all_tiles) : all_tiles;
   const int wave_last_tile = (CAUSAL && qw < S) ? (qw + 31) / kAttnBN : (qw < S ? n_tiles - 1 : -1);
 
-  auto buf = [&](int b) { return reinterpret_cast<bf16_t*>(attn_lds + b * kBwd8DqBufBytes); };
+  auto buf = [&](int b) { return reinterpret_cast<T*>(attn_lds + b * kBwd8DqBufBytes); };
   Bwd8ColStage kt;
   Bwd8RowStage vt;
   auto load_tile = [&](int tile) {
@@ -232,7 +244,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const bf16_t* __restrict__ Q, 
     bwd8_load(vt, Vh + static_cast<size_t>(tile) * kAttnBN * kAttnD, tid);
   };
   auto store_tile = [&](int b) {
-    bf16_t* Ks = buf(b);
+    T* Ks = buf(b);
     bwd8_store_rows(kt, Ks, tid);
     bwd8_store_rows(vt, Ks + kBwd8RowTile, tid);
     bwd8_store_cols(kt, Ks + 2 * kBwd8RowTile, tid);
@@ -240,11 +252,11 @@ __device__ __forceinline__ void attention_bwd8_dq(const bf16_t* __restrict__ Q, 
 
   auto compute = [&](int tile, auto mask_c) {
     constexpr bool MASK = decltype(mask_c)::value;
-    const bf16_t* Ks = buf(tile & 1);
-    const bf16_t* Vs = Ks + kBwd8RowTile;
-    const bf16_t* Kt = Ks + 2 * kBwd8RowTile;
+    const T* Ks = buf(tile & 1);
+    const T* Vs = Ks + kBwd8RowTile;
+    const T* Kt = Ks + 2 * kBwd8RowTile;
     const int key0 = tile * kAttnBN;
-    bf16x8_t dsf[2][2];
+    x8_t dsf[2][2];
 #if BWD8_PREFETCH > 0
     if constexpr (!MASK) {
     // The 32 MFMA steps of a tile (16 score / dP pairs, then 16 dQ updates) read their LDS
@@ -252,7 +264,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const bf16_t* __restrict__ Q, 
     // order pinned by scheduling fences: the softmax arithmetic of a key block then runs while
     // the fragments of the next steps are already in flight.
     constexpr int PF = BWD8_PREFETCH;
-    bf16x8_t ka[16], va[16], ta[16];
+    x8_t ka[16], va[16], ta[16];
     auto issue = [&](auto ic) {
       constexpr int i = decltype(ic)::value;
       if constexpr (i < 16) {
@@ -277,21 +289,21 @@ __device__ __forceinline__ void attention_bwd8_dq(const bf16_t* __restrict__ Q, 
             pacc[r] = 0.f;
           }
         }
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[i], qf[s_], sacc, 0, 0, 0);
-        pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[i], dof[s_], pacc, 0, 0, 0);
+        sacc = E::mfma(ka[i], qf[s_], sacc);
+        pacc = E::mfma(va[i], dof[s_], pacc);
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (s_ == 7) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], c2, -m2));
             if (MASK && key0 + 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3) > qi) p = 0.f;
-            dsf[kb][r >> 3][r & 7] = static_cast<bf16_t>(p * (pacc[r] - delta));
+            dsf[kb][r >> 3][r & 7] = static_cast<T>(p * (pacc[r] - delta));
           }
           __builtin_amdgcn_sched_barrier(0);
         }
       } else {
         constexpr int j = i - 16, t = j >> 2, db = j & 3;
-        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta[j], dsf[t >> 1][t & 1], acc[db], 0, 0, 0);
+        acc[db] = E::mfma(ta[j], dsf[t >> 1][t & 1], acc[db]);
         __builtin_amdgcn_sched_barrier(0);
       }
     });
@@ -308,21 +320,21 @@ __device__ __forceinline__ void attention_bwd8_dq(const bf16_t* __restrict__ Q, 
       }
 #pragma unroll
       for (int s = 0; s < 8; ++s) {
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bwd8_row_frag(Ks, 32 * kb + li, s, g), qf[s], sacc, 0, 0, 0);
-        pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bwd8_row_frag(Vs, 32 * kb + li, s, g), dof[s], pacc, 0, 0, 0);
+        sacc = E::mfma(bwd8_row_frag(Ks, 32 * kb + li, s, g), qf[s], sacc);
+        pacc = E::mfma(bwd8_row_frag(Vs, 32 * kb + li, s, g), dof[s], pacc);
       }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], c2, -m2));
         if (MASK && key0 + 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3) > qi) p = 0.f;
-        dsf[kb][r >> 3][r & 7] = static_cast<bf16_t>(p * (pacc[r] - delta));
+        dsf[kb][r >> 3][r & 7] = static_cast<T>(p * (pacc[r] - delta));
       }
     }
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int db = 0; db < 4; ++db)
-        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bwd8_col_frag(Kt, 32 * db + li, t, g), dsf[t >> 1][t & 1], acc[db], 0, 0, 0);
+        acc[db] = E::mfma(bwd8_col_frag(Kt, 32 * db + li, t, g), dsf[t >> 1][t & 1], acc[db]);
   };
 
   // Under a causal mask only the tiles that overlap the block's own queries (the last four) need
@@ -348,26 +360,28 @@ __device__ __forceinline__ void attention_bwd8_dq(const bf16_t* __restrict__ Q, 
     }
   }
   bwd8_store_acc<!CAUSAL>(dQ + head_off + static_cast<size_t>(qw) * kAttnD, acc, scale,
-                 reinterpret_cast<bf16_t*>(attn_lds) + wave * (32 * kAttnD), lane, S - qw);
+                 reinterpret_cast<T*>(attn_lds) + wave * (32 * kAttnD), lane, S - qw);
   __syncthreads();  // the staging reads are done before a following block refills the tile buffers
 }
 
 // ---------------------------------------------------------------------------------------------
 // dK (WHICH = 0) and dV (WHICH = 1): a wavefront owns 32 keys, loop over query tiles
 // ---------------------------------------------------------------------------------------------
-template <bool CAUSAL, int WHICH>
-__device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q, const bf16_t* __restrict__ K,
-                                                   const bf16_t* __restrict__ V, const bf16_t* __restrict__ dO,
-                                                   const float* __restrict__ stats, bf16_t* __restrict__ dKV,
+template <typename T, bool CAUSAL, int WHICH>
+__device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, const T* __restrict__ K,
+                                                   const T* __restrict__ V, const T* __restrict__ dO,
+                                                   const float* __restrict__ stats, T* __restrict__ dKV,
                                                    int S, int k_block, int head, float scale) {
   constexpr bool DK = WHICH == 0;
   constexpr int BUF = DK ? kBwd8DkBufBytes : kBwd8DvBufBytes;
   constexpr int STAT_OFF = BUF - kBwd8StatBytes;
+  typedef AttnElem<T> E;
+  typedef typename E::x8 x8_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char attn_lds[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, li = lane & 31, g = lane >> 5;
   const size_t head_off = static_cast<size_t>(head) * S * kAttnD;
-  const bf16_t* __restrict__ Qh = Q + head_off;
-  const bf16_t* __restrict__ dOh = dO + head_off;
+  const T* __restrict__ Qh = Q + head_off;
+  const T* __restrict__ dOh = dO + head_off;
   const int k0 = k_block * kBwd8BlockRows;
   const int kw = k0 + wave * 32;  // first key of this wavefront
   const int kj = kw + li;
@@ -375,11 +389,11 @@ __device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q,
   const int kc = valid ? kj : S - 1;
   const size_t krow = head_off + static_cast<size_t>(kc) * kAttnD;
 
-  bf16x8_t kf[8], vf[DK ? 8 : 1];
+  x8_t kf[8], vf[DK ? 8 : 1];
 #pragma unroll
   for (int s = 0; s < 8; ++s) {
-    kf[s] = *reinterpret_cast<const bf16x8_t*>(K + krow + 16 * s + 8 * g);
-    if constexpr (DK) vf[s] = *reinterpret_cast<const bf16x8_t*>(V + krow + 16 * s + 8 * g);
+    kf[s] = *reinterpret_cast<const x8_t*>(K + krow + 16 * s + 8 * g);
+    if constexpr (DK) vf[s] = *reinterpret_cast<const x8_t*>(V + krow + 16 * s + 8 * g);
   }
   f32x16_t acc[4];
   bwd8_zero(acc);
@@ -394,14 +408,14 @@ __device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q,
   Bwd8RowStage rst;  // DK: dO, DV: Q
   Vec<float, 2> sst;
   auto load_tile = [&](int tile) {
-    const bf16_t* qp = Qh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
-    const bf16_t* dp = dOh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
+    const T* qp = Qh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
+    const T* dp = dOh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
     bwd8_load(cst, DK ? qp : dp, tid);
     bwd8_load(rst, DK ? dp : qp, tid);
     if (tid < kAttnBN) sst = load_vec<float, 2>(stats + 2 * (static_cast<size_t>(head) * S + tile * kAttnBN + tid));
   };
   auto store_tile = [&](int b) {
-    bf16_t* base = reinterpret_cast<bf16_t*>(attn_lds + b * BUF);
+    T* base = reinterpret_cast<T*>(attn_lds + b * BUF);
     if constexpr (DK) {
       bwd8_store_rows(cst, base, tid);                        // Q
       bwd8_store_rows(rst, base + kBwd8RowTile, tid);         // dO
@@ -415,13 +429,13 @@ __device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q,
 
   auto compute = [&](int tile, auto mask_c) {
     constexpr bool MASK = decltype(mask_c)::value;
-    const bf16_t* base = reinterpret_cast<const bf16_t*>(attn_lds + (tile & 1) * BUF);
-    const bf16_t* Qs = base;
-    const bf16_t* dOs = base + kBwd8RowTile;                              // DK only
-    const bf16_t* Tt = base + (DK ? 2 * kBwd8RowTile : kBwd8RowTile);     // Q^T (DK) or dO^T (DV)
+    const T* base = reinterpret_cast<const T*>(attn_lds + (tile & 1) * BUF);
+    const T* Qs = base;
+    const T* dOs = base + kBwd8RowTile;                              // DK only
+    const T* Tt = base + (DK ? 2 * kBwd8RowTile : kBwd8RowTile);     // Q^T (DK) or dO^T (DV)
     const float* st = reinterpret_cast<const float*>(attn_lds + (tile & 1) * BUF + STAT_OFF);
     const int q0t = tile * kAttnBN;
-    bf16x8_t bf[2][2];  // [query block][half]: P (dV) or dS (dK) as B operands, contraction over the queries
+    x8_t bf[2][2];  // [query block][half]: P (dV) or dS (dK) as B operands, contraction over the queries
     auto probabilities = [&](auto qbc, const f32x16_t& sacc, const f32x16_t& pacc) {
       constexpr int qb = decltype(qbc)::value;
 #pragma unroll
@@ -438,9 +452,9 @@ __device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q,
           float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], c2, -mrow[e]));
           if (MASK && kj > q0t + row0 + e) p = 0.f;
           if constexpr (DK)
-            bf[qb][r >> 3][r & 7] = static_cast<bf16_t>(p * (pacc[r] - drow[e]));
+            bf[qb][r >> 3][r & 7] = static_cast<T>(p * (pacc[r] - drow[e]));
           else
-            bf[qb][r >> 3][r & 7] = static_cast<bf16_t>(p);
+            bf[qb][r >> 3][r & 7] = static_cast<T>(p);
         }
       }
     };
@@ -448,7 +462,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q,
     constexpr int PF = DK ? (CAUSAL ? BWD8_PREFETCH_DK_CAUSAL : BWD8_PREFETCH_DK) : BWD8_PREFETCH_DV;
     if constexpr (PF > 0 && !MASK) {
       // as in the dQ kernel: LDS fragments read PF steps ahead across the phases of the tile
-      bf16x8_t qa[16], da[DK ? 16 : 1], ta[16];
+      x8_t qa[16], da[DK ? 16 : 1], ta[16];
       auto issue = [&](auto ic) {
         constexpr int i = decltype(ic)::value;
         if constexpr (i < 16) {
@@ -473,8 +487,8 @@ __device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q,
               pacc[r] = 0.f;
             }
           }
-          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[i], kf[s_], sacc, 0, 0, 0);
-          if constexpr (DK) pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da[i], vf[s_], pacc, 0, 0, 0);
+          sacc = E::mfma(qa[i], kf[s_], sacc);
+          if constexpr (DK) pacc = E::mfma(da[i], vf[s_], pacc);
           __builtin_amdgcn_sched_barrier(0);
           if constexpr (s_ == 7) {
             probabilities(std::integral_constant<int, qb>{}, sacc, pacc);
@@ -482,7 +496,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q,
           }
         } else {
           constexpr int j = i - 16, t = j >> 2, db = j & 3;
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta[j], bf[t >> 1][t & 1], acc[db], 0, 0, 0);
+          acc[db] = E::mfma(ta[j], bf[t >> 1][t & 1], acc[db]);
           __builtin_amdgcn_sched_barrier(0);
         }
       });
@@ -498,9 +512,9 @@ __device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q,
       }
 #pragma unroll
       for (int s = 0; s < 8; ++s) {
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bwd8_row_frag(Qs, 32 * qb + li, s, g), kf[s], sacc, 0, 0, 0);
+        sacc = E::mfma(bwd8_row_frag(Qs, 32 * qb + li, s, g), kf[s], sacc);
         if constexpr (DK)
-          pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bwd8_row_frag(dOs, 32 * qb + li, s, g), vf[s], pacc, 0, 0, 0);
+          pacc = E::mfma(bwd8_row_frag(dOs, 32 * qb + li, s, g), vf[s], pacc);
       }
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
@@ -515,9 +529,9 @@ __device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q,
           float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], c2, -mrow[e]));
           if (MASK && kj > q0t + row0 + e) p = 0.f;
           if constexpr (DK)
-            bf[qb][r >> 3][r & 7] = static_cast<bf16_t>(p * (pacc[r] - drow[e]));
+            bf[qb][r >> 3][r & 7] = static_cast<T>(p * (pacc[r] - drow[e]));
           else
-            bf[qb][r >> 3][r & 7] = static_cast<bf16_t>(p);
+            bf[qb][r >> 3][r & 7] = static_cast<T>(p);
         }
       }
     }
@@ -525,7 +539,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q,
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int db = 0; db < 4; ++db)
-        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bwd8_col_frag(Tt, 32 * db + li, t, g), bf[t >> 1][t & 1], acc[db], 0, 0, 0);
+        acc[db] = E::mfma(bwd8_col_frag(Tt, 32 * db + li, t, g), bf[t >> 1][t & 1], acc[db]);
   };
 
   if (first_tile < n_qtiles) {
@@ -552,7 +566,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const bf16_t* __restrict__ Q,
     __syncthreads();
   }
   bwd8_store_acc<!CAUSAL>(dKV + head_off + static_cast<size_t>(kw) * kAttnD, acc, DK ? scale : 1.0f,
-                 reinterpret_cast<bf16_t*>(attn_lds) + wave * (32 * kAttnD), lane, S - kw);
+                 reinterpret_cast<T*>(attn_lds) + wave * (32 * kAttnD), lane, S - kw);
   __syncthreads();  // the staging reads are done before a following block refills the tile buffers
 }
 

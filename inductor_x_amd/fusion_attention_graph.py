@@ -20,7 +20,7 @@ general boolean mask, fp32 operands, other head dimensions and dropout (keep_pro
 mathematics over library GEMMs; padding masks, prefixes, variable sequence lengths and band masks
 raise.
 The backward op recomputes the probabilities from the saved row statistics inside fused gradient
-kernels (bf16, head dimension up to 128, equal lengths that are multiples of 64;
+kernels (bf16 or fp16, head dimension up to 128, equal lengths that are multiples of 64;
 kernels.fused_attention_backward) and falls back to the GEMM formulation otherwise
 (attention_backward.py), which also returns the gradient of pse; the training variant of the
 pattern is registered beside the inference one.
@@ -310,7 +310,7 @@ def _extra_check(match, training: bool = False) -> bool:
     """Only rewrite what the fused kernels run; anything else stays on Inductor's own path.
     Inference graphs: bf16 or fp16 GPU tensors [B, S, N, 128], any sequence lengths, key and value of
     one shape that may differ from the query's in its length (cross attention).  Training graphs,
-    whose backward runs the fused gradient kernels: bf16, query, key and value of one shape, a
+    whose backward runs the fused gradient kernels: query, key and value of one shape and a
     sequence length that is a multiple of 64.  Either way the divisor of the scores, when it is a
     constant, must be positive and finite."""
     try:
@@ -321,10 +321,9 @@ def _extra_check(match, training: bool = False) -> bool:
         return False
     if not (q.device.type == "cuda" and q.dim() == 4 and q.size(3) == 128 and q.size(1) > 0):
         return False
-    if training:
-        if q.dtype != torch.bfloat16 or q.size(1) % 64 != 0 or tuple(k.shape) != tuple(q.shape):
-            return False
-    elif q.dtype not in (torch.bfloat16, torch.float16):
+    if q.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    if training and (q.size(1) % 64 != 0 or tuple(k.shape) != tuple(q.shape)):
         return False
     if k.dim() != 4 or k.size(1) <= 0 or (k.size(0), k.size(2), k.size(3)) != (q.size(0), q.size(2), q.size(3)):
         return False

@@ -666,13 +666,14 @@ _ATTN_BWD8_DV_LDS = 2 * ((64 * 136 + 128 * 64) * 2 + 64 * 2 * 4)
 def _attention_bwd_launchers() -> dict:
     src = codecache.aot_source("attention_bwd_kernels.hip")
     mk = lambda name, sig, cfgs: CachingLauncher(name, src, sig, cfgs, prefer_intree=True)  # noqa: E731
+    types = tuple(_ATTN_DTYPES.values())
     return {
-        "stats": mk("attention_bwd_stats_bf16_d128", "PPPPPi", [LaunchConfig("attention_bwd_stats_bf16_d128", 256)]),
+        "stats": mk("attention_bwd_stats_d128", "PPPPPi", [LaunchConfig(f"attention_bwd_stats_{t}_d128", 256) for t in types]),
         **{
             which: mk(
-                f"attention_bwd8_{which[:2]}_bf16_d128", "PPPPPPiif",
-                [LaunchConfig(f"attention_bwd8_{which[:2]}_bf16_d128_{c}", 512, meta={"CAUSAL": c == "causal"}, lds_bytes=lds)
-                 for c in ("causal", "full")],
+                f"attention_bwd8_{which[:2]}_d128", "PPPPPPiif",
+                [LaunchConfig(f"attention_bwd8_{which[:2]}_{t}_d128_{c}", 512, meta={"CAUSAL": c == "causal"}, lds_bytes=lds)
+                 for t in types for c in ("causal", "full")],
             )
             for which, lds in (("dq8", _ATTN_BWD8_DQ_LDS), ("dk8", _ATTN_BWD8_DK_LDS), ("dv8", _ATTN_BWD8_DV_LDS))
         },
@@ -683,12 +684,13 @@ def fused_attention_backward(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, dout: torch.Tensor,
     softmax_max: torch.Tensor, softmax_sum: torch.Tensor, scale: float, causal: bool,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """Gradients (dq, dk, dv) of fused_attention for [B, N, S, 128] bf16 tensors; softmax_max /
+    """Gradients (dq, dk, dv) of fused_attention for [B, N, S, 128] bf16 or fp16 tensors; softmax_max /
     softmax_sum are the forward's [B, N, S, 8] fp32 statistics.  Workgroups of eight wavefronts on
     256 rows, a statistics pass and separate dQ, dK and dV kernels; S a positive multiple of 64."""
     _check_cuda(q, k, v, out, dout, softmax_max, softmax_sum)
     for t in (q, k, v, out, dout):
-        _require(t.dtype == torch.bfloat16 and t.dim() == 4 and t.shape == q.shape, "q, k, v, out, dout: one [B, N, S, D] bf16 shape")
+        _require(t.dtype == q.dtype and t.dtype in _ATTN_DTYPES and t.dim() == 4 and t.shape == q.shape,
+                 "q, k, v, out, dout: one [B, N, S, D] shape in bf16 or fp16")
         _require(t.is_contiguous() and _aligned(t), "q, k, v, out, dout must be contiguous and 16-byte aligned")
     B, N, S, D = q.shape
     _require(D == 128, "head dimension must be 128")
@@ -705,8 +707,9 @@ def fused_attention_backward(
     st = _stream()
     which = "causal" if causal else "full"
     stats = torch.empty(heads * S, 2, dtype=torch.float32, device=q.device)
+    ty = _ATTN_DTYPES[q.dtype]
     ls["stats"]._launch(
-        _find(ls["stats"], "attention_bwd_stats_bf16_d128"),
+        _find(ls["stats"], f"attention_bwd_stats_{ty}_d128"),
         (out.data_ptr(), dout.data_ptr(), softmax_max.data_ptr(), softmax_sum.data_ptr(), stats.data_ptr(), heads * S),
         (cdiv(heads * S * 16, 256), 1, 1), st,
     )
@@ -715,7 +718,7 @@ def fused_attention_backward(
     for name, dst in (("dk8", dk), ("dv8", dv), ("dq8", dq)):
         l = ls[name]
         l._launch(
-            _find(l, f"attention_bwd8_{name[:2]}_bf16_d128_{which}"),
+            _find(l, f"attention_bwd8_{name[:2]}_{ty}_d128_{which}"),
             (q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), stats.data_ptr(), dst.data_ptr(), heads, S, float(scale)),
             grid, st,
         )

@@ -230,17 +230,18 @@ def test_attention_backward_closed_forms():
     assert q2.grad.float().abs().max().item() <= 2e-2 and k2.grad.float().abs().max().item() <= 2e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,N,S,causal", [(1, 2, 256, True), (1, 3, 384, False), (1, 3, 384, True), (2, 4, 1024, True),
                                           (1, 9, 128, False), (1, 2, 128, True), (1, 2, 640, True), (1, 5, 1280, False)])
-def test_attention_backward_kernels_vs_gemm_path(K, B, N, S, causal):
-    """The fused backward kernels against the same gradients computed with library GEMMs from the
-    same saved statistics.  Both round P and dS to bf16 once, so they agree to two bf16 ulps of the
-    largest entry.  Sequence lengths include last blocks of 128 rows."""
-    announce(f"attention backward vs GEMM path B={B} N={N} S={S} causal={causal}")
+def test_attention_backward_kernels_vs_gemm_path(K, B, N, S, causal, dtype):
+    """The fused backward kernels (bf16 and fp16) against the same gradients computed with library
+    GEMMs from the same saved statistics.  Both round P and dS to the operand type once, so they
+    agree to two bf16 ulps of the largest entry.  Sequence lengths include last blocks of 128 rows."""
+    announce(f"attention backward vs GEMM path {dtype} B={B} N={N} S={S} causal={causal}")
     from inductor_x_amd import attention_backward as AB
 
     torch.manual_seed(7)
-    q, k, v, do = (torch.randn(B, N, S, 128, device=DEV).bfloat16() for _ in range(4))
+    q, k, v, do = (torch.randn(B, N, S, 128, device=DEV).to(dtype) for _ in range(4))
     scale = 128 ** -0.5
     o, m, l = K.fused_attention(q, k, v, scale, causal)
     a = K.fused_attention_backward(q, k, v, o, do, m, l, scale, causal)
@@ -386,6 +387,7 @@ def test_attention_op_cross_attention_gradients(dtype, B, N, Sq, Sk, D):
     (torch.float16, 1, 3, 200, 200, True, 128), (torch.float16, 2, 2, 512, 512, False, 128),
     (torch.bfloat16, 1, 2, 100, 300, False, 128), (torch.bfloat16, 1, 2, 77, 77, True, 128),
     (torch.bfloat16, 2, 3, 256, 256, True, 64), (torch.float16, 1, 2, 130, 130, False, 64), (torch.bfloat16, 1, 2, 192, 192, True, 80),
+    (torch.float16, 2, 2, 320, 320, True, 128), (torch.float16, 1, 3, 128, 128, False, 96),
 ])
 def test_attention_op_reaches_the_fused_kernel_for_fp16_and_any_length(dtype, B, N, Sq, Sk, causal, D):
     """npu_fa with fp16 operands, with sequence lengths that are no multiple of a tile, with
@@ -426,8 +428,8 @@ def test_attention_op_reaches_the_fused_kernel_for_fp16_and_any_length(dtype, B,
             torch.cuda.synchronize()
         finally:
             log, launcher.launch_log = launcher.launch_log, None
-        if dtype == torch.bfloat16 and Sq % 64 == 0:
-            assert any(sym.startswith("attention_bwd8_") for sym in log), log
+        if Sq % 64 == 0:
+            assert any(sym.startswith(f"attention_bwd8_dq_{name}_") for sym in log), log
         ref.backward(do.float())
         for g, r in zip((q.grad, k.grad, v.grad), (qf.grad, kf.grad, vf.grad)):
             assert (g.float() - r).abs().max().item() <= 3e-2 * max(r.abs().max().item(), 1.0)
