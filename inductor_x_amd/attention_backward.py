@@ -1,7 +1,7 @@
 """Backward of the fused attention forward (npu_graph::npu_fa_backward).
 
 Two paths.  bf16 or fp16 with a head dimension up to 128 (a multiple of 8; smaller ones are padded with zero columns)
-and a sequence length that is a multiple of 64 runs the fused MFMA
+runs the fused MFMA
 kernels (kernels.fused_attention_backward, csrc/mi/attention_bwd_w8.h).  Other shapes run the matrix
 products as library GEMMs (torch.bmm, hipBLASLt underneath) on a bounded number of heads at a time
 and move O(S^2) intermediates through HBM.  Both recompute the probabilities from the forward's
@@ -138,8 +138,9 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
                              use_kernels=None, keep_prob: float = 1.0, seed: int = 0, pse=None, atten_mask=None):
     """q, out, dout: [B, N, Sq, D] and k, v: [B, N, Sk, D] of one floating-point type; softmax_max /
     softmax_sum: [B, N, Sq, 8] fp32 from the forward.  Returns (dq, dk, dv) in that type.  use_kernels: None = fused
-    kernels where they apply (bf16 or fp16, head dimension up to 128, one shape for q, k and v, a sequence
-    length that is a multiple of 64, no dropout).
+    kernels where they apply (bf16 or fp16, head dimension up to 128, one shape for q, k and v, no dropout, a
+    sequence length that is a multiple of 64 or, under a causal mask, any; smaller head dimensions and causal
+    lengths in between are zero-padded).
     keep_prob < 1 with the forward's seed regenerates the forward's dropout mask (GEMM path only).
     With pse or atten_mask (GEMM path only) the result has a fourth member, the gradient of pse in
     pse's own shape (None without pse)."""
@@ -148,8 +149,9 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
             raise NotImplementedError("attention backward: the fused kernels take no bias or mask")
         return _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale, causal, keep_prob, seed,
                                     pse=pse, atten_mask=atten_mask)
+    # a length that is no multiple of 64 is served under a causal mask only (see the padding note below)
     fits = (q.dim() == 4 and q.dtype in (torch.bfloat16, torch.float16) and 0 < q.size(3) <= 128 and q.size(3) % 8 == 0
-            and q.size(2) % 64 == 0 and q.size(2) > 0 and q.shape == k.shape and keep_prob == 1.0)
+            and q.size(2) > 0 and (causal or q.size(2) % 64 == 0) and q.shape == k.shape and keep_prob == 1.0)
     if use_kernels is None:
         use_kernels = fits
     if use_kernels:
@@ -157,15 +159,29 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
             raise NotImplementedError("attention backward: the fused kernels have no dropout")
         from . import kernels
 
-        # a head dimension below 128 is padded with zero columns: scores, probabilities and
-        # rowsum(dO * O) do not change, the extra gradient columns are zero and dropped
-        d = q.size(3)
-        widen = (lambda t: torch.nn.functional.pad(t, (0, 128 - d))) if d < 128 else (lambda t: t.contiguous())  # noqa: E731
-        grads = kernels.fused_attention_backward(
-            widen(q), widen(k), widen(v), widen(out), widen(dout),
-            softmax_max.contiguous(), softmax_sum.contiguous(), scale, causal,
-        )
-        return tuple(g[..., :d].contiguous() for g in grads) if d < 128 else grads
+        # A head dimension below 128 is padded with zero columns: scores, probabilities and
+        # rowsum(dO * O) do not change, the extra gradient columns are zero and dropped.
+        # Under a causal mask a sequence length that is no multiple of 64 is padded with zero rows
+        # (statistics m = 0, l = 1): the mask hides every padded key from every real query, so its
+        # probability is exactly zero, and a padded query has dO = 0 and Q = 0, so it adds nothing to
+        # dV or dK; the padded rows of the results are dropped.  Without the mask a padded key would
+        # get the probability exp(-logsumexp of the row), which times K = 0 is zero only while it
+        # stays finite in the operand type, so those lengths run over GEMMs.
+        d, S = q.size(3), q.size(2)
+        pad_d, pad_s = 128 - d, -S % 64
+        if pad_s and not causal:
+            raise NotImplementedError("attention backward: without a causal mask the fused kernels need a sequence "
+                                      "length that is a multiple of 64")
+        if pad_d or pad_s:
+            widen = lambda t: torch.nn.functional.pad(t, (0, pad_d, 0, pad_s))  # noqa: E731
+        else:
+            widen = lambda t: t.contiguous()  # noqa: E731
+        smax, ssum = softmax_max.contiguous(), softmax_sum.contiguous()
+        if pad_s:
+            smax = torch.nn.functional.pad(smax, (0, 0, 0, pad_s), value=0.0)
+            ssum = torch.nn.functional.pad(ssum, (0, 0, 0, pad_s), value=1.0)
+        grads = kernels.fused_attention_backward(widen(q), widen(k), widen(v), widen(out), widen(dout), smax, ssum, scale, causal)
+        return tuple(g[:, :, :S, :d].contiguous() for g in grads) if (pad_d or pad_s) else grads
     return _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale, causal, keep_prob, seed)
 
 

@@ -20,7 +20,7 @@ general boolean mask, fp32 operands, other head dimensions and dropout (keep_pro
 mathematics over library GEMMs; padding masks, prefixes, variable sequence lengths and band masks
 raise.
 The backward op recomputes the probabilities from the saved row statistics inside fused gradient
-kernels (bf16 or fp16, head dimension up to 128, equal lengths that are multiples of 64;
+kernels (bf16 or fp16, head dimension up to 128, equal lengths that are multiples of 64 or, with a causal mask, any;
 kernels.fused_attention_backward) and falls back to the GEMM formulation otherwise
 (attention_backward.py), which also returns the gradient of pse; the training variant of the
 pattern is registered beside the inference one.

@@ -254,6 +254,42 @@ def test_attention_backward_kernels_vs_gemm_path(K, B, N, S, causal, dtype):
                                    l[:, :, :32].contiguous(), scale, causal)
 
 
+@pytest.mark.parametrize("dtype,B,N,S,D", [(torch.bfloat16, 1, 3, 100, 128), (torch.float16, 2, 2, 333, 128), (torch.bfloat16, 1, 2, 77, 64),
+                                            (torch.bfloat16, 1, 2, 1, 128), (torch.float16, 1, 1, 65, 128)])
+def test_attention_backward_causal_any_length(K, dtype, B, N, S, D):
+    """Under a causal mask the gradient kernels serve any sequence length on zero-padded rows: the same
+    gradients as the GEMM formulation from the same saved statistics, and the gradient kernels are
+    what ran.  Without the mask such a length keeps the GEMM formulation."""
+    announce(f"attention backward causal, padded length {dtype} B={B} N={N} S={S} D={D}")
+    from inductor_x_amd import attention_backward as AB
+    from inductor_x_amd import launcher
+
+    torch.manual_seed(17)
+    q, k, v, do = (torch.randn(B, N, S, D, device=DEV).to(dtype) for _ in range(4))
+    scale = D ** -0.5
+    o, m, l = AB.attention_forward_over_gemms(q, k, v, scale, True)
+    launcher.launch_log = []
+    try:
+        a = AB.fused_attention_backward(q, k, v, o, do, m, l, scale, True)
+        torch.cuda.synchronize()
+    finally:
+        log, launcher.launch_log = launcher.launch_log, None
+    assert any(sym.startswith("attention_bwd8_dq_") for sym in log), log
+    b = AB.fused_attention_backward(q, k, v, o, do, m, l, scale, True, use_kernels=False)
+    for x, y in zip(a, b):
+        assert x.shape == q.shape and x.dtype == dtype and torch.isfinite(x).all()
+        assert (x.float() - y.float()).abs().max().item() <= 8e-3 * max(y.float().abs().max().item(), 1.0)
+    if S % 64:
+        launcher.launch_log = []
+        try:
+            AB.fused_attention_backward(q, k, v, o, do, m, l, scale, False)
+        finally:
+            log, launcher.launch_log = launcher.launch_log, None
+        assert not any(sym.startswith("attention_bwd8_") for sym in log), log
+        with pytest.raises(NotImplementedError):
+            AB.fused_attention_backward(q, k, v, o, do, m, l, scale, False, use_kernels=True)
+
+
 @pytest.mark.parametrize("S,causal", [(64, True), (192, False), (320, True), (576, True)])
 def test_attention_backward_sequence_multiple_of_64(K, S, causal):
     """The backward kernels take any multiple of 64: last blocks of 64 and 192 rows (the output and
@@ -428,7 +464,7 @@ def test_attention_op_reaches_the_fused_kernel_for_fp16_and_any_length(dtype, B,
             torch.cuda.synchronize()
         finally:
             log, launcher.launch_log = launcher.launch_log, None
-        if Sq % 64 == 0:
+        if Sq % 64 == 0 or causal:
             assert any(sym.startswith(f"attention_bwd8_dq_{name}_") for sym in log), log
         ref.backward(do.float())
         for g, r in zip((q.grad, k.grad, v.grad), (qf.grad, kf.grad, vf.grad)):
