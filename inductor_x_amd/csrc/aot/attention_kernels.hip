@@ -15,7 +15,7 @@
 
 using namespace mi;
 
-template <typename T, bool CAUSAL, bool RAGGED>
+template <typename T, bool CAUSAL, bool RAGGED, int DH = 128>
 __device__ __forceinline__ void attention_entry_v5(const T* q, const T* k, const T* v, T* o, float* smax,
                                                    float* ssum, int n_heads, int Sq, int Sk,
                                                    float scale_log2e) {
@@ -35,21 +35,22 @@ __device__ __forceinline__ void attention_entry_v5(const T* q, const T* k, const
       const int n_pass = lo != hi ? 2 : 1;
 #pragma nounroll
       for (int pass = 0; pass < n_pass; ++pass)
-        attention_fwd_d128_v5<T, true, RAGGED>(q, k, v, o, smax, ssum, Sq, Sk, pass == 0 ? hi : lo, head, scale_log2e);
+        attention_fwd_d128_v5<T, true, RAGGED, kAttnV5Waves, DH>(q, k, v, o, smax, ssum, Sq, Sk, pass == 0 ? hi : lo, head, scale_log2e);
     } else {
-      attention_fwd_d128_v5<T, false, RAGGED>(q, k, v, o, smax, ssum, Sq, Sk, slot % per_head, head, scale_log2e);
+      attention_fwd_d128_v5<T, false, RAGGED, kAttnV5Waves, DH>(q, k, v, o, smax, ssum, Sq, Sk, slot % per_head, head, scale_log2e);
     }
   }
 }
 
 // 512 threads, 256 queries per workgroup, one workgroup per CU, 64 KiB of LDS.
-#define ATTENTION_V5(NAME, T, CAUSAL, RAGGED)                                                      \
-  extern "C" __global__ __launch_bounds__(512, 1) void NAME(const T* q, const T* k, const T* v,    \
-                                                            T* o, float* smax, float* ssum,        \
-                                                            int n_heads, int Sq, int Sk,           \
-                                                            float scale_log2e) {                   \
-    attention_entry_v5<T, CAUSAL, RAGGED>(q, k, v, o, smax, ssum, n_heads, Sq, Sk, scale_log2e);   \
+#define ATTENTION_V5_DH(NAME, T, CAUSAL, RAGGED, DH)                                                  \
+  extern "C" __global__ __launch_bounds__(512, 1) void NAME(const T* q, const T* k, const T* v,       \
+                                                            T* o, float* smax, float* ssum,           \
+                                                            int n_heads, int Sq, int Sk,              \
+                                                            float scale_log2e) {                      \
+    attention_entry_v5<T, CAUSAL, RAGGED, DH>(q, k, v, o, smax, ssum, n_heads, Sq, Sk, scale_log2e);  \
   }
+#define ATTENTION_V5(NAME, T, CAUSAL, RAGGED) ATTENTION_V5_DH(NAME, T, CAUSAL, RAGGED, 128)
 
 ATTENTION_V5(fused_attention_fwd_bf16_d128_causal_v5, bf16_t, true, false)
 ATTENTION_V5(fused_attention_fwd_bf16_d128_full_v5, bf16_t, false, false)
@@ -59,3 +60,9 @@ ATTENTION_V5(fused_attention_fwd_f16_d128_causal_v5, f16_t, true, false)
 ATTENTION_V5(fused_attention_fwd_f16_d128_full_v5, f16_t, false, false)
 ATTENTION_V5(fused_attention_fwd_f16_d128_causal_v5_ragged, f16_t, true, true)
 ATTENTION_V5(fused_attention_fwd_f16_d128_full_v5_ragged, f16_t, false, true)
+// Heads of at most 64 columns, zero-padded to 128 by the caller: the same tiles, half the matrix work
+// (the all-zero d slices and d blocks are skipped); any sequence lengths.
+ATTENTION_V5_DH(fused_attention_fwd_bf16_d64_causal_v5, bf16_t, true, true, 64)
+ATTENTION_V5_DH(fused_attention_fwd_bf16_d64_full_v5, bf16_t, false, true, 64)
+ATTENTION_V5_DH(fused_attention_fwd_f16_d64_causal_v5, f16_t, true, true, 64)
+ATTENTION_V5_DH(fused_attention_fwd_f16_d64_full_v5, f16_t, false, true, 64)

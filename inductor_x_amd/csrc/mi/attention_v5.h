@@ -36,7 +36,11 @@ constexpr int kAttnV5BM = kAttnV5Waves * 32;
 // WAVES = 8: one workgroup of 256 queries per CU.  WAVES = 4: 128 queries per workgroup and two
 // workgroups per CU (64 KiB of LDS each), so the two wavefronts of a SIMD belong to different
 // workgroups, share no barrier and drift apart in phase.
-template <typename T, bool CAUSAL, bool RAGGED, int WAVES = kAttnV5Waves>
+// DH: columns of the 128-wide head that carry data, 128 or 64.  With 64 (a smaller head zero-padded
+// to 128 by the caller) the d slices and d blocks that hold only zeros are skipped: half the matrix
+// instructions and half the LDS fragment reads per tile; the tiles still travel 128 wide and the
+// upper 64 output columns are left undefined (the caller drops them).
+template <typename T, bool CAUSAL, bool RAGGED, int WAVES = kAttnV5Waves, int DH = 128>
 __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, const T* __restrict__ K,
                                                       const T* __restrict__ V, T* __restrict__ O,
                                                       float* __restrict__ softmax_max,
@@ -66,6 +70,11 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   const T* __restrict__ Vh = V + kv_off;
 
   static_assert(WAVES == 8, "8 wavefronts");
+  static_assert(DH == 128 || DH == 64, "128 or 64 data columns");
+  constexpr int DS = DH / 16;  // d slices of a score product
+  constexpr int DB = DH / 32;  // d blocks of the output
+  constexpr int NA = 4 * DB;   // chunks (= MFMAs) of phase A
+  constexpr int NB = 2 * DS;   // chunks of phase B
   static_assert(sizeof(T) == 2, "16-bit elements");
   constexpr int BM = WAVES * 32;
   const int q0 = q_block * BM;
@@ -80,14 +89,14 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   const int qi = q0 + sub * 32 + li;
   const int qi_ld = RAGGED ? min(qi, Sq - 1) : qi;  // rows past the end work on a copy of the last row
 
-  x8_t qf[8];
+  x8_t qf[DS];
 #pragma unroll
-  for (int s = 0; s < 8; ++s)
+  for (int s = 0; s < DS; ++s)
     qf[s] = *reinterpret_cast<const x8_t*>(Qh + static_cast<size_t>(qi_ld) * kAttnD + 16 * s + 8 * g);
 
-  f32x16_t oacc[4];
+  f32x16_t oacc[DB];
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
   float m_run = -__builtin_inff(), m_true = -__builtin_inff(), l_run = 0.f, alpha = 1.f;
@@ -133,28 +142,28 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   f32x16_t sacc[2];  // [key block]
   u32x4_t pw[4];     // P of the current tile: [key slice of 16] x four 32-bit words
 
-  // K fragment of chunk i of phase B (key block i / 8, d slice i % 8): row 32 kb + li, chunk 2 ks + g
-  int k_off[8];
+  // K fragment of chunk i of phase B (key block i / DS, d slice i % DS): row 32 kb + li, chunk 2 ks + g
+  int k_off[DS];
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) k_off[ks] = li * kAttnD + 8 * ((2 * ks + g) ^ (li & 15));
+  for (int ks = 0; ks < DS; ++ks) k_off[ks] = li * kAttnD + 8 * ((2 * ks + g) ^ (li & 15));
   auto k_frag = [&](const T* Ks, int i) {
-    return *reinterpret_cast<const x8_t*>(Ks + 32 * (i >> 3) * kAttnD + k_off[i & 7]);
+    return *reinterpret_cast<const x8_t*>(Ks + 32 * (i / DS) * kAttnD + k_off[i % DS]);
   };
-  // V^T fragment of chunk i of phase A (key slice t4 = i / 4, d block db = i % 4) by two transposing
+  // V^T fragment of chunk i of phase A (key slice t4 = i / DB, d block db = i % DB) by two transposing
   // LDS reads: in each group of 16 lanes, lane s points at four consecutive d of key
   // 4 g + s / 4 (+ 8 for the second read) and receives, for its own d, the four keys of the group
-  int v_off[4];
+  int v_off[DB];
   {
     const int sl16 = lane & 15, grp = lane >> 4;
     const int key_l = 4 * (grp >> 1) + (sl16 >> 2);
     const int f = (0xE4A0 >> (4 * (key_l & 3))) & 15;
     const int c_l = 2 * (grp & 1) + ((sl16 & 3) >> 1);
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int db = 0; db < DB; ++db)
       v_off[db] = key_l * kAttnD + 8 * (((4 * db) ^ (f & 12)) + (c_l ^ (f & 2))) + 4 * (sl16 & 1);
   }
   auto v_frag = [&](const T* Vt, int i) {
-    const int t4 = i >> 2, db = i & 3;
+    const int t4 = i / DB, db = i % DB;
     const T* p0 = Vt + 16 * t4 * kAttnD + v_off[db];
     const typename E::x4 lo = E::read_tr(p0);
     const typename E::x4 hi = E::read_tr(p0 + 8 * kAttnD);
@@ -222,31 +231,44 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
     constexpr bool GUARD = decltype(guard_c)::value;
     constexpr int ODD = decltype(odd_c)::value ? 1 : 0;
     const T* Vt = Vbuf + (1 - ODD) * kTileElems;
-    x8_t f[16];
+    x8_t f[NA];
     if constexpr (DO_PV) {
       if (!GUARD || do_pv) {
         f[0] = v_frag(Vt, 0);
         f[1] = v_frag(Vt, 1);
       }
     }
-    static_for<16>([&](auto ic) {
+    static_for<NA>([&](auto ic) {
       constexpr int i = decltype(ic)::value;
-      constexpr int t4 = i >> 2, db = i & 3;
+      constexpr int t4 = i / DB, db = i % DB;
       if constexpr (DO_PV) {
         if (!GUARD || do_pv) {
-          if constexpr (i + 2 < 16) f[i + 2] = v_frag(Vt, i + 2);
+          if constexpr (i + 2 < NA) f[i + 2] = v_frag(Vt, i + 2);
           oacc[db] = E::mfma(f[i], __builtin_bit_cast(x8_t, pw[t4]), oacc[db]);
         }
       }
       if constexpr (i == 0) issue_k(k_tile, ODD);
       if constexpr (i == 1) issue_v(v_tile, ODD);
       if (!GUARD || do_sm) {
-        if constexpr (i == 0) softmax_rowmax(std::integral_constant<int, 0>());
-        if constexpr (i == 1) softmax_rowmax(std::integral_constant<int, 1>());
-        if constexpr (i == 2) softmax_ref();
-        // key slice j of P may be rewritten once chunk 4 j + 3 has issued its MFMA
-        if constexpr (i >= 4 && i < 12)
-          softmax_word(std::integral_constant<int, (i >= 4 && i < 12) ? (i >> 2) - 1 : 0>(), std::integral_constant<int, (i & 3)>());
+        if constexpr (DH == 128) {
+          if constexpr (i == 0) softmax_rowmax(std::integral_constant<int, 0>());
+          if constexpr (i == 1) softmax_rowmax(std::integral_constant<int, 1>());
+          if constexpr (i == 2) softmax_ref();
+          // key slice j of P may be rewritten once chunk 4 j + 3 has issued its MFMA
+          if constexpr (i >= 4 && i < 12)
+            softmax_word(std::integral_constant<int, (i >= 4 && i < 12) ? (i >> 2) - 1 : 0>(), std::integral_constant<int, (i & 3)>());
+        } else {
+          // eight chunks: key slice j of P may be rewritten once chunk 2 j + 1 has issued its MFMA
+          if constexpr (i == 0) {
+            softmax_rowmax(std::integral_constant<int, 0>());
+            softmax_rowmax(std::integral_constant<int, 1>());
+          }
+          if constexpr (i == 1) softmax_ref();
+          if constexpr (i >= 2 && i < 6) {
+            softmax_word(std::integral_constant<int, (i >= 2 && i < 6) ? (i - 2) / 2 : 0>(), std::integral_constant<int, 2 * (i & 1)>());
+            softmax_word(std::integral_constant<int, (i >= 2 && i < 6) ? (i - 2) / 2 : 0>(), std::integral_constant<int, 2 * (i & 1) + 1>());
+          }
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -254,7 +276,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   auto rescale = [&]() {
     if (__any(alpha != 1.0f)) {
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
     }
@@ -265,19 +287,19 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
     constexpr bool GUARD = decltype(guard_c)::value;
     constexpr int ODD = decltype(odd_c)::value ? 1 : 0;
     const T* Ks = Kbuf + (1 - ODD) * kTileElems;
-    x8_t f[16];
+    x8_t f[NB];
     if constexpr (DO_QK) {
       if (!GUARD || do_qk) {
         f[0] = k_frag(Ks, 0);
         f[1] = k_frag(Ks, 1);
       }
     }
-    static_for<16>([&](auto ic) {
+    static_for<NB>([&](auto ic) {
       constexpr int i = decltype(ic)::value;
-      constexpr int kb = i >> 3, ks = i & 7;
+      constexpr int kb = i / DS, ks = i % DS;
       if constexpr (DO_QK) {
         if (!GUARD || do_qk) {
-          if constexpr (i + 2 < 16) f[i + 2] = k_frag(Ks, i + 2);
+          if constexpr (i + 2 < NB) f[i + 2] = k_frag(Ks, i + 2);
           if constexpr (ks == 0) {
             f32x16_t z;
 #pragma unroll
@@ -289,11 +311,19 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
         }
       }
       if (!GUARD || do_sm) {
-        // key slices 2 and 3 of P read S's second key block, which chunk 8 starts to overwrite
-        if constexpr (i < 8) softmax_word(std::integral_constant<int, 2 + (i >> 2)>(), std::integral_constant<int, (i & 3)>());
-        if constexpr (i == 7) l_run = fmaf(l_run, alpha, psum);
+        // key slices 2 and 3 of P read S's second key block, which chunk DS starts to overwrite
+        if constexpr (DH == 128) {
+          if constexpr (i < 8) softmax_word(std::integral_constant<int, 2 + (i >> 2)>(), std::integral_constant<int, (i & 3)>());
+          if constexpr (i == 7) l_run = fmaf(l_run, alpha, psum);
+        } else {
+          if constexpr (i < 4) {
+            softmax_word(std::integral_constant<int, 2 + (i >> 1)>(), std::integral_constant<int, 2 * (i & 1)>());
+            softmax_word(std::integral_constant<int, 2 + (i >> 1)>(), std::integral_constant<int, 2 * (i & 1) + 1>());
+          }
+          if constexpr (i == 3) l_run = fmaf(l_run, alpha, psum);
+        }
       }
-      if constexpr (i == 15) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this iteration's tiles have landed
+      if constexpr (i == NB - 1) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this iteration's tiles have landed
       __builtin_amdgcn_sched_barrier(0);
     });
   };
@@ -309,8 +339,8 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
 #pragma unroll
       for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; ++i)
-      sacc[i >> 3] = E::mfma(k_frag(Kbuf, i), qf[i & 7], sacc[i >> 3]);
+    for (int i = 0; i < NB; ++i)
+      sacc[i / DS] = E::mfma(k_frag(Kbuf, i), qf[i % DS], sacc[i / DS]);
   }
   __syncthreads();  // K buffer 0 is rewritten in iteration 0
 
@@ -365,8 +395,8 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
     if (sm) {
       const T* Vt = Vbuf + kTileElems;
 #pragma unroll
-      for (int i = 0; i < 16; ++i)
-        oacc[i & 3] = E::mfma(v_frag(Vt, i), __builtin_bit_cast(x8_t, pw[i >> 2]), oacc[i & 3]);
+      for (int i = 0; i < NA; ++i)
+        oacc[i % DB] = E::mfma(v_frag(Vt, i), __builtin_bit_cast(x8_t, pw[i / DB]), oacc[i % DB]);
     }
   }
 
@@ -385,7 +415,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   {
     T* stage = reinterpret_cast<T*>(attn_lds) + wave * (32 * kAttnD);
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
         typename E::x4 o4;

@@ -131,10 +131,11 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
             and head_dim > 0 and query.size(2) > 0 and key.size(2) > 0 and (not causal or query.size(2) == key.size(2))):
         # the MFMA kernel: bf16 or fp16, head dimension 128, any sequence lengths.  A smaller head
         # dimension is padded with zero columns (scores and statistics do not change, the extra output
-        # columns are zero and dropped): twice the matrix work at 64, but no S x S tensor in memory
+        # columns are dropped); up to 64 columns the kernel skips the matrix work on the zero half
         pad = 128 - head_dim
         widen = (lambda t: torch.nn.functional.pad(t, (0, pad))) if pad else (lambda t: t.contiguous())  # noqa: E731
-        out, smax, ssum = kernels.fused_attention(widen(query), widen(key), widen(value), real_scale, causal)
+        out, smax, ssum = kernels.fused_attention(widen(query), widen(key), widen(value), real_scale, causal,
+                                                  data_columns=64 if head_dim <= 64 else 128)
         if pad:
             out = out[..., :head_dim].contiguous()
     else:

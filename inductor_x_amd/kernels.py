@@ -594,6 +594,15 @@ def _attention_launcher() -> CachingLauncher:
         for t in ("bf16", "f16")
         for c in (1, 0)
         for r in (0, 1)
+    ] + [
+        LaunchConfig(
+            f"fused_attention_fwd_{t}_d64_{'causal' if c else 'full'}_v5",
+            512,
+            meta={"DTYPE": t, "CAUSAL": c, "RAGGED": 1, "WAVES": 8, "DATA_COLUMNS": 64},
+            lds_bytes=_ATTN_LDS_BYTES,
+        )
+        for t in ("bf16", "f16")
+        for c in (1, 0)
     ]
     return CachingLauncher(
         "fused_attention_fwd_d128",
@@ -605,7 +614,7 @@ def _attention_launcher() -> CachingLauncher:
 
 
 def fused_attention(
-    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool, data_columns: int = 128
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """softmax(q k^T * scale [+ causal mask]) v for q [B, N, Sq, 128] and k, v [B, N, Sk, 128], bf16
     or fp16, any positive sequence lengths (a causal mask needs Sq == Sk).
@@ -614,7 +623,10 @@ def fused_attention(
     [B,N,Sq,8]); the statistics are the row maximum of the scaled scores and the row sum of
     exp(score - max), each repeated over the trailing axis.  Lengths that are multiples of 256
     (queries) and 128 (keys) run the kernel without bounds handling, all others the instantiation
-    that masks the ragged end."""
+    that masks the ragged end.
+    data_columns (128, or at most 64): how many leading columns of the 128-wide heads carry data; the
+    caller vouches that the others are zero in q, k and v (a smaller head padded to 128).  With at most 64
+    the kernel skips the matrix work on the zero half and leaves columns 64.. of `out` undefined."""
     _check_cuda(q, k, v)
     _require(q.dtype == k.dtype == v.dtype and q.dtype in _ATTN_DTYPES, "q, k, v must share bf16 or fp16")
     _require(q.dim() == 4 and k.dim() == 4 and k.shape == v.shape, "q [B, N, Sq, D]; k and v one [B, N, Sk, D] shape")
@@ -622,6 +634,7 @@ def fused_attention(
     Sk = k.shape[2]
     _require(k.shape[0] == B and k.shape[1] == N and k.shape[3] == D, "q, k, v must share batch, heads and head dimension")
     _require(D == 128, "head dimension must be 128")
+    _require(0 < data_columns <= 128, "data_columns must lie in 1..128")
     _require(Sq > 0 and Sk > 0, "sequence lengths must be positive")
     _require(not causal or Sq == Sk, "a causal mask needs equal query and key lengths")
     _require(q.is_contiguous() and k.is_contiguous() and v.is_contiguous(), "q, k, v must be contiguous (BNSD)")
@@ -636,8 +649,11 @@ def fused_attention(
         return out, smax, ssum
     ragged = Sq % _ATTN_BLOCK_QUERIES != 0 or Sk % 128 != 0
     l = _attention_launcher()
-    i = _find(l, f"fused_attention_fwd_{_ATTN_DTYPES[q.dtype]}_d128_{'causal' if causal else 'full'}_v5"
-                 f"{'_ragged' if ragged else ''}")
+    if data_columns <= 64:
+        i = _find(l, f"fused_attention_fwd_{_ATTN_DTYPES[q.dtype]}_d64_{'causal' if causal else 'full'}_v5")
+    else:
+        i = _find(l, f"fused_attention_fwd_{_ATTN_DTYPES[q.dtype]}_d128_{'causal' if causal else 'full'}_v5"
+                     f"{'_ragged' if ragged else ''}")
     n_qb = cdiv(Sq, _ATTN_BLOCK_QUERIES)
     per_head = (n_qb + 1) // 2 if causal else n_qb  # causal: query blocks (b, n - 1 - b) are one work item
     items = 8 * cdiv(heads, 8) * per_head

@@ -107,6 +107,33 @@ def test_attention_fp16_vs_oracle(K, O, B, N, Sq, Sk, causal):
     _check_against_oracle(K, O, q, k, v, 128 ** -0.5, causal)
 
 
+@pytest.mark.parametrize("dtype,B,N,Sq,Sk,D,causal", [
+    (torch.bfloat16, 2, 3, 512, 512, 64, True), (torch.bfloat16, 1, 5, 300, 300, 64, True), (torch.float16, 2, 2, 256, 384, 64, False),
+    (torch.float16, 1, 3, 77, 130, 40, False), (torch.bfloat16, 1, 9, 1024, 1024, 32, True), (torch.bfloat16, 1, 2, 1, 1, 8, True),
+])
+def test_attention_small_heads_skip_the_zero_half(K, dtype, B, N, Sq, Sk, D, causal):
+    """Heads of at most 64 columns, zero-padded to 128: the instantiation that skips the all-zero d
+    slices and d blocks returns bit for bit what the full-width kernel returns on the same padded
+    operands (the skipped products only add zeros), and that is right against fp32 attention."""
+    announce(f"attention, 64 data columns {dtype} B={B} N={N} Sq={Sq} Sk={Sk} D={D} causal={causal}")
+    torch.manual_seed(31)
+    pad = lambda t: torch.nn.functional.pad(t, (0, 128 - D))  # noqa: E731
+    q = torch.randn(B, N, Sq, D, device=DEV).to(dtype)
+    k, v = (torch.randn(B, N, Sk, D, device=DEV).to(dtype) for _ in range(2))
+    scale = D ** -0.5
+    narrow = K.fused_attention(pad(q), pad(k), pad(v), scale, causal, data_columns=64)
+    wide = K.fused_attention(pad(q), pad(k), pad(v), scale, causal)
+    assert torch.equal(narrow[0][..., :64], wide[0][..., :64])
+    assert torch.equal(narrow[1], wide[1]) and torch.equal(narrow[2], wide[2])
+    s = (q.float() @ k.float().transpose(-1, -2)) * scale
+    if causal:
+        s = s.masked_fill(torch.ones(Sq, Sk, device=DEV, dtype=torch.bool).triu(1), float("-inf"))
+    ref = torch.softmax(s, -1) @ v.float()
+    assert (narrow[0][..., :D].float() - ref).abs().max().item() <= 2e-2
+    with pytest.raises(ValueError):
+        K.fused_attention(pad(q), pad(k), pad(v), scale, causal, data_columns=0)
+
+
 def test_attention_closed_forms(K):
     """V = 1 gives O = 1 (probabilities sum to one); with a causal mask the first
     query row returns V[0]; identical keys give the running mean of V."""
@@ -448,7 +475,7 @@ def test_attention_op_reaches_the_fused_kernel_for_fp16_and_any_length(dtype, B,
     finally:
         log, launcher.launch_log = launcher.launch_log, None
     name = "f16" if dtype == torch.float16 else "bf16"
-    assert any(sym.startswith(f"fused_attention_fwd_{name}_d128_") for sym in log), log
+    assert any(sym.startswith(f"fused_attention_fwd_{name}_d{64 if D <= 64 else 128}_") for sym in log), log
     qf, kf, vf = (t.detach().float().requires_grad_() for t in (q, k, v))
     s = (qf @ kf.transpose(-1, -2)) / inv
     if causal:
