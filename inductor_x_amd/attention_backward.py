@@ -180,7 +180,9 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
         if pad_s:
             smax = torch.nn.functional.pad(smax, (0, 0, 0, pad_s), value=0.0)
             ssum = torch.nn.functional.pad(ssum, (0, 0, 0, pad_s), value=1.0)
-        grads = kernels.fused_attention_backward(widen(q), widen(k), widen(v), widen(out), widen(dout), smax, ssum, scale, causal)
+        # up to 64 columns the kernels skip the matrix work on the zero half of the padded heads
+        grads = kernels.fused_attention_backward(widen(q), widen(k), widen(v), widen(out), widen(dout), smax, ssum, scale, causal,
+                                                 data_columns=64 if d <= 64 else 128)
         return tuple(g[:, :, :S, :d].contiguous() for g in grads) if (pad_d or pad_s) else grads
     return _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale, causal, keep_prob, seed)
 

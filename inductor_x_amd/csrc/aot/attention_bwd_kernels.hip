@@ -47,27 +47,29 @@ __device__ __forceinline__ void bwd8_for_blocks(int n_heads, int S, Body&& body)
   }
 }
 
-#define BWD8_DQ(NAME, T, CAUSAL)                                                                       \
+#define BWD8_DQ_DH(NAME, T, CAUSAL, DH)                                                                \
   extern "C" __global__ __launch_bounds__(512, 1) void NAME(                                           \
       const T* q, const T* k, const T* v, const T* d_o, const float* stats, T* dq, int n_heads, int S, \
       float scale) {                                                                                   \
     bwd8_for_blocks<CAUSAL>(n_heads, S, [&](int head, int block) {                                     \
-      attention_bwd8_dq<T, CAUSAL>(q, k, v, d_o, stats, dq, S, block, head, scale);                    \
+      attention_bwd8_dq<T, CAUSAL, DH>(q, k, v, d_o, stats, dq, S, block, head, scale);                \
     });                                                                                                \
   }
+#define BWD8_DQ(NAME, T, CAUSAL) BWD8_DQ_DH(NAME, T, CAUSAL, 128)
 BWD8_DQ(attention_bwd8_dq_bf16_d128_causal, bf16_t, true)
 BWD8_DQ(attention_bwd8_dq_bf16_d128_full, bf16_t, false)
 BWD8_DQ(attention_bwd8_dq_f16_d128_causal, f16_t, true)
 BWD8_DQ(attention_bwd8_dq_f16_d128_full, f16_t, false)
 
-#define BWD8_DKV(NAME, T, CAUSAL, WHICH)                                                               \
+#define BWD8_DKV_DH(NAME, T, CAUSAL, WHICH, DH)                                                        \
   extern "C" __global__ __launch_bounds__(512, 1) void NAME(                                           \
       const T* q, const T* k, const T* v, const T* d_o, const float* stats, T* out, int n_heads,       \
       int S, float scale) {                                                                            \
     bwd8_for_blocks<CAUSAL>(n_heads, S, [&](int head, int block) {                                     \
-      attention_bwd8_dkv<T, CAUSAL, WHICH>(q, k, v, d_o, stats, out, S, block, head, scale);           \
+      attention_bwd8_dkv<T, CAUSAL, WHICH, DH>(q, k, v, d_o, stats, out, S, block, head, scale);       \
     });                                                                                                \
   }
+#define BWD8_DKV(NAME, T, CAUSAL, WHICH) BWD8_DKV_DH(NAME, T, CAUSAL, WHICH, 128)
 BWD8_DKV(attention_bwd8_dk_bf16_d128_causal, bf16_t, true, 0)
 BWD8_DKV(attention_bwd8_dk_bf16_d128_full, bf16_t, false, 0)
 BWD8_DKV(attention_bwd8_dv_bf16_d128_causal, bf16_t, true, 1)
@@ -76,3 +78,15 @@ BWD8_DKV(attention_bwd8_dk_f16_d128_causal, f16_t, true, 0)
 BWD8_DKV(attention_bwd8_dk_f16_d128_full, f16_t, false, 0)
 BWD8_DKV(attention_bwd8_dv_f16_d128_causal, f16_t, true, 1)
 BWD8_DKV(attention_bwd8_dv_f16_d128_full, f16_t, false, 1)
+
+// Heads of at most 64 columns, zero-padded to 128 by the caller: the all-zero d slices and d blocks
+// are skipped (half the matrix work, the same tiles).
+#define BWD8_D64(T, TN)                                                           \
+  BWD8_DQ_DH(attention_bwd8_dq_##TN##_d64_causal, T, true, 64)                     \
+  BWD8_DQ_DH(attention_bwd8_dq_##TN##_d64_full, T, false, 64)                      \
+  BWD8_DKV_DH(attention_bwd8_dk_##TN##_d64_causal, T, true, 0, 64)                 \
+  BWD8_DKV_DH(attention_bwd8_dk_##TN##_d64_full, T, false, 0, 64)                  \
+  BWD8_DKV_DH(attention_bwd8_dv_##TN##_d64_causal, T, true, 1, 64)                 \
+  BWD8_DKV_DH(attention_bwd8_dv_##TN##_d64_full, T, false, 1, 64)
+BWD8_D64(bf16_t, bf16)
+BWD8_D64(f16_t, f16)

@@ -154,15 +154,15 @@ __device__ __forceinline__ typename AttnElem<T>::x8 bwd8_col_frag(const T* tile,
 // STAGED = false stores from the registers (the causal kernels: they spill registers already and
 // the staging costs them more than it saves -- measured at [4,32,4096,128]: 2.44 against 2.42 ms for
 // the three causal kernels, 4.19 against 4.24 ms for the unmasked ones).
-template <bool STAGED, typename T>
-__device__ __forceinline__ void bwd8_store_acc(T* __restrict__ dst_block, const f32x16_t (&acc)[4], float factor,
+template <bool STAGED, typename T, int DB>
+__device__ __forceinline__ void bwd8_store_acc(T* __restrict__ dst_block, const f32x16_t (&acc)[DB], float factor,
                                                T* stage, int lane, int rows) {
   typedef typename AttnElem<T>::x4 x4_t;
   const int li = lane & 31, g = lane >> 5;
   if constexpr (!STAGED) {
   if (li < rows) {
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
         x4_t o4;
@@ -174,7 +174,7 @@ __device__ __forceinline__ void bwd8_store_acc(T* __restrict__ dst_block, const 
   return;
   }
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int rq = 0; rq < 4; ++rq) {
       x4_t o4;
@@ -190,9 +190,10 @@ __device__ __forceinline__ void bwd8_store_acc(T* __restrict__ dst_block, const 
     if (row < rows) *reinterpret_cast<u32x4_t*>(dst_block + row * kAttnD + 8 * c16) = v16;
   }
 }
-__device__ __forceinline__ void bwd8_zero(f32x16_t (&acc)[4]) {
+template <int DB>
+__device__ __forceinline__ void bwd8_zero(f32x16_t (&acc)[DB]) {
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
 }
@@ -200,7 +201,10 @@ __device__ __forceinline__ void bwd8_zero(f32x16_t (&acc)[4]) {
 // ---------------------------------------------------------------------------------------------
 // dQ
 // ---------------------------------------------------------------------------------------------
-template <typename T, bool CAUSAL>
+// DH (both kernels below): columns of the 128-wide head that carry data, 128 or 64; with 64 (a smaller
+// head zero-padded by the caller) the d slices and d blocks that hold only zeros are skipped and the
+// upper 64 columns of the result are left undefined.
+template <typename T, bool CAUSAL, int DH = 128>
 __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const T* __restrict__ K,
                                                   const T* __restrict__ V, const T* __restrict__ dO,
                                                   const float* __restrict__ stats, T* __restrict__ dQ,
@@ -219,9 +223,12 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
   const int qc = valid ? qi : S - 1;   // rows past the end read the last row and are never stored
   const size_t qrow = head_off + static_cast<size_t>(qc) * kAttnD;
 
-  x8_t qf[8], dof[8];
+  static_assert(DH == 128 || DH == 64, "128 or 64 data columns");
+  constexpr int DS = DH / 16, DB = DH / 32;   // d slices of a score product, d blocks of the result
+  constexpr int N1 = 2 * DS, N2 = 4 * DB;     // MFMA steps of the score phase and of the update phase
+  x8_t qf[DS], dof[DS];
 #pragma unroll
-  for (int s = 0; s < 8; ++s) {
+  for (int s = 0; s < DS; ++s) {
     qf[s] = *reinterpret_cast<const x8_t*>(Q + qrow + 16 * s + 8 * g);
     dof[s] = *reinterpret_cast<const x8_t*>(dO + qrow + 16 * s + 8 * g);
   }
@@ -229,7 +236,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
   const float m2 = st[0], delta = st[1];
   const float c2 = scale * kBwd8Log2e;
 
-  f32x16_t acc[4];
+  f32x16_t acc[DB];
   bwd8_zero(acc);
 
   const int all_tiles = S / kAttnBN;
@@ -264,24 +271,24 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
     // order pinned by scheduling fences: the softmax arithmetic of a key block then runs while
     // the fragments of the next steps are already in flight.
     constexpr int PF = BWD8_PREFETCH;
-    x8_t ka[16], va[16], ta[16];
+    x8_t ka[N1], va[N1], ta[N2];
     auto issue = [&](auto ic) {
       constexpr int i = decltype(ic)::value;
-      if constexpr (i < 16) {
-        ka[i] = bwd8_row_frag(Ks, 32 * (i >> 3) + li, i & 7, g);
-        va[i] = bwd8_row_frag(Vs, 32 * (i >> 3) + li, i & 7, g);
-      } else if constexpr (i < 32) {
-        ta[i - 16] = bwd8_col_frag(Kt, 32 * ((i - 16) & 3) + li, (i - 16) >> 2, g);
+      if constexpr (i < N1) {
+        ka[i] = bwd8_row_frag(Ks, 32 * (i / DS) + li, i % DS, g);
+        va[i] = bwd8_row_frag(Vs, 32 * (i / DS) + li, i % DS, g);
+      } else if constexpr (i < N1 + N2) {
+        ta[i - N1] = bwd8_col_frag(Kt, 32 * ((i - N1) % DB) + li, (i - N1) / DB, g);
       }
     };
     static_for<PF>([&](auto ic) { issue(ic); });
     f32x16_t sacc, pacc;
-    static_for<32>([&](auto ic) {
+    static_for<N1 + N2>([&](auto ic) {
       constexpr int i = decltype(ic)::value;
       issue(std::integral_constant<int, i + PF>{});
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (i < 16) {
-        constexpr int kb = i >> 3, s_ = i & 7;
+      if constexpr (i < N1) {
+        constexpr int kb = i / DS, s_ = i % DS;
         if constexpr (s_ == 0) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
@@ -292,7 +299,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
         sacc = E::mfma(ka[i], qf[s_], sacc);
         pacc = E::mfma(va[i], dof[s_], pacc);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (s_ == 7) {
+        if constexpr (s_ == DS - 1) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], c2, -m2));
@@ -302,7 +309,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
           __builtin_amdgcn_sched_barrier(0);
         }
       } else {
-        constexpr int j = i - 16, t = j >> 2, db = j & 3;
+        constexpr int j = i - N1, t = j / DB, db = j % DB;
         acc[db] = E::mfma(ta[j], dsf[t >> 1][t & 1], acc[db]);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -319,7 +326,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
         pacc[r] = 0.f;
       }
 #pragma unroll
-      for (int s = 0; s < 8; ++s) {
+      for (int s = 0; s < DS; ++s) {
         sacc = E::mfma(bwd8_row_frag(Ks, 32 * kb + li, s, g), qf[s], sacc);
         pacc = E::mfma(bwd8_row_frag(Vs, 32 * kb + li, s, g), dof[s], pacc);
       }
@@ -333,7 +340,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int db = 0; db < DB; ++db)
         acc[db] = E::mfma(bwd8_col_frag(Kt, 32 * db + li, t, g), dsf[t >> 1][t & 1], acc[db]);
   };
 
@@ -367,7 +374,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
 // ---------------------------------------------------------------------------------------------
 // dK (WHICH = 0) and dV (WHICH = 1): a wavefront owns 32 keys, loop over query tiles
 // ---------------------------------------------------------------------------------------------
-template <typename T, bool CAUSAL, int WHICH>
+template <typename T, bool CAUSAL, int WHICH, int DH = 128>
 __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, const T* __restrict__ K,
                                                    const T* __restrict__ V, const T* __restrict__ dO,
                                                    const float* __restrict__ stats, T* __restrict__ dKV,
@@ -389,13 +396,16 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
   const int kc = valid ? kj : S - 1;
   const size_t krow = head_off + static_cast<size_t>(kc) * kAttnD;
 
-  x8_t kf[8], vf[DK ? 8 : 1];
+  static_assert(DH == 128 || DH == 64, "128 or 64 data columns");
+  constexpr int DS = DH / 16, DB = DH / 32;
+  constexpr int N1 = 2 * DS, N2 = 4 * DB;
+  x8_t kf[DS], vf[DK ? DS : 1];
 #pragma unroll
-  for (int s = 0; s < 8; ++s) {
+  for (int s = 0; s < DS; ++s) {
     kf[s] = *reinterpret_cast<const x8_t*>(K + krow + 16 * s + 8 * g);
     if constexpr (DK) vf[s] = *reinterpret_cast<const x8_t*>(V + krow + 16 * s + 8 * g);
   }
-  f32x16_t acc[4];
+  f32x16_t acc[DB];
   bwd8_zero(acc);
   const float c2 = scale * kBwd8Log2e;
 
@@ -462,24 +472,24 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
     constexpr int PF = DK ? (CAUSAL ? BWD8_PREFETCH_DK_CAUSAL : BWD8_PREFETCH_DK) : BWD8_PREFETCH_DV;
     if constexpr (PF > 0 && !MASK) {
       // as in the dQ kernel: LDS fragments read PF steps ahead across the phases of the tile
-      x8_t qa[16], da[DK ? 16 : 1], ta[16];
+      x8_t qa[N1], da[DK ? N1 : 1], ta[N2];
       auto issue = [&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        if constexpr (i < 16) {
-          qa[i] = bwd8_row_frag(Qs, 32 * (i >> 3) + li, i & 7, g);
-          if constexpr (DK) da[i] = bwd8_row_frag(dOs, 32 * (i >> 3) + li, i & 7, g);
-        } else if constexpr (i < 32) {
-          ta[i - 16] = bwd8_col_frag(Tt, 32 * ((i - 16) & 3) + li, (i - 16) >> 2, g);
+        if constexpr (i < N1) {
+          qa[i] = bwd8_row_frag(Qs, 32 * (i / DS) + li, i % DS, g);
+          if constexpr (DK) da[i] = bwd8_row_frag(dOs, 32 * (i / DS) + li, i % DS, g);
+        } else if constexpr (i < N1 + N2) {
+          ta[i - N1] = bwd8_col_frag(Tt, 32 * ((i - N1) % DB) + li, (i - N1) / DB, g);
         }
       };
       static_for<PF>([&](auto ic) { issue(ic); });
       f32x16_t sacc, pacc;
-      static_for<32>([&](auto ic) {
+      static_for<N1 + N2>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
         issue(std::integral_constant<int, i + PF>{});
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (i < 16) {
-          constexpr int qb = i >> 3, s_ = i & 7;
+        if constexpr (i < N1) {
+          constexpr int qb = i / DS, s_ = i % DS;
           if constexpr (s_ == 0) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -490,12 +500,12 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
           sacc = E::mfma(qa[i], kf[s_], sacc);
           if constexpr (DK) pacc = E::mfma(da[i], vf[s_], pacc);
           __builtin_amdgcn_sched_barrier(0);
-          if constexpr (s_ == 7) {
+          if constexpr (s_ == DS - 1) {
             probabilities(std::integral_constant<int, qb>{}, sacc, pacc);
             __builtin_amdgcn_sched_barrier(0);
           }
         } else {
-          constexpr int j = i - 16, t = j >> 2, db = j & 3;
+          constexpr int j = i - N1, t = j / DB, db = j % DB;
           acc[db] = E::mfma(ta[j], bf[t >> 1][t & 1], acc[db]);
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -511,7 +521,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
         pacc[r] = 0.f;
       }
 #pragma unroll
-      for (int s = 0; s < 8; ++s) {
+      for (int s = 0; s < DS; ++s) {
         sacc = E::mfma(bwd8_row_frag(Qs, 32 * qb + li, s, g), kf[s], sacc);
         if constexpr (DK)
           pacc = E::mfma(bwd8_row_frag(dOs, 32 * qb + li, s, g), vf[s], pacc);
@@ -538,7 +548,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int db = 0; db < DB; ++db)
         acc[db] = E::mfma(bwd8_col_frag(Tt, 32 * db + li, t, g), bf[t >> 1][t & 1], acc[db]);
   };
 

@@ -688,8 +688,9 @@ def _attention_bwd_launchers() -> dict:
         **{
             which: mk(
                 f"attention_bwd8_{which[:2]}_d128", "PPPPPPiif",
-                [LaunchConfig(f"attention_bwd8_{which[:2]}_{t}_d128_{c}", 512, meta={"CAUSAL": c == "causal"}, lds_bytes=lds)
-                 for t in types for c in ("causal", "full")],
+                [LaunchConfig(f"attention_bwd8_{which[:2]}_{t}_d{d}_{c}", 512, meta={"CAUSAL": c == "causal", "DATA_COLUMNS": d},
+                              lds_bytes=lds)
+                 for t in types for d in (128, 64) for c in ("causal", "full")],
             )
             for which, lds in (("dq8", _ATTN_BWD8_DQ_LDS), ("dk8", _ATTN_BWD8_DK_LDS), ("dv8", _ATTN_BWD8_DV_LDS))
         },
@@ -698,11 +699,14 @@ def _attention_bwd_launchers() -> dict:
 
 def fused_attention_backward(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, dout: torch.Tensor,
-    softmax_max: torch.Tensor, softmax_sum: torch.Tensor, scale: float, causal: bool,
+    softmax_max: torch.Tensor, softmax_sum: torch.Tensor, scale: float, causal: bool, data_columns: int = 128,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients (dq, dk, dv) of fused_attention for [B, N, S, 128] bf16 or fp16 tensors; softmax_max /
     softmax_sum are the forward's [B, N, S, 8] fp32 statistics.  Workgroups of eight wavefronts on
-    256 rows, a statistics pass and separate dQ, dK and dV kernels; S a positive multiple of 64."""
+    256 rows, a statistics pass and separate dQ, dK and dV kernels; S a positive multiple of 64.
+    data_columns (128, or at most 64): how many leading columns of the 128-wide heads carry data, the
+    others being zero in q, k, v, out and dout (a smaller head padded to 128): with at most 64 the
+    kernels skip the matrix work on the zero half and leave columns 64.. of the gradients undefined."""
     _check_cuda(q, k, v, out, dout, softmax_max, softmax_sum)
     for t in (q, k, v, out, dout):
         _require(t.dtype == q.dtype and t.dtype in _ATTN_DTYPES and t.dim() == 4 and t.shape == q.shape,
@@ -724,6 +728,8 @@ def fused_attention_backward(
     which = "causal" if causal else "full"
     stats = torch.empty(heads * S, 2, dtype=torch.float32, device=q.device)
     ty = _ATTN_DTYPES[q.dtype]
+    _require(0 < data_columns <= 128, "data_columns must lie in 1..128")
+    dcols = 64 if data_columns <= 64 else 128
     ls["stats"]._launch(
         _find(ls["stats"], f"attention_bwd_stats_{ty}_d128"),
         (out.data_ptr(), dout.data_ptr(), softmax_max.data_ptr(), softmax_sum.data_ptr(), stats.data_ptr(), heads * S),
@@ -734,7 +740,7 @@ def fused_attention_backward(
     for name, dst in (("dk8", dk), ("dv8", dv), ("dq8", dq)):
         l = ls[name]
         l._launch(
-            _find(l, f"attention_bwd8_{name[:2]}_{ty}_d128_{which}"),
+            _find(l, f"attention_bwd8_{name[:2]}_{ty}_d{dcols}_{which}"),
             (q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), stats.data_ptr(), dst.data_ptr(), heads, S, float(scale)),
             grid, st,
         )

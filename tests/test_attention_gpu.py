@@ -317,6 +317,32 @@ def test_attention_backward_causal_any_length(K, dtype, B, N, S, D):
             AB.fused_attention_backward(q, k, v, o, do, m, l, scale, False, use_kernels=True)
 
 
+@pytest.mark.parametrize("dtype,B,N,S,D,causal", [(torch.bfloat16, 2, 3, 512, 64, True), (torch.float16, 1, 5, 320, 64, False),
+                                                   (torch.bfloat16, 1, 2, 256, 32, True), (torch.bfloat16, 1, 3, 1024, 48, False)])
+def test_attention_backward_small_heads_skip_the_zero_half(K, dtype, B, N, S, D, causal):
+    """Gradient kernels for heads of at most 64 columns, zero-padded to 128: the instantiations that
+    skip the all-zero d slices and d blocks return bit for bit what the full-width kernels return on
+    the same padded operands, and the op-level path (which picks them) agrees with the GEMM formulation."""
+    announce(f"attention backward, 64 data columns {dtype} B={B} N={N} S={S} D={D} causal={causal}")
+    from inductor_x_amd import attention_backward as AB
+
+    torch.manual_seed(33)
+    pad = lambda t: torch.nn.functional.pad(t, (0, 128 - D))  # noqa: E731
+    q, k, v, do = (torch.randn(B, N, S, D, device=DEV).to(dtype) for _ in range(4))
+    scale = D ** -0.5
+    o, m, l = K.fused_attention(pad(q), pad(k), pad(v), scale, causal, data_columns=64)
+    o[..., D:] = 0
+    narrow = K.fused_attention_backward(pad(q), pad(k), pad(v), o, pad(do), m, l, scale, causal, data_columns=64)
+    wide = K.fused_attention_backward(pad(q), pad(k), pad(v), o, pad(do), m, l, scale, causal)
+    for a, b in zip(narrow, wide):
+        assert torch.equal(a[..., :64], b[..., :64])
+    got = AB.fused_attention_backward(q, k, v, o[..., :D].contiguous(), do, m, l, scale, causal)
+    ref = AB.fused_attention_backward(q, k, v, o[..., :D].contiguous(), do, m, l, scale, causal, use_kernels=False)
+    for a, b, n in zip(got, ref, narrow):
+        assert a.shape == q.shape and torch.equal(a, n[..., :D])
+        assert (a.float() - b.float()).abs().max().item() <= 8e-3 * max(b.float().abs().max().item(), 1.0)
+
+
 @pytest.mark.parametrize("S,causal", [(64, True), (192, False), (320, True), (576, True)])
 def test_attention_backward_sequence_multiple_of_64(K, S, causal):
     """The backward kernels take any multiple of 64: last blocks of 64 and 192 rows (the output and
