@@ -15,10 +15,12 @@
 
 using namespace mi;
 
-template <typename T, bool CAUSAL, bool RAGGED, int DH = 128>
+template <typename T, bool CAUSAL, bool RAGGED, int DH = 128, bool MASKED = false>
 __device__ __forceinline__ void attention_entry_v5(const T* q, const T* k, const T* v, T* o, float* smax,
                                                    float* ssum, int n_heads, int Sq, int Sk,
-                                                   float scale_log2e) {
+                                                   float scale_log2e, const unsigned char* mask = nullptr,
+                                                   long long mask_batch_stride = 0, long long mask_head_stride = 0,
+                                                   int heads_per_batch = 1) {
   constexpr int XCDS = 8;
   const int n_qb = (Sq + kAttnV5BM - 1) / kAttnV5BM;
   const int per_head = CAUSAL ? (n_qb + 1) / 2 : n_qb;
@@ -29,15 +31,20 @@ __device__ __forceinline__ void attention_entry_v5(const T* q, const T* k, const
     const int slot = id / XCDS;
     const int head = (slot / per_head) * XCDS + xcd;
     if (head >= n_heads) continue;
+    // the [Sq, Sk] byte mask of this head (strides 0 where the mask broadcasts over batch or heads)
+    const unsigned char* hm =
+        MASKED ? mask + (head / heads_per_batch) * mask_batch_stride + (head % heads_per_batch) * mask_head_stride : nullptr;
     if (CAUSAL) {
       const int lo = slot % per_head;
       const int hi = n_qb - 1 - lo;
       const int n_pass = lo != hi ? 2 : 1;
 #pragma nounroll
       for (int pass = 0; pass < n_pass; ++pass)
-        attention_fwd_d128_v5<T, true, RAGGED, kAttnV5Waves, DH>(q, k, v, o, smax, ssum, Sq, Sk, pass == 0 ? hi : lo, head, scale_log2e);
+        attention_fwd_d128_v5<T, true, RAGGED, kAttnV5Waves, DH, MASKED>(q, k, v, o, smax, ssum, Sq, Sk, pass == 0 ? hi : lo, head,
+                                                                         scale_log2e, hm);
     } else {
-      attention_fwd_d128_v5<T, false, RAGGED, kAttnV5Waves, DH>(q, k, v, o, smax, ssum, Sq, Sk, slot % per_head, head, scale_log2e);
+      attention_fwd_d128_v5<T, false, RAGGED, kAttnV5Waves, DH, MASKED>(q, k, v, o, smax, ssum, Sq, Sk, slot % per_head, head,
+                                                                        scale_log2e, hm);
     }
   }
 }
@@ -66,3 +73,18 @@ ATTENTION_V5_DH(fused_attention_fwd_bf16_d64_causal_v5, bf16_t, true, true, 64)
 ATTENTION_V5_DH(fused_attention_fwd_bf16_d64_full_v5, bf16_t, false, true, 64)
 ATTENTION_V5_DH(fused_attention_fwd_f16_d64_causal_v5, f16_t, true, true, 64)
 ATTENTION_V5_DH(fused_attention_fwd_f16_d64_full_v5, f16_t, false, true, 64)
+
+// With a byte mask [B or 1, N or 1, Sq, Sk] (non-zero = hidden), any sequence lengths with Sk % 4 == 0.
+#define ATTENTION_V5_MASKED(NAME, T, CAUSAL)                                                            \
+  extern "C" __global__ __launch_bounds__(512, 1) void NAME(                                            \
+      const T* q, const T* k, const T* v, T* o, float* smax, float* ssum, int n_heads, int Sq, int Sk,  \
+      float scale_log2e, const unsigned char* mask, long long mask_batch_stride,                        \
+      long long mask_head_stride, int heads_per_batch) {                                                \
+    attention_entry_v5<T, CAUSAL, true, 128, true>(q, k, v, o, smax, ssum, n_heads, Sq, Sk, scale_log2e, \
+                                                   mask, mask_batch_stride, mask_head_stride,           \
+                                                   heads_per_batch);                                    \
+  }
+ATTENTION_V5_MASKED(fused_attention_fwd_bf16_d128_causal_v5_masked, bf16_t, true)
+ATTENTION_V5_MASKED(fused_attention_fwd_bf16_d128_full_v5_masked, bf16_t, false)
+ATTENTION_V5_MASKED(fused_attention_fwd_f16_d128_causal_v5_masked, f16_t, true)
+ATTENTION_V5_MASKED(fused_attention_fwd_f16_d128_full_v5_masked, f16_t, false)

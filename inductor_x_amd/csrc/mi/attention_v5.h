@@ -40,12 +40,17 @@ constexpr int kAttnV5BM = kAttnV5Waves * 32;
 // to 128 by the caller) the d slices and d blocks that hold only zeros are skipped: half the matrix
 // instructions and half the LDS fragment reads per tile; the tiles still travel 128 wide and the
 // upper 64 output columns are left undefined (the caller drops them).
-template <typename T, bool CAUSAL, bool RAGGED, int WAVES = kAttnV5Waves, int DH = 128>
+// MASKED: a byte mask [Sq, Sk] for this head (non-zero = the key is hidden from the query) is applied
+// to the scores besides the causal mask; needs RAGGED and Sk % 4 == 0.  A lane fetches the eight
+// dwords of its row that cover its keys of the next tile (bounded buffer loads: zero past the end)
+// while the current tile is worked on.  A row with every key hidden gives zeros, maximum 0 and sum 1.
+template <typename T, bool CAUSAL, bool RAGGED, int WAVES = kAttnV5Waves, int DH = 128, bool MASKED = false>
 __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, const T* __restrict__ K,
                                                       const T* __restrict__ V, T* __restrict__ O,
                                                       float* __restrict__ softmax_max,
                                                       float* __restrict__ softmax_sum, int Sq, int Sk,
-                                                      int q_block, int head, float scale_log2e) {
+                                                      int q_block, int head, float scale_log2e,
+                                                      const unsigned char* __restrict__ head_mask = nullptr) {
   typedef AttnElem<T> E;
   typedef typename E::x8 x8_t;
   constexpr bool GUARDED = CAUSAL || RAGGED;  // the last tiles of a block run the guarded copy of the loop
@@ -71,6 +76,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
 
   static_assert(WAVES == 8, "8 wavefronts");
   static_assert(DH == 128 || DH == 64, "128 or 64 data columns");
+  static_assert(!MASKED || RAGGED, "the masked instantiations are the bounds-checking ones");
   constexpr int DS = DH / 16;  // d slices of a score product
   constexpr int DB = DH / 32;  // d blocks of the output
   constexpr int NA = 4 * DB;   // chunks (= MFMAs) of phase A
@@ -186,6 +192,27 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
       for (int r = 0; r < 16; ++r)
         if (32 * kb + 8 * (r >> 2) + (r & 3) > d) sacc[kb][r] = -__builtin_inff();
   };
+  // ---- byte mask of this head: dwords of row qi_ld that hold the lane's keys of one tile ----
+  uint32_t mk[MASKED ? 8 : 1];
+  auto mask_fetch = [&](int tile) {
+    if constexpr (MASKED) {
+      const auto rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(head_mask), 0, Sq * Sk, 0x00020000);
+      const int row_off = qi_ld * Sk + tile * kAttnBN + 4 * g;
+#pragma unroll
+      for (int w = 0; w < 8; ++w) mk[w] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, row_off + 32 * (w >> 2) + 8 * (w & 3), 0, 0);
+    }
+  };
+  // hides what the fetched dwords mark in S(tile) and requests the dwords of the next tile
+  auto mask_apply = [&](int tile) {
+    if constexpr (MASKED) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if ((mk[4 * kb + (r >> 2)] >> (8 * (r & 3))) & 0xffu) sacc[kb][r] = -__builtin_inff();
+      mask_fetch(tile + 1);
+    }
+  };
   float mpart, mx, m_new, psum;
   auto softmax_rowmax = [&](auto kb_c) {
     constexpr int kb = decltype(kb_c)::value;
@@ -202,6 +229,8 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   };
   auto softmax_ref = [&]() {
     m_true = fmaxf(m_true, mx * scale_log2e);
+    // a finite floor keeps rows whose keys have all been hidden so far free of inf - inf
+    if constexpr (MASKED) m_true = fmaxf(m_true, -1e30f);
     m_new = m_true > m_run + kAttnSlack ? m_true : m_run;
     alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     m_run = m_new;
@@ -329,6 +358,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   };
 
   // ---- prologue: K(0), K(1) in LDS, S(0) ----
+  mask_fetch(0);
   issue_k(0, 0);
   issue_k(1, 1);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): Q fragments and the tiles above have landed
@@ -351,6 +381,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
       CAUSAL ? (RAGGED ? min(min(q0 + sub * 32 + 31, Sq - 1) / kAttnBN, real_tiles - 1) : first_masked + (sub >> 1))
              : real_tiles - 1;
   if (GUARDED && 0 == last_tile) apply_mask(0);
+  mask_apply(0);
   phase_a(No(), No(), min(2, n_tiles - 1), 0, No(), true, true);
   phase_b(Yes(), No(), No(), true, true);
   __syncthreads();
@@ -361,6 +392,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
       if constexpr (MASK) {
         if (t == last_tile) apply_mask(t);
       }
+      mask_apply(t);
       const bool sm = !MASK || t <= last_tile;
       phase_a(Yes(), Yes(), min(t + 2, n_tiles - 1), t, mask_c, t - 1 <= last_tile, sm);  // K past the end: a harmless reload
       if (sm) rescale();
@@ -372,6 +404,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
       if constexpr (MASK) {
         if (u == last_tile) apply_mask(u);
       }
+      mask_apply(u);
       const bool sm = !MASK || u <= last_tile;
       phase_a(Yes(), No(), min(u + 2, n_tiles - 1), u, mask_c, u - 1 <= last_tile, sm);
       if (sm) rescale();
@@ -388,6 +421,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
     t = n_tiles - 1;
     const bool sm = t <= last_tile;
     if (GUARDED && t == last_tile) apply_mask(t);
+    mask_apply(t);
     phase_a(Yes(), Yes(), t, t, std::integral_constant<bool, GUARDED>(), t - 1 <= last_tile, sm);
     if (sm) rescale();
     phase_b(No(), Yes(), std::integral_constant<bool, GUARDED>(), false, sm);
@@ -403,8 +437,9 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   // ---- epilogue ----
   const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
   const float l_tot = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
-  const float inv_l = 1.0f / l_tot;
-  const float l_true = l_tot * __builtin_amdgcn_exp2f(m_run - m_true);
+  const bool hidden_row = MASKED && l_tot == 0.f;  // every key of this query was hidden
+  const float inv_l = hidden_row ? 0.f : 1.0f / l_tot;
+  const float l_true = hidden_row ? 1.0f : l_tot * __builtin_amdgcn_exp2f(m_run - m_true);
   // The accumulators hold O^T: a lane owns one query and, per register quad, four consecutive d.
   // Stored from there a wavefront instruction would write 32 separate 16-byte pieces, one per row;
   // measured on MI355X those partial-line writes kept a workgroup's CU busy for about 5 us per query
@@ -434,7 +469,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   }
   if (g == 0 && (!RAGGED || qi < Sq)) {
     const size_t so = (static_cast<size_t>(head) * Sq + qi) * 8;
-    const float m_nat = m_true * 0.69314718055994530942f;
+    const float m_nat = hidden_row ? 0.f : m_true * 0.69314718055994530942f;
     Vec<float, 4> mv, lv;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {

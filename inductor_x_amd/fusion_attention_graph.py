@@ -15,9 +15,9 @@ through the op's own arguments: sparse_mode 2 or 3, or next_tockens == 0 with
 pre_tockens covering the sequence.  Supported: layouts "BNSD", "BSH", "SBH" ("BSH" and "SBH" are
 viewed as [B, N, S, D], copied once into that order for the kernels and copied back).  The fused
 kernel takes bf16 and fp16 operands with a head dimension that is a multiple of 8 up to 128
-(smaller heads are zero-padded to 128) at any query and key lengths; a positional bias (pse), a
-general boolean mask, fp32 operands, other head dimensions and dropout (keep_prob < 1) run the same
-mathematics over library GEMMs; padding masks, prefixes, variable sequence lengths and band masks
+(smaller heads are zero-padded to 128) at any query and key lengths, also with a general mask (any
+type, non-zero = hidden; key length a multiple of 4); a positional bias (pse), fp32 operands, other
+head dimensions and dropout (keep_prob < 1) run the same mathematics over library GEMMs; padding masks, prefixes, variable sequence lengths and band masks
 raise.
 The backward op recomputes the probabilities from the saved row statistics inside fused gradient
 kernels (bf16 or fp16, head dimension up to 128, equal lengths that are multiples of 64 or, with a causal mask, any;
@@ -127,7 +127,9 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
     mask = None if causal else atten_mask  # under the causal modes the mask tensor is the library's compressed triangle
     seed = numels = 0
     head_dim = query.size(3)
-    if (pse is None and mask is None and keep_prob == 1.0 and query.dtype in (torch.bfloat16, torch.float16) and head_dim <= 128 and head_dim % 8 == 0
+    mask_fits = mask is None or (mask.is_cuda and mask.dim() in (2, 4) and key.size(2) % 4 == 0
+                                 and query.size(2) * key.size(2) < 2 ** 31)
+    if (pse is None and mask_fits and keep_prob == 1.0 and query.dtype in (torch.bfloat16, torch.float16) and head_dim <= 128 and head_dim % 8 == 0
             and head_dim > 0 and query.size(2) > 0 and key.size(2) > 0 and (not causal or query.size(2) == key.size(2))):
         # the MFMA kernel: bf16 or fp16, head dimension 128, any sequence lengths.  A smaller head
         # dimension is padded with zero columns (scores and statistics do not change, the extra output
@@ -135,12 +137,12 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
         pad = 128 - head_dim
         widen = (lambda t: torch.nn.functional.pad(t, (0, pad))) if pad else (lambda t: t.contiguous())  # noqa: E731
         out, smax, ssum = kernels.fused_attention(widen(query), widen(key), widen(value), real_scale, causal,
-                                                  data_columns=64 if head_dim <= 64 else 128)
+                                                  data_columns=64 if head_dim <= 64 else 128, mask=mask)
         if pad:
             out = out[..., :head_dim].contiguous()
     else:
-        # head dimensions above 128 or not a multiple of 8, fp32, dropout, a positional bias or a general mask: the
-        # same mathematics over library GEMMs.  The dropout seed comes from torch's CPU generator (torch.manual_seed makes a
+        # head dimensions above 128 or not a multiple of 8, fp32, dropout, a positional bias, a mask over a key
+        # length that is no multiple of 4: the same mathematics over library GEMMs.  The dropout seed comes from torch's CPU generator (torch.manual_seed makes a
         # run repeatable) and travels to the backward in the op's seed output, as in the reference's op.
         from .attention_backward import attention_forward_over_gemms
 

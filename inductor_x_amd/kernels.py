@@ -613,8 +613,43 @@ def _attention_launcher() -> CachingLauncher:
     )
 
 
+@functools.lru_cache(maxsize=None)
+def _attention_masked_launcher() -> CachingLauncher:
+    cfgs = [
+        LaunchConfig(
+            f"fused_attention_fwd_{t}_d128_{'causal' if c else 'full'}_v5_masked",
+            512,
+            meta={"DTYPE": t, "CAUSAL": c, "RAGGED": 1, "WAVES": 8, "MASKED": 1},
+            lds_bytes=_ATTN_LDS_BYTES,
+        )
+        for t in ("bf16", "f16")
+        for c in (1, 0)
+    ]
+    return CachingLauncher(
+        "fused_attention_fwd_d128_masked",
+        codecache.aot_source("attention_kernels.hip"),
+        "PPPPPPiiifPqqi",
+        cfgs,
+        prefer_intree=True,
+    )
+
+
+def attention_mask_bytes(mask: torch.Tensor, B: int, N: int, Sq: int, Sk: int) -> torch.Tensor:
+    """A mask given as [Sq, Sk] or as a 4-D tensor that broadcasts to [B, N, Sq, Sk] (any type; non-zero =
+    the key is hidden from the query) as contiguous bytes [B or 1, N or 1, Sq, Sk], the form the masked
+    attention kernel reads.  A contiguous boolean mask is reinterpreted, not copied."""
+    if mask.dim() == 2:
+        mask = mask.view(1, 1, *mask.shape)
+    _require(mask.dim() == 4 and tuple(mask.shape[2:]) == (Sq, Sk) and mask.shape[0] in (1, B) and mask.shape[1] in (1, N),
+             f"mask of shape {tuple(mask.shape)} does not broadcast to [{B}, {N}, {Sq}, {Sk}]")
+    if mask.dtype == torch.bool:
+        return mask.contiguous().view(torch.uint8)
+    return (mask != 0).to(torch.uint8).contiguous()
+
+
 def fused_attention(
-    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool, data_columns: int = 128
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool, data_columns: int = 128,
+    mask: Optional[torch.Tensor] = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """softmax(q k^T * scale [+ causal mask]) v for q [B, N, Sq, 128] and k, v [B, N, Sk, 128], bf16
     or fp16, any positive sequence lengths (a causal mask needs Sq == Sk).
@@ -626,7 +661,10 @@ def fused_attention(
     that masks the ragged end.
     data_columns (128, or at most 64): how many leading columns of the 128-wide heads carry data; the
     caller vouches that the others are zero in q, k and v (a smaller head padded to 128).  With at most 64
-    the kernel skips the matrix work on the zero half and leaves columns 64.. of `out` undefined."""
+    the kernel skips the matrix work on the zero half and leaves columns 64.. of `out` undefined.
+    mask ([Sq, Sk] or broadcastable to [B, N, Sq, Sk], non-zero = the key is hidden from the query; needs
+    Sk % 4 == 0) is applied besides the causal mask; a query with every key hidden gets a zero output row,
+    maximum 0 and sum 1."""
     _check_cuda(q, k, v)
     _require(q.dtype == k.dtype == v.dtype and q.dtype in _ATTN_DTYPES, "q, k, v must share bf16 or fp16")
     _require(q.dim() == 4 and k.dim() == 4 and k.shape == v.shape, "q [B, N, Sq, D]; k and v one [B, N, Sk, D] shape")
@@ -647,6 +685,27 @@ def fused_attention(
     heads = B * N
     if heads == 0:
         return out, smax, ssum
+    n_qb = cdiv(Sq, _ATTN_BLOCK_QUERIES)
+    per_head = (n_qb + 1) // 2 if causal else n_qb  # causal: query blocks (b, n - 1 - b) are one work item
+    items = 8 * cdiv(heads, 8) * per_head
+    # persistent launch: at most one workgroup per CU, a multiple of 8 (one per die in turn); every
+    # workgroup walks items blockIdx.x, blockIdx.x + gridDim.x, ...
+    grid = min(items, max(config.hardware().cu_count // 8, 1) * 8)
+    if mask is not None:
+        _check_cuda(mask)
+        _require(Sk % 4 == 0, "a mask needs a key length that is a multiple of 4")
+        _require(Sq * Sk < 2**31, "a mask needs Sq * Sk below 2^31")
+        mb = attention_mask_bytes(mask, B, N, Sq, Sk)
+        lm = _attention_masked_launcher()
+        lm._launch(
+            _find(lm, f"fused_attention_fwd_{_ATTN_DTYPES[q.dtype]}_d128_{'causal' if causal else 'full'}_v5_masked"),
+            (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), smax.data_ptr(), ssum.data_ptr(), heads, Sq, Sk,
+             float(scale) * 1.4426950408889634, mb.data_ptr(), mb.stride(0) if mb.shape[0] > 1 else 0,
+             mb.stride(1) if mb.shape[1] > 1 else 0, N),
+            (grid, 1, 1),
+            _stream(),
+        )
+        return out, smax, ssum
     ragged = Sq % _ATTN_BLOCK_QUERIES != 0 or Sk % 128 != 0
     l = _attention_launcher()
     if data_columns <= 64:
@@ -654,12 +713,6 @@ def fused_attention(
     else:
         i = _find(l, f"fused_attention_fwd_{_ATTN_DTYPES[q.dtype]}_d128_{'causal' if causal else 'full'}_v5"
                      f"{'_ragged' if ragged else ''}")
-    n_qb = cdiv(Sq, _ATTN_BLOCK_QUERIES)
-    per_head = (n_qb + 1) // 2 if causal else n_qb  # causal: query blocks (b, n - 1 - b) are one work item
-    items = 8 * cdiv(heads, 8) * per_head
-    # persistent launch: at most one workgroup per CU, a multiple of 8 (one per die in turn); every
-    # workgroup walks items blockIdx.x, blockIdx.x + gridDim.x, ...
-    grid = min(items, max(config.hardware().cu_count // 8, 1) * 8)
     l._launch(
         i,
         (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), smax.data_ptr(), ssum.data_ptr(), heads, Sq, Sk,

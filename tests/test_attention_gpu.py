@@ -134,6 +134,55 @@ def test_attention_small_heads_skip_the_zero_half(K, dtype, B, N, Sq, Sk, D, cau
         K.fused_attention(pad(q), pad(k), pad(v), scale, causal, data_columns=0)
 
 
+@pytest.mark.parametrize("dtype,B,N,Sq,Sk,causal,mshape", [
+    (torch.bfloat16, 2, 3, 256, 256, False, (2, 1, 256, 256)), (torch.bfloat16, 1, 4, 300, 300, True, (300, 300)),
+    (torch.float16, 2, 2, 130, 200, False, (1, 2, 130, 200)), (torch.bfloat16, 1, 2, 512, 1024, False, (1, 1, 512, 1024)),
+    (torch.float16, 1, 3, 65, 68, False, (1, 3, 65, 68)), (torch.bfloat16, 2, 2, 1, 4, False, (2, 2, 1, 4)),
+])
+def test_attention_with_a_mask(K, dtype, B, N, Sq, Sk, causal, mshape):
+    """A general mask (non-zero = hidden) in the fused kernel, alone and together with the causal mask,
+    broadcast over batch and / or heads: output and statistics against fp32 attention with the same mask;
+    rows with every key hidden (planted) give zeros, maximum 0 and sum 1; a mask of zeros changes nothing."""
+    announce(f"attention with a mask {dtype} B={B} N={N} Sq={Sq} Sk={Sk} causal={causal} mask={mshape}")
+    torch.manual_seed(41)
+    q = torch.randn(B, N, Sq, 128, device=DEV).to(dtype)
+    k, v = (torch.randn(B, N, Sk, 128, device=DEV).to(dtype) for _ in range(2))
+    mask = torch.rand(*mshape, device=DEV) < 0.4
+    mask[..., 0] = False          # every row keeps its first key ...
+    if Sq > 2:
+        mask[..., Sq // 2, :] = True  # ... but one, which loses them all
+    if Sk > 70:
+        mask[..., 1, : 64] = True     # and one whose first tile is hidden entirely
+        mask[..., 1, 64] = False
+    scale = 0.11
+    out, smax, ssum = K.fused_attention(q, k, v, scale, causal, mask=mask)
+    s = (q.float() @ k.float().transpose(-1, -2)) * scale
+    hide = mask if mask.dim() == 4 else mask.view(1, 1, Sq, Sk)
+    hide = hide.expand(B, N, Sq, Sk).clone()
+    if causal:
+        hide |= torch.ones(Sq, Sk, device=DEV, dtype=torch.bool).triu(1)
+    s = s.masked_fill(hide, float("-inf"))
+    dead = hide.all(-1)
+    m = torch.where(dead, torch.zeros_like(s[..., 0]), s.amax(-1))
+    p = torch.exp(s - m.unsqueeze(-1))
+    l = torch.where(dead, torch.ones_like(m), p.sum(-1))
+    ref = torch.where(dead.unsqueeze(-1), torch.zeros_like(v.float()[..., :1, :]).expand(B, N, Sq, 128), (p / l.unsqueeze(-1)) @ v.float())
+    assert torch.isfinite(out).all() and (out.float() - ref).abs().max().item() <= 2e-2
+    torch.testing.assert_close(smax[..., 0], m, rtol=1e-3, atol=1e-3)
+    torch.testing.assert_close(ssum[..., 0], l, rtol=3e-3, atol=1e-6)
+    if Sq > 2:
+        assert dead.any() and out[dead].abs().max().item() == 0
+    # other mask types, and a mask that hides nothing
+    out8 = K.fused_attention(q, k, v, scale, causal, mask=mask.to(torch.int32) * 7)[0]
+    assert torch.equal(out8, out)
+    plain = K.fused_attention(q, k, v, scale, causal)
+    none = K.fused_attention(q, k, v, scale, causal, mask=torch.zeros(Sq, Sk, device=DEV, dtype=torch.bool))
+    assert (none[0].float() - plain[0].float()).abs().max().item() <= 1e-2
+    torch.testing.assert_close(none[1], plain[1], rtol=1e-6, atol=1e-6)
+    with pytest.raises(ValueError):
+        K.fused_attention(q, k, v, scale, causal, mask=torch.zeros(Sq + 1, Sk, device=DEV, dtype=torch.bool))
+
+
 def test_attention_closed_forms(K):
     """V = 1 gives O = 1 (probabilities sum to one); with a causal mask the first
     query row returns V[0]; identical keys give the running mean of V."""
