@@ -31,7 +31,7 @@ __device__ __forceinline__ void attention_entry_v5(const T* q, const T* k, const
     const int slot = id / XCDS;
     const int head = (slot / per_head) * XCDS + xcd;
     if (head >= n_heads) continue;
-    // the [Sq, Sk] byte mask of this head (strides 0 where the mask broadcasts over batch or heads)
+    // the [Sq][tiles] 64-bit mask words of this head (byte strides; 0 where the mask broadcasts over batch or heads)
     const unsigned char* hm =
         MASKED ? mask + (head / heads_per_batch) * mask_batch_stride + (head % heads_per_batch) * mask_head_stride : nullptr;
     if (CAUSAL) {
@@ -74,7 +74,7 @@ ATTENTION_V5_DH(fused_attention_fwd_bf16_d64_full_v5, bf16_t, false, true, 64)
 ATTENTION_V5_DH(fused_attention_fwd_f16_d64_causal_v5, f16_t, true, true, 64)
 ATTENTION_V5_DH(fused_attention_fwd_f16_d64_full_v5, f16_t, false, true, 64)
 
-// With a byte mask [B or 1, N or 1, Sq, Sk] (non-zero = hidden), any sequence lengths with Sk % 4 == 0.
+// With a bit mask, 64-bit words [B or 1, N or 1, Sq, ceil(Sk / 64)] (bit set = hidden), any sequence lengths.
 #define ATTENTION_V5_MASKED(NAME, T, CAUSAL)                                                            \
   extern "C" __global__ __launch_bounds__(512, 1) void NAME(                                            \
       const T* q, const T* k, const T* v, T* o, float* smax, float* ssum, int n_heads, int Sq, int Sk,  \

@@ -40,10 +40,11 @@ constexpr int kAttnV5BM = kAttnV5Waves * 32;
 // to 128 by the caller) the d slices and d blocks that hold only zeros are skipped: half the matrix
 // instructions and half the LDS fragment reads per tile; the tiles still travel 128 wide and the
 // upper 64 output columns are left undefined (the caller drops them).
-// MASKED: a byte mask [Sq, Sk] for this head (non-zero = the key is hidden from the query) is applied
-// to the scores besides the causal mask; needs RAGGED and Sk % 4 == 0.  A lane fetches the eight
-// dwords of its row that cover its keys of the next tile (bounded buffer loads: zero past the end)
-// while the current tile is worked on.  A row with every key hidden gives zeros, maximum 0 and sum 1.
+// MASKED: a bit mask for this head, one 64-bit word per (query, key tile) laid out [Sq][tiles], bit j of
+// a word set = key 64 tile + j is hidden from the query, is applied to the scores besides the causal
+// mask; needs RAGGED.  A lane fetches the word of its query for the next tile (one bounded 8-byte buffer
+// load: zero past the end) while the current tile is worked on.  A row with every key hidden gives zeros,
+// maximum 0 and sum 1.
 template <typename T, bool CAUSAL, bool RAGGED, int WAVES = kAttnV5Waves, int DH = 128, bool MASKED = false>
 __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, const T* __restrict__ K,
                                                       const T* __restrict__ V, T* __restrict__ O,
@@ -193,23 +194,29 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
         if (32 * kb + 8 * (r >> 2) + (r & 3) > d) sacc[kb][r] = -__builtin_inff();
   };
   // ---- byte mask of this head: dwords of row qi_ld that hold the lane's keys of one tile ----
-  uint32_t mk[MASKED ? 8 : 1];
+  u32x2_t mk;  // bits 0..31: the first key block of the tile, 32..63: the second
+  const int mask_tiles = (Sk + kAttnBN - 1) / kAttnBN;
   auto mask_fetch = [&](int tile) {
     if constexpr (MASKED) {
-      const auto rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(head_mask), 0, Sq * Sk, 0x00020000);
-      const int row_off = qi_ld * Sk + tile * kAttnBN + 4 * g;
-#pragma unroll
-      for (int w = 0; w < 8; ++w) mk[w] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, row_off + 32 * (w >> 2) + 8 * (w & 3), 0, 0);
+      const auto rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(head_mask), 0, Sq * mask_tiles * 8, 0x00020000);
+      mk = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (qi_ld * mask_tiles + min(tile, mask_tiles)) * 8, 0, 0);
+      if (tile >= mask_tiles) mk = u32x2_t{0u, 0u};  // tiles past the end hold no keys (already hidden by the length)
     }
   };
   // hides what the fetched dwords mark in S(tile) and requests the dwords of the next tile
   auto mask_apply = [&](int tile) {
     if constexpr (MASKED) {
+      // masks are mostly runs of visible or of hidden keys: a tile none of whose keys is hidden from
+      // any query of the wavefront (all its dwords zero) skips the selects
+      if (__any((mk[0] | mk[1]) != 0)) {
+        // accumulator register r of key block kb is key 32 kb + 8 (r / 4) + 4 g + r % 4
+        const uint32_t b0 = mk[0] >> (4 * g), b1 = mk[1] >> (4 * g);
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if ((mk[4 * kb + (r >> 2)] >> (8 * (r & 3))) & 0xffu) sacc[kb][r] = -__builtin_inff();
+        for (int r = 0; r < 16; ++r) {
+          if ((b0 >> (8 * (r >> 2) + (r & 3))) & 1u) sacc[0][r] = -__builtin_inff();
+          if ((b1 >> (8 * (r >> 2) + (r & 3))) & 1u) sacc[1][r] = -__builtin_inff();
+        }
+      }
       mask_fetch(tile + 1);
     }
   };

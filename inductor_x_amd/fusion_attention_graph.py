@@ -16,7 +16,7 @@ pre_tockens covering the sequence.  Supported: layouts "BNSD", "BSH", "SBH" ("BS
 viewed as [B, N, S, D], copied once into that order for the kernels and copied back).  The fused
 kernel takes bf16 and fp16 operands with a head dimension that is a multiple of 8 up to 128
 (smaller heads are zero-padded to 128) at any query and key lengths, also with a general mask (any
-type, non-zero = hidden; key length a multiple of 4); a positional bias (pse), fp32 operands, other
+type, non-zero = hidden); a positional bias (pse), fp32 operands, other
 head dimensions and dropout (keep_prob < 1) run the same mathematics over library GEMMs; padding masks, prefixes, variable sequence lengths and band masks
 raise.
 The backward op recomputes the probabilities from the saved row statistics inside fused gradient
@@ -127,8 +127,7 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
     mask = None if causal else atten_mask  # under the causal modes the mask tensor is the library's compressed triangle
     seed = numels = 0
     head_dim = query.size(3)
-    mask_fits = mask is None or (mask.is_cuda and mask.dim() in (2, 4) and key.size(2) % 4 == 0
-                                 and query.size(2) * key.size(2) < 2 ** 31)
+    mask_fits = mask is None or (mask.is_cuda and mask.dim() in (2, 4))
     if (pse is None and mask_fits and keep_prob == 1.0 and query.dtype in (torch.bfloat16, torch.float16) and head_dim <= 128 and head_dim % 8 == 0
             and head_dim > 0 and query.size(2) > 0 and key.size(2) > 0 and (not causal or query.size(2) == key.size(2))):
         # the MFMA kernel: bf16 or fp16, head dimension 128, any sequence lengths.  A smaller head
@@ -141,8 +140,8 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
         if pad:
             out = out[..., :head_dim].contiguous()
     else:
-        # head dimensions above 128 or not a multiple of 8, fp32, dropout, a positional bias, a mask over a key
-        # length that is no multiple of 4: the same mathematics over library GEMMs.  The dropout seed comes from torch's CPU generator (torch.manual_seed makes a
+        # head dimensions above 128 or not a multiple of 8, fp32, dropout, a positional bias: the same
+        # mathematics over library GEMMs.  The dropout seed comes from torch's CPU generator (torch.manual_seed makes a
         # run repeatable) and travels to the backward in the op's seed output, as in the reference's op.
         from .attention_backward import attention_forward_over_gemms
 

@@ -634,22 +634,29 @@ def _attention_masked_launcher() -> CachingLauncher:
     )
 
 
-def attention_mask_bytes(mask: torch.Tensor, B: int, N: int, Sq: int, Sk: int) -> torch.Tensor:
+def attention_mask_bits(mask: torch.Tensor, B: int, N: int, Sq: int, Sk: int) -> torch.Tensor:
     """A mask given as [Sq, Sk] or as a 4-D tensor that broadcasts to [B, N, Sq, Sk] (any type; non-zero =
-    the key is hidden from the query) as contiguous bytes [B or 1, N or 1, Sq, Sk], the form the masked
-    attention kernel reads.  A contiguous boolean mask is reinterpreted, not copied."""
+    the key is hidden from the query) packed for the masked attention kernel: bytes
+    [B or 1, N or 1, Sq, 8 * ceil(Sk / 64)], i.e. one little-endian 64-bit word per query and 64-key tile
+    whose bit j is set when key 64 * tile + j is hidden (bits past Sk are clear)."""
     if mask.dim() == 2:
         mask = mask.view(1, 1, *mask.shape)
     _require(mask.dim() == 4 and tuple(mask.shape[2:]) == (Sq, Sk) and mask.shape[0] in (1, B) and mask.shape[1] in (1, N),
              f"mask of shape {tuple(mask.shape)} does not broadcast to [{B}, {N}, {Sq}, {Sk}]")
-    if mask.dtype == torch.bool:
-        return mask.contiguous().view(torch.uint8)
-    return (mask != 0).to(torch.uint8).contiguous()
+    hide = mask if mask.dtype == torch.bool else mask != 0
+    tiles = cdiv(Sk, 64)
+    if tiles * 64 != Sk:
+        hide = torch.nn.functional.pad(hide, (0, tiles * 64 - Sk))
+    # 1, 2, 4, ... 128 made on the device (no host copy, so the packing can be captured in a HIP graph)
+    weights = torch.bitwise_left_shift(torch.ones(8, dtype=torch.uint8, device=mask.device),
+                                       torch.arange(8, dtype=torch.uint8, device=mask.device))
+    groups = hide.reshape(hide.shape[0], hide.shape[1], Sq, tiles * 8, 8).to(torch.uint8)
+    return (groups * weights).sum(-1, dtype=torch.uint8).contiguous()
 
 
 def fused_attention(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool, data_columns: int = 128,
-    mask: Optional[torch.Tensor] = None,
+    mask: Optional[torch.Tensor] = None, mask_is_packed: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """softmax(q k^T * scale [+ causal mask]) v for q [B, N, Sq, 128] and k, v [B, N, Sk, 128], bf16
     or fp16, any positive sequence lengths (a causal mask needs Sq == Sk).
@@ -662,9 +669,10 @@ def fused_attention(
     data_columns (128, or at most 64): how many leading columns of the 128-wide heads carry data; the
     caller vouches that the others are zero in q, k and v (a smaller head padded to 128).  With at most 64
     the kernel skips the matrix work on the zero half and leaves columns 64.. of `out` undefined.
-    mask ([Sq, Sk] or broadcastable to [B, N, Sq, Sk], non-zero = the key is hidden from the query; needs
-    Sk % 4 == 0) is applied besides the causal mask; a query with every key hidden gets a zero output row,
-    maximum 0 and sum 1."""
+    mask ([Sq, Sk] or broadcastable to [B, N, Sq, Sk], any type, non-zero = the key is hidden from the
+    query) is applied besides the causal mask (it is packed to one bit per key first; a caller that uses
+    one mask many times packs it once with attention_mask_bits and passes mask_is_packed=True); a query
+    with every key hidden gets a zero output row, maximum 0 and sum 1."""
     _check_cuda(q, k, v)
     _require(q.dtype == k.dtype == v.dtype and q.dtype in _ATTN_DTYPES, "q, k, v must share bf16 or fp16")
     _require(q.dim() == 4 and k.dim() == 4 and k.shape == v.shape, "q [B, N, Sq, D]; k and v one [B, N, Sk, D] shape")
@@ -693,9 +701,13 @@ def fused_attention(
     grid = min(items, max(config.hardware().cu_count // 8, 1) * 8)
     if mask is not None:
         _check_cuda(mask)
-        _require(Sk % 4 == 0, "a mask needs a key length that is a multiple of 4")
-        _require(Sq * Sk < 2**31, "a mask needs Sq * Sk below 2^31")
-        mb = attention_mask_bytes(mask, B, N, Sq, Sk)
+        if mask_is_packed:
+            mb = mask
+            _require(mb.dtype == torch.uint8 and mb.dim() == 4 and mb.is_contiguous() and mb.shape[0] in (1, B)
+                     and mb.shape[1] in (1, N) and tuple(mb.shape[2:]) == (Sq, 8 * cdiv(Sk, 64)),
+                     "a packed mask is what attention_mask_bits returns for these lengths")
+        else:
+            mb = attention_mask_bits(mask, B, N, Sq, Sk)
         lm = _attention_masked_launcher()
         lm._launch(
             _find(lm, f"fused_attention_fwd_{_ATTN_DTYPES[q.dtype]}_d128_{'causal' if causal else 'full'}_v5_masked"),

@@ -138,6 +138,7 @@ def test_attention_small_heads_skip_the_zero_half(K, dtype, B, N, Sq, Sk, D, cau
     (torch.bfloat16, 2, 3, 256, 256, False, (2, 1, 256, 256)), (torch.bfloat16, 1, 4, 300, 300, True, (300, 300)),
     (torch.float16, 2, 2, 130, 200, False, (1, 2, 130, 200)), (torch.bfloat16, 1, 2, 512, 1024, False, (1, 1, 512, 1024)),
     (torch.float16, 1, 3, 65, 68, False, (1, 3, 65, 68)), (torch.bfloat16, 2, 2, 1, 4, False, (2, 2, 1, 4)),
+    (torch.bfloat16, 1, 2, 77, 131, False, (77, 131)), (torch.float16, 1, 1, 333, 333, True, (1, 1, 333, 333)),
 ])
 def test_attention_with_a_mask(K, dtype, B, N, Sq, Sk, causal, mshape):
     """A general mask (non-zero = hidden) in the fused kernel, alone and together with the causal mask,
@@ -175,6 +176,9 @@ def test_attention_with_a_mask(K, dtype, B, N, Sq, Sk, causal, mshape):
     # other mask types, and a mask that hides nothing
     out8 = K.fused_attention(q, k, v, scale, causal, mask=mask.to(torch.int32) * 7)[0]
     assert torch.equal(out8, out)
+    packed = K.attention_mask_bits(mask, B, N, Sq, Sk)
+    assert packed.dtype == torch.uint8 and packed.shape[-1] == 8 * ((Sk + 63) // 64)
+    assert torch.equal(K.fused_attention(q, k, v, scale, causal, mask=packed, mask_is_packed=True)[0], out)
     plain = K.fused_attention(q, k, v, scale, causal)
     none = K.fused_attention(q, k, v, scale, causal, mask=torch.zeros(Sq, Sk, device=DEV, dtype=torch.bool))
     assert (none[0].float() - plain[0].float()).abs().max().item() <= 1e-2
