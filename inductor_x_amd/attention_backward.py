@@ -142,11 +142,25 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
     sequence length that is a multiple of 64 or, under a causal mask, any; smaller head dimensions and causal
     lengths in between are zero-padded).
     keep_prob < 1 with the forward's seed regenerates the forward's dropout mask (GEMM path only).
-    With pse or atten_mask (GEMM path only) the result has a fourth member, the gradient of pse in
-    pse's own shape (None without pse)."""
+    With pse or atten_mask the result has a fourth member, the gradient of pse in pse's own shape (None
+    without pse); a mask alone runs on the fused kernels under the same shape limits, pse over GEMMs."""
+    masked_fit = (atten_mask is not None and pse is None and keep_prob == 1.0 and q.dim() == 4 and q.shape == k.shape
+                  and q.dtype in (torch.bfloat16, torch.float16) and 0 < q.size(3) <= 128 and q.size(3) % 8 == 0
+                  and q.size(2) > 0 and q.size(2) % 64 == 0 and atten_mask.is_cuda and atten_mask.dim() in (2, 4))
+    if masked_fit and use_kernels is not False:
+        # a general mask on the fused gradient kernels (bit-packed; one shape for q, k, v, a multiple of 64)
+        from . import kernels
+
+        d = q.size(3)
+        widen = (lambda t: torch.nn.functional.pad(t, (0, 128 - d))) if d < 128 else (lambda t: t.contiguous())  # noqa: E731
+        grads = kernels.fused_attention_backward(widen(q), widen(k), widen(v), widen(out), widen(dout),
+                                                 softmax_max.contiguous(), softmax_sum.contiguous(), scale, causal, mask=atten_mask)
+        grads = tuple(g[..., :d].contiguous() for g in grads) if d < 128 else grads
+        return grads + (None,)
     if pse is not None or atten_mask is not None:
         if use_kernels:
-            raise NotImplementedError("attention backward: the fused kernels take no bias or mask")
+            raise NotImplementedError("attention backward: the fused kernels take no bias, and a mask only for one shape "
+                                      "of q, k, v and a sequence length that is a multiple of 64")
         return _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale, causal, keep_prob, seed,
                                     pse=pse, atten_mask=atten_mask)
     # a length that is no multiple of 64 is served under a causal mask only (see the padding note below)

@@ -90,3 +90,32 @@ BWD8_DKV(attention_bwd8_dv_f16_d128_full, f16_t, false, 1)
   BWD8_DKV_DH(attention_bwd8_dv_##TN##_d64_full, T, false, 1, 64)
 BWD8_D64(bf16_t, bf16)
 BWD8_D64(f16_t, f16)
+
+// With a bit mask (64-bit words [B or 1, N or 1, S, S / 64], byte strides; dQ takes the words of the mask,
+// dK and dV those of its transpose): hidden pairs get the probability zero.
+#define BWD8_MASKED(NAME, T, CAUSAL, BODY)                                                             \
+  extern "C" __global__ __launch_bounds__(512, 1) void NAME(                                           \
+      const T* q, const T* k, const T* v, const T* d_o, const float* stats, T* out, int n_heads,       \
+      int S, float scale, const unsigned char* mask, long long mask_batch_stride,                      \
+      long long mask_head_stride, int heads_per_batch) {                                               \
+    bwd8_for_blocks<CAUSAL>(n_heads, S, [&](int head, int block) {                                     \
+      const unsigned char* hm =                                                                        \
+          mask + (head / heads_per_batch) * mask_batch_stride + (head % heads_per_batch) * mask_head_stride; \
+      BODY;                                                                                            \
+    });                                                                                                \
+  }
+#define BWD8_MASKED_ALL(T, TN)                                                                                     \
+  BWD8_MASKED(attention_bwd8_dq_##TN##_d128_causal_masked, T, true,                                               \
+              (attention_bwd8_dq<T, true, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm)))         \
+  BWD8_MASKED(attention_bwd8_dq_##TN##_d128_full_masked, T, false,                                                \
+              (attention_bwd8_dq<T, false, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm)))        \
+  BWD8_MASKED(attention_bwd8_dk_##TN##_d128_causal_masked, T, true,                                               \
+              (attention_bwd8_dkv<T, true, 0, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm)))     \
+  BWD8_MASKED(attention_bwd8_dk_##TN##_d128_full_masked, T, false,                                                \
+              (attention_bwd8_dkv<T, false, 0, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm)))    \
+  BWD8_MASKED(attention_bwd8_dv_##TN##_d128_causal_masked, T, true,                                               \
+              (attention_bwd8_dkv<T, true, 1, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm)))     \
+  BWD8_MASKED(attention_bwd8_dv_##TN##_d128_full_masked, T, false,                                                \
+              (attention_bwd8_dkv<T, false, 1, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm)))
+BWD8_MASKED_ALL(bf16_t, bf16)
+BWD8_MASKED_ALL(f16_t, f16)

@@ -204,11 +204,16 @@ __device__ __forceinline__ void bwd8_zero(f32x16_t (&acc)[DB]) {
 // DH (both kernels below): columns of the 128-wide head that carry data, 128 or 64; with 64 (a smaller
 // head zero-padded by the caller) the d slices and d blocks that hold only zeros are skipped and the
 // upper 64 columns of the result are left undefined.
-template <typename T, bool CAUSAL, int DH = 128>
+// BITS (both kernels below): a bit mask for this head, one 64-bit word per (row, tile of the other axis)
+// laid out [S][S / 64], bit j set = the pair is hidden (dQ: row = query, bit = key of the tile; dK / dV:
+// row = key, bit = query of the tile, i.e. the words of the transposed mask); hidden pairs get the
+// probability zero.  The word of the next tile is fetched with that tile's operands.
+template <typename T, bool CAUSAL, int DH = 128, bool BITS = false>
 __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const T* __restrict__ K,
                                                   const T* __restrict__ V, const T* __restrict__ dO,
                                                   const float* __restrict__ stats, T* __restrict__ dQ,
-                                                  int S, int q_block, int head, float scale) {
+                                                  int S, int q_block, int head, float scale,
+                                                  const unsigned char* __restrict__ head_mask = nullptr) {
   typedef AttnElem<T> E;
   typedef typename E::x8 x8_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char attn_lds[];
@@ -246,11 +251,15 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
   auto buf = [&](int b) { return reinterpret_cast<T*>(attn_lds + b * kBwd8DqBufBytes); };
   Bwd8ColStage kt;
   Bwd8RowStage vt;
+  u32x2_t mk_next, mk_cur;  // mask words of this lane's query: the tile being loaded, the tile being computed
   auto load_tile = [&](int tile) {
     bwd8_load(kt, Kh + static_cast<size_t>(tile) * kAttnBN * kAttnD, tid);
     bwd8_load(vt, Vh + static_cast<size_t>(tile) * kAttnBN * kAttnD, tid);
+    if constexpr (BITS)
+      mk_next = *reinterpret_cast<const u32x2_t*>(head_mask + (static_cast<size_t>(qc) * all_tiles + tile) * 8);
   };
   auto store_tile = [&](int b) {
+    if constexpr (BITS) mk_cur = mk_next;
     T* Ks = buf(b);
     bwd8_store_rows(kt, Ks, tid);
     bwd8_store_rows(vt, Ks + kBwd8RowTile, tid);
@@ -265,7 +274,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
     const int key0 = tile * kAttnBN;
     x8_t dsf[2][2];
 #if BWD8_PREFETCH > 0
-    if constexpr (!MASK) {
+    if constexpr (!MASK && !BITS) {  // the masked instantiations have no registers for fragments in flight
     // The 32 MFMA steps of a tile (16 score / dP pairs, then 16 dQ updates) read their LDS
     // fragments BWD8_PREFETCH steps ahead, across the boundaries between the phases, with the
     // order pinned by scheduling fences: the softmax arithmetic of a key block then runs while
@@ -304,6 +313,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
           for (int r = 0; r < 16; ++r) {
             float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], c2, -m2));
             if (MASK && key0 + 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3) > qi) p = 0.f;
+            if (BITS && ((mk_cur[kb] >> (8 * (r >> 2) + 4 * g + (r & 3))) & 1u)) p = 0.f;
             dsf[kb][r >> 3][r & 7] = static_cast<T>(p * (pacc[r] - delta));
           }
           __builtin_amdgcn_sched_barrier(0);
@@ -334,6 +344,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
       for (int r = 0; r < 16; ++r) {
         float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], c2, -m2));
         if (MASK && key0 + 32 * kb + 8 * (r >> 2) + 4 * g + (r & 3) > qi) p = 0.f;
+        if (BITS && ((mk_cur[kb] >> (8 * (r >> 2) + 4 * g + (r & 3))) & 1u)) p = 0.f;
         dsf[kb][r >> 3][r & 7] = static_cast<T>(p * (pacc[r] - delta));
       }
     }
@@ -374,11 +385,12 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
 // ---------------------------------------------------------------------------------------------
 // dK (WHICH = 0) and dV (WHICH = 1): a wavefront owns 32 keys, loop over query tiles
 // ---------------------------------------------------------------------------------------------
-template <typename T, bool CAUSAL, int WHICH, int DH = 128>
+template <typename T, bool CAUSAL, int WHICH, int DH = 128, bool BITS = false>
 __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, const T* __restrict__ K,
                                                    const T* __restrict__ V, const T* __restrict__ dO,
                                                    const float* __restrict__ stats, T* __restrict__ dKV,
-                                                   int S, int k_block, int head, float scale) {
+                                                   int S, int k_block, int head, float scale,
+                                                   const unsigned char* __restrict__ head_mask = nullptr) {
   constexpr bool DK = WHICH == 0;
   constexpr int BUF = DK ? kBwd8DkBufBytes : kBwd8DvBufBytes;
   constexpr int STAT_OFF = BUF - kBwd8StatBytes;
@@ -417,14 +429,18 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
   Bwd8ColStage cst;  // DK: Q, DV: dO
   Bwd8RowStage rst;  // DK: dO, DV: Q
   Vec<float, 2> sst;
+  u32x2_t mk_next, mk_cur;  // words of the transposed mask for this lane's key: tile being loaded / computed
   auto load_tile = [&](int tile) {
     const T* qp = Qh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
     const T* dp = dOh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
     bwd8_load(cst, DK ? qp : dp, tid);
     bwd8_load(rst, DK ? dp : qp, tid);
+    if constexpr (BITS)
+      mk_next = *reinterpret_cast<const u32x2_t*>(head_mask + (static_cast<size_t>(kc) * n_qtiles + tile) * 8);
     if (tid < kAttnBN) sst = load_vec<float, 2>(stats + 2 * (static_cast<size_t>(head) * S + tile * kAttnBN + tid));
   };
   auto store_tile = [&](int b) {
+    if constexpr (BITS) mk_cur = mk_next;
     T* base = reinterpret_cast<T*>(attn_lds + b * BUF);
     if constexpr (DK) {
       bwd8_store_rows(cst, base, tid);                        // Q
@@ -461,6 +477,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
           const int r = 4 * rq + e;
           float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], c2, -mrow[e]));
           if (MASK && kj > q0t + row0 + e) p = 0.f;
+          if (BITS && ((mk_cur[qb] >> (8 * rq + 4 * g + e)) & 1u)) p = 0.f;
           if constexpr (DK)
             bf[qb][r >> 3][r & 7] = static_cast<T>(p * (pacc[r] - drow[e]));
           else
@@ -470,7 +487,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
     };
     // the causal dK kernel has no registers to spare for fragments in flight beyond one step
     constexpr int PF = DK ? (CAUSAL ? BWD8_PREFETCH_DK_CAUSAL : BWD8_PREFETCH_DK) : BWD8_PREFETCH_DV;
-    if constexpr (PF > 0 && !MASK) {
+    if constexpr (PF > 0 && !MASK && !BITS) {
       // as in the dQ kernel: LDS fragments read PF steps ahead across the phases of the tile
       x8_t qa[N1], da[DK ? N1 : 1], ta[N2];
       auto issue = [&](auto ic) {
@@ -538,6 +555,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
           const int r = 4 * rq + e;
           float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], c2, -mrow[e]));
           if (MASK && kj > q0t + row0 + e) p = 0.f;
+          if (BITS && ((mk_cur[qb] >> (8 * rq + 4 * g + e)) & 1u)) p = 0.f;
           if constexpr (DK)
             bf[qb][r >> 3][r & 7] = static_cast<T>(p * (pacc[r] - drow[e]));
           else

@@ -22,7 +22,8 @@ raise.
 The backward op recomputes the probabilities from the saved row statistics inside fused gradient
 kernels (bf16 or fp16, head dimension up to 128, equal lengths that are multiples of 64 or, with a causal mask, any;
 kernels.fused_attention_backward) and falls back to the GEMM formulation otherwise
-(attention_backward.py), which also returns the gradient of pse; the training variant of the
+(attention_backward.py), which also returns the gradient of pse; a general mask runs the fused
+gradient kernels too (one shape for q, k, v, a multiple of 64); the training variant of the
 pattern is registered beside the inference one.
 """
 from __future__ import annotations

@@ -762,16 +762,34 @@ def _attention_bwd_launchers() -> dict:
     }
 
 
+@functools.lru_cache(maxsize=None)
+def _attention_bwd_masked_launchers() -> dict:
+    src = codecache.aot_source("attention_bwd_kernels.hip")
+    return {
+        which: CachingLauncher(
+            f"attention_bwd8_{which[:2]}_d128_masked", src, "PPPPPPiifPqqi",
+            [LaunchConfig(f"attention_bwd8_{which[:2]}_{t}_d128_{c}_masked", 512, meta={"CAUSAL": c == "causal", "MASKED": 1},
+                          lds_bytes=lds)
+             for t in _ATTN_DTYPES.values() for c in ("causal", "full")],
+            prefer_intree=True,
+        )
+        for which, lds in (("dq8", _ATTN_BWD8_DQ_LDS), ("dk8", _ATTN_BWD8_DK_LDS), ("dv8", _ATTN_BWD8_DV_LDS))
+    }
+
+
 def fused_attention_backward(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, dout: torch.Tensor,
     softmax_max: torch.Tensor, softmax_sum: torch.Tensor, scale: float, causal: bool, data_columns: int = 128,
+    mask: Optional[torch.Tensor] = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients (dq, dk, dv) of fused_attention for [B, N, S, 128] bf16 or fp16 tensors; softmax_max /
     softmax_sum are the forward's [B, N, S, 8] fp32 statistics.  Workgroups of eight wavefronts on
     256 rows, a statistics pass and separate dQ, dK and dV kernels; S a positive multiple of 64.
     data_columns (128, or at most 64): how many leading columns of the 128-wide heads carry data, the
     others being zero in q, k, v, out and dout (a smaller head padded to 128): with at most 64 the
-    kernels skip the matrix work on the zero half and leave columns 64.. of the gradients undefined."""
+    kernels skip the matrix work on the zero half and leave columns 64.. of the gradients undefined.
+    mask: the forward's mask ([S, S] or broadcastable to [B, N, S, S], non-zero = hidden); it is packed to
+    bits, once as it stands for dQ and once transposed for dK and dV."""
     _check_cuda(q, k, v, out, dout, softmax_max, softmax_sum)
     for t in (q, k, v, out, dout):
         _require(t.dtype == q.dtype and t.dtype in _ATTN_DTYPES and t.dim() == 4 and t.shape == q.shape,
@@ -802,6 +820,22 @@ def fused_attention_backward(
     )
     blocks = cdiv(S, 256)
     grid = (8 * cdiv(heads, 8) * (cdiv(blocks, 2) if causal else blocks), 1, 1)  # causal: pairs of blocks
+    if mask is not None:
+        _check_cuda(mask)
+        m4 = mask.view(1, 1, *mask.shape) if mask.dim() == 2 else mask
+        rows = attention_mask_bits(m4, B, N, S, S)                     # [.., query, key tiles]
+        cols = attention_mask_bits(m4.transpose(-1, -2), B, N, S, S)   # [.., key, query tiles]
+        lm = _attention_bwd_masked_launchers()
+        for name, dst, words in (("dk8", dk, cols), ("dv8", dv, cols), ("dq8", dq, rows)):
+            l = lm[name]
+            l._launch(
+                _find(l, f"attention_bwd8_{name[:2]}_{ty}_d128_{which}_masked"),
+                (q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), stats.data_ptr(), dst.data_ptr(), heads, S,
+                 float(scale), words.data_ptr(), words.stride(0) if words.shape[0] > 1 else 0,
+                 words.stride(1) if words.shape[1] > 1 else 0, N),
+                grid, st,
+            )
+        return dq, dk, dv
     for name, dst in (("dk8", dk), ("dv8", dv), ("dq8", dq)):
         l = ls[name]
         l._launch(

@@ -396,6 +396,70 @@ def test_attention_backward_small_heads_skip_the_zero_half(K, dtype, B, N, S, D,
         assert (a.float() - b.float()).abs().max().item() <= 8e-3 * max(b.float().abs().max().item(), 1.0)
 
 
+@pytest.mark.parametrize("dtype,B,N,S,D,causal,mshape", [
+    (torch.bfloat16, 2, 3, 256, 128, False, (2, 1, 256, 256)), (torch.float16, 1, 2, 320, 128, True, (320, 320)),
+    (torch.bfloat16, 1, 4, 512, 64, False, (1, 4, 512, 512)), (torch.bfloat16, 1, 2, 64, 128, False, (1, 1, 64, 64)),
+])
+def test_attention_backward_with_a_mask(K, dtype, B, N, S, D, causal, mshape):
+    """Gradients under a general mask on the fused kernels (bit-packed mask for dQ, its transpose for
+    dK and dV), alone and together with the causal mask, with planted rows that lose every key: against
+    fp32 autograd of the unfused graph and against the GEMM formulation from the same saved statistics;
+    the masked kernels are what ran (through npu_fa as well, where the mask is not paired with a causal
+    mode: under those the op does not read the mask tensor, as in the reference)."""
+    announce(f"attention backward with a mask {dtype} B={B} N={N} S={S} D={D} causal={causal} mask={mshape}")
+    from inductor_x_amd import attention_backward as AB
+    from inductor_x_amd import launcher
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
+    torch.manual_seed(43)
+    q, k, v = (torch.randn(B, N, S, D, device=DEV).to(dtype) for _ in range(3))
+    do = torch.randn(B, N, S, D, device=DEV).to(dtype)
+    mask = torch.rand(*mshape, device=DEV) < 0.35
+    mask[..., 0] = False
+    mask[..., S // 3, :] = True   # a query that sees nothing
+    mask[..., :, 5] = True        # a key nobody sees
+    mask[..., 0, 5] = False
+    scale = D ** -0.5
+    pad = (lambda t: torch.nn.functional.pad(t, (0, 128 - D))) if D < 128 else (lambda t: t)  # noqa: E731
+    launcher.launch_log = []
+    try:
+        o, m, l = K.fused_attention(pad(q), pad(k), pad(v), scale, causal, mask=mask)
+        o = o[..., :D].contiguous()
+        got = AB.fused_attention_backward(q, k, v, o, do, m, l, scale, causal, atten_mask=mask)
+        torch.cuda.synchronize()
+    finally:
+        log, launcher.launch_log = launcher.launch_log, None
+    assert sum(sym.endswith("_masked") and sym.startswith("attention_bwd8_") for sym in log) == 3, log
+    qf, kf, vf = (t.float().requires_grad_() for t in (q, k, v))
+    hide = (mask if mask.dim() == 4 else mask.view(1, 1, S, S)).expand(B, N, S, S).clone()
+    if causal:
+        hide |= torch.ones(S, S, device=DEV, dtype=torch.bool).triu(1)
+    s = ((qf @ kf.transpose(-1, -2)) * scale).masked_fill(hide, float("-inf"))
+    dead = hide.all(-1, keepdim=True)
+    p = torch.where(dead, torch.zeros_like(s), torch.softmax(torch.where(dead, torch.zeros_like(s), s), -1))
+    ref = p @ vf
+    ref.backward(do.float())
+    assert (o.float() - ref).abs().max().item() <= 2e-2
+    for g, r in zip(got[:3], (qf.grad, kf.grad, vf.grad)):
+        assert g.shape == q.shape and torch.isfinite(g).all()
+        assert (g.float() - r).abs().max().item() <= 3e-2 * max(r.abs().max().item(), 1.0)
+    gemm = AB.fused_attention_backward(q, k, v, o, do, m, l, scale, causal, atten_mask=mask, use_kernels=False)
+    for x, y in zip(got[:3], gemm[:3]):
+        assert (x.float() - y.float()).abs().max().item() <= 8e-3 * max(y.float().abs().max().item(), 1.0)
+    if not causal:
+        qo, ko, vo = (t.clone().requires_grad_() for t in (q, k, v))
+        launcher.launch_log = []
+        try:
+            npu_fusion_attention_graph(qo, ko, vo, N, "BNSD", atten_mask=mask, scale=1 / scale)[0].backward(do)
+            torch.cuda.synchronize()
+        finally:
+            log, launcher.launch_log = launcher.launch_log, None
+        assert any(sym.endswith("_masked") and sym.startswith("fused_attention_fwd_") for sym in log), log
+        assert sum(sym.endswith("_masked") and sym.startswith("attention_bwd8_") for sym in log) == 3, log
+        for g, x in zip((qo.grad, ko.grad, vo.grad), got[:3]):
+            assert torch.equal(g, x)
+
+
 @pytest.mark.parametrize("S,causal", [(64, True), (192, False), (320, True), (576, True)])
 def test_attention_backward_sequence_multiple_of_64(K, S, causal):
     """The backward kernels take any multiple of 64: last blocks of 64 and 192 rows (the output and
