@@ -144,28 +144,52 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
     keep_prob < 1 with the forward's seed regenerates the forward's dropout mask (GEMM path only).
     With pse or atten_mask the result has a fourth member, the gradient of pse in pse's own shape (None
     without pse); a mask alone runs on the fused kernels under the same shape limits, pse over GEMMs."""
-    masked_fit = (atten_mask is not None and pse is None and keep_prob == 1.0 and q.dim() == 4 and q.shape == k.shape
-                  and q.dtype in (torch.bfloat16, torch.float16) and 0 < q.size(3) <= 128 and q.size(3) % 8 == 0
-                  and q.size(2) > 0 and q.size(2) % 64 == 0 and atten_mask.is_cuda and atten_mask.dim() in (2, 4))
-    if masked_fit and use_kernels is not False:
-        # a general mask on the fused gradient kernels (bit-packed; one shape for q, k, v, a multiple of 64)
+    kernel_shape = (q.dim() == 4 and q.shape == k.shape and q.dtype in (torch.bfloat16, torch.float16)
+                    and 0 < q.size(3) <= 128 and q.size(3) % 8 == 0 and q.size(2) > 0 and keep_prob == 1.0)
+    masked_fit = (kernel_shape and pse is None and atten_mask is not None and atten_mask.is_cuda and atten_mask.dim() in (2, 4))
+    # without a causal mask a length that is no multiple of 64 needs the padded keys hidden exactly: a bit mask
+    ragged_fit = kernel_shape and pse is None and atten_mask is None and not causal and q.size(2) % 64 != 0
+    if (masked_fit or ragged_fit) and use_kernels is not False:
+        # The gradient kernels with a bit mask (one shape for q, k, v).  The length is padded to a multiple
+        # of 64 with zero rows (statistics m = 0, l = 1); the mask hides the padded keys from every query
+        # and, where the caller gave a mask, is that mask padded with "hidden".
         from . import kernels
 
-        d = q.size(3)
-        widen = (lambda t: torch.nn.functional.pad(t, (0, 128 - d))) if d < 128 else (lambda t: t.contiguous())  # noqa: E731
-        grads = kernels.fused_attention_backward(widen(q), widen(k), widen(v), widen(out), widen(dout),
-                                                 softmax_max.contiguous(), softmax_sum.contiguous(), scale, causal, mask=atten_mask)
-        grads = tuple(g[..., :d].contiguous() for g in grads) if d < 128 else grads
-        return grads + (None,)
+        d, S = q.size(3), q.size(2)
+        pad_d, pad_s = 128 - d, -S % 64
+        Sp = S + pad_s
+        widen = (lambda t: torch.nn.functional.pad(t, (0, pad_d, 0, pad_s))) if (pad_d or pad_s) else (lambda t: t.contiguous())  # noqa: E731
+        smax, ssum = softmax_max.contiguous(), softmax_sum.contiguous()
+        if pad_s:
+            smax = torch.nn.functional.pad(smax, (0, 0, 0, pad_s), value=0.0)
+            ssum = torch.nn.functional.pad(ssum, (0, 0, 0, pad_s), value=1.0)
+        if atten_mask is not None:
+            m4 = atten_mask.view(1, 1, *atten_mask.shape) if atten_mask.dim() == 2 else atten_mask
+            hide = m4 if m4.dtype == torch.bool else m4 != 0
+            if pad_s:
+                hide = torch.nn.functional.pad(hide, (0, pad_s, 0, pad_s), value=True)
+            packed = (kernels.attention_mask_bits(hide, q.size(0), q.size(1), Sp, Sp),
+                      kernels.attention_mask_bits(hide.transpose(-1, -2), q.size(0), q.size(1), Sp, Sp))
+        else:
+            # keys S .. Sp - 1 hidden from everybody: the same word row for every query (only the last key
+            # tile has bits set); transposed, a padded key hides every query and a real key none
+            tiles = Sp // 64
+            words = torch.zeros(tiles, dtype=torch.int64, device=q.device)
+            words[tiles - 1] = -1 << (S % 64)
+            rows = words.view(1, 1, 1, tiles).expand(1, 1, Sp, tiles).contiguous().view(torch.uint8)
+            cols = torch.zeros(Sp, tiles, dtype=torch.int64, device=q.device)
+            cols[S:] = -1
+            packed = (rows, cols.view(1, 1, Sp, tiles).view(torch.uint8))
+        grads = kernels.fused_attention_backward(widen(q), widen(k), widen(v), widen(out), widen(dout), smax, ssum, scale, causal,
+                                                 packed_masks=packed)
+        grads = tuple(g[:, :, :S, :d].contiguous() for g in grads) if (pad_d or pad_s) else grads
+        return grads + (None,) if atten_mask is not None else grads
     if pse is not None or atten_mask is not None:
         if use_kernels:
-            raise NotImplementedError("attention backward: the fused kernels take no bias, and a mask only for one shape "
-                                      "of q, k, v and a sequence length that is a multiple of 64")
+            raise NotImplementedError("attention backward: the fused kernels take no bias, and a mask only for one shape of q, k, v")
         return _backward_over_gemms(q, k, v, out, dout, softmax_max, softmax_sum, scale, causal, keep_prob, seed,
                                     pse=pse, atten_mask=atten_mask)
-    # a length that is no multiple of 64 is served under a causal mask only (see the padding note below)
-    fits = (q.dim() == 4 and q.dtype in (torch.bfloat16, torch.float16) and 0 < q.size(3) <= 128 and q.size(3) % 8 == 0
-            and q.size(2) > 0 and (causal or q.size(2) % 64 == 0) and q.shape == k.shape and keep_prob == 1.0)
+    fits = kernel_shape  # (without a causal mask, lengths that are no multiple of 64 took the masked kernels above)
     if use_kernels is None:
         use_kernels = fits
     if use_kernels:
@@ -180,12 +204,12 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
         # probability is exactly zero, and a padded query has dO = 0 and Q = 0, so it adds nothing to
         # dV or dK; the padded rows of the results are dropped.  Without the mask a padded key would
         # get the probability exp(-logsumexp of the row), which times K = 0 is zero only while it
-        # stays finite in the operand type, so those lengths run over GEMMs.
+        # stays finite in the operand type: those lengths took the kernels with a bit mask above.
         d, S = q.size(3), q.size(2)
         pad_d, pad_s = 128 - d, -S % 64
         if pad_s and not causal:
-            raise NotImplementedError("attention backward: without a causal mask the fused kernels need a sequence "
-                                      "length that is a multiple of 64")
+            raise NotImplementedError("attention backward: without a causal mask a sequence length that is no multiple "
+                                      "of 64 needs the masked kernels")
         if pad_d or pad_s:
             widen = lambda t: torch.nn.functional.pad(t, (0, pad_d, 0, pad_s))  # noqa: E731
         else:

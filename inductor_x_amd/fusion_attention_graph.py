@@ -20,10 +20,10 @@ type, non-zero = hidden); a positional bias (pse), fp32 operands, other
 head dimensions and dropout (keep_prob < 1) run the same mathematics over library GEMMs; padding masks, prefixes, variable sequence lengths and band masks
 raise.
 The backward op recomputes the probabilities from the saved row statistics inside fused gradient
-kernels (bf16 or fp16, head dimension up to 128, equal lengths that are multiples of 64 or, with a causal mask, any;
+kernels (bf16 or fp16, head dimension up to 128, one shape for q, k, v;
 kernels.fused_attention_backward) and falls back to the GEMM formulation otherwise
 (attention_backward.py), which also returns the gradient of pse; a general mask runs the fused
-gradient kernels too (one shape for q, k, v, a multiple of 64); the training variant of the
+gradient kernels too; the training variant of the
 pattern is registered beside the inference one.
 """
 from __future__ import annotations
@@ -313,8 +313,7 @@ def _extra_check(match, training: bool = False) -> bool:
     """Only rewrite what the fused kernels run; anything else stays on Inductor's own path.
     Inference graphs: bf16 or fp16 GPU tensors [B, S, N, 128], any sequence lengths, key and value of
     one shape that may differ from the query's in its length (cross attention).  Training graphs,
-    whose backward runs the fused gradient kernels: query, key and value of one shape and a
-    sequence length that is a multiple of 64.  Either way the divisor of the scores, when it is a
+    whose backward runs the fused gradient kernels: query, key and value of one shape.  Either way the divisor of the scores, when it is a
     constant, must be positive and finite."""
     try:
         q = match.kwargs["query"].meta["val"]
@@ -326,7 +325,7 @@ def _extra_check(match, training: bool = False) -> bool:
         return False
     if q.dtype not in (torch.bfloat16, torch.float16):
         return False
-    if training and (q.size(1) % 64 != 0 or tuple(k.shape) != tuple(q.shape)):
+    if training and tuple(k.shape) != tuple(q.shape):
         return False
     if k.dim() != 4 or k.size(1) <= 0 or (k.size(0), k.size(2), k.size(3)) != (q.size(0), q.size(2), q.size(3)):
         return False

@@ -780,7 +780,7 @@ def _attention_bwd_masked_launchers() -> dict:
 def fused_attention_backward(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, dout: torch.Tensor,
     softmax_max: torch.Tensor, softmax_sum: torch.Tensor, scale: float, causal: bool, data_columns: int = 128,
-    mask: Optional[torch.Tensor] = None,
+    mask: Optional[torch.Tensor] = None, packed_masks: Optional[tuple] = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients (dq, dk, dv) of fused_attention for [B, N, S, 128] bf16 or fp16 tensors; softmax_max /
     softmax_sum are the forward's [B, N, S, 8] fp32 statistics.  Workgroups of eight wavefronts on
@@ -789,7 +789,8 @@ def fused_attention_backward(
     others being zero in q, k, v, out and dout (a smaller head padded to 128): with at most 64 the
     kernels skip the matrix work on the zero half and leave columns 64.. of the gradients undefined.
     mask: the forward's mask ([S, S] or broadcastable to [B, N, S, S], non-zero = hidden); it is packed to
-    bits, once as it stands for dQ and once transposed for dK and dV."""
+    bits, once as it stands for dQ and once transposed for dK and dV.  packed_masks: those two packings
+    (attention_mask_bits of the mask and of its transpose), for a caller that holds them already."""
     _check_cuda(q, k, v, out, dout, softmax_max, softmax_sum)
     for t in (q, k, v, out, dout):
         _require(t.dtype == q.dtype and t.dtype in _ATTN_DTYPES and t.dim() == 4 and t.shape == q.shape,
@@ -820,11 +821,19 @@ def fused_attention_backward(
     )
     blocks = cdiv(S, 256)
     grid = (8 * cdiv(heads, 8) * (cdiv(blocks, 2) if causal else blocks), 1, 1)  # causal: pairs of blocks
-    if mask is not None:
-        _check_cuda(mask)
-        m4 = mask.view(1, 1, *mask.shape) if mask.dim() == 2 else mask
-        rows = attention_mask_bits(m4, B, N, S, S)                     # [.., query, key tiles]
-        cols = attention_mask_bits(m4.transpose(-1, -2), B, N, S, S)   # [.., key, query tiles]
+    if mask is not None or packed_masks is not None:
+        if packed_masks is not None:
+            rows, cols = packed_masks
+            for w in (rows, cols):
+                _check_cuda(w)
+                _require(w.dtype == torch.uint8 and w.dim() == 4 and w.is_contiguous() and w.shape[0] in (1, B)
+                         and w.shape[1] in (1, N) and tuple(w.shape[2:]) == (S, S // 8),
+                         "packed masks are what attention_mask_bits returns for this length")
+        else:
+            _check_cuda(mask)
+            m4 = mask.view(1, 1, *mask.shape) if mask.dim() == 2 else mask
+            rows = attention_mask_bits(m4, B, N, S, S)                     # [.., query, key tiles]
+            cols = attention_mask_bits(m4.transpose(-1, -2), B, N, S, S)   # [.., key, query tiles]
         lm = _attention_bwd_masked_launchers()
         for name, dst, words in (("dk8", dk, cols), ("dv8", dv, cols), ("dq8", dq, rows)):
             l = lm[name]

@@ -337,9 +337,9 @@ def test_attention_backward_kernels_vs_gemm_path(K, B, N, S, causal, dtype):
 @pytest.mark.parametrize("dtype,B,N,S,D", [(torch.bfloat16, 1, 3, 100, 128), (torch.float16, 2, 2, 333, 128), (torch.bfloat16, 1, 2, 77, 64),
                                             (torch.bfloat16, 1, 2, 1, 128), (torch.float16, 1, 1, 65, 128)])
 def test_attention_backward_causal_any_length(K, dtype, B, N, S, D):
-    """Under a causal mask the gradient kernels serve any sequence length on zero-padded rows: the same
-    gradients as the GEMM formulation from the same saved statistics, and the gradient kernels are
-    what ran.  Without the mask such a length keeps the GEMM formulation."""
+    """The gradient kernels serve any sequence length on zero-padded rows: under a causal mask as they are
+    (the mask hides the padded keys), without it through the instantiations with a bit mask that hides
+    them.  The same gradients as the GEMM formulation from the same saved statistics."""
     announce(f"attention backward causal, padded length {dtype} B={B} N={N} S={S} D={D}")
     from inductor_x_amd import attention_backward as AB
     from inductor_x_amd import launcher
@@ -360,14 +360,19 @@ def test_attention_backward_causal_any_length(K, dtype, B, N, S, D):
         assert x.shape == q.shape and x.dtype == dtype and torch.isfinite(x).all()
         assert (x.float() - y.float()).abs().max().item() <= 8e-3 * max(y.float().abs().max().item(), 1.0)
     if S % 64:
+        # without the causal mask the padded keys are hidden by a bit mask: the masked kernels run
+        o2, m2, l2 = AB.attention_forward_over_gemms(q, k, v, scale, False)
         launcher.launch_log = []
         try:
-            AB.fused_attention_backward(q, k, v, o, do, m, l, scale, False)
+            a2 = AB.fused_attention_backward(q, k, v, o2, do, m2, l2, scale, False)
+            torch.cuda.synchronize()
         finally:
             log, launcher.launch_log = launcher.launch_log, None
-        assert not any(sym.startswith("attention_bwd8_") for sym in log), log
-        with pytest.raises(NotImplementedError):
-            AB.fused_attention_backward(q, k, v, o, do, m, l, scale, False, use_kernels=True)
+        assert sum(sym.startswith("attention_bwd8_") and sym.endswith("_masked") for sym in log) == 3, log
+        b2 = AB.fused_attention_backward(q, k, v, o2, do, m2, l2, scale, False, use_kernels=False)
+        for x, y in zip(a2, b2):
+            assert x.shape == q.shape and torch.isfinite(x).all()
+            assert (x.float() - y.float()).abs().max().item() <= 8e-3 * max(y.float().abs().max().item(), 1.0)
 
 
 @pytest.mark.parametrize("dtype,B,N,S,D,causal", [(torch.bfloat16, 2, 3, 512, 64, True), (torch.float16, 1, 5, 320, 64, False),
