@@ -730,6 +730,100 @@ def _attention_ceiling(torch) -> dict:
     }
 
 
+def _attention_timeline(torch) -> dict:
+    """Where a workgroup of the fused attention forward spends its time at q, k, v [4,32,4096,128] bf16: the
+    measurement build of the shipped kernel template (csrc/probes/attention_timeline.hip) records the 100 MHz
+    clock at seven points of every query block; ten launches back to back, the last one is read."""
+    import numpy as np
+
+    from inductor_x_amd import codecache, kernels as K, launcher
+
+    path = codecache.compile_source(codecache.probe_source("attention_timeline.hip"), label="attention_timeline", prefer_intree=True)
+    with open(path, "rb") as f:
+        mod = launcher.Module(f.read(), label="attention_timeline")
+    dev = "cuda:0"
+    torch.manual_seed(0)
+    B, N, S, D = 4, 32, 4096, 128
+    q, k, v = (torch.randn(B, N, S, D, device=dev).bfloat16() for _ in range(3))
+    scale = D ** -0.5
+    n_qb = S // 256
+    n_blocks = B * N * n_qb
+    out = torch.empty_like(q)
+    smax = torch.empty(B, N, S, 8, device=dev)
+    ssum = torch.empty_like(smax)
+    times = torch.zeros(n_blocks * 2 * 8, dtype=torch.int64, device=dev)
+    stream = torch._C._cuda_getCurrentRawStream(0)
+    cus = launcher.device_props(0).cu_count
+    res = {"shape": [B, N, S, D], "clock": "s_memrealtime, 100 MHz", "launches": "10 back to back after 10 warm-ups, last one read"}
+    for causal, name in ((True, "causal"), (False, "full")):
+        fn = mod.function(f"attention_timeline_bf16_d128_{name}")
+        per_head = (n_qb + 1) // 2 if causal else n_qb
+        grid = (min(8 * ((B * N + 7) // 8) * per_head, 8 * (cus // 8)), 1, 1)
+        launch = lambda: fn.launch("PPPPPPiiifP", (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), smax.data_ptr(),  # noqa: E731
+                                                   ssum.data_ptr(), B * N, S, S, scale * 1.4426950408889634, times.data_ptr()),
+                                   grid, (512,), stream, 65536)
+        ref = K.fused_attention(q, k, v, scale, causal)
+        for _ in range(10):
+            launch()
+        torch.cuda.synchronize()
+        same = bool(torch.equal(out, ref[0]) and torch.equal(smax, ref[1]) and torch.equal(ssum, ref[2]))
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        for _ in range(10):
+            launch()
+        t1.record()
+        t1.synchronize()
+        tr = times.cpu().numpy().reshape(n_blocks, 2, 8).astype(np.float64)
+        us = tr[:, :, :7] * 0.01
+        w0 = us[:, 0, :]
+        qb = np.arange(n_blocks) % n_qb
+        tiles = (4 * qb + 4) if causal else np.full(n_blocks, S // 64)
+        seg = lambda a, b, m=slice(None): float(np.mean(w0[m, b] - w0[m, a]))  # noqa: E731
+        unguarded_tiles = np.maximum(tiles - (6 if causal else 2), 0)  # first step and last step lie outside, causal: the diagonal too
+        long_blocks = unguarded_tiles >= 8
+        per_tile = float(np.sum((w0[:, 3] - w0[:, 2])[long_blocks]) / np.sum(unguarded_tiles[long_blocks]))
+        start = w0[:, 0].min()
+        wg = tr[:, 0, 7].astype(np.int64)
+        ends, gaps = {}, []
+        for g in np.unique(wg):
+            m = np.where(wg == g)[0]
+            o = m[np.argsort(w0[m, 0])]
+            block_end = us[o, :, 6].max(axis=1)
+            ends[int(g)] = block_end[-1] - start
+            gaps += list(w0[o[1:], 0] - block_end[:-1])
+        end = np.array([ends[g] for g in sorted(ends)])
+        die = np.array(sorted(ends)) % 8
+        row = {
+            "matches_shipped_kernel": same,
+            "launch_us_mean_of_10": round(t0.elapsed_time(t1) * 100, 1),
+            "traced_launch_span_us": round(float(us[:, :, 6].max() - start), 1),
+            "mean_us_per_query_block": {
+                "queries_and_first_two_k_tiles_land": round(seg(0, 1), 2),
+                "first_score_product_and_first_step": round(seg(1, 2), 2),
+                "unguarded_steps": round(seg(2, 3), 2),
+                "guarded_steps_and_last_step": round(seg(3, 4), 2),
+                "normalise_stage_issue_stores": round(seg(4, 5), 2),
+                "statistics_and_barrier": round(seg(5, 6), 2),
+                "whole_block": round(seg(0, 6), 2),
+                "idle_before_next_block": round(float(np.mean(gaps)), 2),
+            },
+            "us_per_unguarded_tile_step": round(per_tile, 3),
+            "mean_tiles_per_block": float(np.mean(tiles)),
+            "us_per_block_beyond_tiles_times_step": round(seg(0, 6) + float(np.mean(gaps)) - float(np.mean(tiles)) * per_tile, 2),
+            "workgroup_end_us": {"mean": round(float(end.mean()), 1), "max": round(float(end.max()), 1),
+                                 "per_die_mean": [round(float(end[die == x].mean()), 1) for x in range(8)],
+                                 "spread_within_a_die_max": round(float(max(end[die == x].max() - end[die == x].min() for x in range(8))), 1)},
+        }
+        if causal:
+            row["by_query_block"] = {
+                str(b): {"tiles": 4 * b + 4, "land": round(seg(0, 1, qb == b), 2), "first": round(seg(1, 2, qb == b), 2),
+                         "unguarded": round(seg(2, 3, qb == b), 2), "guarded_and_last": round(seg(3, 4, qb == b), 2),
+                         "epilogue": round(seg(4, 6, qb == b), 2), "block": round(seg(0, 6, qb == b), 2)}
+                for b in (0, 1, 7, 8, 15)}
+        res[name] = row
+    return res
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=int(os.environ.get("WORLD_SIZE", "1")))
@@ -746,6 +840,9 @@ def main() -> None:
     ap.add_argument("--launch-floor", action="store_true",
                     help="time a 4 KiB copy (one workgroup) and the cfg 1 row sum the same way, 20 dependent launches per "
                          "HIP graph: what a launch costs on this machine before any data moves")
+    ap.add_argument("--attention-timeline", action="store_true",
+                    help="run the measurement build of the fused attention forward (csrc/probes/attention_timeline.hip) "
+                         "and print where a workgroup's time goes per query block")
     ap.add_argument("--attention-ceiling", action="store_true",
                     help="run the resource probes of csrc/probes/probe_kernels.hip: what one CU sustains of MFMA, LDS operand "
                          "reads and softmax-like vector work, alone and together (the ceiling of the attention design)")
@@ -772,6 +869,9 @@ def main() -> None:
         return
     if args.launch_floor:
         print(json.dumps(_launch_floor(K, torch)))
+        return
+    if args.attention_timeline:
+        print(json.dumps(_attention_timeline(torch)))
         return
     if args.attention_ceiling:
         print(json.dumps(_attention_ceiling(torch)))

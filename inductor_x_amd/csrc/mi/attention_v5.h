@@ -33,6 +33,14 @@ namespace mi {
 constexpr int kAttnV5Waves = 8;
 constexpr int kAttnV5BM = kAttnV5Waves * 32;
 
+// Timeline hook: the kernel calls mark(point, head, q_block) at seven fixed points of a query block
+// (0 entry, 1 queries and first two K tiles landed, 2 first score product and tile step done, 3 unguarded
+// tile steps done, 4 all tile steps done, 5 output stores issued, 6 block done).  The default does nothing
+// and leaves no code; the measurement build under csrc/probes records a clock there.
+struct AttnNoTimeline {
+  __device__ __forceinline__ void mark(int, int, int) const {}
+};
+
 // WAVES = 8: one workgroup of 256 queries per CU.  WAVES = 4: 128 queries per workgroup and two
 // workgroups per CU (64 KiB of LDS each), so the two wavefronts of a SIMD belong to different
 // workgroups, share no barrier and drift apart in phase.
@@ -45,13 +53,15 @@ constexpr int kAttnV5BM = kAttnV5Waves * 32;
 // mask; needs RAGGED.  A lane fetches the word of its query for the next tile (one bounded 8-byte buffer
 // load: zero past the end) while the current tile is worked on.  A row with every key hidden gives zeros,
 // maximum 0 and sum 1.
-template <typename T, bool CAUSAL, bool RAGGED, int WAVES = kAttnV5Waves, int DH = 128, bool MASKED = false>
+template <typename T, bool CAUSAL, bool RAGGED, int WAVES = kAttnV5Waves, int DH = 128, bool MASKED = false,
+          typename TL = AttnNoTimeline>
 __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, const T* __restrict__ K,
                                                       const T* __restrict__ V, T* __restrict__ O,
                                                       float* __restrict__ softmax_max,
                                                       float* __restrict__ softmax_sum, int Sq, int Sk,
                                                       int q_block, int head, float scale_log2e,
-                                                      const unsigned char* __restrict__ head_mask = nullptr) {
+                                                      const unsigned char* __restrict__ head_mask = nullptr,
+                                                      TL timeline = TL()) {
   typedef AttnElem<T> E;
   typedef typename E::x8 x8_t;
   constexpr bool GUARDED = CAUSAL || RAGGED;  // the last tiles of a block run the guarded copy of the loop
@@ -96,6 +106,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   const int qi = q0 + sub * 32 + li;
   const int qi_ld = RAGGED ? min(qi, Sq - 1) : qi;  // rows past the end work on a copy of the last row
 
+  timeline.mark(0, head, q_block);
   x8_t qf[DS];
 #pragma unroll
   for (int s = 0; s < DS; ++s)
@@ -370,6 +381,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   issue_k(1, 1);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): Q fragments and the tiles above have landed
   __syncthreads();
+  timeline.mark(1, head, q_block);
   {
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
@@ -419,8 +431,10 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
       __syncthreads();
     }
   };
+  timeline.mark(2, head, q_block);
   int t = 1;
   for (; t + 1 < first_masked; t += 2) pair(t, No());
+  timeline.mark(3, head, q_block);
   if constexpr (GUARDED) {
     for (; t < n_tiles - 1; t += 2) pair(t, Yes());
   }
@@ -441,6 +455,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
     }
   }
 
+  timeline.mark(4, head, q_block);
   // ---- epilogue ----
   const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
   const float l_tot = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
@@ -474,6 +489,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
       if (!RAGGED || q0 + sub * 32 + row < Sq) *reinterpret_cast<u32x4_t*>(oblk + row * kAttnD + 8 * c16) = v16;
     }
   }
+  timeline.mark(5, head, q_block);
   if (g == 0 && (!RAGGED || qi < Sq)) {
     const size_t so = (static_cast<size_t>(head) * Sq + qi) * 8;
     const float m_nat = hidden_row ? 0.f : m_true * 0.69314718055994530942f;
@@ -489,6 +505,48 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
     store_vec<float, 4>(softmax_sum + so + 4, lv);
   }
   __syncthreads();  // the staging reads are done before a following query block refills the K buffers
+  timeline.mark(6, head, q_block);
+}
+
+// One workgroup of a persistent launch.  Workgroup -> (head, query block) mapping: hardware deals consecutive
+// workgroup ids round-robin to the 8 accelerator dies, each with its own L2.  Ids that land on one die walk
+// the query blocks of one head before moving to the next head, so a head's K and V are fetched into a single
+// L2.  Under a causal mask query block b visits 4 b + 4 key tiles; a work item is the pair (b, n - 1 - b), the
+// longer member first, so every item is the same amount of work.  The grid is at most one workgroup per CU and
+// every workgroup walks the work items id = blockIdx.x, blockIdx.x + gridDim.x, ... (gridDim.x is a multiple
+// of 8, so a workgroup stays on the heads of its own die).
+template <typename T, bool CAUSAL, bool RAGGED, int DH = 128, bool MASKED = false, typename TL = AttnNoTimeline>
+__device__ __forceinline__ void attention_entry_v5(const T* q, const T* k, const T* v, T* o, float* smax,
+                                                   float* ssum, int n_heads, int Sq, int Sk,
+                                                   float scale_log2e, const unsigned char* mask = nullptr,
+                                                   long long mask_batch_stride = 0, long long mask_head_stride = 0,
+                                                   int heads_per_batch = 1, TL timeline = TL()) {
+  constexpr int XCDS = 8;
+  const int n_qb = (Sq + kAttnV5BM - 1) / kAttnV5BM;
+  const int per_head = CAUSAL ? (n_qb + 1) / 2 : n_qb;
+  const int total = XCDS * ((n_heads + XCDS - 1) / XCDS) * per_head;
+#pragma nounroll
+  for (int id = blockIdx.x; id < total; id += gridDim.x) {
+    const int xcd = id % XCDS;
+    const int slot = id / XCDS;
+    const int head = (slot / per_head) * XCDS + xcd;
+    if (head >= n_heads) continue;
+    // the [Sq][tiles] 64-bit mask words of this head (byte strides; 0 where the mask broadcasts over batch or heads)
+    const unsigned char* hm =
+        MASKED ? mask + (head / heads_per_batch) * mask_batch_stride + (head % heads_per_batch) * mask_head_stride : nullptr;
+    if (CAUSAL) {
+      const int lo = slot % per_head;
+      const int hi = n_qb - 1 - lo;
+      const int n_pass = lo != hi ? 2 : 1;
+#pragma nounroll
+      for (int pass = 0; pass < n_pass; ++pass)
+        attention_fwd_d128_v5<T, true, RAGGED, kAttnV5Waves, DH, MASKED, TL>(q, k, v, o, smax, ssum, Sq, Sk, pass == 0 ? hi : lo,
+                                                                             head, scale_log2e, hm, timeline);
+    } else {
+      attention_fwd_d128_v5<T, false, RAGGED, kAttnV5Waves, DH, MASKED, TL>(q, k, v, o, smax, ssum, Sq, Sk, slot % per_head, head,
+                                                                            scale_log2e, hm, timeline);
+    }
+  }
 }
 
 }  // namespace mi

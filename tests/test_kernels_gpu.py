@@ -462,3 +462,22 @@ def test_attention_resource_probes_run():
     assert all(math.isfinite(v) and v > 0 for v in ns.values())
     assert all(math.isfinite(v) and v > 0 for v in r["lds_bytes_per_clock_per_cu"].values())
     assert math.isfinite(r["ceiling_of_datasheet_peak"]) and r["ceiling_of_datasheet_peak"] > 0
+
+
+def test_attention_timeline_probe_matches_the_shipped_kernel():
+    """The measurement build behind `bench.py --attention-timeline` is the shipped kernel template plus clock
+    reads: its outputs are bit-identical to `kernels.fused_attention` and every query block of both launches
+    leaves a complete, ordered record (the durations themselves are measurements, not pass criteria)."""
+    announce("attention timeline probe")
+    import math
+
+    import bench
+
+    r = bench._attention_timeline(torch)
+    for mode in ("causal", "full"):
+        row = r[mode]
+        assert row["matches_shipped_kernel"], mode
+        seg = row["mean_us_per_query_block"]
+        assert all(math.isfinite(v) for v in seg.values()) and seg["whole_block"] > 0 and seg["unguarded_steps"] > 0
+        assert 0 < row["us_per_unguarded_tile_step"] < 50
+        assert row["workgroup_end_us"]["max"] >= row["workgroup_end_us"]["mean"] > 0
