@@ -9,10 +9,10 @@
 //
 //   dQ kernel   a wavefront owns 32 queries (lane = query), a workgroup 256; loop over 64-key tiles:
 //               S^T = K Q^T, dP^T = V dO^T (A from LDS, B = Q / dO fragments in registers),
-//               dS^T is at once the B operand of dQ^T += K^T dS^T (A = transposed K tile).
+//               dS^T is at once the B operand of dQ^T += K^T dS^T (A = the K tile read transposed).
 //   dK kernel   a wavefront owns 32 keys (lane = key), loop over 64-query tiles:
 //               S = Q K^T, dP = dO V^T (A from LDS, B = K / V fragments in registers),
-//               dK^T += Q^T dS (A = transposed Q tile, query axis permuted as attn_vt_pos).
+//               dK^T += Q^T dS (A = the Q tile read transposed).
 //   dV kernel   same orientation: S = Q K^T, dV^T += dO^T P.
 //
 // dK and dV are separate kernels (the scores are recomputed three times in all, eight matrix
@@ -21,7 +21,13 @@
 // wavefronts per SIMD -- one in its MFMAs while the other recomputes probabilities -- is worth
 // more than the product saved.
 //
-// Every 64-row tile travels global -> registers -> LDS (double-buffered, one barrier per tile).
+// Every 64-row tile travels memory -> LDS by direct 16-byte `buffer_load ... lds` copies exactly as it
+// lies in memory ([64][128], one 1 KiB block = four rows per wavefront instruction, double-buffered, one
+// barrier per tile), the 16-byte chunks of a row XOR-swizzled on the way in by the choice of the global
+// chunk a lane fetches.  An operand that is read along its rows (K, V for dQ; Q, dO for dK / dV) is
+// swizzled by row mod 16; the transposed operand of the update product (K^T, Q^T, dO^T) is formed by
+// transposing LDS reads (`ds_read_b64_tr_b16`) of a second copy of the same tile, swizzled by a 4-entry
+// table that keeps those reads on distinct banks.  No tile passes through registers.
 // Sequence lengths need only be multiples of 64: rows of a last partial block are clamped for
 // loads and not stored.
 #pragma once
@@ -33,12 +39,11 @@ namespace mi {
 constexpr int kBwd8Waves = 8;
 constexpr int kBwd8Threads = 64 * kBwd8Waves;
 constexpr int kBwd8BlockRows = 32 * kBwd8Waves;  // queries (dQ) or keys (dK, dV) per workgroup
-constexpr int kBwd8RowTile = kAttnBN * kAttnKStride;  // [64][136] row-major tile, elements
-constexpr int kBwd8ColTile = kAttnD * kAttnVStride;   // [128][64] transposed tile, elements
+constexpr int kBwd8Tile = kAttnBN * kAttnD;           // [64][128] tile as it lies in memory, elements
 constexpr int kBwd8StatBytes = kAttnBN * 2 * 4;       // (exponent offset, D) of a query tile
-constexpr int kBwd8DqBufBytes = (2 * kBwd8RowTile + kBwd8ColTile) * 2;                    // K, V, K^T
-constexpr int kBwd8DkBufBytes = (2 * kBwd8RowTile + kBwd8ColTile) * 2 + kBwd8StatBytes;   // Q, dO, Q^T
-constexpr int kBwd8DvBufBytes = (kBwd8RowTile + kBwd8ColTile) * 2 + kBwd8StatBytes;       // Q, dO^T
+constexpr int kBwd8DqBufBytes = 3 * kBwd8Tile * 2;                    // K, V, K for transposing reads
+constexpr int kBwd8DkBufBytes = 3 * kBwd8Tile * 2 + kBwd8StatBytes;   // Q, dO, Q for transposing reads
+constexpr int kBwd8DvBufBytes = 2 * kBwd8Tile * 2 + kBwd8StatBytes;   // Q, dO for transposing reads
 constexpr int kBwd8DqLdsBytes = 2 * kBwd8DqBufBytes;
 constexpr int kBwd8DkLdsBytes = 2 * kBwd8DkBufBytes;
 constexpr int kBwd8DvLdsBytes = 2 * kBwd8DvBufBytes;
@@ -51,10 +56,13 @@ constexpr float kBwd8Log2e = 1.4426950408889634f;
 #define BWD8_PREFETCH_DK 2
 #endif
 #ifndef BWD8_PREFETCH_DK_CAUSAL
-#define BWD8_PREFETCH_DK_CAUSAL 0
+#define BWD8_PREFETCH_DK_CAUSAL 2
 #endif
 #ifndef BWD8_PREFETCH_DV
-#define BWD8_PREFETCH_DV 0
+#define BWD8_PREFETCH_DV 2
+#endif
+#ifndef BWD8_STAGED_CAUSAL
+#define BWD8_STAGED_CAUSAL 1
 #endif
 
 // stats[row] = (m log2 e + log2 l, sum_d dO[row, d] * O[row, d]); 16 lanes per row.
@@ -89,62 +97,56 @@ __device__ __forceinline__ void attention_bwd_stats(const T* __restrict__ O, con
 // row-major.  Column form: 4 rows x 4 columns per thread (4 x 8 bytes), stored transposed with the
 // row index (the contraction axis of the MFMA that reads the tile) permuted, and optionally
 // row-major as well.
-struct Bwd8RowStage {
-  u32x4_t r[2];
-};
-struct Bwd8ColStage {
-  u32x2_t r[4];
-};
-template <typename T>
-__device__ __forceinline__ void bwd8_load(Bwd8RowStage& t, const T* __restrict__ src, int tid) {
-  const int row = tid >> 4, col = (tid & 15) * 8;
+// One [64][128] tile, memory -> LDS: the eight wavefronts copy two 1 KiB blocks (four rows) each; lane l of
+// an instruction fills LDS chunk l of the block (row 4 b + l / 16, chunk position l % 16) with the global
+// chunk that the swizzle puts there.  TR: the copy that the transposing reads use.
+template <bool TR, typename T>
+__device__ __forceinline__ void bwd8_copy_tile(const T* __restrict__ src, T* dst, int wave, int lane) {
+  const int blk_row = lane >> 4, blk_pos = lane & 15;
 #pragma unroll
-  for (int u = 0; u < 2; ++u)
-    t.r[u] = *reinterpret_cast<const u32x4_t*>(src + static_cast<size_t>(row + 32 * u) * kAttnD + col);
-}
-template <typename T>
-__device__ __forceinline__ void bwd8_store_rows(const Bwd8RowStage& t, T* dst, int tid) {
-  const int row = tid >> 4, col = (tid & 15) * 8;
-#pragma unroll
-  for (int u = 0; u < 2; ++u) *reinterpret_cast<u32x4_t*>(dst + (row + 32 * u) * kAttnKStride + col) = t.r[u];
-}
-template <typename T>
-__device__ __forceinline__ void bwd8_load(Bwd8ColStage& t, const T* __restrict__ src, int tid) {
-  const int rg = tid >> 5, cg = tid & 31;
-#pragma unroll
-  for (int u = 0; u < 4; ++u)
-    t.r[u] = *reinterpret_cast<const u32x2_t*>(src + static_cast<size_t>(4 * rg + u) * kAttnD + 4 * cg);
-}
-template <typename T>
-__device__ __forceinline__ void bwd8_store_rows(const Bwd8ColStage& t, T* dst, int tid) {
-  const int rg = tid >> 5, cg = tid & 31;
-#pragma unroll
-  for (int u = 0; u < 4; ++u) *reinterpret_cast<u32x2_t*>(dst + (4 * rg + u) * kAttnKStride + 4 * cg) = t.r[u];
-}
-template <typename T>
-__device__ __forceinline__ void bwd8_store_cols(const Bwd8ColStage& t, T* dst, int tid) {
-  const int rg = tid >> 5, cg = tid & 31;
-  const int pos = attn_vt_pos(4 * rg);
-#pragma unroll
-  for (int e2 = 0; e2 < 2; ++e2) {
-    // dword e2 of each row holds columns 4 cg + 2 e2 (low half) and + 1 (high half)
-    const uint32_t a0 = t.r[0][e2], a1 = t.r[1][e2], a2 = t.r[2][e2], a3 = t.r[3][e2];
-    u32x2_t lo, hi;
-    lo[0] = __builtin_amdgcn_perm(a1, a0, 0x05040100u);
-    lo[1] = __builtin_amdgcn_perm(a3, a2, 0x05040100u);
-    hi[0] = __builtin_amdgcn_perm(a1, a0, 0x07060302u);
-    hi[1] = __builtin_amdgcn_perm(a3, a2, 0x07060302u);
-    *reinterpret_cast<u32x2_t*>(dst + attn_vt_offset(4 * cg + 2 * e2, pos)) = lo;
-    *reinterpret_cast<u32x2_t*>(dst + attn_vt_offset(4 * cg + 2 * e2 + 1, pos)) = hi;
+  for (int u = 0; u < 2; ++u) {
+    const int b = 2 * wave + u;
+    const int row = 4 * b + blk_row;
+    const int swz = TR ? ((0xE4A0 >> (4 * (row & 3))) & 15) : (row & 15);
+    const int voff = (row * kAttnD + 8 * (blk_pos ^ swz)) * 2;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(src), 0, kBwd8Tile * 2, 0x00020000),
+        (__attribute__((address_space(3))) void*)(dst + b * 512), 16, voff, 0, 0, 0);
   }
 }
+// A operand along the rows of a tile: row `row`, d slice s, half g
 template <typename T>
 __device__ __forceinline__ typename AttnElem<T>::x8 bwd8_row_frag(const T* tile, int row, int s, int g) {
-  return *reinterpret_cast<const typename AttnElem<T>::x8*>(tile + row * kAttnKStride + 16 * s + 8 * g);
+  return *reinterpret_cast<const typename AttnElem<T>::x8*>(tile + row * kAttnD + 8 * ((2 * s + g) ^ (row & 15)));
 }
+// Per-lane element offsets of the transposing reads, one per d block: in every group of 16 lanes, lane s
+// points at four consecutive d of row 4 g + s / 4 (+ 8 for the second read) and receives, for its own d,
+// the four rows of the group -- the order in which the accumulator layout of the first product delivers
+// the rows as a B operand.
+template <int DB>
+__device__ __forceinline__ void bwd8_tr_offsets(int (&off)[DB], int lane) {
+  const int sl16 = lane & 15, grp = lane >> 4;
+  const int row_l = 4 * (grp >> 1) + (sl16 >> 2);
+  const int f = (0xE4A0 >> (4 * (row_l & 3))) & 15;
+  const int c_l = 2 * (grp & 1) + ((sl16 & 3) >> 1);
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+    off[db] = row_l * kAttnD + 8 * (((4 * db) ^ (f & 12)) + (c_l ^ (f & 2))) + 4 * (sl16 & 1);
+}
+// A operand across the rows of a tile (the tile transposed): d block via its offset, row slice t of 16
 template <typename T>
-__device__ __forceinline__ typename AttnElem<T>::x8 bwd8_col_frag(const T* tile, int row, int t, int g) {
-  return *reinterpret_cast<const typename AttnElem<T>::x8*>(tile + attn_vt_offset(row, 16 * t + 8 * g));
+__device__ __forceinline__ typename AttnElem<T>::x8 bwd8_tr_frag(const T* tile, int off, int t) {
+  typedef AttnElem<T> E;
+  const T* p0 = tile + 16 * t * kAttnD + off;
+  const typename E::x4 lo = E::read_tr(p0);
+  const typename E::x4 hi = E::read_tr(p0 + 8 * kAttnD);
+  typename E::x8 r;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    r[e] = lo[e];
+    r[4 + e] = hi[e];
+  }
+  return r;
 }
 // Accumulators (transposed: lane = row of the output, registers = head dimension) of one wavefront's
 // 32 rows -> memory.  Stored from the registers a wavefront instruction would write 32 separate
@@ -249,28 +251,30 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
   const int wave_last_tile = (CAUSAL && qw < S) ? (qw + 31) / kAttnBN : (qw < S ? n_tiles - 1 : -1);
 
   auto buf = [&](int b) { return reinterpret_cast<T*>(attn_lds + b * kBwd8DqBufBytes); };
-  Bwd8ColStage kt;
-  Bwd8RowStage vt;
+  int tr_off[DB];
+  bwd8_tr_offsets(tr_off, lane);
   u32x2_t mk_next, mk_cur;  // mask words of this lane's query: the tile being loaded, the tile being computed
+  // requests tile `tile` into its buffer (free since the barrier that ended the tile before last)
   auto load_tile = [&](int tile) {
-    bwd8_load(kt, Kh + static_cast<size_t>(tile) * kAttnBN * kAttnD, tid);
-    bwd8_load(vt, Vh + static_cast<size_t>(tile) * kAttnBN * kAttnD, tid);
+    const T* kp = Kh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
+    T* Ks = buf(tile & 1);
+    bwd8_copy_tile<false>(kp, Ks, wave, lane);
+    bwd8_copy_tile<false>(Vh + static_cast<size_t>(tile) * kAttnBN * kAttnD, Ks + kBwd8Tile, wave, lane);
+    bwd8_copy_tile<true>(kp, Ks + 2 * kBwd8Tile, wave, lane);
     if constexpr (BITS)
       mk_next = *reinterpret_cast<const u32x2_t*>(head_mask + (static_cast<size_t>(qc) * all_tiles + tile) * 8);
   };
-  auto store_tile = [&](int b) {
+  // the requested tile has landed (for this wavefront's copies; the barrier that follows covers the rest)
+  auto finish_tile = [&]() {
     if constexpr (BITS) mk_cur = mk_next;
-    T* Ks = buf(b);
-    bwd8_store_rows(kt, Ks, tid);
-    bwd8_store_rows(vt, Ks + kBwd8RowTile, tid);
-    bwd8_store_cols(kt, Ks + 2 * kBwd8RowTile, tid);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   };
 
   auto compute = [&](int tile, auto mask_c) {
     constexpr bool MASK = decltype(mask_c)::value;
     const T* Ks = buf(tile & 1);
-    const T* Vs = Ks + kBwd8RowTile;
-    const T* Kt = Ks + 2 * kBwd8RowTile;
+    const T* Vs = Ks + kBwd8Tile;
+    const T* Kt = Ks + 2 * kBwd8Tile;
     const int key0 = tile * kAttnBN;
     x8_t dsf[2][2];
 #if BWD8_PREFETCH > 0
@@ -287,7 +291,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
         ka[i] = bwd8_row_frag(Ks, 32 * (i / DS) + li, i % DS, g);
         va[i] = bwd8_row_frag(Vs, 32 * (i / DS) + li, i % DS, g);
       } else if constexpr (i < N1 + N2) {
-        ta[i - N1] = bwd8_col_frag(Kt, 32 * ((i - N1) % DB) + li, (i - N1) / DB, g);
+        ta[i - N1] = bwd8_tr_frag(Kt, tr_off[(i - N1) % DB], (i - N1) / DB);
       }
     };
     static_for<PF>([&](auto ic) { issue(ic); });
@@ -352,7 +356,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int db = 0; db < DB; ++db)
-        acc[db] = E::mfma(bwd8_col_frag(Kt, 32 * db + li, t, g), dsf[t >> 1][t & 1], acc[db]);
+        acc[db] = E::mfma(bwd8_tr_frag(Kt, tr_off[db], t), dsf[t >> 1][t & 1], acc[db]);
   };
 
   // Under a causal mask only the tiles that overlap the block's own queries (the last four) need
@@ -360,12 +364,12 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
   // over the tiles before them carries no masking code.
   const int first_diag = CAUSAL ? min(q0 / kAttnBN, n_tiles) : n_tiles;
   load_tile(0);
-  store_tile(0);
+  finish_tile();
   __syncthreads();
   for (int tile = 0; tile < first_diag; ++tile) {
     if (tile + 1 < n_tiles) load_tile(tile + 1);
     if (tile <= wave_last_tile) compute(tile, attn_flag<false>{});
-    if (tile + 1 < n_tiles) store_tile((tile + 1) & 1);
+    finish_tile();
     __syncthreads();
   }
   if constexpr (CAUSAL) {
@@ -373,11 +377,11 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
     for (int tile = first_diag; tile < n_tiles; ++tile) {
       if (tile + 1 < n_tiles) load_tile(tile + 1);
       if (tile <= wave_last_tile) compute(tile, attn_flag<true>{});
-      if (tile + 1 < n_tiles) store_tile((tile + 1) & 1);
+      finish_tile();
       __syncthreads();
     }
   }
-  bwd8_store_acc<!CAUSAL>(dQ + head_off + static_cast<size_t>(qw) * kAttnD, acc, scale,
+  bwd8_store_acc<!CAUSAL || BWD8_STAGED_CAUSAL>(dQ + head_off + static_cast<size_t>(qw) * kAttnD, acc, scale,
                  reinterpret_cast<T*>(attn_lds) + wave * (32 * kAttnD), lane, S - qw);
   __syncthreads();  // the staging reads are done before a following block refills the tile buffers
 }
@@ -425,40 +429,41 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
   const int first_tile = CAUSAL ? k0 / kAttnBN : 0;  // first query tile that sees a key of the block
   const int wave_first_tile = kw < S ? (CAUSAL ? kw / kAttnBN : 0) : n_qtiles;
 
-  // DK: Q both ways + dO rows; DV: Q rows + dO transposed
-  Bwd8ColStage cst;  // DK: Q, DV: dO
-  Bwd8RowStage rst;  // DK: dO, DV: Q
+  // DK: Q for both kinds of read + dO rows; DV: Q rows + dO for transposing reads
+  int tr_off[DB];
+  bwd8_tr_offsets(tr_off, lane);
   Vec<float, 2> sst;
   u32x2_t mk_next, mk_cur;  // words of the transposed mask for this lane's key: tile being loaded / computed
+  // requests query tile `tile` into its buffer (free since the barrier that ended the tile before last)
   auto load_tile = [&](int tile) {
     const T* qp = Qh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
     const T* dp = dOh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
-    bwd8_load(cst, DK ? qp : dp, tid);
-    bwd8_load(rst, DK ? dp : qp, tid);
+    T* base = reinterpret_cast<T*>(attn_lds + (tile & 1) * BUF);
+    bwd8_copy_tile<false>(qp, base, wave, lane);                              // Q
+    if constexpr (DK) {
+      bwd8_copy_tile<false>(dp, base + kBwd8Tile, wave, lane);                // dO
+      bwd8_copy_tile<true>(qp, base + 2 * kBwd8Tile, wave, lane);             // Q, read transposed
+    } else {
+      bwd8_copy_tile<true>(dp, base + kBwd8Tile, wave, lane);                 // dO, read transposed
+    }
     if constexpr (BITS)
       mk_next = *reinterpret_cast<const u32x2_t*>(head_mask + (static_cast<size_t>(kc) * n_qtiles + tile) * 8);
     if (tid < kAttnBN) sst = load_vec<float, 2>(stats + 2 * (static_cast<size_t>(head) * S + tile * kAttnBN + tid));
   };
-  auto store_tile = [&](int b) {
+  // the requested tile has landed (this wavefront's copies; the barrier that follows covers the rest) and its
+  // row statistics go to their place behind the tiles
+  auto finish_tile = [&](int b) {
     if constexpr (BITS) mk_cur = mk_next;
-    T* base = reinterpret_cast<T*>(attn_lds + b * BUF);
-    if constexpr (DK) {
-      bwd8_store_rows(cst, base, tid);                        // Q
-      bwd8_store_rows(rst, base + kBwd8RowTile, tid);         // dO
-      bwd8_store_cols(cst, base + 2 * kBwd8RowTile, tid);     // Q^T
-    } else {
-      bwd8_store_rows(rst, base, tid);                        // Q
-      bwd8_store_cols(cst, base + kBwd8RowTile, tid);         // dO^T
-    }
     if (tid < kAttnBN) store_vec<float, 2>(reinterpret_cast<float*>(attn_lds + b * BUF + STAT_OFF) + 2 * tid, sst);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   };
 
   auto compute = [&](int tile, auto mask_c) {
     constexpr bool MASK = decltype(mask_c)::value;
     const T* base = reinterpret_cast<const T*>(attn_lds + (tile & 1) * BUF);
     const T* Qs = base;
-    const T* dOs = base + kBwd8RowTile;                              // DK only
-    const T* Tt = base + (DK ? 2 * kBwd8RowTile : kBwd8RowTile);     // Q^T (DK) or dO^T (DV)
+    const T* dOs = base + kBwd8Tile;                                 // DK only
+    const T* Tt = base + (DK ? 2 * kBwd8Tile : kBwd8Tile);           // the tile read transposed: Q (DK) or dO (DV)
     const float* st = reinterpret_cast<const float*>(attn_lds + (tile & 1) * BUF + STAT_OFF);
     const int q0t = tile * kAttnBN;
     x8_t bf[2][2];  // [query block][half]: P (dV) or dS (dK) as B operands, contraction over the queries
@@ -496,7 +501,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
           qa[i] = bwd8_row_frag(Qs, 32 * (i / DS) + li, i % DS, g);
           if constexpr (DK) da[i] = bwd8_row_frag(dOs, 32 * (i / DS) + li, i % DS, g);
         } else if constexpr (i < N1 + N2) {
-          ta[i - N1] = bwd8_col_frag(Tt, 32 * ((i - N1) % DB) + li, (i - N1) / DB, g);
+          ta[i - N1] = bwd8_tr_frag(Tt, tr_off[(i - N1) % DB], (i - N1) / DB);
         }
       };
       static_for<PF>([&](auto ic) { issue(ic); });
@@ -567,12 +572,12 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int db = 0; db < DB; ++db)
-        acc[db] = E::mfma(bwd8_col_frag(Tt, 32 * db + li, t, g), bf[t >> 1][t & 1], acc[db]);
+        acc[db] = E::mfma(bwd8_tr_frag(Tt, tr_off[db], t), bf[t >> 1][t & 1], acc[db]);
   };
 
   if (first_tile < n_qtiles) {
     load_tile(first_tile);
-    store_tile(first_tile & 1);
+    finish_tile(first_tile & 1);
   }
   __syncthreads();
   // Under a causal mask the first four query tiles overlap the block's own keys: a loop of their
@@ -583,17 +588,17 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
     for (int tile = first_tile; tile < after_diag; ++tile) {
       if (tile + 1 < n_qtiles) load_tile(tile + 1);
       if (tile >= wave_first_tile) compute(tile, attn_flag<true>{});
-      if (tile + 1 < n_qtiles) store_tile((tile + 1) & 1);
+      if (tile + 1 < n_qtiles) finish_tile((tile + 1) & 1);
       __syncthreads();
     }
   }
   for (int tile = after_diag; tile < n_qtiles; ++tile) {
     if (tile + 1 < n_qtiles) load_tile(tile + 1);
     if (kw < S) compute(tile, attn_flag<false>{});
-    if (tile + 1 < n_qtiles) store_tile((tile + 1) & 1);
+    if (tile + 1 < n_qtiles) finish_tile((tile + 1) & 1);
     __syncthreads();
   }
-  bwd8_store_acc<!CAUSAL>(dKV + head_off + static_cast<size_t>(kw) * kAttnD, acc, DK ? scale : 1.0f,
+  bwd8_store_acc<!CAUSAL || BWD8_STAGED_CAUSAL>(dKV + head_off + static_cast<size_t>(kw) * kAttnD, acc, DK ? scale : 1.0f,
                  reinterpret_cast<T*>(attn_lds) + wave * (32 * kAttnD), lane, S - kw);
   __syncthreads();  // the staging reads are done before a following block refills the tile buffers
 }

@@ -738,9 +738,11 @@ def fused_attention(
 # ---------------------------------------------------------------------------
 # fused attention backward (bf16, head dim 128): row statistics, then dQ, dK and dV kernels
 # ---------------------------------------------------------------------------
-_ATTN_BWD8_DQ_LDS = 2 * (2 * 64 * 136 + 128 * 64) * 2
-_ATTN_BWD8_DK_LDS = 2 * ((2 * 64 * 136 + 128 * 64) * 2 + 64 * 2 * 4)
-_ATTN_BWD8_DV_LDS = 2 * ((64 * 136 + 128 * 64) * 2 + 64 * 2 * 4)
+# two buffers of [64][128] tiles as they lie in memory (dQ: K, V and K again for the transposing reads; dK: Q, dO, Q;
+# dV: Q, dO), dK / dV with the 64 (offset, D) pairs of the query tile behind them
+_ATTN_BWD8_DQ_LDS = 2 * (3 * 64 * 128 * 2)
+_ATTN_BWD8_DK_LDS = 2 * (3 * 64 * 128 * 2 + 64 * 2 * 4)
+_ATTN_BWD8_DV_LDS = 2 * (2 * 64 * 128 * 2 + 64 * 2 * 4)
 
 
 @functools.lru_cache(maxsize=None)
