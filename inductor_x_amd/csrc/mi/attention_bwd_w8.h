@@ -48,7 +48,8 @@ constexpr int kBwd8DqLdsBytes = 2 * kBwd8DqBufBytes;
 constexpr int kBwd8DkLdsBytes = 2 * kBwd8DkBufBytes;
 constexpr int kBwd8DvLdsBytes = 2 * kBwd8DvBufBytes;
 constexpr float kBwd8Log2e = 1.4426950408889634f;
-// LDS fragments are read this many MFMA steps ahead in the unmasked loops (0: left to the compiler)
+// LDS fragments are read this many MFMA steps ahead in the unmasked loops (0: left to the compiler); measured at
+// [4,32,4096,128]: two steps ahead is worth 6 % in the causal dK and 8 % in the unmasked dV, more changes nothing
 #ifndef BWD8_PREFETCH
 #define BWD8_PREFETCH 2
 #endif
@@ -153,9 +154,9 @@ __device__ __forceinline__ typename AttnElem<T>::x8 bwd8_tr_frag(const T* tile, 
 // 16-byte pieces; instead the block goes through the wavefront's own 8 KiB of the (idle) tile
 // buffers, 16-byte chunks XOR-swizzled by the row, and leaves as whole 256-byte rows, four per
 // instruction.  The caller has passed the barrier that ends the last tile; `rows` of the 32 exist.
-// STAGED = false stores from the registers (the causal kernels: they spill registers already and
-// the staging costs them more than it saves -- measured at [4,32,4096,128]: 2.44 against 2.42 ms for
-// the three causal kernels, 4.19 against 4.24 ms for the unmasked ones).
+// STAGED = false stores from the registers (BWD8_STAGED_CAUSAL = 0 selects it for the causal kernels; measured
+// at [4,32,4096,128] the staged form is 2 % faster in dK and dV since the tiles stopped passing through
+// registers, and was slower before, when those kernels spilled).
 template <bool STAGED, typename T, int DB>
 __device__ __forceinline__ void bwd8_store_acc(T* __restrict__ dst_block, const f32x16_t (&acc)[DB], float factor,
                                                T* stage, int lane, int rows) {
@@ -490,7 +491,6 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
         }
       }
     };
-    // the causal dK kernel has no registers to spare for fragments in flight beyond one step
     constexpr int PF = DK ? (CAUSAL ? BWD8_PREFETCH_DK_CAUSAL : BWD8_PREFETCH_DK) : BWD8_PREFETCH_DV;
     if constexpr (PF > 0 && !MASK && !BITS) {
       // as in the dQ kernel: LDS fragments read PF steps ahead across the phases of the tile
