@@ -24,10 +24,9 @@
 // Every 64-row tile travels memory -> LDS by direct 16-byte `buffer_load ... lds` copies exactly as it
 // lies in memory ([64][128], one 1 KiB block = four rows per wavefront instruction, double-buffered, one
 // barrier per tile), the 16-byte chunks of a row XOR-swizzled on the way in by the choice of the global
-// chunk a lane fetches.  An operand that is read along its rows (K, V for dQ; Q, dO for dK / dV) is
-// swizzled by row mod 16; the transposed operand of the update product (K^T, Q^T, dO^T) is formed by
-// transposing LDS reads (`ds_read_b64_tr_b16`) of a second copy of the same tile, swizzled by a 4-entry
-// table that keeps those reads on distinct banks.  No tile passes through registers.
+// chunk a lane fetches (bwd8_swz).  The transposed operand of the update product (K^T, Q^T, dO^T) is
+// formed by transposing LDS reads (`ds_read_b64_tr_b16`) of the same tile that a score product reads
+// along its rows: one copy serves both.  No tile passes through registers.
 // Sequence lengths need only be multiples of 64: rows of a last partial block are clamped for
 // loads and not stored.
 #pragma once
@@ -41,9 +40,9 @@ constexpr int kBwd8Threads = 64 * kBwd8Waves;
 constexpr int kBwd8BlockRows = 32 * kBwd8Waves;  // queries (dQ) or keys (dK, dV) per workgroup
 constexpr int kBwd8Tile = kAttnBN * kAttnD;           // [64][128] tile as it lies in memory, elements
 constexpr int kBwd8StatBytes = kAttnBN * 2 * 4;       // (exponent offset, D) of a query tile
-constexpr int kBwd8DqBufBytes = 3 * kBwd8Tile * 2;                    // K, V, K for transposing reads
-constexpr int kBwd8DkBufBytes = 3 * kBwd8Tile * 2 + kBwd8StatBytes;   // Q, dO, Q for transposing reads
-constexpr int kBwd8DvBufBytes = 2 * kBwd8Tile * 2 + kBwd8StatBytes;   // Q, dO for transposing reads
+constexpr int kBwd8DqBufBytes = 2 * kBwd8Tile * 2;                    // K, V
+constexpr int kBwd8DkBufBytes = 2 * kBwd8Tile * 2 + kBwd8StatBytes;   // Q, dO
+constexpr int kBwd8DvBufBytes = 2 * kBwd8Tile * 2 + kBwd8StatBytes;   // Q, dO
 constexpr int kBwd8DqLdsBytes = 2 * kBwd8DqBufBytes;
 constexpr int kBwd8DkLdsBytes = 2 * kBwd8DkBufBytes;
 constexpr int kBwd8DvLdsBytes = 2 * kBwd8DvBufBytes;
@@ -98,18 +97,28 @@ __device__ __forceinline__ void attention_bwd_stats(const T* __restrict__ O, con
 // row-major.  Column form: 4 rows x 4 columns per thread (4 x 8 bytes), stored transposed with the
 // row index (the contraction axis of the MFMA that reads the tile) permuted, and optionally
 // row-major as well.
+// Chunk swizzle of a tile row: the 16-byte chunk c of row r lies at position c ^ bwd8_swz(r), a linear map
+// of the four low row bits (r0 -> chunk bits 1 and 3, r1 -> bit 2, r2 -> bit 0, r3 -> bit 3).  Sixteen
+// consecutive rows get sixteen different positions, which keeps the 16-byte reads along the rows (one row per
+// lane) off each other's banks; and the four consecutive rows that one pass of a transposing read touches
+// (32 bytes of each) differ in chunk bits 1, 2 and 3 the way the forward's V swizzle makes them differ.
+// Measured at [4,32,4096,128]: as fast as two copies under the two separate swizzles, one tile copy less.
+__device__ __forceinline__ int bwd8_swz(int row) {
+  const int r0 = row & 1, r1 = (row >> 1) & 1, r2 = (row >> 2) & 1, r3 = (row >> 3) & 1;
+  return (r0 << 1) | (r1 << 2) | r2 | ((r0 ^ r3) << 3);
+}
+
 // One [64][128] tile, memory -> LDS: the eight wavefronts copy two 1 KiB blocks (four rows) each; lane l of
 // an instruction fills LDS chunk l of the block (row 4 b + l / 16, chunk position l % 16) with the global
-// chunk that the swizzle puts there.  TR: the copy that the transposing reads use.
-template <bool TR, typename T>
+// chunk that the swizzle puts there.
+template <typename T>
 __device__ __forceinline__ void bwd8_copy_tile(const T* __restrict__ src, T* dst, int wave, int lane) {
   const int blk_row = lane >> 4, blk_pos = lane & 15;
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int b = 2 * wave + u;
     const int row = 4 * b + blk_row;
-    const int swz = TR ? ((0xE4A0 >> (4 * (row & 3))) & 15) : (row & 15);
-    const int voff = (row * kAttnD + 8 * (blk_pos ^ swz)) * 2;
+    const int voff = (row * kAttnD + 8 * (blk_pos ^ bwd8_swz(row))) * 2;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(
         __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(src), 0, kBwd8Tile * 2, 0x00020000),
         (__attribute__((address_space(3))) void*)(dst + b * 512), 16, voff, 0, 0, 0);
@@ -118,7 +127,7 @@ __device__ __forceinline__ void bwd8_copy_tile(const T* __restrict__ src, T* dst
 // A operand along the rows of a tile: row `row`, d slice s, half g
 template <typename T>
 __device__ __forceinline__ typename AttnElem<T>::x8 bwd8_row_frag(const T* tile, int row, int s, int g) {
-  return *reinterpret_cast<const typename AttnElem<T>::x8*>(tile + row * kAttnD + 8 * ((2 * s + g) ^ (row & 15)));
+  return *reinterpret_cast<const typename AttnElem<T>::x8*>(tile + row * kAttnD + 8 * ((2 * s + g) ^ bwd8_swz(row)));
 }
 // Per-lane element offsets of the transposing reads, one per d block: in every group of 16 lanes, lane s
 // points at four consecutive d of row 4 g + s / 4 (+ 8 for the second read) and receives, for its own d,
@@ -128,11 +137,10 @@ template <int DB>
 __device__ __forceinline__ void bwd8_tr_offsets(int (&off)[DB], int lane) {
   const int sl16 = lane & 15, grp = lane >> 4;
   const int row_l = 4 * (grp >> 1) + (sl16 >> 2);
-  const int f = (0xE4A0 >> (4 * (row_l & 3))) & 15;
   const int c_l = 2 * (grp & 1) + ((sl16 & 3) >> 1);
 #pragma unroll
   for (int db = 0; db < DB; ++db)
-    off[db] = row_l * kAttnD + 8 * (((4 * db) ^ (f & 12)) + (c_l ^ (f & 2))) + 4 * (sl16 & 1);
+    off[db] = row_l * kAttnD + 8 * ((4 * db + c_l) ^ bwd8_swz(row_l)) + 4 * (sl16 & 1);
 }
 // A operand across the rows of a tile (the tile transposed): d block via its offset, row slice t of 16
 template <typename T>
@@ -140,7 +148,8 @@ __device__ __forceinline__ typename AttnElem<T>::x8 bwd8_tr_frag(const T* tile, 
   typedef AttnElem<T> E;
   const T* p0 = tile + 16 * t * kAttnD + off;
   const typename E::x4 lo = E::read_tr(p0);
-  const typename E::x4 hi = E::read_tr(p0 + 8 * kAttnD);
+  // eight rows further down the chunk sits bwd8_swz(8) positions away (the swizzle is linear in the row bits)
+  const typename E::x4 hi = E::read_tr(tile + (16 * t + 8) * kAttnD + (off ^ (8 * bwd8_swz(8))));
   typename E::x8 r;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
@@ -258,10 +267,9 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
   // requests tile `tile` into its buffer (free since the barrier that ended the tile before last)
   auto load_tile = [&](int tile) {
     const T* kp = Kh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
-    T* Ks = buf(tile & 1);
-    bwd8_copy_tile<false>(kp, Ks, wave, lane);
-    bwd8_copy_tile<false>(Vh + static_cast<size_t>(tile) * kAttnBN * kAttnD, Ks + kBwd8Tile, wave, lane);
-    bwd8_copy_tile<true>(kp, Ks + 2 * kBwd8Tile, wave, lane);
+    T* Ks = buf(tile & 1);  // K for both kinds of read, V behind it
+    bwd8_copy_tile(kp, Ks, wave, lane);
+    bwd8_copy_tile(Vh + static_cast<size_t>(tile) * kAttnBN * kAttnD, Ks + kBwd8Tile, wave, lane);
     if constexpr (BITS)
       mk_next = *reinterpret_cast<const u32x2_t*>(head_mask + (static_cast<size_t>(qc) * all_tiles + tile) * 8);
   };
@@ -275,7 +283,7 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
     constexpr bool MASK = decltype(mask_c)::value;
     const T* Ks = buf(tile & 1);
     const T* Vs = Ks + kBwd8Tile;
-    const T* Kt = Ks + 2 * kBwd8Tile;
+    const T* Kt = Ks;  // the same tile, read transposed
     const int key0 = tile * kAttnBN;
     x8_t dsf[2][2];
 #if BWD8_PREFETCH > 0
@@ -430,7 +438,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
   const int first_tile = CAUSAL ? k0 / kAttnBN : 0;  // first query tile that sees a key of the block
   const int wave_first_tile = kw < S ? (CAUSAL ? kw / kAttnBN : 0) : n_qtiles;
 
-  // DK: Q for both kinds of read + dO rows; DV: Q rows + dO for transposing reads
+  // DK reads Q both ways and dO along its rows; DV reads Q along its rows and dO transposed
   int tr_off[DB];
   bwd8_tr_offsets(tr_off, lane);
   Vec<float, 2> sst;
@@ -440,13 +448,8 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
     const T* qp = Qh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
     const T* dp = dOh + static_cast<size_t>(tile) * kAttnBN * kAttnD;
     T* base = reinterpret_cast<T*>(attn_lds + (tile & 1) * BUF);
-    bwd8_copy_tile<false>(qp, base, wave, lane);                              // Q
-    if constexpr (DK) {
-      bwd8_copy_tile<false>(dp, base + kBwd8Tile, wave, lane);                // dO
-      bwd8_copy_tile<true>(qp, base + 2 * kBwd8Tile, wave, lane);             // Q, read transposed
-    } else {
-      bwd8_copy_tile<true>(dp, base + kBwd8Tile, wave, lane);                 // dO, read transposed
-    }
+    bwd8_copy_tile(qp, base, wave, lane);               // Q: along its rows, and transposed for dK
+    bwd8_copy_tile(dp, base + kBwd8Tile, wave, lane);   // dO: along its rows for dK, transposed for dV
     if constexpr (BITS)
       mk_next = *reinterpret_cast<const u32x2_t*>(head_mask + (static_cast<size_t>(kc) * n_qtiles + tile) * 8);
     if (tid < kAttnBN) sst = load_vec<float, 2>(stats + 2 * (static_cast<size_t>(head) * S + tile * kAttnBN + tid));
@@ -464,7 +467,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
     const T* base = reinterpret_cast<const T*>(attn_lds + (tile & 1) * BUF);
     const T* Qs = base;
     const T* dOs = base + kBwd8Tile;                                 // DK only
-    const T* Tt = base + (DK ? 2 * kBwd8Tile : kBwd8Tile);           // the tile read transposed: Q (DK) or dO (DV)
+    const T* Tt = DK ? base : base + kBwd8Tile;                      // the tile read transposed: Q (DK) or dO (DV)
     const float* st = reinterpret_cast<const float*>(attn_lds + (tile & 1) * BUF + STAT_OFF);
     const int q0t = tile * kAttnBN;
     x8_t bf[2][2];  // [query block][half]: P (dV) or dS (dK) as B operands, contraction over the queries

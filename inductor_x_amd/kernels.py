@@ -738,10 +738,10 @@ def fused_attention(
 # ---------------------------------------------------------------------------
 # fused attention backward (bf16, head dim 128): row statistics, then dQ, dK and dV kernels
 # ---------------------------------------------------------------------------
-# two buffers of [64][128] tiles as they lie in memory (dQ: K, V and K again for the transposing reads; dK: Q, dO, Q;
-# dV: Q, dO), dK / dV with the 64 (offset, D) pairs of the query tile behind them
-_ATTN_BWD8_DQ_LDS = 2 * (3 * 64 * 128 * 2)
-_ATTN_BWD8_DK_LDS = 2 * (3 * 64 * 128 * 2 + 64 * 2 * 4)
+# two buffers of two [64][128] tiles as they lie in memory (dQ: K, V; dK and dV: Q, dO, with the 64 (offset, D)
+# pairs of the query tile behind them); the row staging of the result at the end uses the first 64 KiB
+_ATTN_BWD8_DQ_LDS = 2 * (2 * 64 * 128 * 2)
+_ATTN_BWD8_DK_LDS = 2 * (2 * 64 * 128 * 2 + 64 * 2 * 4)
 _ATTN_BWD8_DV_LDS = 2 * (2 * 64 * 128 * 2 + 64 * 2 * 4)
 
 
