@@ -95,9 +95,9 @@ KERNEL_TRACE_US: dict = {
     ('4acold', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "us": [24.02], "profile": "profiles/kernel_traces_per_config.txt"},
     ('4bcold', 'kernel'): {"symbols": ["permute_copy_b16_b256_p16_t8x2"], "us": [84.4], "profile": "profiles/kernel_traces_per_config.txt"},
     ('4bcold', 'torch.compile'): {"symbols": ["hip_pointwise_0"], "us": [86.53], "profile": "profiles/kernel_traces_per_config.txt"},
-    ('5', 'kernel'): {"symbols": ["fused_attention_fwd_bf16_d128_causal_v5"], "us": [583.17], "profile": "profiles/kernel_traces_per_config.txt"},
-    ('5', 'torch.compile'): {"symbols": ["fused_attention_fwd_bf16_d128_causal_v5"], "us": [583.17], "profile": "profiles/kernel_traces_per_config.txt"},
-    ('5b', 'kernel'): {"symbols": ["attention_bwd_stats_bf16_d128", "attention_bwd8_dk_bf16_d128_causal", "attention_bwd8_dv_bf16_d128_causal", "attention_bwd8_dq_bf16_d128_causal"], "us": [51.86, 825.16, 598.8, 775.52], "profile": "profiles/kernel_traces_per_config.txt"},
+    ('5', 'kernel'): {"symbols": ["fused_attention_fwd_bf16_d128_causal_v5"], "us": [575.06], "profile": "profiles/kernel_traces_per_config.txt"},
+    ('5', 'torch.compile'): {"symbols": ["fused_attention_fwd_bf16_d128_causal_v5"], "us": [575.06], "profile": "profiles/kernel_traces_per_config.txt"},
+    ('5b', 'kernel'): {"symbols": ["attention_bwd_stats_bf16_d128", "attention_bwd8_dk_bf16_d128_causal", "attention_bwd8_dv_bf16_d128_causal", "attention_bwd8_dq_bf16_d128_causal"], "us": [53.94, 796.63, 587.58, 759.39], "profile": "profiles/kernel_traces_per_config.txt"},
 }
 
 ALGO_BYTES = {
