@@ -17,8 +17,10 @@ viewed as [B, N, S, D], copied once into that order for the kernels and copied b
 kernel takes bf16 and fp16 operands with a head dimension that is a multiple of 8 up to 128
 (smaller heads are zero-padded to 128) at any query and key lengths, also with a general mask (any
 type, non-zero = hidden); a positional bias (pse), fp32 operands, other
-head dimensions and dropout (keep_prob < 1) run the same mathematics over library GEMMs; padding masks, prefixes, variable sequence lengths and band masks
-raise.
+head dimensions and dropout (keep_prob < 1) run the same mathematics over library GEMMs.  pre_tockens / next_tockens
+short of the sequence (sparse_mode 0) describe a sliding window, key j visible to query i when
+-pre_tockens <= j - i <= next_tockens: it becomes a mask for the fused kernels, joined with atten_mask if one is
+given.  Padding masks, prefixes, variable sequence lengths and the other sparse modes raise.
 The backward op recomputes the probabilities from the saved row statistics inside fused gradient
 kernels (bf16 or fp16, head dimension up to 128, one shape for q, k, v;
 kernels.fused_attention_backward) and falls back to the GEMM formulation otherwise
@@ -90,20 +92,36 @@ def _check_layout(op: str, layout: str):
         raise NotImplementedError(f"{op}: layout {layout!r} (supported: {', '.join(LAYOUTS)})")
 
 
-def _is_causal(seq_len: int, atten_mask, pre_tockens: int, next_tockens: int, sparse_mode: int) -> bool:
-    """True when the arguments describe the plain causal mask (which the kernels apply themselves and
-    for which a mask tensor, if given, is the compressed triangle of the reference's device library and is
-    not read).  Otherwise a given atten_mask is applied as it stands."""
+@functools.lru_cache(maxsize=4)
+def _band_mask(sq: int, sk: int, pre_tockens: int, next_tockens: int, device: str) -> torch.Tensor:
+    """[sq, sk] bool, True = hidden: key j is visible to query i when -pre_tockens <= j - i <= next_tockens."""
+    dist = torch.arange(sk, device=device).view(1, sk) - torch.arange(sq, device=device).view(sq, 1)
+    return (dist > next_tockens) | (dist < -pre_tockens)
+
+
+def _mask_plan(query, key, atten_mask, pre_tockens: int, next_tockens: int, sparse_mode: int):
+    """(causal, mask) for the op's mask arguments.  causal: the plain causal mask, which the kernels apply
+    themselves (sparse_mode 2 or 3, or next_tockens == 0 with pre_tockens covering the sequence; a mask tensor,
+    if given, is then the compressed triangle of the reference's device library and is not read).  Otherwise
+    mask is what hides keys: a given atten_mask as it stands, a band when pre_tockens / next_tockens are short
+    of the sequence (a sliding window: key j visible to query i when -pre_tockens <= j - i <= next_tockens),
+    or both."""
+    sq, sk = query.size(2), key.size(2)
     if sparse_mode in (2, 3):
-        return True
-    if sparse_mode == 0 and next_tockens == 0 and pre_tockens >= seq_len:
-        return True
-    if sparse_mode != 0 or (atten_mask is None and (next_tockens < seq_len or pre_tockens < seq_len)):
-        raise NotImplementedError(
-            "npu_fa: band masks (pre_tockens / next_tockens short of the sequence length) and sparse modes other "
-            "than 0, 2 and 3 are not supported"
-        )
-    return False
+        return True, None
+    if sparse_mode != 0:
+        raise NotImplementedError("npu_fa: sparse modes other than 0, 2 and 3 are not supported")
+    if next_tockens == 0 and pre_tockens >= sq:
+        return True, None
+    mask = atten_mask
+    if next_tockens < sk - 1 or pre_tockens < sq - 1:
+        band = _band_mask(sq, sk, max(int(pre_tockens), -TOKEN_MAX), max(int(next_tockens), -TOKEN_MAX), str(query.device))
+        if mask is None:
+            mask = band
+        else:
+            hide = mask if mask.dtype == torch.bool else mask != 0
+            mask = hide | (band if hide.dim() == 2 else band.view(1, 1, sq, sk))
+    return False, mask
 
 
 def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask=None, atten_mask=None, scale=1.0,
@@ -124,8 +142,7 @@ def npu_fa_gpu(query, key, value, head_num, input_layout, pse=None, padding_mask
         raise ZeroDivisionError("npu_fa: the inverse scale factor is zero")
     # the graph pattern passes the divisor of the scores; the kernel multiplies
     real_scale = 1.0 / scale
-    causal = _is_causal(query.size(2), atten_mask, pre_tockens, next_tockens, sparse_mode)
-    mask = None if causal else atten_mask  # under the causal modes the mask tensor is the library's compressed triangle
+    causal, mask = _mask_plan(query, key, atten_mask, pre_tockens, next_tockens, sparse_mode)
     seed = numels = 0
     head_dim = query.size(3)
     mask_fits = mask is None or (mask.is_cuda and mask.dim() in (2, 4))
@@ -183,8 +200,7 @@ def npu_fa_backward_gpu(query, key, value, dy, head_num, input_layout, *, pse=No
     query, key, value, attention_in, dy = (
         _to_bnsd(t, head_num, layout).contiguous() for t in (query, key, value, attention_in, dy)
     )
-    causal = _is_causal(query.size(2), atten_mask, pre_tockens, next_tockens, sparse_mode)
-    mask = None if causal else atten_mask
+    causal, mask = _mask_plan(query, key, atten_mask, pre_tockens, next_tockens, sparse_mode)
     grads = fused_attention_backward(
         query, key, value, attention_in, dy, softmax_max, softmax_sum, 1.0 / scale_value, causal,
         keep_prob=keep_prob, seed=int(seed.item()) if keep_prob < 1.0 else 0, pse=pse, atten_mask=mask,

@@ -810,3 +810,66 @@ def test_attention_op_dropout(dtype, B, N, S, D, causal, keep_prob):
     assert zero[0].abs().max().item() == 0.0
     with pytest.raises(ValueError):
         npu_fusion_attention_graph(q, k, v, N, "BNSD", scale=inv, keep_prob=1.5)
+
+
+@pytest.mark.parametrize("dtype,B,N,Sq,Sk,D,pre,nxt,extra", [
+    (torch.bfloat16, 2, 3, 320, 320, 128, 63, 0, False),     # causal sliding window of 64 keys
+    (torch.float16, 1, 4, 256, 256, 64, 100, 17, False),      # a band around the diagonal, small heads
+    (torch.bfloat16, 2, 2, 200, 200, 128, 40, 40, True),      # band joined with a key-padding mask, ragged length
+    (torch.bfloat16, 1, 2, 130, 300, 128, 20, 150, False),    # query and key lengths differ (forward only)
+    (torch.bfloat16, 1, 2, 256, 256, 128, 2147483647, 2147483647, False),  # the defaults: no band at all
+])
+def test_attention_op_sliding_window(dtype, B, N, Sq, Sk, D, pre, nxt, extra):
+    """pre_tockens / next_tockens short of the sequence (op schema, reference
+    inductor_x/npu_fusion_attention_graph.py:17): key j is visible to query i when -pre <= j - i <= next.
+    The band runs on the fused kernels as a bit mask, forward and gradients, alone or joined with atten_mask."""
+    announce(f"attention op sliding window {dtype} [{B},{N},{Sq}/{Sk},{D}] pre={pre} next={nxt} mask={extra}")
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
+    torch.manual_seed(17)
+    same = Sq == Sk
+    q = torch.randn(B, N, Sq, D, device=DEV).to(dtype).requires_grad_(same)
+    k = torch.randn(B, N, Sk, D, device=DEV).to(dtype).requires_grad_(same)
+    v = torch.randn(B, N, Sk, D, device=DEV).to(dtype).requires_grad_(same)
+    user = None
+    if extra:
+        user = torch.zeros(B, 1, Sq, Sk, device=DEV, dtype=torch.bool)
+        user[0, :, :, Sk - 30:] = True
+    inv = D ** 0.5
+    out = npu_fusion_attention_graph(q, k, v, N, "BNSD", atten_mask=user, scale=inv, pre_tockens=pre, next_tockens=nxt)[0]
+    dist = torch.arange(Sk, device=DEV).view(1, Sk) - torch.arange(Sq, device=DEV).view(Sq, 1)
+    hide = ((dist > nxt) | (dist < -pre)).view(1, 1, Sq, Sk)
+    if user is not None:
+        hide = hide | user
+    qf, kf, vf = (t.detach().float().requires_grad_(same) for t in (q, k, v))
+    s = (qf @ kf.transpose(-1, -2)) / inv
+    s = s.masked_fill(hide, float("-inf"))
+    gone = hide.expand(B, N, Sq, Sk).all(-1, keepdim=True)
+    p = torch.softmax(s.masked_fill(gone, 0.0), -1).masked_fill(gone, 0.0)
+    want = p @ vf
+    assert (out.float() - want).abs().max().item() <= 2e-2
+    if same:
+        go = torch.randn_like(want)
+        want.backward(go)
+        out.backward(go.to(dtype))
+        for g, r in zip((q.grad, k.grad, v.grad), (qf.grad, kf.grad, vf.grad)):
+            assert torch.isfinite(g).all()
+            assert (g.float() - r).abs().max().item() <= 3e-2 * max(r.abs().max().item(), 1.0)
+
+
+def test_attention_op_sliding_window_launches_the_masked_kernels():
+    announce("attention op sliding window launches the masked kernels")
+    from inductor_x_amd import launcher as L
+    from inductor_x_amd.fusion_attention_graph import npu_fusion_attention_graph
+
+    torch.manual_seed(3)
+    q, k, v = (torch.randn(1, 2, 256, 128, device=DEV).bfloat16().requires_grad_() for _ in range(3))
+    L.launch_log = []
+    try:
+        out = npu_fusion_attention_graph(q, k, v, 2, "BNSD", scale=128 ** 0.5, pre_tockens=31, next_tockens=0)[0]
+        out.sum().backward()
+        torch.cuda.synchronize()
+    finally:
+        names, L.launch_log = L.launch_log, None
+    assert "fused_attention_fwd_bf16_d128_full_v5_masked" in names, names
+    assert {f"attention_bwd8_{w}_bf16_d128_full_masked" for w in ("dq", "dk", "dv")} <= set(names), names
