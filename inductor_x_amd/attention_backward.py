@@ -170,7 +170,11 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
                 hide = torch.nn.functional.pad(hide, (0, pad_s, 0, pad_s), value=True)
             packed = (kernels.attention_mask_bits(hide, q.size(0), q.size(1), Sp, Sp),
                       kernels.attention_mask_bits(hide.transpose(-1, -2), q.size(0), q.size(1), Sp, Sp))
+            # the tiles of the other axis each block of 256 rows has to visit (a sliding window visits few)
+            ranges = (kernels.attention_mask_tile_ranges(packed[0], Sp, Sp, causal),
+                      kernels.attention_mask_tile_ranges(packed[1], Sp, Sp, causal, transposed=True))
         else:
+            ranges = None
             # keys S .. Sp - 1 hidden from everybody: the same word row for every query (only the last key
             # tile has bits set); transposed, a padded key hides every query and a real key none
             tiles = Sp // 64
@@ -181,7 +185,7 @@ def fused_attention_backward(q, k, v, out, dout, softmax_max, softmax_sum, scale
             cols[S:] = -1
             packed = (rows, cols.view(1, 1, Sp, tiles).view(torch.uint8))
         grads = kernels.fused_attention_backward(widen(q), widen(k), widen(v), widen(out), widen(dout), smax, ssum, scale, causal,
-                                                 packed_masks=packed)
+                                                 packed_masks=packed, tile_ranges=ranges)
         grads = tuple(g[:, :, :S, :d].contiguous() for g in grads) if (pad_d or pad_s) else grads
         return grads + (None,) if atten_mask is not None else grads
     if pse is not None or atten_mask is not None:

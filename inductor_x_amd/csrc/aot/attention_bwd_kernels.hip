@@ -92,30 +92,37 @@ BWD8_D64(bf16_t, bf16)
 BWD8_D64(f16_t, f16)
 
 // With a bit mask (64-bit words [B or 1, N or 1, S, S / 64], byte strides; dQ takes the words of the mask,
-// dK and dV those of its transpose): hidden pairs get the probability zero.
+// dK and dV those of its transpose): hidden pairs get the probability zero.  tile_ranges (may be null): per
+// block of 256 rows the first and last tile of the other axis with a visible pair, int [B or 1, N or 1,
+// ceil(S / 256), 2] with batch and head strides in elements; tiles outside are not visited.
 #define BWD8_MASKED(NAME, T, CAUSAL, BODY)                                                             \
   extern "C" __global__ __launch_bounds__(512, 1) void NAME(                                           \
       const T* q, const T* k, const T* v, const T* d_o, const float* stats, T* out, int n_heads,       \
       int S, float scale, const unsigned char* mask, long long mask_batch_stride,                      \
-      long long mask_head_stride, int heads_per_batch) {                                               \
+      long long mask_head_stride, int heads_per_batch, const int* tile_ranges, int range_batch_stride, \
+      int range_head_stride) {                                                                         \
     bwd8_for_blocks<CAUSAL>(n_heads, S, [&](int head, int block) {                                     \
       const unsigned char* hm =                                                                        \
           mask + (head / heads_per_batch) * mask_batch_stride + (head % heads_per_batch) * mask_head_stride; \
+      const int* hr = tile_ranges ? tile_ranges + (head / heads_per_batch) * range_batch_stride +      \
+                                        (head % heads_per_batch) * range_head_stride + 2 * block       \
+                                  : nullptr;                                                           \
+      const int lo = hr ? hr[0] : 0, hi = hr ? hr[1] : 0x7fffff;                                       \
       BODY;                                                                                            \
     });                                                                                                \
   }
 #define BWD8_MASKED_ALL(T, TN)                                                                                     \
   BWD8_MASKED(attention_bwd8_dq_##TN##_d128_causal_masked, T, true,                                               \
-              (attention_bwd8_dq<T, true, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm)))         \
+              (attention_bwd8_dq<T, true, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm, lo, hi)))         \
   BWD8_MASKED(attention_bwd8_dq_##TN##_d128_full_masked, T, false,                                                \
-              (attention_bwd8_dq<T, false, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm)))        \
+              (attention_bwd8_dq<T, false, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm, lo, hi)))        \
   BWD8_MASKED(attention_bwd8_dk_##TN##_d128_causal_masked, T, true,                                               \
-              (attention_bwd8_dkv<T, true, 0, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm)))     \
+              (attention_bwd8_dkv<T, true, 0, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm, lo, hi)))     \
   BWD8_MASKED(attention_bwd8_dk_##TN##_d128_full_masked, T, false,                                                \
-              (attention_bwd8_dkv<T, false, 0, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm)))    \
+              (attention_bwd8_dkv<T, false, 0, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm, lo, hi)))    \
   BWD8_MASKED(attention_bwd8_dv_##TN##_d128_causal_masked, T, true,                                               \
-              (attention_bwd8_dkv<T, true, 1, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm)))     \
+              (attention_bwd8_dkv<T, true, 1, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm, lo, hi)))     \
   BWD8_MASKED(attention_bwd8_dv_##TN##_d128_full_masked, T, false,                                                \
-              (attention_bwd8_dkv<T, false, 1, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm)))
+              (attention_bwd8_dkv<T, false, 1, 128, true>(q, k, v, d_o, stats, out, S, block, head, scale, hm, lo, hi)))
 BWD8_MASKED_ALL(bf16_t, bf16)
 BWD8_MASKED_ALL(f16_t, f16)

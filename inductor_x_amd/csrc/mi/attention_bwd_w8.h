@@ -219,13 +219,16 @@ __device__ __forceinline__ void bwd8_zero(f32x16_t (&acc)[DB]) {
 // BITS (both kernels below): a bit mask for this head, one 64-bit word per (row, tile of the other axis)
 // laid out [S][S / 64], bit j set = the pair is hidden (dQ: row = query, bit = key of the tile; dK / dV:
 // row = key, bit = query of the tile, i.e. the words of the transposed mask); hidden pairs get the
-// probability zero.  The word of the next tile is fetched with that tile's operands.
+// probability zero.  The word of the next tile is fetched with that tile's operands.  tile_lo .. tile_hi (BITS
+// only): the tiles of the other axis outside this range hold no visible pair for any row of the block (the
+// host derives the range from the mask words) and are left out of the loop.
 template <typename T, bool CAUSAL, int DH = 128, bool BITS = false>
 __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const T* __restrict__ K,
                                                   const T* __restrict__ V, const T* __restrict__ dO,
                                                   const float* __restrict__ stats, T* __restrict__ dQ,
                                                   int S, int q_block, int head, float scale,
-                                                  const unsigned char* __restrict__ head_mask = nullptr) {
+                                                  const unsigned char* __restrict__ head_mask = nullptr,
+                                                  int tile_lo = 0, int tile_hi = 0x7fffff) {
   typedef AttnElem<T> E;
   typedef typename E::x8 x8_t;
   extern __shared__ __attribute__((aligned(16))) unsigned char attn_lds[];
@@ -257,7 +260,9 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
   bwd8_zero(acc);
 
   const int all_tiles = S / kAttnBN;
-  const int n_tiles = CAUSAL ? min((q0 + kBwd8BlockRows) / kAttnBN, all_tiles) : all_tiles;
+  const int end_tiles = CAUSAL ? min((q0 + kBwd8BlockRows) / kAttnBN, all_tiles) : all_tiles;
+  const int n_tiles = BITS ? min(end_tiles, max(tile_hi, 0) + 1) : end_tiles;  // one past the last tile visited
+  const int first = BITS ? min(max(tile_lo, 0), n_tiles - 1) : 0;            // first tile visited
   const int wave_last_tile = (CAUSAL && qw < S) ? (qw + 31) / kAttnBN : (qw < S ? n_tiles - 1 : -1);
 
   auto buf = [&](int b) { return reinterpret_cast<T*>(attn_lds + b * kBwd8DqBufBytes); };
@@ -371,11 +376,11 @@ __device__ __forceinline__ void attention_bwd8_dq(const T* __restrict__ Q, const
   // Under a causal mask only the tiles that overlap the block's own queries (the last four) need
   // the mask or are skipped by some wavefronts; they run in a loop of their own so that the loop
   // over the tiles before them carries no masking code.
-  const int first_diag = CAUSAL ? min(q0 / kAttnBN, n_tiles) : n_tiles;
-  load_tile(0);
+  const int first_diag = CAUSAL ? max(min(q0 / kAttnBN, n_tiles), first) : n_tiles;
+  load_tile(first);
   finish_tile();
   __syncthreads();
-  for (int tile = 0; tile < first_diag; ++tile) {
+  for (int tile = first; tile < first_diag; ++tile) {
     if (tile + 1 < n_tiles) load_tile(tile + 1);
     if (tile <= wave_last_tile) compute(tile, attn_flag<false>{});
     finish_tile();
@@ -403,7 +408,8 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
                                                    const T* __restrict__ V, const T* __restrict__ dO,
                                                    const float* __restrict__ stats, T* __restrict__ dKV,
                                                    int S, int k_block, int head, float scale,
-                                                   const unsigned char* __restrict__ head_mask = nullptr) {
+                                                   const unsigned char* __restrict__ head_mask = nullptr,
+                                                   int tile_lo = 0, int tile_hi = 0x7fffff) {
   constexpr bool DK = WHICH == 0;
   constexpr int BUF = DK ? kBwd8DkBufBytes : kBwd8DvBufBytes;
   constexpr int STAT_OFF = BUF - kBwd8StatBytes;
@@ -434,9 +440,11 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
   bwd8_zero(acc);
   const float c2 = scale * kBwd8Log2e;
 
-  const int n_qtiles = S / kAttnBN;
-  const int first_tile = CAUSAL ? k0 / kAttnBN : 0;  // first query tile that sees a key of the block
-  const int wave_first_tile = kw < S ? (CAUSAL ? kw / kAttnBN : 0) : n_qtiles;
+  const int all_qtiles = S / kAttnBN;
+  const int n_qtiles = BITS ? min(all_qtiles, max(tile_hi, 0) + 1) : all_qtiles;  // one past the last query tile visited
+  // first query tile visited: under a causal mask the first one that sees a key of the block
+  const int first_tile = BITS ? min(max(CAUSAL ? k0 / kAttnBN : 0, tile_lo), n_qtiles) : (CAUSAL ? k0 / kAttnBN : 0);
+  const int wave_first_tile = kw < S ? (CAUSAL ? kw / kAttnBN : 0) : all_qtiles;
 
   // DK reads Q both ways and dO along its rows; DV reads Q along its rows and dO transposed
   int tr_off[DB];
@@ -451,7 +459,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
     bwd8_copy_tile(qp, base, wave, lane);               // Q: along its rows, and transposed for dK
     bwd8_copy_tile(dp, base + kBwd8Tile, wave, lane);   // dO: along its rows for dK, transposed for dV
     if constexpr (BITS)
-      mk_next = *reinterpret_cast<const u32x2_t*>(head_mask + (static_cast<size_t>(kc) * n_qtiles + tile) * 8);
+      mk_next = *reinterpret_cast<const u32x2_t*>(head_mask + (static_cast<size_t>(kc) * all_qtiles + tile) * 8);
     if (tid < kAttnBN) sst = load_vec<float, 2>(stats + 2 * (static_cast<size_t>(head) * S + tile * kAttnBN + tid));
   };
   // the requested tile has landed (this wavefront's copies; the barrier that follows covers the rest) and its
@@ -585,7 +593,7 @@ __device__ __forceinline__ void attention_bwd8_dkv(const T* __restrict__ Q, cons
   __syncthreads();
   // Under a causal mask the first four query tiles overlap the block's own keys: a loop of their
   // own with the mask (and wavefronts whose keys come later skipping), then the unmasked rest.
-  const int after_diag = CAUSAL ? min(first_tile + kBwd8BlockRows / kAttnBN, n_qtiles) : first_tile;
+  const int after_diag = CAUSAL ? max(min(k0 / kAttnBN + kBwd8BlockRows / kAttnBN, n_qtiles), first_tile) : first_tile;
   if constexpr (CAUSAL) {
 #pragma nounroll
     for (int tile = first_tile; tile < after_diag; ++tile) {

@@ -52,7 +52,9 @@ struct AttnNoTimeline {
 // a word set = key 64 tile + j is hidden from the query, is applied to the scores besides the causal
 // mask; needs RAGGED.  A lane fetches the word of its query for the next tile (one bounded 8-byte buffer
 // load: zero past the end) while the current tile is worked on.  A row with every key hidden gives zeros,
-// maximum 0 and sum 1.
+// maximum 0 and sum 1.  tile_lo .. tile_hi (MASKED only): the key tiles outside this range hold no key that
+// any query of the block may see (the host derives the range from the mask words); they are neither
+// copied nor computed, which is what makes a sliding window or a block-sparse mask cheaper than a dense one.
 template <typename T, bool CAUSAL, bool RAGGED, int WAVES = kAttnV5Waves, int DH = 128, bool MASKED = false,
           typename TL = AttnNoTimeline>
 __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, const T* __restrict__ K,
@@ -61,7 +63,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
                                                       float* __restrict__ softmax_sum, int Sq, int Sk,
                                                       int q_block, int head, float scale_log2e,
                                                       const unsigned char* __restrict__ head_mask = nullptr,
-                                                      TL timeline = TL()) {
+                                                      TL timeline = TL(), int tile_lo = 0, int tile_hi = 0x7fffff) {
   typedef AttnElem<T> E;
   typedef typename E::x8 x8_t;
   constexpr bool GUARDED = CAUSAL || RAGGED;  // the last tiles of a block run the guarded copy of the loop
@@ -79,8 +81,21 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   const int li = lane & 31;
   const int g = lane >> 5;
 
+  constexpr int BM = WAVES * 32;
+  const int q0 = q_block * BM;
+  // MASKED: key tiles before tile_lo and after tile_hi are left out; the loop below then walks tiles relative to
+  // tile_lo, keys are counted from `shift` and the sequence ends with tile tile_hi
+  const int all_tiles = (Sk + kAttnBN - 1) / kAttnBN;
+  if constexpr (MASKED) {
+    tile_lo = max(0, min(tile_lo, CAUSAL ? min(q0 / kAttnBN, all_tiles - 1) : all_tiles - 1));
+    tile_hi = max(tile_lo, tile_hi);
+  }
+  const int shift = MASKED ? tile_lo * kAttnBN : 0;
+  const int Sk_end = MASKED ? min(Sk, (tile_hi + 1) * kAttnBN) : Sk;  // first key that is not looked at
+  const int Sk_rel = Sk_end - shift;                                  // keys the loop covers
+
   const size_t head_off = static_cast<size_t>(head) * Sq * kAttnD;
-  const size_t kv_off = static_cast<size_t>(head) * Sk * kAttnD;
+  const size_t kv_off = static_cast<size_t>(head) * Sk * kAttnD + static_cast<size_t>(shift) * kAttnD;
   const T* __restrict__ Qh = Q + head_off;
   const T* __restrict__ Kh = K + kv_off;
   const T* __restrict__ Vh = V + kv_off;
@@ -93,8 +108,6 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   constexpr int NA = 4 * DB;   // chunks (= MFMAs) of phase A
   constexpr int NB = 2 * DS;   // chunks of phase B
   static_assert(sizeof(T) == 2, "16-bit elements");
-  constexpr int BM = WAVES * 32;
-  const int q0 = q_block * BM;
   // Wavefronts 4..7 take the 32-query sub-blocks in reverse order: with a causal mask a sub-block
   // needs 1 + sub / 2 of the four diagonal tiles, and the two wavefronts that share a SIMD
   // (w and w + 4) then have five tiles of diagonal work between them on every SIMD instead of
@@ -123,18 +136,18 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   // the pipeline below is unrolled over pairs of tiles, so an odd count is padded with one tile
   // that lies wholly past the end (zeros from the bounded loads, skipped like a tile above the
   // diagonal).
-  const int real_tiles = RAGGED ? (Sk + kAttnBN - 1) / kAttnBN : Sk / kAttnBN;
-  const int vis_tiles = CAUSAL ? min(real_tiles, (q0 + BM) / kAttnBN) : real_tiles;
+  const int real_tiles = RAGGED ? (Sk_rel + kAttnBN - 1) / kAttnBN : Sk / kAttnBN;
+  const int vis_tiles = CAUSAL ? min(real_tiles, (q0 + BM - shift) / kAttnBN) : real_tiles;
   const int n_tiles = RAGGED ? 2 * ((vis_tiles + 1) / 2) : vis_tiles;
   // first tile that needs the guarded loop: the diagonal, or the tile that holds the end of the keys
-  const int first_masked = CAUSAL ? q0 / kAttnBN : (RAGGED ? Sk / kAttnBN : n_tiles);
+  const int first_masked = CAUSAL ? (q0 - shift) / kAttnBN : (RAGGED ? Sk_rel / kAttnBN : n_tiles);
 
   // direct global -> LDS copies: block b of a tile (rows 4 b .. 4 b + 3) is written by one wavefront
   // instruction, lane l filling LDS chunk l of the block (row 4 b + l / 16, chunk position l % 16)
   // with the global chunk that the swizzle puts there
   const int blk_row = lane >> 4;
   const int blk_pos = lane & 15;
-  const int kv_bytes = RAGGED ? Sk * kAttnD * 2 : 0x7fffffff;  // loads past a head's keys return zeros
+  const int kv_bytes = RAGGED ? Sk_rel * kAttnD * 2 : 0x7fffffff;  // loads past a head's keys return zeros
   auto issue_tile = [&](const T* __restrict__ src, T* dst, int tile, auto swz) {
 #pragma unroll
     for (int u = 0; u < 16 / WAVES; ++u) {
@@ -195,7 +208,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   };
 
   // last key this lane's query may see: itself under a causal mask, the last key there is otherwise
-  const int key_limit = CAUSAL ? (RAGGED ? min(qi_ld, Sk - 1) : qi) : Sk - 1;
+  const int key_limit = (CAUSAL ? (RAGGED ? min(qi_ld, Sk_end - 1) : qi) : Sk_end - 1) - shift;
   auto apply_mask = [&](int tile) {
     const int d = key_limit - (tile * kAttnBN + 4 * g);  // keys with local offset > d are masked
 #pragma unroll
@@ -210,8 +223,8 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   auto mask_fetch = [&](int tile) {
     if constexpr (MASKED) {
       const auto rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(head_mask), 0, Sq * mask_tiles * 8, 0x00020000);
-      mk = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (qi_ld * mask_tiles + min(tile, mask_tiles)) * 8, 0, 0);
-      if (tile >= mask_tiles) mk = u32x2_t{0u, 0u};  // tiles past the end hold no keys (already hidden by the length)
+      mk = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (qi_ld * mask_tiles + min(tile + tile_lo, mask_tiles)) * 8, 0, 0);
+      if (tile + tile_lo >= mask_tiles) mk = u32x2_t{0u, 0u};  // tiles past the end hold no keys (already hidden by the length)
     }
   };
   // hides what the fetched dwords mark in S(tile) and requests the dwords of the next tile
@@ -397,7 +410,7 @@ __device__ __forceinline__ void attention_fwd_d128_v5(const T* __restrict__ Q, c
   using No = std::false_type;
   // last key tile this wavefront's queries can see (only the diagonal tiles differ between wavefronts)
   const int last_tile =
-      CAUSAL ? (RAGGED ? min(min(q0 + sub * 32 + 31, Sq - 1) / kAttnBN, real_tiles - 1) : first_masked + (sub >> 1))
+      CAUSAL ? (RAGGED ? min((min(q0 + sub * 32 + 31, Sq - 1) - shift) / kAttnBN, real_tiles - 1) : first_masked + (sub >> 1))
              : real_tiles - 1;
   if (GUARDED && 0 == last_tile) apply_mask(0);
   mask_apply(0);
@@ -520,7 +533,9 @@ __device__ __forceinline__ void attention_entry_v5(const T* q, const T* k, const
                                                    float* ssum, int n_heads, int Sq, int Sk,
                                                    float scale_log2e, const unsigned char* mask = nullptr,
                                                    long long mask_batch_stride = 0, long long mask_head_stride = 0,
-                                                   int heads_per_batch = 1, TL timeline = TL()) {
+                                                   int heads_per_batch = 1, TL timeline = TL(),
+                                                   const int* tile_ranges = nullptr, int range_batch_stride = 0,
+                                                   int range_head_stride = 0) {
   constexpr int XCDS = 8;
   const int n_qb = (Sq + kAttnV5BM - 1) / kAttnV5BM;
   const int per_head = CAUSAL ? (n_qb + 1) / 2 : n_qb;
@@ -534,6 +549,12 @@ __device__ __forceinline__ void attention_entry_v5(const T* q, const T* k, const
     // the [Sq][tiles] 64-bit mask words of this head (byte strides; 0 where the mask broadcasts over batch or heads)
     const unsigned char* hm =
         MASKED ? mask + (head / heads_per_batch) * mask_batch_stride + (head % heads_per_batch) * mask_head_stride : nullptr;
+    // (first, last) key tile that holds a visible key, per query block: [B or 1][N or 1][query blocks][2]
+    const int* hr = (MASKED && tile_ranges)
+                        ? tile_ranges + (head / heads_per_batch) * range_batch_stride + (head % heads_per_batch) * range_head_stride
+                        : nullptr;
+    auto range_lo = [&](int qb) { return hr ? hr[2 * qb] : 0; };
+    auto range_hi = [&](int qb) { return hr ? hr[2 * qb + 1] : 0x7fffff; };
     if (CAUSAL) {
       const int lo = slot % per_head;
       const int hi = n_qb - 1 - lo;
@@ -541,10 +562,12 @@ __device__ __forceinline__ void attention_entry_v5(const T* q, const T* k, const
 #pragma nounroll
       for (int pass = 0; pass < n_pass; ++pass)
         attention_fwd_d128_v5<T, true, RAGGED, kAttnV5Waves, DH, MASKED, TL>(q, k, v, o, smax, ssum, Sq, Sk, pass == 0 ? hi : lo,
-                                                                             head, scale_log2e, hm, timeline);
+                                                                             head, scale_log2e, hm, timeline,
+                                                                             range_lo(pass == 0 ? hi : lo), range_hi(pass == 0 ? hi : lo));
     } else {
       attention_fwd_d128_v5<T, false, RAGGED, kAttnV5Waves, DH, MASKED, TL>(q, k, v, o, smax, ssum, Sq, Sk, slot % per_head, head,
-                                                                            scale_log2e, hm, timeline);
+                                                                            scale_log2e, hm, timeline, range_lo(slot % per_head),
+                                                                            range_hi(slot % per_head));
     }
   }
 }

@@ -628,7 +628,7 @@ def _attention_masked_launcher() -> CachingLauncher:
     return CachingLauncher(
         "fused_attention_fwd_d128_masked",
         codecache.aot_source("attention_kernels.hip"),
-        "PPPPPPiiifPqqi",
+        "PPPPPPiiifPqqiPii",
         cfgs,
         prefer_intree=True,
     )
@@ -654,9 +654,45 @@ def attention_mask_bits(mask: torch.Tensor, B: int, N: int, Sq: int, Sk: int) ->
     return (groups * weights).sum(-1, dtype=torch.uint8).contiguous()
 
 
+def attention_mask_tile_ranges(packed: torch.Tensor, Sq: int, Sk: int, causal: bool = False,
+                               transposed: bool = False) -> torch.Tensor:
+    """For a packed mask (attention_mask_bits) the key tiles each block of 256 queries has to visit: int32
+    [B or 1, N or 1, ceil(Sq / 256), 2] holding the first and the last 64-key tile in which some query of the
+    block sees a key (under `causal` only tiles up to the block's diagonal count); (0, 0) for a block that sees
+    nothing.  The masked kernels leave the tiles outside the range alone, so a sliding window or a block-sparse
+    mask costs what it shows.  transposed: `packed` is the packing of the transposed mask (rows = keys, tiles of
+    queries, what the dK and dV kernels read), for which `causal` keeps the tiles from the block's diagonal on.
+    Device work only (no host copy)."""
+    tiles = cdiv(Sk, 64)
+    dev = packed.device
+    words = packed.view(torch.int64)  # [b, n, Sq, tiles]
+    # bits a fully hidden tile has set: all 64, in the last tile only those of existing keys
+    full = torch.full((tiles,), -1, dtype=torch.int64, device=dev)
+    if Sk % 64:
+        full[tiles - 1] = (1 << (Sk % 64)) - 1
+    seen = (words & full) != full  # [b, n, Sq, tiles]: the query sees a key of the tile
+    blocks = cdiv(Sq, _ATTN_BLOCK_QUERIES)
+    if blocks * _ATTN_BLOCK_QUERIES != Sq:
+        seen = torch.nn.functional.pad(seen, (0, 0, 0, blocks * _ATTN_BLOCK_QUERIES - Sq))
+    seen = seen.view(seen.shape[0], seen.shape[1], blocks, _ATTN_BLOCK_QUERIES, tiles).any(dim=3)  # [b, n, blocks, tiles]
+    t = torch.arange(tiles, device=dev)
+    if causal and transposed:
+        first_visible = (torch.arange(blocks, device=dev) * _ATTN_BLOCK_QUERIES) // 64
+        seen = seen & (t.view(1, 1, 1, tiles) >= first_visible.view(1, 1, blocks, 1))
+    elif causal:
+        last_visible = (torch.arange(blocks, device=dev) * _ATTN_BLOCK_QUERIES + _ATTN_BLOCK_QUERIES - 1) // 64
+        seen = seen & (t.view(1, 1, 1, tiles) <= last_visible.view(1, 1, blocks, 1))
+    lo = torch.where(seen, t, tiles).amin(dim=-1)
+    hi = torch.where(seen, t, -1).amax(dim=-1)
+    none = hi < 0
+    lo = torch.where(none, 0, lo)
+    hi = torch.where(none, 0, hi)
+    return torch.stack((lo, hi), dim=-1).to(torch.int32).contiguous()
+
+
 def fused_attention(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, causal: bool, data_columns: int = 128,
-    mask: Optional[torch.Tensor] = None, mask_is_packed: bool = False,
+    mask: Optional[torch.Tensor] = None, mask_is_packed: bool = False, tile_ranges: Optional[torch.Tensor] = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """softmax(q k^T * scale [+ causal mask]) v for q [B, N, Sq, 128] and k, v [B, N, Sk, 128], bf16
     or fp16, any positive sequence lengths (a causal mask needs Sq == Sk).
@@ -671,8 +707,9 @@ def fused_attention(
     the kernel skips the matrix work on the zero half and leaves columns 64.. of `out` undefined.
     mask ([Sq, Sk] or broadcastable to [B, N, Sq, Sk], any type, non-zero = the key is hidden from the
     query) is applied besides the causal mask (it is packed to one bit per key first; a caller that uses
-    one mask many times packs it once with attention_mask_bits and passes mask_is_packed=True); a query
-    with every key hidden gets a zero output row, maximum 0 and sum 1."""
+    one mask many times packs it once with attention_mask_bits and passes mask_is_packed=True, best together with
+    tile_ranges=attention_mask_tile_ranges(packed, ...), without which a packed mask visits every key tile); a
+    query with every key hidden gets a zero output row, maximum 0 and sum 1."""
     _check_cuda(q, k, v)
     _require(q.dtype == k.dtype == v.dtype and q.dtype in _ATTN_DTYPES, "q, k, v must share bf16 or fp16")
     _require(q.dim() == 4 and k.dim() == 4 and k.shape == v.shape, "q [B, N, Sq, D]; k and v one [B, N, Sk, D] shape")
@@ -708,12 +745,21 @@ def fused_attention(
                      "a packed mask is what attention_mask_bits returns for these lengths")
         else:
             mb = attention_mask_bits(mask, B, N, Sq, Sk)
+            tile_ranges = attention_mask_tile_ranges(mb, Sq, Sk, causal)
+        if tile_ranges is not None:
+            _check_cuda(tile_ranges)
+            _require(tile_ranges.dtype == torch.int32 and tile_ranges.is_contiguous()
+                     and tuple(tile_ranges.shape) == (mb.shape[0], mb.shape[1], cdiv(Sq, _ATTN_BLOCK_QUERIES), 2),
+                     "tile_ranges is what attention_mask_tile_ranges returns for this packed mask")
+        tr = tile_ranges
         lm = _attention_masked_launcher()
         lm._launch(
             _find(lm, f"fused_attention_fwd_{_ATTN_DTYPES[q.dtype]}_d128_{'causal' if causal else 'full'}_v5_masked"),
             (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), smax.data_ptr(), ssum.data_ptr(), heads, Sq, Sk,
              float(scale) * 1.4426950408889634, mb.data_ptr(), mb.stride(0) if mb.shape[0] > 1 else 0,
-             mb.stride(1) if mb.shape[1] > 1 else 0, N),
+             mb.stride(1) if mb.shape[1] > 1 else 0, N, tr.data_ptr() if tr is not None else 0,
+             (tr.stride(0) if tr.shape[0] > 1 else 0) if tr is not None else 0,
+             (tr.stride(1) if tr.shape[1] > 1 else 0) if tr is not None else 0),
             (grid, 1, 1),
             _stream(),
         )
@@ -769,7 +815,7 @@ def _attention_bwd_masked_launchers() -> dict:
     src = codecache.aot_source("attention_bwd_kernels.hip")
     return {
         which: CachingLauncher(
-            f"attention_bwd8_{which[:2]}_d128_masked", src, "PPPPPPiifPqqi",
+            f"attention_bwd8_{which[:2]}_d128_masked", src, "PPPPPPiifPqqiPii",
             [LaunchConfig(f"attention_bwd8_{which[:2]}_{t}_d128_{c}_masked", 512, meta={"CAUSAL": c == "causal", "MASKED": 1},
                           lds_bytes=lds)
              for t in _ATTN_DTYPES.values() for c in ("causal", "full")],
@@ -782,7 +828,7 @@ def _attention_bwd_masked_launchers() -> dict:
 def fused_attention_backward(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, dout: torch.Tensor,
     softmax_max: torch.Tensor, softmax_sum: torch.Tensor, scale: float, causal: bool, data_columns: int = 128,
-    mask: Optional[torch.Tensor] = None, packed_masks: Optional[tuple] = None,
+    mask: Optional[torch.Tensor] = None, packed_masks: Optional[tuple] = None, tile_ranges: Optional[tuple] = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients (dq, dk, dv) of fused_attention for [B, N, S, 128] bf16 or fp16 tensors; softmax_max /
     softmax_sum are the forward's [B, N, S, 8] fp32 statistics.  Workgroups of eight wavefronts on
@@ -792,7 +838,9 @@ def fused_attention_backward(
     kernels skip the matrix work on the zero half and leave columns 64.. of the gradients undefined.
     mask: the forward's mask ([S, S] or broadcastable to [B, N, S, S], non-zero = hidden); it is packed to
     bits, once as it stands for dQ and once transposed for dK and dV.  packed_masks: those two packings
-    (attention_mask_bits of the mask and of its transpose), for a caller that holds them already."""
+    (attention_mask_bits of the mask and of its transpose), for a caller that holds them already; tile_ranges:
+    attention_mask_tile_ranges of the two (the second with transposed=True), computed here when a mask is
+    given unpacked; without them packed masks visit every tile."""
     _check_cuda(q, k, v, out, dout, softmax_max, softmax_sum)
     for t in (q, k, v, out, dout):
         _require(t.dtype == q.dtype and t.dtype in _ATTN_DTYPES and t.dim() == 4 and t.shape == q.shape,
@@ -836,14 +884,24 @@ def fused_attention_backward(
             m4 = mask.view(1, 1, *mask.shape) if mask.dim() == 2 else mask
             rows = attention_mask_bits(m4, B, N, S, S)                     # [.., query, key tiles]
             cols = attention_mask_bits(m4.transpose(-1, -2), B, N, S, S)   # [.., key, query tiles]
+            tile_ranges = (attention_mask_tile_ranges(rows, S, S, causal),
+                           attention_mask_tile_ranges(cols, S, S, causal, transposed=True))
+        if tile_ranges is not None:
+            for r, w in zip(tile_ranges, (rows, cols)):
+                _check_cuda(r)
+                _require(r.dtype == torch.int32 and r.is_contiguous() and tuple(r.shape) == (w.shape[0], w.shape[1], cdiv(S, 256), 2),
+                         "tile_ranges are what attention_mask_tile_ranges returns for the two packed masks")
+        rr, rc = tile_ranges if tile_ranges is not None else (None, None)
         lm = _attention_bwd_masked_launchers()
-        for name, dst, words in (("dk8", dk, cols), ("dv8", dv, cols), ("dq8", dq, rows)):
+        for name, dst, words, tr in (("dk8", dk, cols, rc), ("dv8", dv, cols, rc), ("dq8", dq, rows, rr)):
             l = lm[name]
             l._launch(
                 _find(l, f"attention_bwd8_{name[:2]}_{ty}_d128_{which}_masked"),
                 (q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), stats.data_ptr(), dst.data_ptr(), heads, S,
                  float(scale), words.data_ptr(), words.stride(0) if words.shape[0] > 1 else 0,
-                 words.stride(1) if words.shape[1] > 1 else 0, N),
+                 words.stride(1) if words.shape[1] > 1 else 0, N, tr.data_ptr() if tr is not None else 0,
+                 (tr.stride(0) if tr.shape[0] > 1 else 0) if tr is not None else 0,
+                 (tr.stride(1) if tr.shape[1] > 1 else 0) if tr is not None else 0),
                 grid, st,
             )
         return dq, dk, dv

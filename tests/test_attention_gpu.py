@@ -873,3 +873,103 @@ def test_attention_op_sliding_window_launches_the_masked_kernels():
         names, L.launch_log = L.launch_log, None
     assert "fused_attention_fwd_bf16_d128_full_v5_masked" in names, names
     assert {f"attention_bwd8_{w}_bf16_d128_full_masked" for w in ("dq", "dk", "dv")} <= set(names), names
+
+
+@pytest.mark.parametrize("dtype,B,N,S,causal,kind", [
+    (torch.bfloat16, 2, 3, 1024, False, "window"),     # keys i-200 .. i+100
+    (torch.bfloat16, 1, 4, 1280, True, "window"),      # causal and the last 300 keys only
+    (torch.float16, 2, 2, 777, False, "blocks"),       # block-diagonal (documents packed into one sequence), ragged length
+    (torch.bfloat16, 1, 2, 512, False, "nothing"),     # one block of queries sees no key at all
+])
+def test_attention_mask_tile_ranges(K, dtype, B, N, S, causal, kind):
+    """The masked kernel visits, per block of 256 queries, only the key tiles between the first and the last one in
+    which a query of the block sees a key (kernels.attention_mask_tile_ranges): the result is bit-identical to the
+    same launch over all tiles and matches the fp32 definition."""
+    announce(f"attention mask tile ranges {dtype} [{B},{N},{S},128] causal={causal} {kind}")
+    torch.manual_seed(23)
+    q, k, v = (torch.randn(B, N, S, 128, device=DEV).to(dtype) for _ in range(3))
+    i = torch.arange(S, device=DEV).view(S, 1)
+    j = torch.arange(S, device=DEV).view(1, S)
+    if kind == "window":
+        hide = (j > i + (0 if causal else 100)) | (j < i - (299 if causal else 200))
+    elif kind == "blocks":
+        doc = torch.tensor([0, 130, 400, 401, 700, S], device=DEV)
+        seg = torch.bucketize(torch.arange(S, device=DEV), doc[1:], right=True)
+        hide = seg.view(S, 1) != seg.view(1, S)
+    else:
+        hide = torch.zeros(S, S, device=DEV, dtype=torch.bool)
+        hide[256:512, :] = True
+        hide[:256, 300:] = True
+    hide = hide.view(1, 1, S, S).expand(B if kind == "blocks" else 1, 1, S, S).contiguous()
+    packed = K.attention_mask_bits(hide, B, N, S, S)
+    ranges = K.attention_mask_tile_ranges(packed, S, S, causal)
+    assert ranges.shape == (packed.shape[0], 1, -(-S // 256), 2) and ranges.dtype == torch.int32
+    lo, hi = ranges[..., 0], ranges[..., 1]
+    assert (lo >= 0).all() and (hi >= lo).all() and (hi < -(-S // 64)).all()
+    if kind == "window":
+        assert (hi - lo).max().item() <= (256 + 300) // 64 + 2  # a band: a few tiles per block, not all of them
+    scale = 128 ** -0.5
+    got = K.fused_attention(q, k, v, scale, causal, mask=packed, mask_is_packed=True, tile_ranges=ranges)
+    every = K.fused_attention(q, k, v, scale, causal, mask=packed, mask_is_packed=True)
+    for a, b in zip(got, every):
+        assert torch.equal(a, b)
+    auto = K.fused_attention(q, k, v, scale, causal, mask=hide)
+    assert torch.equal(auto[0], got[0])
+    full_hide = hide | (torch.ones(S, S, device=DEV, dtype=torch.bool).triu(1) if causal else False)
+    s = (q.float() @ k.float().transpose(-1, -2)) * scale
+    s = s.masked_fill(full_hide, float("-inf"))
+    gone = full_hide.expand(B, N, S, S).all(-1, keepdim=True)
+    p = torch.softmax(s.masked_fill(gone, 0.0), -1).masked_fill(gone, 0.0)
+    want = p @ v.float()
+    assert (got[0].float() - want).abs().max().item() <= 2e-2
+    assert torch.isfinite(got[1]).all() and torch.isfinite(got[2]).all()
+
+
+@pytest.mark.parametrize("dtype,B,N,S,causal,kind", [
+    (torch.bfloat16, 2, 2, 1024, False, "window"),
+    (torch.bfloat16, 1, 3, 1280, True, "window"),
+    (torch.float16, 1, 2, 768, False, "blocks"),
+    (torch.bfloat16, 1, 2, 512, False, "nothing"),
+])
+def test_attention_backward_mask_tile_ranges(K, dtype, B, N, S, causal, kind):
+    """The masked gradient kernels with tile ranges (dQ: key tiles per block of queries from the mask, dK / dV:
+    query tiles per block of keys from its transpose) give bit-identical gradients to the same kernels over all
+    tiles, and match autograd on the fp32 definition."""
+    announce(f"attention backward mask tile ranges {dtype} [{B},{N},{S},128] causal={causal} {kind}")
+    torch.manual_seed(29)
+    q, k, v, go = (torch.randn(B, N, S, 128, device=DEV).to(dtype) for _ in range(4))
+    i = torch.arange(S, device=DEV).view(S, 1)
+    j = torch.arange(S, device=DEV).view(1, S)
+    if kind == "window":
+        hide = (j > i + (0 if causal else 100)) | (j < i - (299 if causal else 200))
+    elif kind == "blocks":
+        doc = torch.tensor([0, 130, 400, 401, 700, S], device=DEV)
+        seg = torch.bucketize(torch.arange(S, device=DEV), doc[1:], right=True)
+        hide = seg.view(S, 1) != seg.view(1, S)
+    else:
+        hide = torch.zeros(S, S, device=DEV, dtype=torch.bool)
+        hide[256:512, :] = True
+        hide[:256, 300:] = True
+    hide = hide.view(1, 1, S, S).contiguous()
+    scale = 128 ** -0.5
+    out, smax, ssum = K.fused_attention(q, k, v, scale, causal, mask=hide)
+    rows = K.attention_mask_bits(hide, B, N, S, S)
+    cols = K.attention_mask_bits(hide.transpose(-1, -2), B, N, S, S)
+    ranges = (K.attention_mask_tile_ranges(rows, S, S, causal), K.attention_mask_tile_ranges(cols, S, S, causal, transposed=True))
+    got = K.fused_attention_backward(q, k, v, out, go, smax, ssum, scale, causal, packed_masks=(rows, cols), tile_ranges=ranges)
+    every = K.fused_attention_backward(q, k, v, out, go, smax, ssum, scale, causal, packed_masks=(rows, cols))
+    for a, b in zip(got, every):
+        assert torch.equal(a, b)
+    auto = K.fused_attention_backward(q, k, v, out, go, smax, ssum, scale, causal, mask=hide)
+    for a, b in zip(got, auto):
+        assert torch.equal(a, b)
+    full_hide = hide | (torch.ones(S, S, device=DEV, dtype=torch.bool).triu(1) if causal else False)
+    qf, kf, vf = (t.float().requires_grad_() for t in (q, k, v))
+    s = (qf @ kf.transpose(-1, -2)) * scale
+    s = s.masked_fill(full_hide, float("-inf"))
+    gone = full_hide.expand(B, N, S, S).all(-1, keepdim=True)
+    p = torch.softmax(s.masked_fill(gone, 0.0), -1).masked_fill(gone, 0.0)
+    (p @ vf).backward(go.float())
+    for g, r in zip(got, (qf.grad, kf.grad, vf.grad)):
+        assert torch.isfinite(g).all()
+        assert (g.float() - r).abs().max().item() <= 3e-2 * max(r.abs().max().item(), 1.0)
